@@ -1,0 +1,252 @@
+/*
+ * thrust_amd.h -- C ABI of the MI355X (gfx950) device system for the Thrust API.
+ *
+ * Every compute entry point follows the two-phase temporary-storage protocol the
+ * reference's CUDA device system uses for its `doit_step` functions
+ * (thrust/system/cuda/detail/reduce.h:689-848, sort.h:1149-1269, copy_if.h:602-690,
+ * merge.h:676-782):
+ *
+ *   size_t bytes = 0;
+ *   fn(NULL, &bytes, ...);          // size query: writes the bytes needed, launches nothing
+ *   fn(temp, &bytes, ...);          // run: enqueues kernels on `stream` and returns
+ *
+ * Rules that hold for all of them:
+ *   - The caller owns every buffer.  Entry points never allocate, free or synchronise.
+ *   - All data pointers are DEVICE pointers unless a parameter is documented as a host
+ *     pointer (`init`, `threshold`: one scalar of the stated dtype, read during the call).
+ *   - Scalar results (`d_out`, `d_num_*`) are written to caller-supplied device memory;
+ *     the caller copies them to the host after synchronising the stream.
+ *   - `stream` is a hipStream_t passed as void* (NULL = the default stream).
+ *   - The return value is a hipError_t as int; 0 means success.  No exception crosses
+ *     the boundary and nothing aborts.
+ *   - n == 0 is legal everywhere.
+ *   - Calls are re-entrant and thread-safe as long as they use distinct temp buffers.
+ *   - `temp` must be 256-byte aligned (anything from hipMalloc / thrust_amd_malloc is).
+ */
+#ifndef THRUST_AMD_H
+#define THRUST_AMD_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define THRUST_AMD_VERSION 100 /* major*100 + minor */
+
+/* Element types understood across the boundary. */
+typedef enum thrust_amd_dtype {
+  THRUST_AMD_I8 = 0,
+  THRUST_AMD_U8 = 1,
+  THRUST_AMD_I16 = 2,
+  THRUST_AMD_U16 = 3,
+  THRUST_AMD_I32 = 4,
+  THRUST_AMD_U32 = 5,
+  THRUST_AMD_I64 = 6,
+  THRUST_AMD_U64 = 7,
+  THRUST_AMD_F32 = 8,
+  THRUST_AMD_F64 = 9,
+  THRUST_AMD_DTYPE_COUNT = 10
+} thrust_amd_dtype;
+
+/* Binary operators: the closed set the front end maps thrust::plus / minimum / maximum
+ * (and their <void> forms) to.  Integer PLUS wraps modulo 2^bits, which is what the
+ * reference's accumulator does (thrust/system/detail/generic/reduce.inl:40-53). */
+typedef enum thrust_amd_binop {
+  THRUST_AMD_PLUS = 0,
+  THRUST_AMD_MIN = 1,
+  THRUST_AMD_MAX = 2,
+  THRUST_AMD_BINOP_COUNT = 3
+} thrust_amd_binop;
+
+/* Unary predicates `x CMP threshold` (threshold has the dtype of the tested array).
+ * NONZERO is the reference's default "stencil element converted to bool". */
+typedef enum thrust_amd_cmp {
+  THRUST_AMD_LT = 0,
+  THRUST_AMD_LE = 1,
+  THRUST_AMD_GT = 2,
+  THRUST_AMD_GE = 3,
+  THRUST_AMD_EQ = 4,
+  THRUST_AMD_NE = 5,
+  THRUST_AMD_NONZERO = 6,
+  THRUST_AMD_CMP_COUNT = 7
+} thrust_amd_cmp;
+
+typedef enum thrust_amd_memcpy_kind {
+  THRUST_AMD_H2D = 1,
+  THRUST_AMD_D2H = 2,
+  THRUST_AMD_D2D = 3
+} thrust_amd_memcpy_kind;
+
+/* ------------------------------------------------------------------ library */
+
+/* Library version (THRUST_AMD_VERSION of the build). */
+int thrust_amd_version(void);
+
+/* Static, NUL-terminated description of a status code returned by any entry point.
+ * Replaces thrust::system::cuda_category().message() (thrust/system/cuda/detail/error.inl). */
+const char* thrust_amd_error_string(int status);
+
+/* Size in bytes of one element of `dtype`, 0 for an unknown code. */
+size_t thrust_amd_dtype_size(int dtype);
+
+/* ------------------------------------------------------------- memory model */
+
+/* Device allocation / release.  Replace cuda_cub::malloc / cuda_cub::free
+ * (thrust/system/cuda/detail/malloc_and_free.h:51-100).  bytes == 0 yields *ptr = NULL. */
+int thrust_amd_malloc(void** ptr, size_t bytes);
+int thrust_amd_free(void* ptr);
+
+/* Copy between host and device or device and device, ordered on `stream`; the H2D/D2H
+ * forms return after the copy has completed (pageable host memory), the D2D form is
+ * asynchronous.  Replaces cuda_cub::trivial_copy_{to,from}_device / trivial_copy_device_to_device
+ * (thrust/system/cuda/detail/util.h:107-162) behind copy_cross_system.h:50-200. */
+int thrust_amd_memcpy(void* dst, const void* src, size_t bytes, int kind, void* stream);
+
+/* Block until all work enqueued on `stream` has finished.  Replaces
+ * cuda_cub::synchronize (thrust/system/cuda/detail/util.h:75-104). */
+int thrust_amd_stream_synchronize(void* stream);
+
+/* Fill n elements of `elem_bytes` (1, 2, 4 or 8) with the host value *value.  Replaces
+ * cuda_cub::fill_n (thrust/system/cuda/detail/fill.h) as used by
+ * device_vector(n, value) (thrust/detail/vector_base.inl:214-234). */
+int thrust_amd_fill(void* dst, uint64_t n, size_t elem_bytes, const void* value, void* stream);
+
+/* Temporary-storage arena: a size-bucketed cache of device blocks, so that the blocking
+ * thrust:: front end performs no hipMalloc in steady state.  `acquire` returns a block
+ * of at least `bytes`, 256-byte aligned; `release` returns it to the cache once the
+ * work enqueued so far on `stream` may be assumed ordered before its next use (blocks
+ * are reused in stream order on the stream they were released on; a block released on
+ * one stream is handed to another stream only after that stream was synchronised).
+ * `trim` frees every cached block.  Replaces temporary_array<uint8_t,Derived> over
+ * get_temporary_buffer (thrust/detail/temporary_array.inl:62-140,
+ * thrust/system/detail/generic/temporary_buffer.inl:33-47). */
+int thrust_amd_temp_acquire(void** ptr, size_t bytes, void* stream);
+int thrust_amd_temp_release(void* ptr, void* stream);
+int thrust_amd_temp_trim(void);
+/* Bytes currently held by the arena (cached + handed out). */
+size_t thrust_amd_temp_bytes_held(void);
+
+/* ------------------------------------------------------------------- reduce */
+
+/* *d_out = init OP in[0] OP ... OP in[n-1]; accumulator type = dtype.
+ * `init` is a host pointer to one dtype element.  d_out: one dtype element on device.
+ * Replaces cuda_cub::detail::reduce_n_impl -> cub::DispatchReduce::Dispatch
+ * (thrust/system/cuda/detail/reduce.h:927-1000). */
+int thrust_amd_reduce(void* temp, size_t* temp_bytes, const void* in, uint64_t n, int dtype,
+                      int op, const void* init, void* d_out, void* stream);
+
+/* --------------------------------------------------------------------- scan */
+
+/* out[i] = in[0] OP ... OP in[i]; accumulator type = dtype; out == in allowed.
+ * Replaces cuda_cub::inclusive_scan_n -> cub::DispatchScan
+ * (thrust/system/cuda/detail/scan.h:55-122). */
+int thrust_amd_inclusive_scan(void* temp, size_t* temp_bytes, const void* in, void* out,
+                              uint64_t n, int dtype, int op, void* stream);
+
+/* out[0] = init, out[i] = init OP in[0] OP ... OP in[i-1]; out == in allowed.
+ * `init` is a host pointer to one dtype element.
+ * Replaces cuda_cub::exclusive_scan_n (thrust/system/cuda/detail/scan.h:132-200). */
+int thrust_amd_exclusive_scan(void* temp, size_t* temp_bytes, const void* in, void* out,
+                              uint64_t n, int dtype, int op, const void* init, void* stream);
+
+/* --------------------------------------------------------------------- sort */
+
+/* Stable in-place sort of n keys by the total order of their radix encoding:
+ * unsigned = value, signed = sign bit flipped, float = IEEE bits ^ (-(bits>>31) | signbit)
+ * (-0.0 before +0.0, NaNs by bit pattern), the reference's encoders
+ * (thrust/system/detail/sequential/stable_radix_sort.inl:41-138).  Only key bits
+ * [begin_bit, end_bit) take part (0 and 8*sizeof(key) sort fully).  descending != 0
+ * yields the order thrust::greater<Key> gives, still stable.
+ * Replaces cuda_cub::__radix_sort::dispatch -> cub::DeviceRadixSort::SortKeys[Descending]
+ * (thrust/system/cuda/detail/sort.h:1326-1429,1438-1508). */
+int thrust_amd_sort_keys(void* temp, size_t* temp_bytes, void* keys, uint64_t n, int key_dtype,
+                         int descending, int begin_bit, int end_bit, void* stream);
+
+/* Same for key-value pairs; values are opaque items of value_bytes (1, 2, 4 or 8) that
+ * travel with their key.  Replaces cub::DeviceRadixSort::SortPairs[Descending]
+ * (thrust/system/cuda/detail/sort.h:1383-1427). */
+int thrust_amd_sort_pairs(void* temp, size_t* temp_bytes, void* keys, void* values, uint64_t n,
+                          int key_dtype, size_t value_bytes, int descending, int begin_bit,
+                          int end_bit, void* stream);
+
+/* ----------------------------------------------------- selection / partition */
+
+/* Stable compaction: copies in[i] (items of item_bytes = 1, 2, 4 or 8) to out, in order,
+ * for every i whose tested element satisfies `tested CMP *threshold`; the tested
+ * element is stencil[i] (dtype stencil_dtype) or, when stencil == NULL, in[i] itself
+ * (then stencil_dtype is the dtype of `in`).  *d_num_selected (uint64 on device)
+ * receives the count.  out may alias in.
+ * Replaces cuda_cub::__copy_if::copy_if (thrust/system/cuda/detail/copy_if.h:699-773). */
+int thrust_amd_copy_if(void* temp, size_t* temp_bytes, const void* in, const void* stencil,
+                       void* out, uint64_t* d_num_selected, uint64_t n, size_t item_bytes,
+                       int stencil_dtype, int cmp, const void* threshold, void* stream);
+
+/* Stable two-way split: selected items go to out_true, the others to out_false, both
+ * in their original order; *d_num_true (uint64 on device) receives the number selected.
+ * out_true may alias in.
+ * Replaces cuda_cub::__partition::partition with two outputs
+ * (thrust/system/cuda/detail/partition.h:612-795, stable_partition_copy :925-1010). */
+int thrust_amd_partition_copy(void* temp, size_t* temp_bytes, const void* in,
+                              const void* stencil, void* out_true, void* out_false,
+                              uint64_t* d_num_true, uint64_t n, size_t item_bytes,
+                              int stencil_dtype, int cmp, const void* threshold, void* stream);
+
+/* In-place stable partition of `data`: selected items first, then the rest, each group
+ * in its original order; *d_num_true receives the split point.
+ * Replaces cuda_cub::__partition::partition_inplace + the trailing reverse
+ * (thrust/system/cuda/detail/partition.h:796-824,1068-1120). */
+int thrust_amd_stable_partition(void* temp, size_t* temp_bytes, void* data, const void* stencil,
+                                uint64_t* d_num_true, uint64_t n, size_t item_bytes,
+                                int stencil_dtype, int cmp, const void* threshold, void* stream);
+
+/* Keeps the first element of every run of equal consecutive elements
+ * (run boundary at i where in[i-1] != in[i]; element 0 always kept).  Floating-point
+ * keys compare with ==, as thrust::equal_to does.  out may alias in.
+ * Replaces cuda_cub::__unique::unique (thrust/system/cuda/detail/unique.h:635-700). */
+int thrust_amd_unique(void* temp, size_t* temp_bytes, const void* in, void* out,
+                      uint64_t* d_num_out, uint64_t n, int dtype, void* stream);
+
+/* Same on keys, carrying the FIRST value of each run along; values are opaque items of
+ * value_bytes (1, 2, 4 or 8).  keys_out / values_out may alias the inputs.
+ * Replaces cuda_cub::__unique_by_key::unique_by_key
+ * (thrust/system/cuda/detail/unique_by_key.h:732-800). */
+int thrust_amd_unique_by_key(void* temp, size_t* temp_bytes, const void* keys_in,
+                             const void* values_in, void* keys_out, void* values_out,
+                             uint64_t* d_num_out, uint64_t n, int key_dtype, size_t value_bytes,
+                             void* stream);
+
+/* For every run of equal consecutive keys writes the run's first key and the OP-fold of
+ * its values (accumulator = value_dtype; floating-point sums use a tree order inside a
+ * run, so they agree with a left fold to rounding only).  *d_num_runs receives the
+ * number of runs.  Outputs must not alias inputs.
+ * Replaces cuda_cub::__reduce_by_key::reduce_by_key
+ * (thrust/system/cuda/detail/reduce_by_key.h:974-1055). */
+int thrust_amd_reduce_by_key(void* temp, size_t* temp_bytes, const void* keys_in,
+                             const void* values_in, void* keys_out, void* values_out,
+                             uint64_t* d_num_runs, uint64_t n, int key_dtype, int value_dtype,
+                             int op, void* stream);
+
+/* -------------------------------------------------------------------- merge */
+
+/* Stable merge of two ranges sorted in the radix-encoding order of dtype (ascending, or
+ * descending when descending != 0) into out (na + nb elements).  Ties: every equal
+ * element of `a` precedes those of `b`
+ * (thrust/system/detail/sequential/merge.inl:56-65).  out must not alias a or b.
+ * Replaces cuda_cub::__merge::merge keys-only (thrust/system/cuda/detail/merge.h:785-853). */
+int thrust_amd_merge(void* temp, size_t* temp_bytes, const void* a, uint64_t na, const void* b,
+                     uint64_t nb, void* out, int dtype, int descending, void* stream);
+
+/* Same with values (opaque items of value_bytes = 1, 2, 4 or 8) travelling with the keys.
+ * Replaces cuda_cub::__merge::merge with items (thrust/system/cuda/detail/merge.h:785-853,
+ * merge_by_key :930-1010). */
+int thrust_amd_merge_by_key(void* temp, size_t* temp_bytes, const void* keys_a, uint64_t na,
+                            const void* keys_b, uint64_t nb, const void* values_a,
+                            const void* values_b, void* keys_out, void* values_out,
+                            int key_dtype, size_t value_bytes, int descending, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* THRUST_AMD_H */

@@ -1,0 +1,298 @@
+// TEST INFRASTRUCTURE -- NOT PART OF THE PRODUCT.
+//
+// C bindings around the REAL reference (the Thrust headers under the reference tree),
+// compiled twice by oracle/Makefile: once with the OpenMP device system and once with
+// the sequential CPP device system.  This file contains no algorithm; it only
+// instantiates the reference's templates and gives them the same host-pointer C
+// interface as thrust_oracle.c, so that tests can compare the restatement with the
+// real thing and write golden vectors, and the benchmark can time the reference's
+// OMP path as CPU baseline.  Built only into oracle/_ref/, which is not committed.
+#include <thrust/copy.h>
+#include <thrust/device_ptr.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/merge.h>
+#include <thrust/partition.h>
+#include <thrust/reduce.h>
+#include <thrust/scan.h>
+#include <thrust/sort.h>
+#include <thrust/unique.h>
+
+#include <cstdint>
+#include <cstring>
+
+#include "../include/thrust_amd.h"
+
+#define REF_API extern "C" __attribute__((visibility("default")))
+
+namespace {
+
+template <typename T> thrust::device_ptr<T> dp(void* p) { return thrust::device_pointer_cast((T*)p); }
+template <typename T> thrust::device_ptr<const T> dp(const void* p) { return thrust::device_pointer_cast((const T*)p); }
+
+template <typename F>
+int with_dtype(int dtype, F&& f) {
+  switch (dtype) {
+    case THRUST_AMD_I8: return f((int8_t)0);
+    case THRUST_AMD_U8: return f((uint8_t)0);
+    case THRUST_AMD_I16: return f((int16_t)0);
+    case THRUST_AMD_U16: return f((uint16_t)0);
+    case THRUST_AMD_I32: return f((int32_t)0);
+    case THRUST_AMD_U32: return f((uint32_t)0);
+    case THRUST_AMD_I64: return f((int64_t)0);
+    case THRUST_AMD_U64: return f((uint64_t)0);
+    case THRUST_AMD_F32: return f((float)0);
+    case THRUST_AMD_F64: return f((double)0);
+    default: return -1;
+  }
+}
+
+template <typename F>
+int with_bytes(uint64_t bytes, F&& f) {
+  switch (bytes) {
+    case 1: return f((uint8_t)0);
+    case 2: return f((uint16_t)0);
+    case 4: return f((uint32_t)0);
+    case 8: return f((uint64_t)0);
+    default: return -1;
+  }
+}
+
+template <typename T, typename F>
+int with_op(int op, F&& f) {
+  switch (op) {
+    case THRUST_AMD_PLUS: return f(thrust::plus<T>());
+    case THRUST_AMD_MIN: return f(thrust::minimum<T>());
+    case THRUST_AMD_MAX: return f(thrust::maximum<T>());
+    default: return -1;
+  }
+}
+
+template <typename T>
+struct cmp_pred {
+  int cmp;
+  T t;
+  __host__ __device__ bool operator()(const T& x) const {
+    switch (cmp) {
+      case THRUST_AMD_LT: return x < t;
+      case THRUST_AMD_LE: return x <= t;
+      case THRUST_AMD_GT: return x > t;
+      case THRUST_AMD_GE: return x >= t;
+      case THRUST_AMD_EQ: return x == t;
+      case THRUST_AMD_NE: return x != t;
+      default: return x != T(0);
+    }
+  }
+};
+
+template <typename T>
+cmp_pred<T> make_pred(int cmp, const void* thr) {
+  cmp_pred<T> p;
+  p.cmp = cmp;
+  p.t = thr ? *(const T*)thr : T(0);
+  return p;
+}
+
+}  // namespace
+
+// 1 = OMP device system, 0 = CPP
+REF_API int ref_is_omp(void) { return THRUST_DEVICE_SYSTEM == THRUST_DEVICE_SYSTEM_OMP; }
+
+REF_API int ref_reduce(const void* in, uint64_t n, int dtype, int op, const void* init, void* out) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    return with_op<T>(op, [&](auto o) {
+      *(T*)out = thrust::reduce(thrust::device, dp<T>(in), dp<T>(in) + n, *(const T*)init, o);
+      return 0;
+    });
+  });
+}
+
+REF_API int ref_inclusive_scan(const void* in, void* out, uint64_t n, int dtype, int op) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    return with_op<T>(op, [&](auto o) {
+      thrust::inclusive_scan(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), o);
+      return 0;
+    });
+  });
+}
+
+REF_API int ref_exclusive_scan(const void* in, void* out, uint64_t n, int dtype, int op,
+                               const void* init) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    return with_op<T>(op, [&](auto o) {
+      thrust::exclusive_scan(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), *(const T*)init, o);
+      return 0;
+    });
+  });
+}
+
+REF_API int ref_sort_keys(void* keys, uint64_t n, int dtype, int descending) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    if (descending) thrust::sort(thrust::device, dp<T>(keys), dp<T>(keys) + n, thrust::greater<T>());
+    else thrust::sort(thrust::device, dp<T>(keys), dp<T>(keys) + n);
+    return 0;
+  });
+}
+
+REF_API int ref_sort_pairs(void* keys, void* values, uint64_t n, int dtype, uint64_t value_bytes,
+                           int descending) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    return with_bytes(value_bytes, [&](auto vz) {
+      using V = decltype(vz);
+      if (descending)
+        thrust::stable_sort_by_key(thrust::device, dp<T>(keys), dp<T>(keys) + n, dp<V>(values), thrust::greater<T>());
+      else
+        thrust::stable_sort_by_key(thrust::device, dp<T>(keys), dp<T>(keys) + n, dp<V>(values));
+      return 0;
+    });
+  });
+}
+
+REF_API int ref_merge(const void* a, uint64_t na, const void* b, uint64_t nb, void* out, int dtype,
+                      int descending) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    if (descending)
+      thrust::merge(thrust::device, dp<T>(a), dp<T>(a) + na, dp<T>(b), dp<T>(b) + nb, dp<T>(out), thrust::greater<T>());
+    else
+      thrust::merge(thrust::device, dp<T>(a), dp<T>(a) + na, dp<T>(b), dp<T>(b) + nb, dp<T>(out));
+    return 0;
+  });
+}
+
+REF_API int ref_merge_by_key(const void* ka, uint64_t na, const void* kb, uint64_t nb,
+                             const void* va, const void* vb, void* kout, void* vout, int dtype,
+                             uint64_t value_bytes, int descending) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    return with_bytes(value_bytes, [&](auto vz) {
+      using V = decltype(vz);
+      if (descending)
+        thrust::merge_by_key(thrust::device, dp<T>(ka), dp<T>(ka) + na, dp<T>(kb), dp<T>(kb) + nb,
+                             dp<V>(va), dp<V>(vb), dp<T>(kout), dp<V>(vout), thrust::greater<T>());
+      else
+        thrust::merge_by_key(thrust::device, dp<T>(ka), dp<T>(ka) + na, dp<T>(kb), dp<T>(kb) + nb,
+                             dp<V>(va), dp<V>(vb), dp<T>(kout), dp<V>(vout));
+      return 0;
+    });
+  });
+}
+
+REF_API int ref_copy_if(const void* in, const void* stencil, void* out, uint64_t* num, uint64_t n,
+                        uint64_t item_bytes, int stencil_dtype, int cmp, const void* threshold) {
+  return with_dtype(stencil_dtype, [&](auto z) {
+    using T = decltype(z);
+    const cmp_pred<T> pred = make_pred<T>(cmp, threshold);
+    if (!stencil) {
+      *num = thrust::copy_if(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), pred) - dp<T>(out);
+      return 0;
+    }
+    return with_bytes(item_bytes, [&](auto vz) {
+      using V = decltype(vz);
+      *num = thrust::copy_if(thrust::device, dp<V>(in), dp<V>(in) + n, dp<T>(stencil), dp<V>(out), pred) - dp<V>(out);
+      return 0;
+    });
+  });
+}
+
+REF_API int ref_partition_copy(const void* in, const void* stencil, void* out_true, void* out_false,
+                               uint64_t* num_true, uint64_t n, uint64_t item_bytes,
+                               int stencil_dtype, int cmp, const void* threshold) {
+  return with_dtype(stencil_dtype, [&](auto z) {
+    using T = decltype(z);
+    const cmp_pred<T> pred = make_pred<T>(cmp, threshold);
+    if (!stencil) {
+      *num_true = thrust::stable_partition_copy(thrust::device, dp<T>(in), dp<T>(in) + n,
+                                                dp<T>(out_true), dp<T>(out_false), pred).first - dp<T>(out_true);
+      return 0;
+    }
+    return with_bytes(item_bytes, [&](auto vz) {
+      using V = decltype(vz);
+      *num_true = thrust::stable_partition_copy(thrust::device, dp<V>(in), dp<V>(in) + n, dp<T>(stencil),
+                                                dp<V>(out_true), dp<V>(out_false), pred).first - dp<V>(out_true);
+      return 0;
+    });
+  });
+}
+
+REF_API int ref_stable_partition(void* data, const void* stencil, uint64_t* num_true, uint64_t n,
+                                 uint64_t item_bytes, int stencil_dtype, int cmp,
+                                 const void* threshold) {
+  return with_dtype(stencil_dtype, [&](auto z) {
+    using T = decltype(z);
+    const cmp_pred<T> pred = make_pred<T>(cmp, threshold);
+    if (!stencil) {
+      *num_true = thrust::stable_partition(thrust::device, dp<T>(data), dp<T>(data) + n, pred) - dp<T>(data);
+      return 0;
+    }
+    return with_bytes(item_bytes, [&](auto vz) {
+      using V = decltype(vz);
+      *num_true = thrust::stable_partition(thrust::device, dp<V>(data), dp<V>(data) + n, dp<T>(stencil), pred) - dp<V>(data);
+      return 0;
+    });
+  });
+}
+
+REF_API int ref_unique(const void* in, void* out, uint64_t* num, uint64_t n, int dtype) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    if (in == out) *num = thrust::unique(thrust::device, dp<T>(out), dp<T>(out) + n) - dp<T>(out);
+    else *num = thrust::unique_copy(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out)) - dp<T>(out);
+    return 0;
+  });
+}
+
+REF_API int ref_unique_by_key(const void* keys_in, const void* values_in, void* keys_out,
+                              void* values_out, uint64_t* num, uint64_t n, int key_dtype,
+                              uint64_t value_bytes) {
+  return with_dtype(key_dtype, [&](auto z) {
+    using T = decltype(z);
+    return with_bytes(value_bytes, [&](auto vz) {
+      using V = decltype(vz);
+      if (keys_in == keys_out)
+        *num = thrust::unique_by_key(thrust::device, dp<T>(keys_out), dp<T>(keys_out) + n, dp<V>(values_out)).first - dp<T>(keys_out);
+      else
+        *num = thrust::unique_by_key_copy(thrust::device, dp<T>(keys_in), dp<T>(keys_in) + n, dp<V>(values_in),
+                                          dp<T>(keys_out), dp<V>(values_out)).first - dp<T>(keys_out);
+      return 0;
+    });
+  });
+}
+
+// Value types are limited to the ones the library's tests and configs use, to keep the
+// compile time of the reference's zip-iterator scan in bounds.
+REF_API int ref_reduce_by_key(const void* keys_in, const void* values_in, void* keys_out,
+                              void* values_out, uint64_t* num_runs, uint64_t n, int key_dtype,
+                              int value_dtype, int op) {
+  auto run = [&](auto kz, auto vz) {
+    using K = decltype(kz);
+    using V = decltype(vz);
+    return with_op<V>(op, [&](auto o) {
+      *num_runs = thrust::reduce_by_key(thrust::device, dp<K>(keys_in), dp<K>(keys_in) + n, dp<V>(values_in),
+                                        dp<K>(keys_out), dp<V>(values_out), thrust::equal_to<K>(), o).first - dp<K>(keys_out);
+      return 0;
+    });
+  };
+  auto by_value = [&](auto kz) {
+    switch (value_dtype) {
+      case THRUST_AMD_I32: return run(kz, (int32_t)0);
+      case THRUST_AMD_I64: return run(kz, (int64_t)0);
+      case THRUST_AMD_F32: return run(kz, (float)0);
+      case THRUST_AMD_F64: return run(kz, (double)0);
+      default: return -1;
+    }
+  };
+  switch (key_dtype) {
+    case THRUST_AMD_I32: return by_value((int32_t)0);
+    case THRUST_AMD_U32: return by_value((uint32_t)0);
+    case THRUST_AMD_I64: return by_value((int64_t)0);
+    case THRUST_AMD_U64: return by_value((uint64_t)0);
+    case THRUST_AMD_F32: return by_value((float)0);
+    default: return -1;
+  }
+}

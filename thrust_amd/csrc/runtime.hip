@@ -1,0 +1,238 @@
+// Memory model and plumbing of the device system: allocation, copies, synchronisation,
+// fill, and the temporary-storage arena.  These are the only entry points that
+// allocate or block; every compute entry point works on caller-owned memory.
+#include "common.hpp"
+#include "dispatch.hpp"
+
+#include <map>
+#include <mutex>
+#include <vector>
+
+TA_EXPORT int thrust_amd_version(void) { return THRUST_AMD_VERSION; }
+
+TA_EXPORT const char* thrust_amd_error_string(int status) {
+  return hipGetErrorString((hipError_t)status);
+}
+
+TA_EXPORT size_t thrust_amd_dtype_size(int dtype) {
+  switch (dtype) {
+    case THRUST_AMD_I8: case THRUST_AMD_U8: return 1;
+    case THRUST_AMD_I16: case THRUST_AMD_U16: return 2;
+    case THRUST_AMD_I32: case THRUST_AMD_U32: case THRUST_AMD_F32: return 4;
+    case THRUST_AMD_I64: case THRUST_AMD_U64: case THRUST_AMD_F64: return 8;
+    default: return 0;
+  }
+}
+
+TA_EXPORT int thrust_amd_malloc(void** ptr, size_t bytes) {
+  if (!ptr) return (int)hipErrorInvalidValue;
+  *ptr = nullptr;
+  if (bytes == 0) return 0;
+  hipError_t e = hipMalloc(ptr, bytes);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();  // an allocation failure must not poison later calls
+    *ptr = nullptr;
+  }
+  return (int)e;
+}
+
+TA_EXPORT int thrust_amd_free(void* ptr) {
+  if (!ptr) return 0;
+  return (int)hipFree(ptr);
+}
+
+TA_EXPORT int thrust_amd_memcpy(void* dst, const void* src, size_t bytes, int kind, void* stream) {
+  if (bytes == 0) return 0;
+  if (!dst || !src) return (int)hipErrorInvalidValue;
+  hipStream_t s = (hipStream_t)stream;
+  switch (kind) {
+    case THRUST_AMD_H2D:
+      TA_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s));
+      return (int)hipStreamSynchronize(s);
+    case THRUST_AMD_D2H:
+      TA_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
+      return (int)hipStreamSynchronize(s);
+    case THRUST_AMD_D2D:
+      return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s);
+    default:
+      return (int)hipErrorInvalidValue;
+  }
+}
+
+TA_EXPORT int thrust_amd_stream_synchronize(void* stream) {
+  return (int)hipStreamSynchronize((hipStream_t)stream);
+}
+
+namespace ta {
+
+template <typename U>
+__global__ __launch_bounds__(256) void fill_kernel(U* __restrict__ dst, uint64_t n, U value) {
+  constexpr int VEC = Vec16<U>::N;
+  const uint64_t vecs = n / VEC;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  const uint64_t tid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  // dst is element-aligned only; peel to the first 16-byte boundary.
+  const uint64_t mis = (reinterpret_cast<uintptr_t>(dst) & 15u) / sizeof(U);
+  const uint64_t head = mis ? ((VEC - mis) < n ? (VEC - mis) : n) : 0;
+  if (tid < head) dst[tid] = value;
+  U* body = dst + head;
+  const uint64_t body_vecs = (n - head) / VEC;
+  Vec16<U> v;
+#pragma unroll
+  for (int i = 0; i < VEC; ++i) v.v[i] = value;
+  for (uint64_t i = tid; i < body_vecs; i += stride) reinterpret_cast<Vec16<U>*>(body)[i] = v;
+  const uint64_t tail_begin = head + body_vecs * VEC;
+  if (tail_begin + tid < n) dst[tail_begin + tid] = value;  // < VEC elements, grid has >= 256 threads
+  (void)vecs;
+}
+
+}  // namespace ta
+
+TA_EXPORT int thrust_amd_fill(void* dst, uint64_t n, size_t elem_bytes, const void* value,
+                               void* stream) {
+  using namespace ta;
+  if (!valid_item_bytes(elem_bytes)) return (int)hipErrorInvalidValue;
+  if (n == 0) return 0;
+  if (!dst || !value) return (int)hipErrorInvalidValue;
+  return with_item_bytes(elem_bytes, [&](auto tt) {
+    using U = typename decltype(tt)::type;
+    U v;
+    __builtin_memcpy(&v, value, sizeof(U));
+    const uint64_t vecs = n / Vec16<U>::N + 1;
+    uint64_t blocks = (vecs + 255) / 256;
+    const uint64_t cap = (uint64_t)NUM_CU * 16;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL((fill_kernel<U>), dim3((uint32_t)blocks), dim3(256), 0, (hipStream_t)stream,
+                       static_cast<U*>(dst), n, v);
+    TA_CHECK_LAUNCH();
+    return 0;
+  });
+}
+
+// ------------------------------------------------------------------ temp arena
+// Blocks are rounded up to size classes (powers of two from 4 KiB to 64 MiB, then
+// multiples of 64 MiB -- a 2^28-key radix sort needs ~1.2 GiB and must not round to
+// 2 GiB).  A released block remembers the stream it was released on.  It is handed out
+// again without further ado on the same stream (stream order makes the reuse safe);
+// for a different stream the releasing stream is synchronised first.
+namespace ta {
+
+struct ArenaBlock {
+  void* ptr;
+  size_t bytes;
+  hipStream_t released_on;
+};
+
+struct Arena {
+  std::mutex mu;
+  std::multimap<size_t, ArenaBlock> free_blocks;  // by size class
+  std::map<void*, size_t> live;                   // handed out -> size class
+  size_t held = 0;
+};
+
+static Arena& arena() {
+  static Arena* a = new Arena;  // leaked on purpose: no hipFree during static destruction
+  return *a;
+}
+
+static size_t size_class(size_t bytes) {
+  const size_t lo = 4096, hi = (size_t)64 << 20;
+  if (bytes <= lo) return lo;
+  if (bytes <= hi) {
+    size_t c = lo;
+    while (c < bytes) c <<= 1;
+    return c;
+  }
+  return align_up(bytes, hi);
+}
+
+}  // namespace ta
+
+TA_EXPORT int thrust_amd_temp_acquire(void** ptr, size_t bytes, void* stream) {
+  using namespace ta;
+  if (!ptr) return (int)hipErrorInvalidValue;
+  *ptr = nullptr;
+  if (bytes == 0) return 0;
+  const size_t cls = size_class(bytes);
+  Arena& a = arena();
+  ArenaBlock blk{nullptr, 0, nullptr};
+  {
+    std::lock_guard<std::mutex> g(a.mu);
+    auto range = a.free_blocks.equal_range(cls);
+    auto pick = range.second;
+    for (auto it = range.first; it != range.second; ++it) {
+      if (it->second.released_on == (hipStream_t)stream) { pick = it; break; }
+      if (pick == range.second) pick = it;
+    }
+    if (pick != range.second) {
+      blk = pick->second;
+      a.free_blocks.erase(pick);
+      a.live[blk.ptr] = cls;
+    }
+  }
+  if (blk.ptr) {
+    if (blk.released_on != (hipStream_t)stream) {
+      hipError_t e = hipStreamSynchronize(blk.released_on);
+      if (e != hipSuccess) return (int)e;
+    }
+    *ptr = blk.ptr;
+    return 0;
+  }
+  void* p = nullptr;
+  hipError_t e = hipMalloc(&p, cls);
+  if (e != hipSuccess) {
+    // Out of memory: give the cached blocks back to the driver and try once more.
+    (void)hipGetLastError();
+    thrust_amd_temp_trim();
+    e = hipMalloc(&p, cls);
+    if (e != hipSuccess) {
+      (void)hipGetLastError();
+      return (int)e;
+    }
+  }
+  {
+    std::lock_guard<std::mutex> g(a.mu);
+    a.live[p] = cls;
+    a.held += cls;
+  }
+  *ptr = p;
+  return 0;
+}
+
+TA_EXPORT int thrust_amd_temp_release(void* ptr, void* stream) {
+  using namespace ta;
+  if (!ptr) return 0;
+  Arena& a = arena();
+  std::lock_guard<std::mutex> g(a.mu);
+  auto it = a.live.find(ptr);
+  if (it == a.live.end()) return (int)hipErrorInvalidValue;
+  const size_t cls = it->second;
+  a.live.erase(it);
+  a.free_blocks.emplace(cls, ArenaBlock{ptr, cls, (hipStream_t)stream});
+  return 0;
+}
+
+TA_EXPORT int thrust_amd_temp_trim(void) {
+  using namespace ta;
+  Arena& a = arena();
+  std::vector<ArenaBlock> victims;
+  {
+    std::lock_guard<std::mutex> g(a.mu);
+    for (auto& kv : a.free_blocks) victims.push_back(kv.second);
+    a.free_blocks.clear();
+    for (auto& b : victims) a.held -= b.bytes;
+  }
+  int rc = 0;
+  for (auto& b : victims) {
+    hipError_t e = hipFree(b.ptr);  // hipFree waits for outstanding work on the block
+    if (e != hipSuccess && rc == 0) rc = (int)e;
+  }
+  return rc;
+}
+
+TA_EXPORT size_t thrust_amd_temp_bytes_held(void) {
+  using namespace ta;
+  Arena& a = arena();
+  std::lock_guard<std::mutex> g(a.mu);
+  return a.held;
+}
