@@ -1,0 +1,145 @@
+"""GPU parity: thrust_amd_sort_keys / thrust_amd_sort_pairs against the CPU oracle.
+
+Sort results have a unique answer (total order on the radix encoding; stability fixes
+the order of values of equal keys), so everything is compared bit for bit -- floats
+through their bit patterns, against the one-thread oracle (= the reference's CPP
+system; the multi-thread OMP layout of +-0.0 depends on the thread count).
+Mirrors testing/sort.cu:80-90, testing/stable_sort_by_key.cu:99-116 and
+testing/sort_variable_bits.cu:18-43.
+"""
+import numpy as np
+import pytest
+
+from thrust_amd import datagen
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [0, 1, 2, 63, 64, 65, 1000, 4096, 8191, 8192, 8193, 16383, 16384, 16385, 65537, 100003,
+         (1 << 20) + 13]
+KEY_DTYPES = [np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64,
+              np.float32, np.float64]
+
+
+def _keys(n, dtype, seed):
+    raw = datagen.splitmix64(seed, n)
+    dt = np.dtype(dtype)
+    if dt.kind == "f":
+        u = raw if dt.itemsize == 8 else (raw >> np.uint64(32)).astype(np.uint32)
+        f = u.view(dtype).copy()
+        f[~np.isfinite(f)] = 0  # NaN/inf patterns are exercised separately
+        return f
+    return raw.astype(dtype) if dt.itemsize == 8 else (raw >> np.uint64(13)).astype(dtype)
+
+
+def _bits(a):
+    return a.view({1: np.uint8, 2: np.uint16, 4: np.uint32, 8: np.uint64}[a.dtype.itemsize])
+
+
+@pytest.mark.parametrize("dtype", KEY_DTYPES)
+def test_sort_keys_all_types(dev, oracle_seq, dtype):
+    for n in SIZES:
+        k = _keys(n, dtype, 3)
+        d = dev.DeviceArray.from_numpy(k)
+        dev.sort_keys(d)
+        assert np.array_equal(_bits(d.numpy()), _bits(oracle_seq.sort_keys(k))), (dtype, n)
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.uint32, np.float32, np.uint64, np.float64])
+def test_sort_keys_descending(dev, oracle_seq, dtype):
+    for n in [1, 77, 16385, 100003]:
+        k = _keys(n, dtype, 5)
+        d = dev.DeviceArray.from_numpy(k)
+        dev.sort_keys(d, descending=True)
+        assert np.array_equal(_bits(d.numpy()), _bits(oracle_seq.sort_keys(k, descending=True)))
+
+
+def test_sort_float_special_values(dev, oracle_seq):
+    n = 70001
+    k = datagen.c2_float32(n)
+    k[::997] = np.float32("nan")
+    k[5::997] = -np.float32("nan")
+    k[7::997] = np.float32("inf")
+    k[9::997] = -np.float32("inf")
+    d = dev.DeviceArray.from_numpy(k)
+    dev.sort_keys(d)
+    assert np.array_equal(_bits(d.numpy()), _bits(oracle_seq.sort_keys(k)))
+
+
+@pytest.mark.parametrize("kdtype", [np.uint32, np.int32, np.float32, np.uint64, np.int64, np.uint16])
+@pytest.mark.parametrize("vdtype", [np.uint32, np.uint64])
+def test_sort_pairs_stable(dev, oracle_seq, kdtype, vdtype):
+    for n in [0, 1, 1000, 8193, 16385, 100003, (1 << 19) + 5]:
+        k = _keys(n, kdtype, 7)
+        if n > 10:
+            k[1::3] = k[0]  # many duplicates: stability becomes visible in the values
+        v = np.arange(n, dtype=vdtype)
+        dk, dv = dev.DeviceArray.from_numpy(k), dev.DeviceArray.from_numpy(v)
+        dev.sort_pairs(dk, dv)
+        rk, rv = oracle_seq.sort_pairs(k, v)
+        assert np.array_equal(_bits(dk.numpy()), _bits(rk)), (kdtype, n)
+        assert np.array_equal(dv.numpy(), rv), (kdtype, n)
+
+
+def test_sort_pairs_descending_is_stable(dev, oracle_seq):
+    n = 50001
+    k = (_keys(n, np.uint32, 9) % 50).astype(np.uint32)
+    v = np.arange(n, dtype=np.uint32)
+    dk, dv = dev.DeviceArray.from_numpy(k), dev.DeviceArray.from_numpy(v)
+    dev.sort_pairs(dk, dv, descending=True)
+    rk, rv = oracle_seq.sort_pairs(k, v, descending=True)
+    assert np.array_equal(dk.numpy(), rk) and np.array_equal(dv.numpy(), rv)
+
+
+def test_sort_variable_bits(dev):
+    """Keys masked to their low b bits (testing/sort_variable_bits.cu:18-43): skipped passes."""
+    n = 40001
+    for b in [0, 1, 7, 8, 9, 16, 21, 32]:
+        k = _keys(n, np.uint32, 11) & np.uint32((1 << b) - 1 if b < 32 else 0xFFFFFFFF)
+        d = dev.DeviceArray.from_numpy(k)
+        dev.sort_keys(d)
+        assert np.array_equal(d.numpy(), np.sort(k, kind="stable")), b
+
+
+def test_sort_bit_range(dev):
+    n = 30001
+    k = _keys(n, np.uint32, 13)
+    v = np.arange(n, dtype=np.uint32)
+    for lo, hi in [(0, 8), (4, 20), (8, 32), (5, 6), (12, 12)]:
+        dk, dv = dev.DeviceArray.from_numpy(k), dev.DeviceArray.from_numpy(v)
+        dev.sort_pairs(dk, dv, begin_bit=lo, end_bit=hi)
+        digit = (k.astype(np.uint64) >> np.uint64(lo)) & np.uint64((1 << (hi - lo)) - 1)
+        order = np.argsort(digit, kind="stable")
+        assert np.array_equal(dk.numpy(), k[order]) and np.array_equal(dv.numpy(), v[order])
+
+
+@pytest.mark.parametrize("kind", ["full", "low16", "skew90"])
+def test_config3_key_distributions(dev, oracle_seq, kind):
+    n = (1 << 21) + 17
+    k = datagen.c3_uint64(n, kind)
+    v = np.arange(n, dtype=np.uint32)
+    dk, dv = dev.DeviceArray.from_numpy(k), dev.DeviceArray.from_numpy(v)
+    dev.sort_pairs(dk, dv)
+    rk, rv = oracle_seq.sort_pairs(k, v)
+    assert np.array_equal(dk.numpy(), rk) and np.array_equal(dv.numpy(), rv)
+
+
+def test_config2_full_size_properties(dev):
+    """Config 2 at N=2^28: sortedness, multiset preservation (histogram of all bytes and a
+    64-bit sum/xor checksum) for uint32; the float32 case is checked on its encoded bits."""
+    n = 1 << 28
+    for gen in (datagen.c2_uint32, datagen.c2_float32):
+        k = gen(n)
+        d = dev.DeviceArray.from_numpy(k)
+        dev.sort_keys(d)
+        out = d.numpy()
+        b_in, b_out = _bits(k), _bits(out)
+        if k.dtype == np.float32:
+            enc = lambda u: u ^ (np.where(u >> 31, np.uint32(0xFFFFFFFF), np.uint32(0x80000000)))
+            e_out = enc(b_out)
+        else:
+            e_out = b_out
+        assert np.all(e_out[:-1] <= e_out[1:])
+        assert int(np.sum(b_in, dtype=np.uint64)) == int(np.sum(b_out, dtype=np.uint64))
+        assert int(np.bitwise_xor.reduce(b_in)) == int(np.bitwise_xor.reduce(b_out))
+        assert np.array_equal(np.bincount(b_in >> 20, minlength=4096),
+                              np.bincount(b_out >> 20, minlength=4096))

@@ -1,0 +1,497 @@
+// thrust_amd_sort_keys / thrust_amd_sort_pairs: onesweep least-significant-digit radix sort.
+//
+//   init       zeroes the digit histograms, the per-pass tile descriptors and tickets
+//   histogram  one read of the keys builds the 256-bin histogram of EVERY 8-bit digit
+//   scan       exclusive scan of each histogram -> global digit offsets; a digit whose one
+//              bin holds all n keys is marked "skip" (the reference's sequential radix
+//              sort does the same, thrust/system/detail/sequential/stable_radix_sort.inl:
+//              264-283), and the ping-pong source of every pass is derived from that
+//   pass x P   chained digit-binning pass ("onesweep"): a tile ranks its keys by digit,
+//              learns the global offset of each of its 256 digit runs by decoupled
+//              look-back over the tiles before it, and scatters keys (and values)
+//   copy-back  only if an odd number of passes ran
+//
+// Ranking inside a tile uses the wave64 match pattern: for each of the 8 digit bits one
+// ballot, folded into a 64-bit peer mask with v_bitop3; rank = wave-private LDS counter
+// + number of peers in lower lanes.  Lanes hold keys wave-striped (lane l of wave w holds
+// keys l, 64+l, ... of the wave's span), so (round, lane) order is memory order and the
+// pass is stable.  Keys and values are then exchanged through LDS so that global stores
+// are contiguous per digit run.
+//
+// Tile order is a dynamic ticket, so the look-back only waits for tiles that have
+// started.  Tile descriptors are one 32-bit word per (tile, digit): 2 status bits and a
+// 30-bit count, which limits one call to n < 2^30 keys.
+//
+// Algorithmic HBM traffic for K-byte keys, V-byte values, P = K passes:
+// K*n (histogram) + P * 2*(K+V)*n.  Replaces cub::DeviceRadixSort as called from
+// thrust/system/cuda/detail/sort.h:1326-1508.
+#include "common.hpp"
+#include "dispatch.hpp"
+
+namespace ta {
+
+constexpr int RADIX_BITS = 8;
+constexpr int RADIX_SIZE = 1 << RADIX_BITS;
+constexpr int MAX_PASSES = 8;
+constexpr uint64_t SORT_MAX_N = (1ull << 30) - 1;
+
+constexpr uint32_t ST_FLAG_SHIFT = 30;
+constexpr uint32_t ST_VALUE_MASK = (1u << ST_FLAG_SHIFT) - 1;
+constexpr uint32_t ST_PARTIAL = 1u << ST_FLAG_SHIFT;
+constexpr uint32_t ST_INCLUSIVE = 2u << ST_FLAG_SHIFT;
+
+// Key <-> radix encoding, decided at run time (uniform across the grid).
+//   sign:   sign bit for signed integers and floats, else 0
+//   fmask:  all ones for floating point, else 0
+//   dmask:  all ones for descending order, else 0
+template <typename K>
+struct KeyCodec {
+  K sign, fmask, dmask;
+  TA_DEVICE K encode(K k) const {
+    using SK = typename std::make_signed<K>::type;
+    const K neg = (K)((SK)k >> (sizeof(K) * 8 - 1));
+    return k ^ ((neg & fmask) | sign) ^ dmask;
+  }
+  TA_DEVICE K decode(K e) const {
+    using SK = typename std::make_signed<K>::type;
+    e ^= dmask;
+    const K pos = (K)((SK)e >> (sizeof(K) * 8 - 1));
+    return e ^ ((~pos & fmask) | sign);
+  }
+};
+
+struct SortCtl {
+  uint32_t skip[MAX_PASSES];     // pass moves nothing
+  uint32_t src_alt[MAX_PASSES];  // pass reads the alternate buffer
+  uint32_t final_in_alt;         // result sits in the alternate buffer after the last pass
+};
+
+struct SortGeometry {
+  int passes;
+  int begin_bit;
+  int end_bit;
+};
+
+// ------------------------------------------------------------------ init
+__global__ __launch_bounds__(256) void sort_init_kernel(uint32_t* __restrict__ words, uint64_t count) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < count; i += stride)
+    words[i] = 0;
+}
+
+// ------------------------------------------------------------------ histogram
+constexpr int HIST_BLOCK = 512;
+constexpr int HIST_ITEMS = 16;  // keys per lane per tile
+
+template <typename K>
+__global__ __launch_bounds__(HIST_BLOCK) void sort_histogram_kernel(const K* __restrict__ keys,
+                                                                     uint64_t n, KeyCodec<K> codec,
+                                                                     SortGeometry geo,
+                                                                     uint32_t* __restrict__ hist) {
+  __shared__ uint32_t s_hist[MAX_PASSES * RADIX_SIZE];
+  for (int i = threadIdx.x; i < geo.passes * RADIX_SIZE; i += HIST_BLOCK) s_hist[i] = 0;
+  __syncthreads();
+
+  constexpr uint64_t TILE = (uint64_t)HIST_BLOCK * HIST_ITEMS;
+  const uint64_t tiles = (n + TILE - 1) / TILE;
+  for (uint64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const uint64_t base = tile * TILE;
+    K k[HIST_ITEMS];
+    bool ok[HIST_ITEMS];
+#pragma unroll
+    for (int i = 0; i < HIST_ITEMS; ++i) {
+      const uint64_t idx = base + (uint64_t)i * HIST_BLOCK + threadIdx.x;
+      ok[i] = idx < n;
+      k[i] = ok[i] ? keys[idx] : (K)0;
+    }
+#pragma unroll
+    for (int i = 0; i < HIST_ITEMS; ++i) {
+      if (ok[i]) {
+        const K e = codec.encode(k[i]);
+        for (int p = 0; p < geo.passes; ++p) {
+          const int lo = geo.begin_bit + p * RADIX_BITS;
+          const int nb = (geo.end_bit - lo) < RADIX_BITS ? (geo.end_bit - lo) : RADIX_BITS;
+          const uint32_t d = (uint32_t)(e >> lo) & ((1u << nb) - 1u);
+          atomicAdd(&s_hist[p * RADIX_SIZE + d], 1u);
+        }
+      }
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < geo.passes * RADIX_SIZE; i += HIST_BLOCK) {
+    const uint32_t c = s_hist[i];
+    if (c) atomicAdd(&hist[i], c);
+  }
+}
+
+// ------------------------------------------------------------------ scan of the histograms
+// One workgroup of 256 threads; thread d owns bin d.  hist[p][d] becomes the exclusive
+// prefix (the global offset of digit d in pass p).
+__global__ __launch_bounds__(RADIX_SIZE) void sort_scan_kernel(uint32_t* __restrict__ hist,
+                                                               uint32_t n, SortGeometry geo,
+                                                               SortCtl* __restrict__ ctl) {
+  __shared__ uint32_t s_wave[RADIX_SIZE / WAVE];
+  __shared__ uint32_t s_full;
+  const int d = threadIdx.x;
+  uint32_t parity = 0;
+  for (int p = 0; p < geo.passes; ++p) {
+    if (d == 0) s_full = 0;
+    __syncthreads();
+    const uint32_t c = hist[p * RADIX_SIZE + d];
+    if (c == n) s_full = 1;
+    const uint32_t incl = wave_inclusive_scan(c, OpPlus{});
+    if ((d % WAVE) == WAVE - 1) s_wave[d / WAVE] = incl;
+    __syncthreads();
+    uint32_t base = 0;
+    for (int w = 0; w < d / WAVE; ++w) base += s_wave[w];
+    hist[p * RADIX_SIZE + d] = base + incl - c;
+    const uint32_t skip = s_full;
+    if (d == 0) {
+      ctl->skip[p] = skip;
+      ctl->src_alt[p] = parity;
+    }
+    parity ^= (skip ? 0u : 1u);
+    __syncthreads();
+  }
+  if (d == 0) ctl->final_in_alt = parity;
+}
+
+// ------------------------------------------------------------------ onesweep pass
+// f(a, b, c) = a & ~(b ^ c): truth table index = a*4 + b*2 + c.
+constexpr int BITOP_AND_XNOR = 0x90;
+
+template <typename K, typename V, bool HAS_VALUES, int BLOCK, int ITEMS>
+struct PassShape {
+  static constexpr int WAVES = BLOCK / WAVE;
+  static constexpr int TILE = BLOCK * ITEMS;
+  static constexpr size_t EXCH_ITEM = (HAS_VALUES && sizeof(V) > sizeof(K)) ? sizeof(V) : sizeof(K);
+  static constexpr size_t EXCH_BYTES = (size_t)TILE * EXCH_ITEM;
+  static constexpr size_t CNT_BYTES = (size_t)WAVES * RADIX_SIZE * sizeof(uint32_t);
+  static constexpr size_t UNION_BYTES = EXCH_BYTES > CNT_BYTES ? EXCH_BYTES : CNT_BYTES;
+};
+
+template <typename K, typename V, bool HAS_VALUES, int BLOCK, int ITEMS>
+__global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
+    K* __restrict__ keys_a, K* __restrict__ keys_b, V* __restrict__ vals_a, V* __restrict__ vals_b,
+    uint32_t n, int pass, SortGeometry geo, KeyCodec<K> codec,
+    const uint32_t* __restrict__ bin_base,  // [RADIX_SIZE] global digit offsets of this pass
+    uint32_t* __restrict__ status,          // [tiles][RADIX_SIZE]
+    uint32_t* __restrict__ ticket, const SortCtl* __restrict__ ctl) {
+  using Shape = PassShape<K, V, HAS_VALUES, BLOCK, ITEMS>;
+  constexpr int WAVES = Shape::WAVES;
+  constexpr int TILE = Shape::TILE;
+  static_assert(BLOCK >= RADIX_SIZE, "one thread per digit is required");
+
+  if (ctl->skip[pass]) return;
+  const bool from_alt = ctl->src_alt[pass] != 0;
+  const K* __restrict__ keys_in = from_alt ? keys_b : keys_a;
+  K* __restrict__ keys_out = from_alt ? keys_a : keys_b;
+  const V* __restrict__ vals_in = from_alt ? vals_b : vals_a;
+  V* __restrict__ vals_out = from_alt ? vals_a : vals_b;
+
+  __shared__ __attribute__((aligned(16))) unsigned char s_union[Shape::UNION_BYTES];
+  __shared__ uint32_t s_scatter_base[RADIX_SIZE];  // global offset - local offset, per digit
+  __shared__ uint32_t s_digit_wave[RADIX_SIZE / WAVE];
+  __shared__ uint32_t s_tile;
+  uint32_t* s_cnt = reinterpret_cast<uint32_t*>(s_union);  // [WAVES][RADIX_SIZE]
+  K* s_keys = reinterpret_cast<K*>(s_union);
+  V* s_vals = reinterpret_cast<V*>(s_union);
+
+  if (threadIdx.x == 0) s_tile = atomicAdd(ticket, 1u);
+  for (int i = threadIdx.x; i < WAVES * RADIX_SIZE; i += BLOCK) s_cnt[i] = 0;
+  __syncthreads();
+  const uint32_t tile = s_tile;
+  const uint32_t tile_base = tile * (uint32_t)TILE;
+  const uint32_t valid = (n - tile_base < (uint32_t)TILE) ? (n - tile_base) : (uint32_t)TILE;
+  const int wave = threadIdx.x / WAVE;
+  const int lane = threadIdx.x % WAVE;
+  const uint32_t span = (uint32_t)wave * (WAVE * ITEMS) + lane;  // + r*64
+
+  const int shift = geo.begin_bit + pass * RADIX_BITS;
+  const int nbits = (geo.end_bit - shift) < RADIX_BITS ? (geo.end_bit - shift) : RADIX_BITS;
+  const uint32_t dmask = (1u << nbits) - 1u;
+
+  // ---- load (wave-striped) and encode; slots past the end sort last inside the tile
+  K e[ITEMS];
+  if (valid == (uint32_t)TILE) {
+#pragma unroll
+    for (int r = 0; r < ITEMS; ++r) e[r] = codec.encode(keys_in[tile_base + span + r * WAVE]);
+  } else {
+#pragma unroll
+    for (int r = 0; r < ITEMS; ++r) {
+      const uint32_t pos = span + r * WAVE;
+      e[r] = (pos < valid) ? codec.encode(keys_in[tile_base + pos]) : (K)~(K)0;
+    }
+  }
+
+  // ---- rank inside the wave by digit
+  uint32_t* my_cnt = s_cnt + wave * RADIX_SIZE;
+  uint32_t rank[ITEMS];
+#pragma unroll
+  for (int r = 0; r < ITEMS; ++r) {
+    const uint32_t d = (uint32_t)(e[r] >> shift) & dmask;
+    uint32_t peers_lo = ~0u, peers_hi = ~0u;
+#pragma unroll
+    for (int b = 0; b < RADIX_BITS; ++b) {
+      const int sb = __builtin_amdgcn_sbfe(d, b, 1);  // -1 where the bit is set
+      const uint64_t m = __builtin_amdgcn_ballot_w64(sb != 0);
+      peers_lo = __builtin_amdgcn_bitop3_b32(peers_lo, (uint32_t)m, (uint32_t)sb, BITOP_AND_XNOR);
+      peers_hi = __builtin_amdgcn_bitop3_b32(peers_hi, (uint32_t)(m >> 32), (uint32_t)sb, BITOP_AND_XNOR);
+    }
+    const uint32_t below = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
+    const uint32_t total = __builtin_popcount(peers_lo) + __builtin_popcount(peers_hi);
+    const uint32_t old = my_cnt[d];
+    rank[r] = old + below;
+    if (below == total - 1) my_cnt[d] = old + total;  // the highest peer lane updates
+  }
+  __syncthreads();
+
+  // ---- per digit: offsets of the waves, tile count; publish the tile's partial counts
+  uint32_t digit_count = 0;
+  uint32_t* my_status = status + (size_t)tile * RADIX_SIZE;
+  if (threadIdx.x < RADIX_SIZE) {
+    const int d = threadIdx.x;
+    uint32_t sum = 0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const uint32_t c = s_cnt[w * RADIX_SIZE + d];
+      s_cnt[w * RADIX_SIZE + d] = sum;
+      sum += c;
+    }
+    digit_count = sum;
+    // padding slots carry the all-ones key and must not be counted
+    if (d == (int)dmask) digit_count -= ((uint32_t)TILE - valid);
+    if (tile != 0)
+      __hip_atomic_store(my_status + d, ST_PARTIAL | digit_count, __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    // exclusive scan of the (padded) counts over the digits -> local run offsets;
+    // the part inside this wave of 64 digits now, the preceding waves after the barrier
+    const uint32_t incl = wave_inclusive_scan(sum, OpPlus{});
+    if (lane == WAVE - 1) s_digit_wave[wave] = incl;
+    s_scatter_base[d] = incl - sum;
+  }
+  __syncthreads();
+  uint32_t local_base = 0;
+  if (threadIdx.x < RADIX_SIZE) {
+    const int d = threadIdx.x;
+    local_base = s_scatter_base[d];
+    for (int w = 0; w < wave; ++w) local_base += s_digit_wave[w];
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) s_cnt[w * RADIX_SIZE + d] += local_base;
+  }
+  __syncthreads();
+
+  // ---- final position of every key inside the tile
+#pragma unroll
+  for (int r = 0; r < ITEMS; ++r) {
+    const uint32_t d = (uint32_t)(e[r] >> shift) & dmask;
+    rank[r] += my_cnt[d];
+  }
+  __syncthreads();  // all reads of s_cnt done: the exchange buffer may overwrite it
+
+#pragma unroll
+  for (int r = 0; r < ITEMS; ++r) s_keys[rank[r]] = e[r];
+
+  // ---- look-back: global offset of each digit run of this tile
+  if (threadIdx.x < RADIX_SIZE) {
+    const int d = threadIdx.x;
+    uint32_t excl;
+    if (tile == 0) {
+      excl = bin_base[d];
+    } else {
+      uint32_t acc = 0;
+      int64_t t = (int64_t)tile - 1;
+      for (;;) {
+        const uint32_t s = __hip_atomic_load(status + (size_t)t * RADIX_SIZE + d, __ATOMIC_RELAXED,
+                                             __HIP_MEMORY_SCOPE_AGENT);
+        const uint32_t flag = s & ~ST_VALUE_MASK;
+        if (flag == 0) {
+          __builtin_amdgcn_s_sleep(1);
+          continue;
+        }
+        acc += s & ST_VALUE_MASK;
+        if (flag == ST_INCLUSIVE) break;
+        --t;
+      }
+      excl = acc;
+    }
+    __hip_atomic_store(my_status + d, ST_INCLUSIVE | (excl + digit_count), __ATOMIC_RELAXED,
+                       __HIP_MEMORY_SCOPE_AGENT);
+    s_scatter_base[d] = excl - local_base;
+  }
+  __syncthreads();
+
+  // ---- keys leave in tile-sorted order: consecutive lanes write consecutive addresses
+  uint32_t gpos[ITEMS];
+#pragma unroll
+  for (int k = 0; k < ITEMS; ++k) {
+    const uint32_t q = (uint32_t)k * BLOCK + threadIdx.x;
+    const K ek = s_keys[q];
+    const uint32_t d = (uint32_t)(ek >> shift) & dmask;
+    gpos[k] = s_scatter_base[d] + q;
+    if (q < valid) keys_out[gpos[k]] = codec.decode(ek);
+  }
+
+  if constexpr (HAS_VALUES) {
+    V v[ITEMS];
+#pragma unroll
+    for (int r = 0; r < ITEMS; ++r) {
+      const uint32_t pos = span + r * WAVE;
+      v[r] = (pos < valid) ? vals_in[tile_base + pos] : V{};
+    }
+    __syncthreads();  // keys have been read out of the exchange buffer
+#pragma unroll
+    for (int r = 0; r < ITEMS; ++r) s_vals[rank[r]] = v[r];
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k) {
+      const uint32_t q = (uint32_t)k * BLOCK + threadIdx.x;
+      if (q < valid) vals_out[gpos[k]] = s_vals[q];
+    }
+  }
+}
+
+// ------------------------------------------------------------------ copy-back
+template <typename K, typename V, bool HAS_VALUES>
+__global__ __launch_bounds__(256) void sort_copy_back_kernel(K* __restrict__ keys,
+                                                             const K* __restrict__ keys_alt,
+                                                             V* __restrict__ vals,
+                                                             const V* __restrict__ vals_alt,
+                                                             uint64_t n,
+                                                             const SortCtl* __restrict__ ctl) {
+  if (!ctl->final_in_alt) return;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    keys[i] = keys_alt[i];
+    if constexpr (HAS_VALUES) vals[i] = vals_alt[i];
+  }
+}
+
+// ------------------------------------------------------------------ host side
+template <typename K>
+static KeyCodec<K> make_codec(int dtype, int descending) {
+  KeyCodec<K> c;
+  const bool is_float = dtype == THRUST_AMD_F32 || dtype == THRUST_AMD_F64;
+  const bool is_signed = is_float || dtype == THRUST_AMD_I8 || dtype == THRUST_AMD_I16 ||
+                         dtype == THRUST_AMD_I32 || dtype == THRUST_AMD_I64;
+  c.sign = is_signed ? (K)((K)1 << (sizeof(K) * 8 - 1)) : (K)0;
+  c.fmask = is_float ? (K)~(K)0 : (K)0;
+  c.dmask = descending ? (K)~(K)0 : (K)0;
+  return c;
+}
+
+template <typename K, typename V, bool HAS_VALUES>
+struct SortPlan {
+  // 16384-key tiles for 4-byte keys keep the ticket rate (one same-address atomic per
+  // tile) far below what a pass needs; 8-byte keys halve the tile to fit LDS.
+  static constexpr int BLOCK = 1024;
+  static constexpr int ITEMS = (sizeof(K) == 8 || (HAS_VALUES && sizeof(V) == 8)) ? 8 : 16;
+  static constexpr int TILE = BLOCK * ITEMS;
+};
+
+template <typename K, typename V, bool HAS_VALUES>
+static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, uint64_t n, int dtype,
+                     int descending, int begin_bit, int end_bit, hipStream_t stream) {
+  using Plan = SortPlan<K, V, HAS_VALUES>;
+  const int key_bits = (int)sizeof(K) * 8;
+  if (begin_bit < 0 || end_bit > key_bits || begin_bit > end_bit) return (int)hipErrorInvalidValue;
+  if (n > SORT_MAX_N) return (int)hipErrorInvalidValue;
+  SortGeometry geo;
+  geo.begin_bit = begin_bit;
+  geo.end_bit = end_bit;
+  geo.passes = (end_bit - begin_bit + RADIX_BITS - 1) / RADIX_BITS;
+  const uint64_t tiles = (n + Plan::TILE - 1) / Plan::TILE;
+
+  TempLayout lay;
+  const size_t off_ctl = lay.add(sizeof(SortCtl));
+  // contiguous zero-initialised region: tickets, histograms, tile descriptors
+  const size_t zero_words = (size_t)MAX_PASSES + (size_t)MAX_PASSES * RADIX_SIZE +
+                            (size_t)geo.passes * tiles * RADIX_SIZE;
+  const size_t off_zero = lay.add(zero_words * sizeof(uint32_t));
+  const size_t off_keys = lay.add((size_t)n * sizeof(K));
+  const size_t off_vals = lay.add(HAS_VALUES ? (size_t)n * sizeof(V) : 0);
+  if (temp == nullptr) {
+    *temp_bytes = lay.total;
+    return 0;
+  }
+  if (*temp_bytes < lay.total) return (int)hipErrorInvalidValue;
+  if (n <= 1 || geo.passes == 0) return 0;
+  if (!keys || (HAS_VALUES && !values)) return (int)hipErrorInvalidValue;
+
+  char* base = static_cast<char*>(temp);
+  SortCtl* ctl = reinterpret_cast<SortCtl*>(base + off_ctl);
+  uint32_t* zero = reinterpret_cast<uint32_t*>(base + off_zero);
+  uint32_t* tickets = zero;
+  uint32_t* hist = zero + MAX_PASSES;
+  uint32_t* status = hist + MAX_PASSES * RADIX_SIZE;
+  K* keys_a = static_cast<K*>(keys);
+  K* keys_b = reinterpret_cast<K*>(base + off_keys);
+  V* vals_a = static_cast<V*>(values);
+  V* vals_b = reinterpret_cast<V*>(base + off_vals);
+  const KeyCodec<K> codec = make_codec<K>(dtype, descending);
+
+  {
+    uint64_t blocks = (zero_words + 255) / 256;
+    if (blocks > (uint64_t)NUM_CU * 8) blocks = (uint64_t)NUM_CU * 8;
+    hipLaunchKernelGGL(sort_init_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, zero,
+                       (uint64_t)zero_words);
+    TA_CHECK_LAUNCH();
+  }
+  {
+    constexpr uint64_t HT = (uint64_t)HIST_BLOCK * HIST_ITEMS;
+    uint64_t blocks = (n + HT - 1) / HT;
+    if (blocks > (uint64_t)NUM_CU * 4) blocks = (uint64_t)NUM_CU * 4;
+    hipLaunchKernelGGL((sort_histogram_kernel<K>), dim3((uint32_t)blocks), dim3(HIST_BLOCK), 0,
+                       stream, (const K*)keys_a, n, codec, geo, hist);
+    TA_CHECK_LAUNCH();
+  }
+  hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(RADIX_SIZE), 0, stream, hist, (uint32_t)n, geo,
+                     ctl);
+  TA_CHECK_LAUNCH();
+  for (int p = 0; p < geo.passes; ++p) {
+    hipLaunchKernelGGL((onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS>),
+                       dim3((uint32_t)tiles), dim3(Plan::BLOCK), 0, stream, keys_a, keys_b, vals_a,
+                       vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE,
+                       status + (size_t)p * tiles * RADIX_SIZE, tickets + p, (const SortCtl*)ctl);
+    TA_CHECK_LAUNCH();
+  }
+  {
+    uint64_t blocks = (n + 255) / 256;
+    if (blocks > (uint64_t)NUM_CU * 8) blocks = (uint64_t)NUM_CU * 8;
+    hipLaunchKernelGGL((sort_copy_back_kernel<K, V, HAS_VALUES>), dim3((uint32_t)blocks), dim3(256),
+                       0, stream, keys_a, (const K*)keys_b, vals_a, (const V*)vals_b, n,
+                       (const SortCtl*)ctl);
+    TA_CHECK_LAUNCH();
+  }
+  return 0;
+}
+
+}  // namespace ta
+
+TA_EXPORT int thrust_amd_sort_keys(void* temp, size_t* temp_bytes, void* keys, uint64_t n,
+                                   int key_dtype, int descending, int begin_bit, int end_bit,
+                                   void* stream) {
+  using namespace ta;
+  if (!temp_bytes || !valid_dtype(key_dtype)) return (int)hipErrorInvalidValue;
+  return with_item_bytes(thrust_amd_dtype_size(key_dtype), [&](auto kt) {
+    using K = typename decltype(kt)::type;
+    return sort_impl<K, uint32_t, false>(temp, temp_bytes, keys, nullptr, n, key_dtype, descending,
+                                         begin_bit, end_bit, (hipStream_t)stream);
+  });
+}
+
+TA_EXPORT int thrust_amd_sort_pairs(void* temp, size_t* temp_bytes, void* keys, void* values,
+                                    uint64_t n, int key_dtype, size_t value_bytes, int descending,
+                                    int begin_bit, int end_bit, void* stream) {
+  using namespace ta;
+  if (!temp_bytes || !valid_dtype(key_dtype) || !valid_item_bytes(value_bytes))
+    return (int)hipErrorInvalidValue;
+  return with_item_bytes(thrust_amd_dtype_size(key_dtype), [&](auto kt) {
+    using K = typename decltype(kt)::type;
+    return with_item_bytes(value_bytes, [&](auto vt) {
+      using V = typename decltype(vt)::type;
+      return sort_impl<K, V, true>(temp, temp_bytes, keys, values, n, key_dtype, descending,
+                                   begin_bit, end_bit, (hipStream_t)stream);
+    });
+  });
+}

@@ -17,8 +17,12 @@
 
 namespace ta {
 
-constexpr int SCAN_BLOCK = 256;
-constexpr int SCAN_CHUNKS = 4;
+// Tile shapes (threads x 16-byte vectors per lane).  The per-tile cost of the ticket
+// (a same-address atomic retires every ~12 ns on MI355X) and of the look-back makes large
+// tiles win once there are enough of them to fill 256 CUs; small inputs use small tiles.
+struct ScanShapeLarge { static constexpr int BLOCK = 1024, CHUNKS = 12; };
+struct ScanShapeSmall { static constexpr int BLOCK = 256, CHUNKS = 4; };
+constexpr uint64_t SCAN_LARGE_MIN_BYTES = (uint64_t)32 << 20;
 
 __global__ void tile_state_init_kernel(uint64_t* __restrict__ words, uint64_t count,
                                        uint32_t* __restrict__ counters, uint32_t num_counters) {
@@ -33,10 +37,12 @@ TA_DEVICE T wave_shift_up(T v, T id) {
   return dpp_move<0x138 /* wave_shr:1 */>(id, v);
 }
 
-template <typename T, typename Op, bool EXCLUSIVE, bool ALIGNED>
-__global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(const T* in, T* out, uint64_t n, T init,
+template <typename T, typename Op, bool EXCLUSIVE, bool ALIGNED, typename Shape>
+__global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out, uint64_t n, T init,
                                                           uint64_t* __restrict__ status,
                                                           uint32_t* __restrict__ ticket) {
+  constexpr int SCAN_BLOCK = Shape::BLOCK;
+  constexpr int SCAN_CHUNKS = Shape::CHUNKS;
   constexpr int VEC = Vec16<T>::N;
   constexpr int WAVES = SCAN_BLOCK / WAVE;
   constexpr uint32_t WAVE_SPAN = WAVE * SCAN_CHUNKS * VEC;  // elements per wave
@@ -148,19 +154,14 @@ __global__ __launch_bounds__(SCAN_BLOCK) void scan_kernel(const T* in, T* out, u
   }
 }
 
-template <typename T>
-static uint64_t scan_tiles(uint64_t n) {
-  constexpr uint64_t TILE = (uint64_t)SCAN_BLOCK * SCAN_CHUNKS * Vec16<T>::N;
-  return (n + TILE - 1) / TILE;
-}
-
 template <bool EXCLUSIVE>
 struct ScanLaunch {
-  template <typename T, typename Op>
-  static int run(void* temp, size_t* temp_bytes, const void* in, void* out, uint64_t n,
-                 const void* init, hipStream_t stream) {
+  template <typename T, typename Op, typename Shape>
+  static int run_shape(void* temp, size_t* temp_bytes, const void* in, void* out, uint64_t n,
+                       const void* init, hipStream_t stream) {
     constexpr int W = TileWords<T>::W;
-    const uint64_t tiles = scan_tiles<T>(n);
+    constexpr uint64_t TILE = (uint64_t)Shape::BLOCK * Shape::CHUNKS * Vec16<T>::N;
+    const uint64_t tiles = (n + TILE - 1) / TILE;
     if (tiles > 0xffffffffull) return (int)hipErrorInvalidValue;
     TempLayout lay;
     const size_t off_ticket = lay.add(sizeof(uint32_t));
@@ -186,13 +187,21 @@ struct ScanLaunch {
     const T* src = static_cast<const T*>(in);
     T* dst = static_cast<T*>(out);
     if (is_aligned16(in) && is_aligned16(out))
-      hipLaunchKernelGGL((scan_kernel<T, Op, EXCLUSIVE, true>), dim3((uint32_t)tiles),
-                         dim3(SCAN_BLOCK), 0, stream, src, dst, n, init_v, status, ticket);
+      hipLaunchKernelGGL((scan_kernel<T, Op, EXCLUSIVE, true, Shape>), dim3((uint32_t)tiles),
+                         dim3(Shape::BLOCK), 0, stream, src, dst, n, init_v, status, ticket);
     else
-      hipLaunchKernelGGL((scan_kernel<T, Op, EXCLUSIVE, false>), dim3((uint32_t)tiles),
-                         dim3(SCAN_BLOCK), 0, stream, src, dst, n, init_v, status, ticket);
+      hipLaunchKernelGGL((scan_kernel<T, Op, EXCLUSIVE, false, Shape>), dim3((uint32_t)tiles),
+                         dim3(Shape::BLOCK), 0, stream, src, dst, n, init_v, status, ticket);
     TA_CHECK_LAUNCH();
     return 0;
+  }
+
+  template <typename T, typename Op>
+  static int run(void* temp, size_t* temp_bytes, const void* in, void* out, uint64_t n,
+                 const void* init, hipStream_t stream) {
+    if (n * sizeof(T) >= SCAN_LARGE_MIN_BYTES)
+      return run_shape<T, Op, ScanShapeLarge>(temp, temp_bytes, in, out, n, init, stream);
+    return run_shape<T, Op, ScanShapeSmall>(temp, temp_bytes, in, out, n, init, stream);
   }
 };
 
