@@ -47,6 +47,7 @@ constexpr uint32_t ST_INCLUSIVE = 2u << ST_FLAG_SHIFT;
 template <typename K>
 struct KeyCodec {
   K sign, fmask, dmask;
+  uint32_t plain;  // all three masks are zero: encode/decode are the identity
   TA_DEVICE K encode(K k) const {
     using SK = typename std::make_signed<K>::type;
     const K neg = (K)((SK)k >> (sizeof(K) * 8 - 1));
@@ -80,48 +81,94 @@ __global__ __launch_bounds__(256) void sort_init_kernel(uint32_t* __restrict__ w
 }
 
 // ------------------------------------------------------------------ histogram
-constexpr int HIST_BLOCK = 512;
-constexpr int HIST_ITEMS = 16;  // keys per lane per tile
+// One workgroup per CU with up to 128 KiB of LDS: every bin exists in COPIES copies and
+// lane l only ever touches copy l % COPIES, so with 32 copies the 64 lanes of an LDS
+// atomic fall on 32 distinct banks whatever the digits are (random digits on a single
+// copy serialise about five-fold on bank conflicts).  Keys are read with 16-byte loads;
+// their order does not matter here.
+constexpr int HIST_BLOCK = 1024;
+constexpr int HIST_UNROLL = 4;  // 16-byte vectors in flight per lane
 
-template <typename K>
+template <typename K, int NP>
 __global__ __launch_bounds__(HIST_BLOCK) void sort_histogram_kernel(const K* __restrict__ keys,
                                                                      uint64_t n, KeyCodec<K> codec,
                                                                      SortGeometry geo,
                                                                      uint32_t* __restrict__ hist) {
-  __shared__ uint32_t s_hist[MAX_PASSES * RADIX_SIZE];
-  for (int i = threadIdx.x; i < geo.passes * RADIX_SIZE; i += HIST_BLOCK) s_hist[i] = 0;
+  constexpr int COPIES = NP <= 4 ? 32 : 16;
+  constexpr int BINS = NP * RADIX_SIZE;
+  constexpr int VEC = Vec16<K>::N;
+  __shared__ uint32_t s_hist[BINS * COPIES];
+  for (int i = threadIdx.x; i < BINS * COPIES; i += HIST_BLOCK) s_hist[i] = 0;
   __syncthreads();
+  uint32_t* my_copy = s_hist + (threadIdx.x % COPIES);
 
-  constexpr uint64_t TILE = (uint64_t)HIST_BLOCK * HIST_ITEMS;
-  const uint64_t tiles = (n + TILE - 1) / TILE;
-  for (uint64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const uint64_t base = tile * TILE;
-    K k[HIST_ITEMS];
-    bool ok[HIST_ITEMS];
+  auto count = [&](K k) {
+    const K e = codec.plain ? k : codec.encode(k);
 #pragma unroll
-    for (int i = 0; i < HIST_ITEMS; ++i) {
-      const uint64_t idx = base + (uint64_t)i * HIST_BLOCK + threadIdx.x;
-      ok[i] = idx < n;
-      k[i] = ok[i] ? keys[idx] : (K)0;
+    for (int p = 0; p < NP; ++p) {
+      const int lo = geo.begin_bit + p * RADIX_BITS;
+      const int nb = (p == NP - 1) ? (geo.end_bit - lo) : RADIX_BITS;
+      const uint32_t d = (uint32_t)(e >> lo) & ((1u << nb) - 1u);
+      __hip_atomic_fetch_add(my_copy + (p * RADIX_SIZE + d) * COPIES, 1u, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_WORKGROUP);
+    }
+  };
+
+  // head: elements before the first 16-byte boundary; tail: what the vectors leave over
+  const uint64_t mis = (reinterpret_cast<uintptr_t>(keys) & 15u) / sizeof(K);
+  const uint64_t head = mis ? ((VEC - mis) < n ? (VEC - mis) : n) : 0;
+  const uint64_t vecs = (n - head) / VEC;
+  const uint64_t tail_begin = head + vecs * VEC;
+  if (blockIdx.x == 0) {
+    if (threadIdx.x < head) count(keys[threadIdx.x]);
+    if (tail_begin + threadIdx.x < n) count(keys[tail_begin + threadIdx.x]);
+  }
+  const Vec16<K>* body = reinterpret_cast<const Vec16<K>*>(keys + head);
+  constexpr uint64_t TILE_VECS = (uint64_t)HIST_BLOCK * HIST_UNROLL;
+  const uint64_t tiles = (vecs + TILE_VECS - 1) / TILE_VECS;
+  for (uint64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
+    const uint64_t base = tile * TILE_VECS + threadIdx.x;
+    Vec16<K> x[HIST_UNROLL];
+    bool ok[HIST_UNROLL];
+#pragma unroll
+    for (int u = 0; u < HIST_UNROLL; ++u) {
+      const uint64_t i = base + (uint64_t)u * HIST_BLOCK;
+      ok[u] = i < vecs;
+      if (ok[u]) x[u] = body[i];
     }
 #pragma unroll
-    for (int i = 0; i < HIST_ITEMS; ++i) {
-      if (ok[i]) {
-        const K e = codec.encode(k[i]);
-        for (int p = 0; p < geo.passes; ++p) {
-          const int lo = geo.begin_bit + p * RADIX_BITS;
-          const int nb = (geo.end_bit - lo) < RADIX_BITS ? (geo.end_bit - lo) : RADIX_BITS;
-          const uint32_t d = (uint32_t)(e >> lo) & ((1u << nb) - 1u);
-          atomicAdd(&s_hist[p * RADIX_SIZE + d], 1u);
-        }
+    for (int u = 0; u < HIST_UNROLL; ++u) {
+      if (ok[u]) {
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) count(x[u].v[i]);
       }
     }
   }
   __syncthreads();
-  for (int i = threadIdx.x; i < geo.passes * RADIX_SIZE; i += HIST_BLOCK) {
-    const uint32_t c = s_hist[i];
-    if (c) atomicAdd(&hist[i], c);
+  // fold the copies; thread t starts at copy t so that a wave spreads over all banks
+  for (int bin = threadIdx.x; bin < BINS; bin += HIST_BLOCK) {
+    uint32_t c = 0;
+#pragma unroll 8
+    for (int j = 0; j < COPIES; ++j) c += s_hist[bin * COPIES + ((j + threadIdx.x) % COPIES)];
+    if (c) atomicAdd(&hist[bin], c);
   }
+}
+
+template <typename K>
+static void launch_histogram(int passes, uint32_t blocks, hipStream_t stream, const K* keys,
+                             uint64_t n, const KeyCodec<K>& codec, const SortGeometry& geo,
+                             uint32_t* hist) {
+#define TA_HIST_CASE(NP)                                                                       \
+  case NP:                                                                                     \
+    hipLaunchKernelGGL((sort_histogram_kernel<K, NP>), dim3(blocks), dim3(HIST_BLOCK), 0,      \
+                       stream, keys, n, codec, geo, hist);                                     \
+    break;
+  switch (passes) {
+    TA_HIST_CASE(1) TA_HIST_CASE(2) TA_HIST_CASE(3) TA_HIST_CASE(4)
+    TA_HIST_CASE(5) TA_HIST_CASE(6) TA_HIST_CASE(7) TA_HIST_CASE(8)
+    default: break;
+  }
+#undef TA_HIST_CASE
 }
 
 // ------------------------------------------------------------------ scan of the histograms
@@ -157,6 +204,19 @@ __global__ __launch_bounds__(RADIX_SIZE) void sort_scan_kernel(uint32_t* __restr
 }
 
 // ------------------------------------------------------------------ onesweep pass
+#ifdef TA_DBG_PHASES
+__device__ unsigned long long g_phase[16384 * 16];
+#define TA_PHASE(i)                                                                   \
+  do {                                                                                \
+    if (threadIdx.x == TA_DBG_PHASE_THREAD) {                                         \
+      const unsigned long long _now = __builtin_readcyclecounter();                   \
+      g_phase[blockIdx.x * 16 + (i)] += _now - _t_prev;                                         \
+      _t_prev = _now;                                                                 \
+    }                                                                                 \
+  } while (0)
+#else
+#define TA_PHASE(i)
+#endif
 // f(a, b, c) = a & ~(b ^ c): truth table index = a*4 + b*2 + c.
 constexpr int BITOP_AND_XNOR = 0x90;
 
@@ -170,8 +230,20 @@ struct PassShape {
   static constexpr size_t UNION_BYTES = EXCH_BYTES > CNT_BYTES ? EXCH_BYTES : CNT_BYTES;
 };
 
+#ifndef TA_RANK_VARIANT
+#define TA_RANK_VARIANT 1
+#endif
+#ifndef TA_BFE_ASM
+#define TA_BFE_ASM 1
+#endif
+#ifndef TA_RANK_GROUP
+#define TA_RANK_GROUP 2
+#endif
+#ifndef TA_SORT_MIN_WAVES
+#define TA_SORT_MIN_WAVES 1
+#endif
 template <typename K, typename V, bool HAS_VALUES, int BLOCK, int ITEMS>
-__global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
+__global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel(
     K* __restrict__ keys_a, K* __restrict__ keys_b, V* __restrict__ vals_a, V* __restrict__ vals_b,
     uint32_t n, int pass, SortGeometry geo, KeyCodec<K> codec,
     const uint32_t* __restrict__ bin_base,  // [RADIX_SIZE] global digit offsets of this pass
@@ -183,6 +255,9 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   static_assert(BLOCK >= RADIX_SIZE, "one thread per digit is required");
 
   if (ctl->skip[pass]) return;
+#ifdef TA_DBG_PHASES
+  unsigned long long _t_prev = __builtin_readcyclecounter();
+#endif
   const bool from_alt = ctl->src_alt[pass] != 0;
   const K* __restrict__ keys_in = from_alt ? keys_b : keys_a;
   K* __restrict__ keys_out = from_alt ? keys_a : keys_b;
@@ -197,9 +272,14 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   K* s_keys = reinterpret_cast<K*>(s_union);
   V* s_vals = reinterpret_cast<V*>(s_union);
 
+#ifdef TA_DBG_NOTICKET
+  if (threadIdx.x == 0) s_tile = blockIdx.x;
+#else
   if (threadIdx.x == 0) s_tile = atomicAdd(ticket, 1u);
+#endif
   for (int i = threadIdx.x; i < WAVES * RADIX_SIZE; i += BLOCK) s_cnt[i] = 0;
   __syncthreads();
+  TA_PHASE(0);
   const uint32_t tile = s_tile;
   const uint32_t tile_base = tile * (uint32_t)TILE;
   const uint32_t valid = (n - tile_base < (uint32_t)TILE) ? (n - tile_base) : (uint32_t)TILE;
@@ -215,7 +295,11 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   K e[ITEMS];
   if (valid == (uint32_t)TILE) {
 #pragma unroll
-    for (int r = 0; r < ITEMS; ++r) e[r] = codec.encode(keys_in[tile_base + span + r * WAVE]);
+    for (int r = 0; r < ITEMS; ++r) e[r] = keys_in[tile_base + span + r * WAVE];
+    if (!codec.plain) {  // uniform branch: unsigned ascending keys need no transform
+#pragma unroll
+      for (int r = 0; r < ITEMS; ++r) e[r] = codec.encode(e[r]);
+    }
   } else {
 #pragma unroll
     for (int r = 0; r < ITEMS; ++r) {
@@ -224,27 +308,62 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     }
   }
 
+  TA_PHASE(1);
   // ---- rank inside the wave by digit
+  // Per digit bit: v_bfe_i32 (lane's bit as 0 / -1), one ballot, and two v_bitop3 folding
+  // "same bit as mine" into the 64-bit peer mask.  The wave-private counter is read, then
+  // bumped by one per peer with an LDS atomic; LDS executes a wave's instructions in
+  // order, so the next round reads the updated count.
   uint32_t* my_cnt = s_cnt + wave * RADIX_SIZE;
-  uint32_t rank[ITEMS];
+  // ranks are < TILE <= 65536: two per register
+  static_assert(TILE <= 65536 && ITEMS % 2 == 0, "rank packing");
+  uint32_t rank2[ITEMS / 2];
 #pragma unroll
   for (int r = 0; r < ITEMS; ++r) {
     const uint32_t d = (uint32_t)(e[r] >> shift) & dmask;
     uint32_t peers_lo = ~0u, peers_hi = ~0u;
 #pragma unroll
     for (int b = 0; b < RADIX_BITS; ++b) {
-      const int sb = __builtin_amdgcn_sbfe(d, b, 1);  // -1 where the bit is set
+      int sb;
+#if TA_BFE_ASM
+      // opaque to the optimiser so that the compare below is made on sb itself
+      asm volatile("v_bfe_i32 %0, %1, %2, 1" : "=v"(sb) : "v"(d), "n"(b));
+#else
+      sb = __builtin_amdgcn_sbfe(d, b, 1);
+#endif
       const uint64_t m = __builtin_amdgcn_ballot_w64(sb != 0);
       peers_lo = __builtin_amdgcn_bitop3_b32(peers_lo, (uint32_t)m, (uint32_t)sb, BITOP_AND_XNOR);
       peers_hi = __builtin_amdgcn_bitop3_b32(peers_hi, (uint32_t)(m >> 32), (uint32_t)sb, BITOP_AND_XNOR);
     }
     const uint32_t below = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
+#if TA_RANK_VARIANT == 3
+    const uint32_t old = 0; (void)my_cnt;
+#elif TA_RANK_VARIANT == 2
     const uint32_t total = __builtin_popcount(peers_lo) + __builtin_popcount(peers_hi);
     const uint32_t old = my_cnt[d];
-    rank[r] = old + below;
-    if (below == total - 1) my_cnt[d] = old + total;  // the highest peer lane updates
+    if (below == total - 1) my_cnt[d] = old + total;
+#elif TA_RANK_VARIANT == 4
+    const uint32_t total = __builtin_popcount(peers_lo) + __builtin_popcount(peers_hi);
+    const uint32_t old = my_cnt[d];
+    my_cnt[d] = old + total;
+#else
+    const uint32_t old = my_cnt[d];
+    __hip_atomic_fetch_add(&my_cnt[d], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+#endif
+    if (r % 2 == 0) rank2[r / 2] = old + below;
+    else rank2[r / 2] |= (old + below) << 16;
+    // pin the packed rank here: otherwise the add is sunk past the barrier and `old` and
+    // `below` of every round stay live
+    asm volatile("" : "+v"(rank2[r / 2]));
+#if TA_RANK_GROUP > 0
+    // keep the scheduler from computing all peer masks first (two live registers per
+    // round): rounds are finished in groups
+    if (r % TA_RANK_GROUP == TA_RANK_GROUP - 1) __builtin_amdgcn_sched_barrier(0);
+#endif
   }
+  TA_PHASE(2);
   __syncthreads();
+  TA_PHASE(3);
 
   // ---- per digit: offsets of the waves, tile count; publish the tile's partial counts
   uint32_t digit_count = 0;
@@ -281,17 +400,19 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   }
   __syncthreads();
 
+  TA_PHASE(4);
   // ---- final position of every key inside the tile
 #pragma unroll
   for (int r = 0; r < ITEMS; ++r) {
     const uint32_t d = (uint32_t)(e[r] >> shift) & dmask;
-    rank[r] += my_cnt[d];
+    rank2[r / 2] += my_cnt[d] << (16 * (r % 2));  // no carry: each half stays < TILE
   }
   __syncthreads();  // all reads of s_cnt done: the exchange buffer may overwrite it
 
 #pragma unroll
-  for (int r = 0; r < ITEMS; ++r) s_keys[rank[r]] = e[r];
+  for (int r = 0; r < ITEMS; ++r) s_keys[(rank2[r / 2] >> (16 * (r % 2))) & 0xffffu] = e[r];
 
+  TA_PHASE(5);
   // ---- look-back: global offset of each digit run of this tile
   if (threadIdx.x < RADIX_SIZE) {
     const int d = threadIdx.x;
@@ -301,6 +422,9 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     } else {
       uint32_t acc = 0;
       int64_t t = (int64_t)tile - 1;
+#ifdef TA_DBG_NOLOOKBACK
+      if (false)
+#endif
       for (;;) {
         const uint32_t s = __hip_atomic_load(status + (size_t)t * RADIX_SIZE + d, __ATOMIC_RELAXED,
                                              __HIP_MEMORY_SCOPE_AGENT);
@@ -319,19 +443,34 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
                        __HIP_MEMORY_SCOPE_AGENT);
     s_scatter_base[d] = excl - local_base;
   }
+  TA_PHASE(6);
   __syncthreads();
+  TA_PHASE(7);
 
   // ---- keys leave in tile-sorted order: consecutive lanes write consecutive addresses
+  // Batched so that the 2*ITEMS LDS reads are independent and in flight together.
   uint32_t gpos[ITEMS];
+  {
+    K ek[ITEMS];
 #pragma unroll
-  for (int k = 0; k < ITEMS; ++k) {
-    const uint32_t q = (uint32_t)k * BLOCK + threadIdx.x;
-    const K ek = s_keys[q];
-    const uint32_t d = (uint32_t)(ek >> shift) & dmask;
-    gpos[k] = s_scatter_base[d] + q;
-    if (q < valid) keys_out[gpos[k]] = codec.decode(ek);
+    for (int k = 0; k < ITEMS; ++k) ek[k] = s_keys[(uint32_t)k * BLOCK + threadIdx.x];
+#pragma unroll
+    for (int k = 0; k < ITEMS; ++k)
+      gpos[k] = s_scatter_base[(uint32_t)(ek[k] >> shift) & dmask] + (uint32_t)k * BLOCK + threadIdx.x;
+    if (!codec.plain) {
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) ek[k] = codec.decode(ek[k]);
+    }
+    if (valid == (uint32_t)TILE) {
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k) keys_out[gpos[k]] = ek[k];
+    } else {
+#pragma unroll
+      for (int k = 0; k < ITEMS; ++k)
+        if ((uint32_t)k * BLOCK + threadIdx.x < valid) keys_out[gpos[k]] = ek[k];
+    }
   }
-
+  TA_PHASE(8);
   if constexpr (HAS_VALUES) {
     V v[ITEMS];
 #pragma unroll
@@ -341,7 +480,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     }
     __syncthreads();  // keys have been read out of the exchange buffer
 #pragma unroll
-    for (int r = 0; r < ITEMS; ++r) s_vals[rank[r]] = v[r];
+    for (int r = 0; r < ITEMS; ++r) s_vals[(rank2[r / 2] >> (16 * (r % 2))) & 0xffffu] = v[r];
     __syncthreads();
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
@@ -377,6 +516,7 @@ static KeyCodec<K> make_codec(int dtype, int descending) {
   c.sign = is_signed ? (K)((K)1 << (sizeof(K) * 8 - 1)) : (K)0;
   c.fmask = is_float ? (K)~(K)0 : (K)0;
   c.dmask = descending ? (K)~(K)0 : (K)0;
+  c.plain = (!is_signed && !descending) ? 1u : 0u;
   return c;
 }
 
@@ -384,8 +524,13 @@ template <typename K, typename V, bool HAS_VALUES>
 struct SortPlan {
   // 16384-key tiles for 4-byte keys keep the ticket rate (one same-address atomic per
   // tile) far below what a pass needs; 8-byte keys halve the tile to fit LDS.
+#if defined(TA_SORT_BLOCK)
+  static constexpr int BLOCK = TA_SORT_BLOCK;
+  static constexpr int ITEMS = TA_SORT_ITEMS;
+#else
   static constexpr int BLOCK = 1024;
   static constexpr int ITEMS = (sizeof(K) == 8 || (HAS_VALUES && sizeof(V) == 8)) ? 8 : 16;
+#endif
   static constexpr int TILE = BLOCK * ITEMS;
 };
 
@@ -438,11 +583,10 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
     TA_CHECK_LAUNCH();
   }
   {
-    constexpr uint64_t HT = (uint64_t)HIST_BLOCK * HIST_ITEMS;
+    constexpr uint64_t HT = (uint64_t)HIST_BLOCK * HIST_UNROLL * Vec16<K>::N;
     uint64_t blocks = (n + HT - 1) / HT;
-    if (blocks > (uint64_t)NUM_CU * 4) blocks = (uint64_t)NUM_CU * 4;
-    hipLaunchKernelGGL((sort_histogram_kernel<K>), dim3((uint32_t)blocks), dim3(HIST_BLOCK), 0,
-                       stream, (const K*)keys_a, n, codec, geo, hist);
+    if (blocks > (uint64_t)NUM_CU) blocks = NUM_CU;
+    launch_histogram<K>(geo.passes, (uint32_t)blocks, stream, (const K*)keys_a, n, codec, geo, hist);
     TA_CHECK_LAUNCH();
   }
   hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(RADIX_SIZE), 0, stream, hist, (uint32_t)n, geo,
