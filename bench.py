@@ -1,0 +1,207 @@
+#!/usr/bin/env python3
+"""Headline benchmark: thrust::sort of 2^28 uint32 keys (BASELINE.json configs[1]) on one MI355X,
+with thrust::reduce / inclusive_scan over 2^28 int32 measured beside it.
+
+One step = one full radix sort of a device-resident, never-before-sorted copy of the seeded
+input (the sort is in place, so every step gets its own copy; the copies are made before the
+timed region).  Exactly K steps are timed between two device synchronisations; the printed
+JSON line follows the driver's contract.  `roofline` describes the dominant kernel (one
+onesweep digit-binning pass: n keys read + n keys written), timed with events on the launch
+stream; `cpu_baseline` is the reference's own OpenMP device system (oracle/_ref, built from
+the reference sources) when that library travelled with the tree, else the C restatement,
+timed on a bounded sample on this machine's host cores.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
+N_SORT = 1 << 28
+N_C1 = 1 << 28
+
+# HBM bytes per onesweep pass launch at n = 2^28 uint32, from rocprofv3 --pmc FETCH_SIZE /
+# WRITE_SIZE, scaled by the same counters on a plain copy kernel of known size (see the
+# profiles/ summary for the sort kernels); None until measured.
+PASS_TRAFFIC_BYTES = None
+
+
+def device_random_u32(torch, n, seed):
+    """uint32 keys, uniform over the full range, generated on the device (seeded)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    x = torch.randint(-(1 << 31), 1 << 31, (n,), dtype=torch.int32, device="cuda", generator=g)
+    return x.view(torch.uint8)
+
+
+def time_region(torch, fn, steps, warmup):
+    for i in range(warmup):
+        fn(i, True)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(i, False)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
+def bench_sort(torch, capi, steps, warmup):
+    n = N_SORT
+    src = device_random_u32(torch, n, 1)
+    temp = capi.Temp()
+    bufs = [capi.DeviceArray(n, capi.U32, src.clone()) for _ in range(steps)]
+    warm = [capi.DeviceArray(n, capi.U32, src.clone()) for _ in range(max(warmup, 1))]
+    capi.sort_keys(warm[0], temp=temp)  # sizes the temp storage once
+
+    def step(i, is_warm):
+        capi.sort_keys(warm[i] if is_warm else bufs[i], temp=temp)
+
+    ms = time_region(torch, step, steps, warmup)
+    # parity spot-check of the last sorted buffer: order + multiset (checksum) preserved
+    out = bufs[-1].storage.view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    inp = src.view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    ok = bool((out[1:] >= out[:-1]).all().item()) and int(out.sum().item()) == int(inp.sum().item())
+    if not ok:
+        raise SystemExit("bench: sorted output failed the order/checksum check")
+    del bufs, warm
+
+    # per-kernel durations of the same call, events on the launch stream
+    capi.profile_enable(True)
+    reps = 5
+    prof_bufs = [capi.DeviceArray(n, capi.U32, src.clone()) for _ in range(reps)]
+    for b in prof_bufs:
+        capi.sort_keys(b, temp=temp)
+    torch.cuda.synchronize()
+    prof = capi.profile_collect()
+    capi.profile_enable(False)
+    launches, total_ms = prof["onesweep_pass"]
+    pass_ms = total_ms / launches
+    kernels_ms = {k: v[1] / reps for k, v in prof.items()}
+    return ms, pass_ms, kernels_ms
+
+
+def bench_c1(torch, capi, steps, warmup):
+    n = N_C1
+    g = torch.Generator(device="cuda")
+    g.manual_seed(42)
+    x = torch.randint(0, 1001, (n,), dtype=torch.int32, device="cuda", generator=g)
+    d = capi.DeviceArray(n, capi.I32, x.view(torch.uint8))
+    out1 = capi.DeviceArray(1, capi.I32)
+    outn = capi.DeviceArray(n, capi.I32)
+    t_r, t_s = capi.Temp(), capi.Temp()
+    capi.reduce(d, temp=t_r, out=out1)
+    capi.inclusive_scan(d, out=outn, temp=t_s)
+    total = int(x.sum(dtype=torch.int64).item())
+    got = int(out1.numpy()[0])
+    if (got - total) % (1 << 32) != 0:
+        raise SystemExit("bench: reduce result differs from the int64 sum modulo 2^32")
+    last = int(outn.storage.view(torch.int32)[n - 1].item())
+    if (last - total) % (1 << 32) != 0:
+        raise SystemExit("bench: inclusive_scan total differs from the int64 sum modulo 2^32")
+    ms_reduce = time_region(torch, lambda i, w: capi.reduce(d, temp=t_r, out=out1), steps, warmup)
+    ms_scan = time_region(torch, lambda i, w: capi.inclusive_scan(d, out=outn, temp=t_s), steps, warmup)
+    return ms_reduce, ms_scan
+
+
+def cpu_baseline():
+    """Reference OMP back end (or the restatement) on a bounded sample: sort of 2^26 uint32."""
+    from oracle import cpu as ocpu
+    from thrust_amd import datagen
+    cores = len(os.sched_getaffinity(0))
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    n = 1 << 26
+    keys = datagen.c2_uint32(n)
+    if ocpu.ref_available("omp"):
+        impl, kind = ocpu.Reference("omp"), "reference"
+    else:
+        if not os.path.exists(ocpu.ORACLE_LIB):
+            ocpu.build(with_ref=False)
+        impl, kind = ocpu.Oracle(), "port"
+    best = None
+    for _ in range(2):
+        k = keys.copy()
+        t0 = time.perf_counter()
+        out = impl.sort_keys(k)
+        dt = time.perf_counter() - t0
+        best = dt if best is None else min(best, dt)
+    if not np.all(out[:-1] <= out[1:]):
+        raise SystemExit("bench: CPU baseline output is not sorted")
+    x = datagen.c1_int32(1 << 26)
+    t0 = time.perf_counter(); impl.reduce(x); t_red = time.perf_counter() - t0
+    t0 = time.perf_counter(); impl.inclusive_scan(x); t_scan = time.perf_counter() - t0
+    return {
+        "value": n / best / 1e9, "unit": "Gkeys/s", "cores": cores, "kind": kind,
+        "sample": "thrust::sort of 2^26 uint32 (same generator as the GPU run's key space), best of 2, "
+                  "timing includes one copy of the input made by the binding",
+        "reduce_GBps": 4.0 * x.size / t_red / 1e9, "inclusive_scan_GBps": 8.0 * x.size / t_scan / 1e9,
+        "note": "OMP back end: sort = per-thread LSD radix + serial pairwise merges; "
+                "inclusive_scan is single-threaded by construction",
+    }
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        raise SystemExit("bench.py: this build measures one GPU only (the device system is "
+                         "single-GPU by design); run with --gpus 1")
+    if not 1 <= args.steps <= 200:
+        raise SystemExit("bench.py: --steps must be in [1, 200] (each step sorts its own 1 GiB copy)")
+
+    import torch
+    from thrust_amd import capi
+    if not torch.cuda.is_available():
+        raise SystemExit("bench.py needs a GPU")
+    capi.load()  # raises if the HIP library is missing: there is no fallback
+
+    ms_sort, pass_ms, kernels_ms = bench_sort(torch, capi, args.steps, args.warmup)
+    ms_reduce, ms_scan = bench_c1(torch, capi, args.steps, args.warmup)
+    torch.cuda.empty_cache()
+
+    n = N_SORT
+    gkeys = n / ms_sort / 1e6
+    pass_bytes = 2.0 * 4.0 * n  # keys read + keys written by one digit-binning pass
+    pass_gbs = pass_bytes / pass_ms / 1e6
+    line = {
+        "metric": "sort Gkeys/s (2^28 u32) + scan/reduce GB/s as % of HBM peak, 1 GPU",
+        "value": round(gkeys, 3),
+        "unit": "Gkeys/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_sort, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "u32",
+        "data": "synthetic",
+        "config": {"workload": "thrust::sort, N=2^28 uint32 keys uniform over the full range (seeded), "
+                               "in place, keys resident in HBM"},
+        "sort_model_bytes_pct_of_peak": round(36.0 * n / ms_sort / 1e6 / HBM_PEAK_GBS * 100, 2),
+        "sort_kernels_ms": {k: round(v, 4) for k, v in kernels_ms.items()},
+        "reduce_i32_2p28": {"ms": round(ms_reduce, 4), "GBps": round(4.0 * N_C1 / ms_reduce / 1e6, 1),
+                            "pct_of_peak": round(4.0 * N_C1 / ms_reduce / 1e6 / HBM_PEAK_GBS * 100, 2)},
+        "inclusive_scan_i32_2p28": {"ms": round(ms_scan, 4), "GBps": round(8.0 * N_C1 / ms_scan / 1e6, 1),
+                                    "pct_of_peak": round(8.0 * N_C1 / ms_scan / 1e6 / HBM_PEAK_GBS * 100, 2)},
+        "roofline": {"bound": "hbm", "kernel": "onesweep_pass (one of 4 per sort)",
+                     "achieved": round(pass_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(pass_gbs / HBM_PEAK_GBS, 4), "traffic": PASS_TRAFFIC_BYTES,
+                     "launch_ms": round(pass_ms, 4)},
+    }
+    if not args.no_cpu_baseline:
+        line["cpu_baseline"] = cpu_baseline()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

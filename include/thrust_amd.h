@@ -128,6 +128,15 @@ int thrust_amd_temp_trim(void);
 /* Bytes currently held by the arena (cached + handed out). */
 size_t thrust_amd_temp_bytes_held(void);
 
+/* Per-kernel timing, a debugging aid in the place of the reference's THRUST_DEBUG_SYNC
+ * launch log (thrust/system/cuda/config.h:65-69, core/agent_launcher.h:518-535).  While
+ * enabled, every kernel the library launches is bracketed by two events on its stream.
+ * `collect` waits for the recorded events, writes one line "label launches total_ms" per
+ * kernel label into text (NUL-terminated, truncated to capacity; *needed = full size) and
+ * forgets them.  Not meant to be left on: it creates two events per launch. */
+int thrust_amd_profile_enable(int on);
+int thrust_amd_profile_collect(char* text, size_t capacity, size_t* needed);
+
 /* ------------------------------------------------------------------- reduce */
 
 /* *d_out = init OP in[0] OP ... OP in[n-1]; accumulator type = dtype.

@@ -46,6 +46,8 @@ SIGNATURES = {
     "thrust_amd_temp_release": (_int, [_vp, _vp]),
     "thrust_amd_temp_trim": (_int, []),
     "thrust_amd_temp_bytes_held": (_sz, []),
+    "thrust_amd_profile_enable": (_int, [_int]),
+    "thrust_amd_profile_collect": (_int, [_c.c_char_p, _sz, _szp]),
     "thrust_amd_reduce": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp, _vp, _vp]),
     "thrust_amd_inclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _vp]),
     "thrust_amd_exclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _vp, _vp]),
@@ -166,6 +168,23 @@ def _run(fn_name, temp, call):
     tptr = temp.ensure(lambda t, b: call(fn, t, b))
     check(call(fn, tptr, ctypes.byref(temp.bytes)), fn_name)
     return temp
+
+
+def profile_enable(on=True):
+    check(load().thrust_amd_profile_enable(int(on)), "profile_enable")
+
+
+def profile_collect():
+    """Returns {label: (launches, total_ms)} for the kernels launched since the last call."""
+    lib = load()
+    buf = ctypes.create_string_buffer(1 << 16)
+    need = ctypes.c_size_t(0)
+    check(lib.thrust_amd_profile_collect(buf, len(buf), ctypes.byref(need)), "profile_collect")
+    out = {}
+    for line in buf.value.decode().splitlines():
+        label, launches, ms = line.split()
+        out[label] = (int(launches), float(ms))
+    return out
 
 
 def reduce(x, op=PLUS, init=0, temp=None, out=None):

@@ -27,6 +27,7 @@
 // thrust/system/cuda/detail/sort.h:1326-1508.
 #include "common.hpp"
 #include "dispatch.hpp"
+#include "launch.hpp"
 
 namespace ta {
 
@@ -160,8 +161,8 @@ static void launch_histogram(int passes, uint32_t blocks, hipStream_t stream, co
                              uint32_t* hist) {
 #define TA_HIST_CASE(NP)                                                                       \
   case NP:                                                                                     \
-    hipLaunchKernelGGL((sort_histogram_kernel<K, NP>), dim3(blocks), dim3(HIST_BLOCK), 0,      \
-                       stream, keys, n, codec, geo, hist);                                     \
+    TA_LAUNCH("sort_histogram", \
+                       stream, (sort_histogram_kernel<K, NP>), dim3(blocks), dim3(HIST_BLOCK), keys, n, codec, geo, hist);                                     \
     break;
   switch (passes) {
     TA_HIST_CASE(1) TA_HIST_CASE(2) TA_HIST_CASE(3) TA_HIST_CASE(4)
@@ -578,8 +579,7 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
   {
     uint64_t blocks = (zero_words + 255) / 256;
     if (blocks > (uint64_t)NUM_CU * 8) blocks = (uint64_t)NUM_CU * 8;
-    hipLaunchKernelGGL(sort_init_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, zero,
-                       (uint64_t)zero_words);
+    TA_LAUNCH("sort_init", stream, sort_init_kernel, dim3((uint32_t)blocks), dim3(256), zero, (uint64_t)zero_words);
     TA_CHECK_LAUNCH();
   }
   {
@@ -589,22 +589,16 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
     launch_histogram<K>(geo.passes, (uint32_t)blocks, stream, (const K*)keys_a, n, codec, geo, hist);
     TA_CHECK_LAUNCH();
   }
-  hipLaunchKernelGGL(sort_scan_kernel, dim3(1), dim3(RADIX_SIZE), 0, stream, hist, (uint32_t)n, geo,
-                     ctl);
+  TA_LAUNCH("sort_scan", stream, sort_scan_kernel, dim3(1), dim3(RADIX_SIZE), hist, (uint32_t)n, geo, ctl);
   TA_CHECK_LAUNCH();
   for (int p = 0; p < geo.passes; ++p) {
-    hipLaunchKernelGGL((onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS>),
-                       dim3((uint32_t)tiles), dim3(Plan::BLOCK), 0, stream, keys_a, keys_b, vals_a,
-                       vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE,
-                       status + (size_t)p * tiles * RADIX_SIZE, tickets + p, (const SortCtl*)ctl);
+    TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + (size_t)p * tiles * RADIX_SIZE, tickets + p, (const SortCtl*)ctl);
     TA_CHECK_LAUNCH();
   }
   {
     uint64_t blocks = (n + 255) / 256;
     if (blocks > (uint64_t)NUM_CU * 8) blocks = (uint64_t)NUM_CU * 8;
-    hipLaunchKernelGGL((sort_copy_back_kernel<K, V, HAS_VALUES>), dim3((uint32_t)blocks), dim3(256),
-                       0, stream, keys_a, (const K*)keys_b, vals_a, (const V*)vals_b, n,
-                       (const SortCtl*)ctl);
+    TA_LAUNCH("sort_copy_back", stream, (sort_copy_back_kernel<K, V, HAS_VALUES>), dim3((uint32_t)blocks), dim3(256), keys_a, (const K*)keys_b, vals_a, (const V*)vals_b, n, (const SortCtl*)ctl);
     TA_CHECK_LAUNCH();
   }
   return 0;

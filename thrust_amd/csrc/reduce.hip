@@ -11,6 +11,7 @@
 // (thrust/system/cuda/detail/reduce.h:151-665) and cub::DispatchReduce (:946-954).
 #include "common.hpp"
 #include "dispatch.hpp"
+#include "launch.hpp"
 
 namespace ta {
 
@@ -95,20 +96,16 @@ struct ReduceLaunch {
     const uint32_t grid = reduce_grid(n, sizeof(T));
     const T* src = static_cast<const T*>(in);
     if (n == 0) {
-      hipLaunchKernelGGL((reduce_final_kernel<T, Op>), dim3(1), dim3(REDUCE_BLOCK), 0, stream,
-                         partials, 0u, init_v, static_cast<T*>(d_out));
+      TA_LAUNCH("reduce_final", stream, (reduce_final_kernel<T, Op>), dim3(1), dim3(REDUCE_BLOCK), partials, 0u, init_v, static_cast<T*>(d_out));
       TA_CHECK_LAUNCH();
       return 0;
     }
     if (is_aligned16(in))
-      hipLaunchKernelGGL((reduce_partials_kernel<T, Op, true>), dim3(grid), dim3(REDUCE_BLOCK), 0,
-                         stream, src, n, partials);
+      TA_LAUNCH("reduce_partials", stream, (reduce_partials_kernel<T, Op, true>), dim3(grid), dim3(REDUCE_BLOCK), src, n, partials);
     else
-      hipLaunchKernelGGL((reduce_partials_kernel<T, Op, false>), dim3(grid), dim3(REDUCE_BLOCK), 0,
-                         stream, src, n, partials);
+      TA_LAUNCH("reduce_partials", stream, (reduce_partials_kernel<T, Op, false>), dim3(grid), dim3(REDUCE_BLOCK), src, n, partials);
     TA_CHECK_LAUNCH();
-    hipLaunchKernelGGL((reduce_final_kernel<T, Op>), dim3(1), dim3(REDUCE_BLOCK), 0, stream,
-                       partials, grid, init_v, static_cast<T*>(d_out));
+    TA_LAUNCH("reduce_final", stream, (reduce_final_kernel<T, Op>), dim3(1), dim3(REDUCE_BLOCK), partials, grid, init_v, static_cast<T*>(d_out));
     TA_CHECK_LAUNCH();
     return 0;
   }

@@ -3,8 +3,15 @@
 // allocate or block; every compute entry point works on caller-owned memory.
 #include "common.hpp"
 #include "dispatch.hpp"
+#include "launch.hpp"
 
+#include "launch.hpp"
+
+#include <atomic>
+#include <cstdio>
+#include <cstring>
 #include <map>
+#include <string>
 #include <mutex>
 #include <vector>
 
@@ -102,8 +109,7 @@ TA_EXPORT int thrust_amd_fill(void* dst, uint64_t n, size_t elem_bytes, const vo
     uint64_t blocks = (vecs + 255) / 256;
     const uint64_t cap = (uint64_t)NUM_CU * 16;
     if (blocks > cap) blocks = cap;
-    hipLaunchKernelGGL((fill_kernel<U>), dim3((uint32_t)blocks), dim3(256), 0, (hipStream_t)stream,
-                       static_cast<U*>(dst), n, v);
+    TA_LAUNCH("fill", (hipStream_t)stream, (fill_kernel<U>), dim3((uint32_t)blocks), dim3(256), static_cast<U*>(dst), n, v);
     TA_CHECK_LAUNCH();
     return 0;
   });
@@ -235,4 +241,91 @@ TA_EXPORT size_t thrust_amd_temp_bytes_held(void) {
   Arena& a = arena();
   std::lock_guard<std::mutex> g(a.mu);
   return a.held;
+}
+
+// ------------------------------------------------------------------ per-kernel timing
+namespace ta {
+
+struct ProfileRecord {
+  const char* label;
+  hipEvent_t begin, end;
+};
+
+struct Profile {
+  std::mutex mu;
+  std::vector<ProfileRecord> records;
+  hipEvent_t pending = nullptr;
+};
+
+static std::atomic<int> g_profile_on{0};
+static Profile& profile() {
+  static Profile* p = new Profile;
+  return *p;
+}
+
+bool profile_on() { return g_profile_on.load(std::memory_order_relaxed) != 0; }
+
+void profile_mark(const char* label, hipStream_t stream, bool begin) {
+  Profile& p = profile();
+  std::lock_guard<std::mutex> g(p.mu);
+  hipEvent_t ev = nullptr;
+  if (hipEventCreate(&ev) != hipSuccess) return;
+  (void)hipEventRecord(ev, stream);
+  if (begin) {
+    p.pending = ev;
+  } else {
+    p.records.push_back(ProfileRecord{label, p.pending, ev});
+    p.pending = nullptr;
+  }
+}
+
+}  // namespace ta
+
+TA_EXPORT int thrust_amd_profile_enable(int on) {
+  ta::g_profile_on.store(on ? 1 : 0);
+  return 0;
+}
+
+TA_EXPORT int thrust_amd_profile_collect(char* text, size_t capacity, size_t* needed) {
+  using namespace ta;
+  Profile& p = profile();
+  std::vector<ProfileRecord> recs;
+  {
+    std::lock_guard<std::mutex> g(p.mu);
+    recs.swap(p.records);
+  }
+  // label -> (launches, total ms), in order of first appearance
+  std::vector<std::pair<const char*, std::pair<uint64_t, double>>> agg;
+  int rc = 0;
+  for (auto& r : recs) {
+    float ms = 0.f;
+    hipError_t e = hipEventSynchronize(r.end);
+    if (e == hipSuccess) e = hipEventElapsedTime(&ms, r.begin, r.end);
+    if (e != hipSuccess && rc == 0) rc = (int)e;
+    (void)hipEventDestroy(r.begin);
+    (void)hipEventDestroy(r.end);
+    bool found = false;
+    for (auto& a : agg)
+      if (std::string(a.first) == r.label) {
+        a.second.first++;
+        a.second.second += ms;
+        found = true;
+        break;
+      }
+    if (!found) agg.push_back({r.label, {1, (double)ms}});
+  }
+  std::string out;
+  for (auto& a : agg) {
+    char line[160];
+    snprintf(line, sizeof line, "%s %llu %.6f\n", a.first, (unsigned long long)a.second.first,
+             a.second.second);
+    out += line;
+  }
+  if (needed) *needed = out.size() + 1;
+  if (text && capacity) {
+    const size_t nbytes = out.size() < capacity - 1 ? out.size() : capacity - 1;
+    memcpy(text, out.data(), nbytes);
+    text[nbytes] = 0;
+  }
+  return rc;
 }

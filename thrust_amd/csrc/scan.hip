@@ -14,6 +14,7 @@
 // from thrust/system/cuda/detail/scan.h:55-200.
 #include "common.hpp"
 #include "dispatch.hpp"
+#include "launch.hpp"
 
 namespace ta {
 
@@ -181,17 +182,14 @@ struct ScanLaunch {
     uint32_t* ticket = reinterpret_cast<uint32_t*>(static_cast<char*>(temp) + off_ticket);
     uint64_t* status = reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + off_status);
     const uint64_t words = tiles * W;
-    hipLaunchKernelGGL(tile_state_init_kernel, dim3((uint32_t)((words + 255) / 256)), dim3(256), 0,
-                       stream, status, words, ticket, 1u);
+    TA_LAUNCH("tile_state_init", stream, tile_state_init_kernel, dim3((uint32_t)((words + 255) / 256)), dim3(256), status, words, ticket, 1u);
     TA_CHECK_LAUNCH();
     const T* src = static_cast<const T*>(in);
     T* dst = static_cast<T*>(out);
     if (is_aligned16(in) && is_aligned16(out))
-      hipLaunchKernelGGL((scan_kernel<T, Op, EXCLUSIVE, true, Shape>), dim3((uint32_t)tiles),
-                         dim3(Shape::BLOCK), 0, stream, src, dst, n, init_v, status, ticket);
+      TA_LAUNCH("scan", stream, (scan_kernel<T, Op, EXCLUSIVE, true, Shape>), dim3((uint32_t)tiles), dim3(Shape::BLOCK), src, dst, n, init_v, status, ticket);
     else
-      hipLaunchKernelGGL((scan_kernel<T, Op, EXCLUSIVE, false, Shape>), dim3((uint32_t)tiles),
-                         dim3(Shape::BLOCK), 0, stream, src, dst, n, init_v, status, ticket);
+      TA_LAUNCH("scan", stream, (scan_kernel<T, Op, EXCLUSIVE, false, Shape>), dim3((uint32_t)tiles), dim3(Shape::BLOCK), src, dst, n, init_v, status, ticket);
     TA_CHECK_LAUNCH();
     return 0;
   }
