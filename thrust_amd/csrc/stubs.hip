@@ -1,11 +1,6 @@
 // Entry points whose kernels are not written yet: they report hipErrorNotSupported.
 #include "common.hpp"
 #define NS return (int)hipErrorNotSupported
-TA_EXPORT int thrust_amd_copy_if(void*, size_t*, const void*, const void*, void*, uint64_t*, uint64_t, size_t, int, int, const void*, void*) { NS; }
-TA_EXPORT int thrust_amd_partition_copy(void*, size_t*, const void*, const void*, void*, void*, uint64_t*, uint64_t, size_t, int, int, const void*, void*) { NS; }
-TA_EXPORT int thrust_amd_stable_partition(void*, size_t*, void*, const void*, uint64_t*, uint64_t, size_t, int, int, const void*, void*) { NS; }
-TA_EXPORT int thrust_amd_unique(void*, size_t*, const void*, void*, uint64_t*, uint64_t, int, void*) { NS; }
-TA_EXPORT int thrust_amd_unique_by_key(void*, size_t*, const void*, const void*, void*, void*, uint64_t*, uint64_t, int, size_t, void*) { NS; }
 TA_EXPORT int thrust_amd_reduce_by_key(void*, size_t*, const void*, const void*, void*, void*, uint64_t*, uint64_t, int, int, int, void*) { NS; }
 TA_EXPORT int thrust_amd_merge(void*, size_t*, const void*, uint64_t, const void*, uint64_t, void*, int, int, void*) { NS; }
 TA_EXPORT int thrust_amd_merge_by_key(void*, size_t*, const void*, uint64_t, const void*, uint64_t, const void*, const void*, void*, void*, int, size_t, int, void*) { NS; }
