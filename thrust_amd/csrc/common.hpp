@@ -156,11 +156,17 @@ TA_DEVICE T dpp_move(T old, T src) {
     __builtin_memcpy(&out, &r, sizeof(T));
     return out;
   } else {
-    static_assert(sizeof(T) == 8, "dpp_move: unsupported size");
-    uint64_t o = bit_cast<uint64_t>(old), s = bit_cast<uint64_t>(src);
-    uint32_t lo = (uint32_t)__builtin_amdgcn_update_dpp((int)(uint32_t)o, (int)(uint32_t)s, CTRL, ROW_MASK, BANK_MASK, false);
-    uint32_t hi = (uint32_t)__builtin_amdgcn_update_dpp((int)(uint32_t)(o >> 32), (int)(uint32_t)(s >> 32), CTRL, ROW_MASK, BANK_MASK, false);
-    return bit_cast<T>(((uint64_t)hi << 32) | lo);
+    static_assert(sizeof(T) % 4 == 0, "dpp_move: size must be a multiple of 4 bytes");
+    constexpr int WORDS = sizeof(T) / 4;
+    uint32_t o[WORDS], s[WORDS], r[WORDS];
+    __builtin_memcpy(o, &old, sizeof(T));
+    __builtin_memcpy(s, &src, sizeof(T));
+#pragma unroll
+    for (int i = 0; i < WORDS; ++i)
+      r[i] = (uint32_t)__builtin_amdgcn_update_dpp((int)o[i], (int)s[i], CTRL, ROW_MASK, BANK_MASK, false);
+    T out;
+    __builtin_memcpy(&out, r, sizeof(T));
+    return out;
   }
 }
 
@@ -174,10 +180,15 @@ TA_DEVICE T readlane(T v, int lane) {
     __builtin_memcpy(&out, &r, sizeof(T));
     return out;
   } else {
-    uint64_t s = bit_cast<uint64_t>(v);
-    uint32_t lo = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)s, lane);
-    uint32_t hi = (uint32_t)__builtin_amdgcn_readlane((int)(uint32_t)(s >> 32), lane);
-    return bit_cast<T>(((uint64_t)hi << 32) | lo);
+    static_assert(sizeof(T) % 4 == 0, "readlane: size must be a multiple of 4 bytes");
+    constexpr int WORDS = sizeof(T) / 4;
+    uint32_t s[WORDS], r[WORDS];
+    __builtin_memcpy(s, &v, sizeof(T));
+#pragma unroll
+    for (int i = 0; i < WORDS; ++i) r[i] = (uint32_t)__builtin_amdgcn_readlane((int)s[i], lane);
+    T out;
+    __builtin_memcpy(&out, r, sizeof(T));
+    return out;
   }
 }
 

@@ -96,7 +96,7 @@ def c4_segments(n, mean, seed=4):
         start += c
         lens = np.floor(np.log(u) / log1mp).astype(np.int64) + 1
         ends = np.cumsum(lens)
-        take = int(np.searchsorted(ends, n - filled, side="left")) + 1
+        take = min(int(np.searchsorted(ends, n - filled, side="left")) + 1, c)
         lens = lens[:take]
         ids = np.repeat(np.arange(run, run + take, dtype=np.int64), lens)[: n - filled]
         keys[filled:filled + ids.size] = ids.astype(np.int32)
