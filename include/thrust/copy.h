@@ -1,0 +1,196 @@
+// thrust::copy, thrust::copy_n and thrust::copy_if.
+//
+// copy moves trivially copyable elements inside one system or across the two
+// (the reference: thrust/system/cuda/detail/internal/copy_cross_system.h:50-200,
+// util.h:107-162).  copy_if is a stable compaction, with or without a stencil
+// (thrust/system/detail/generic/copy_if.inl:97-154); on the device system the predicate
+// must be one of the recognised forms listed in thrust/functional.h.
+#pragma once
+#include <algorithm>
+#include <vector>
+
+#include <thrust/functional.h>
+#include <thrust/system/hip/detail/backend.h>
+
+namespace thrust {
+
+namespace detail {
+// Copy n elements between any two of {host, device} given raw element addresses.
+template <typename T>
+inline void copy_raw(const T* src, bool src_device, T* dst, bool dst_device, std::size_t n, void* stream) {
+  if (n == 0) return;
+  using thrust::system::hip::detail::throw_on_error;
+  if (!src_device && !dst_device) {
+    std::copy(src, src + n, dst);
+  } else if (src_device && dst_device) {
+    throw_on_error(thrust_amd_memcpy(dst, src, n * sizeof(T), THRUST_AMD_D2D, stream), "copy (device to device)");
+    throw_on_error(thrust_amd_stream_synchronize(stream), "copy: synchronize");
+  } else {
+    throw_on_error(thrust_amd_memcpy(dst, src, n * sizeof(T), src_device ? THRUST_AMD_D2H : THRUST_AMD_H2D, stream),
+                   "copy (across systems)");
+  }
+}
+
+template <typename In, typename Out>
+inline Out copy_dispatch(In first, In last, Out result, bool in_device, bool out_device, void* stream) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  typedef typename iterator_value<Out>::type U;
+  const std::size_t n = (std::size_t)std::distance(first, last);
+  if (n == 0) return result;
+  if (!in_device && !out_device) return std::copy(first, last, result);
+  static_assert(std::is_trivially_copyable<T>::value, "thrust::copy involving the device needs trivially copyable elements");
+  if (std::is_same<T, U>::value && (in_device || is_contiguous_host_iterator<In>::value) &&
+      (out_device || is_contiguous_host_iterator<Out>::value)) {
+    copy_raw<T>(raw(first), in_device, reinterpret_cast<T*>(raw(result)), out_device, n, stream);
+  } else if (in_device) {
+    // device -> host with conversion or a non-contiguous destination: stage on the host
+    std::vector<T> staged(n);
+    copy_raw<T>(raw(first), true, staged.data(), false, n, stream);
+    if (out_device) {
+      std::vector<U> converted(staged.begin(), staged.end());
+      copy_raw<U>(converted.data(), false, reinterpret_cast<U*>(raw(result)), true, n, stream);
+    } else {
+      std::copy(staged.begin(), staged.end(), result);
+    }
+  } else {
+    std::vector<U> staged(first, last);
+    copy_raw<U>(staged.data(), false, reinterpret_cast<U*>(raw(result)), true, n, stream);
+  }
+  return result + n;
+}
+}  // namespace detail
+
+template <typename D, typename In, typename Out, typename Pred>
+Out copy_if(const detail::execution_policy_base<D>& exec, In first, In last, Out result, Pred pred);
+template <typename D, typename In, typename St, typename Out, typename Pred>
+Out copy_if(const detail::execution_policy_base<D>& exec, In first, In last, St stencil, Out result, Pred pred);
+
+namespace system {
+namespace cpp {
+template <typename D, typename In, typename Out>
+Out copy(execution_policy<D>&, In first, In last, Out result) {
+  return thrust::detail::copy_dispatch(first, last, result, thrust::detail::is_device_iterator<In>::value,
+                                       thrust::detail::is_device_iterator<Out>::value, nullptr);
+}
+template <typename D, typename In, typename St, typename Out, typename Pred>
+Out copy_if(execution_policy<D>&, In first, In last, St stencil, Out result, Pred pred) {
+  for (; first != last; ++first, ++stencil)
+    if (pred(*stencil)) { *result = *first; ++result; }
+  return result;
+}
+template <typename D, typename In, typename Out, typename Pred>
+Out copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred) {
+  return copy_if(exec, first, last, first, result, pred);
+}
+}  // namespace cpp
+
+namespace hip {
+template <typename D, typename In, typename Out>
+Out copy(execution_policy<D>& exec, In first, In last, Out result) {
+  // explicit device policy: raw pointers are device pointers
+  const bool in_dev = thrust::detail::is_device_iterator<In>::value || std::is_pointer<In>::value;
+  const bool out_dev = thrust::detail::is_device_iterator<Out>::value || std::is_pointer<Out>::value;
+  return thrust::detail::copy_dispatch(first, last, result, in_dev, out_dev, detail::stream_of(exec));
+}
+
+namespace detail {
+// Shared by copy_if and the partition family: runs `entry` (one of the three selection
+// entry points bound by the caller) and returns the number of selected elements.
+template <typename Tested, typename Pred, typename Call>
+inline uint64_t run_selection(void* stream, const Pred& pred, const char* what, Call call) {
+  static_assert(is_abi_type<Tested>::value,
+                "selection on the device system needs an arithmetic type to test");
+  static_assert(unary_pred<Pred, Tested>::supported,
+                "selection on the device system supports placeholder comparisons (_1 < t, ...), "
+                "thrust::identity and thrust::logical_not as predicate");
+  const int cmp = unary_pred<Pred, Tested>::cmp(pred);
+  const Tested thr = unary_pred<Pred, Tested>::threshold(pred);
+  temp_storage temp(stream);
+  std::size_t need = 0;
+  uint64_t* d_num = nullptr;
+  throw_on_error(call((void*)nullptr, &need, d_num, cmp, (const void*)&thr), what);
+  const std::size_t aligned = (need + 255) / 256 * 256;
+  temp.ensure(aligned + 256);
+  d_num = reinterpret_cast<uint64_t*>(static_cast<char*>(temp.ptr()) + aligned);
+  std::size_t bytes = aligned;
+  throw_on_error(call(temp.ptr(), &bytes, d_num, cmp, (const void*)&thr), what);
+  return read_scalar<uint64_t>(d_num, stream, what);
+}
+}  // namespace detail
+
+template <typename D, typename In, typename Out, typename Pred>
+Out copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  static_assert(std::is_same<typename iterator_value<Out>::type, T>::value,
+                "thrust::copy_if on the device system: input and output element types must match");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  const uint64_t cnt = detail::run_selection<T>(stream, pred, "copy_if failed",
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_copy_if(t, b, thrust::detail::raw(first), nullptr, thrust::detail::raw(result), d_num, n,
+                                  sizeof(T), detail::dtype_of<T>::value, cmp, thr, stream);
+      });
+  return result + cnt;
+}
+template <typename D, typename In, typename St, typename Out, typename Pred>
+Out copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
+                "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  const uint64_t cnt = detail::run_selection<S>(stream, pred, "copy_if failed",
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_copy_if(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil),
+                                  thrust::detail::raw(result), d_num, n, sizeof(T), detail::dtype_of<S>::value, cmp,
+                                  thr, stream);
+      });
+  return result + cnt;
+}
+}  // namespace hip
+}  // namespace system
+
+// ------------------------------------------------------------------ copy
+template <typename D, typename In, typename Out>
+Out copy(const detail::execution_policy_base<D>& exec, In first, In last, Out result) {
+  return copy(detail::derived_cast(detail::strip_const(exec)), first, last, result);
+}
+// Without a policy the two iterators may live in different systems.
+template <typename In, typename Out>
+Out copy(In first, In last, Out result) {
+  return thrust::detail::copy_dispatch(first, last, result, detail::is_device_iterator<In>::value,
+                                       detail::is_device_iterator<Out>::value, nullptr);
+}
+template <typename D, typename In, typename Size, typename Out>
+Out copy_n(const detail::execution_policy_base<D>& exec, In first, Size n, Out result) {
+  return thrust::copy(exec, first, first + n, result);
+}
+template <typename In, typename Size, typename Out,
+          typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>
+Out copy_n(In first, Size n, Out result) {
+  return thrust::copy(first, first + n, result);
+}
+
+// ------------------------------------------------------------------ copy_if
+template <typename D, typename In, typename Out, typename Pred>
+Out copy_if(const detail::execution_policy_base<D>& exec, In first, In last, Out result, Pred pred) {
+  return copy_if(detail::derived_cast(detail::strip_const(exec)), first, last, result, pred);
+}
+template <typename D, typename In, typename St, typename Out, typename Pred>
+Out copy_if(const detail::execution_policy_base<D>& exec, In first, In last, St stencil, Out result, Pred pred) {
+  return copy_if(detail::derived_cast(detail::strip_const(exec)), first, last, stencil, result, pred);
+}
+template <typename In, typename Out, typename Pred>
+Out copy_if(In first, In last, Out result, Pred pred) {
+  return thrust::copy_if(detail::policy_for<In>(), first, last, result, pred);
+}
+template <typename In, typename St, typename Out, typename Pred,
+          typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>
+Out copy_if(In first, In last, St stencil, Out result, Pred pred) {
+  return thrust::copy_if(detail::policy_for<In>(), first, last, stencil, result, pred);
+}
+
+}  // namespace thrust

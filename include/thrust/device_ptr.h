@@ -1,0 +1,145 @@
+// thrust::device_ptr<T>, thrust::device_reference<T>, raw_pointer_cast, device_pointer_cast,
+// device_malloc / device_free.
+//
+// A device_ptr is a typed pointer tagged with the device system: algorithms given
+// device_ptr iterators (device_vector::iterator is one) run on the GPU without an
+// explicit policy.  Dereferencing on the host yields a device_reference, a proxy whose
+// reads and writes are one-element copies across the bus -- the reference's
+// tagged_reference over get_value / assign_value
+// (thrust/system/cuda/detail/get_value.h:35-92, assign_value.h:32-100).
+#pragma once
+#include <cstddef>
+#include <iterator>
+#include <type_traits>
+
+#include <thrust/detail/execution_policy.h>
+#include <thrust/system_error.h>
+
+namespace thrust {
+
+template <typename T> class device_ptr;
+
+template <typename T>
+class device_reference {
+ public:
+  typedef typename std::remove_const<T>::type value_type;
+  explicit device_reference(T* p) : ptr_(p) {}
+  device_reference(const device_reference&) = default;
+
+  operator value_type() const {
+    value_type v;
+    system::hip::detail::throw_on_error(
+        thrust_amd_memcpy(&v, ptr_, sizeof(value_type), THRUST_AMD_D2H, nullptr), "device_reference read");
+    return v;
+  }
+  device_reference& operator=(const value_type& v) {
+    system::hip::detail::throw_on_error(
+        thrust_amd_memcpy(const_cast<value_type*>(ptr_), &v, sizeof(value_type), THRUST_AMD_H2D, nullptr),
+        "device_reference write");
+    return *this;
+  }
+  device_reference& operator=(const device_reference& other) { return *this = (value_type)other; }
+  device_ptr<T> operator&() const { return device_ptr<T>(ptr_); }
+#define THRUST_AMD_REF_COMPOUND(OP)                               \
+  device_reference& operator OP##=(const value_type& v) {         \
+    value_type t = *this;                                         \
+    t OP##= v;                                                    \
+    return *this = t;                                             \
+  }
+  THRUST_AMD_REF_COMPOUND(+) THRUST_AMD_REF_COMPOUND(-) THRUST_AMD_REF_COMPOUND(*) THRUST_AMD_REF_COMPOUND(/)
+#undef THRUST_AMD_REF_COMPOUND
+  device_reference& operator++() { return *this += value_type(1); }
+  device_reference& operator--() { return *this -= value_type(1); }
+
+ private:
+  T* ptr_;
+};
+
+template <typename T>
+class device_ptr {
+ public:
+  typedef std::random_access_iterator_tag iterator_category;
+  typedef typename std::remove_const<T>::type value_type;
+  typedef std::ptrdiff_t difference_type;
+  typedef device_ptr pointer;
+  typedef device_reference<T> reference;
+  typedef T element_type;
+  typedef thrust::device_system_tag system_tag;
+
+  device_ptr() : ptr_(nullptr) {}
+  device_ptr(std::nullptr_t) : ptr_(nullptr) {}
+  explicit device_ptr(T* p) : ptr_(p) {}
+  template <typename U, typename = typename std::enable_if<std::is_convertible<U*, T*>::value>::type>
+  device_ptr(const device_ptr<U>& o) : ptr_(o.get()) {}
+
+  T* get() const { return ptr_; }
+  reference operator*() const { return reference(ptr_); }
+  reference operator[](difference_type i) const { return reference(ptr_ + i); }
+  T* operator->() const { return ptr_; }
+  explicit operator bool() const { return ptr_ != nullptr; }
+
+  device_ptr& operator++() { ++ptr_; return *this; }
+  device_ptr operator++(int) { device_ptr t(*this); ++ptr_; return t; }
+  device_ptr& operator--() { --ptr_; return *this; }
+  device_ptr operator--(int) { device_ptr t(*this); --ptr_; return t; }
+  device_ptr& operator+=(difference_type n) { ptr_ += n; return *this; }
+  device_ptr& operator-=(difference_type n) { ptr_ -= n; return *this; }
+  device_ptr operator+(difference_type n) const { return device_ptr(ptr_ + n); }
+  device_ptr operator-(difference_type n) const { return device_ptr(ptr_ - n); }
+  difference_type operator-(const device_ptr& o) const { return ptr_ - o.ptr_; }
+  bool operator==(const device_ptr& o) const { return ptr_ == o.ptr_; }
+  bool operator!=(const device_ptr& o) const { return ptr_ != o.ptr_; }
+  bool operator<(const device_ptr& o) const { return ptr_ < o.ptr_; }
+  bool operator>(const device_ptr& o) const { return ptr_ > o.ptr_; }
+  bool operator<=(const device_ptr& o) const { return ptr_ <= o.ptr_; }
+  bool operator>=(const device_ptr& o) const { return ptr_ >= o.ptr_; }
+
+ private:
+  T* ptr_;
+};
+
+template <>
+class device_ptr<void> {
+ public:
+  device_ptr() : ptr_(nullptr) {}
+  explicit device_ptr(void* p) : ptr_(p) {}
+  void* get() const { return ptr_; }
+
+ private:
+  void* ptr_;
+};
+
+template <typename T>
+inline device_ptr<T> operator+(std::ptrdiff_t n, const device_ptr<T>& p) { return p + n; }
+
+template <typename T>
+inline device_ptr<T> device_pointer_cast(T* p) { return device_ptr<T>(p); }
+template <typename T>
+inline device_ptr<T> device_pointer_cast(const device_ptr<T>& p) { return p; }
+
+template <typename T>
+inline T* raw_pointer_cast(const device_ptr<T>& p) { return p.get(); }
+template <typename T>
+inline T* raw_pointer_cast(T* p) { return p; }
+template <typename T>
+inline T* raw_pointer_cast(const device_reference<T>& r) { return (&r).get(); }
+
+// Allocation through the device system (cuda_cub::malloc / free in the reference,
+// thrust/system/cuda/detail/malloc_and_free.h:51-100).
+inline device_ptr<void> device_malloc(std::size_t bytes) {
+  void* p = nullptr;
+  const int rc = thrust_amd_malloc(&p, bytes);
+  if (rc != 0) throw system::detail::bad_alloc(thrust_amd_error_string(rc));
+  return device_ptr<void>(p);
+}
+template <typename T>
+inline device_ptr<T> device_malloc(std::size_t n) {
+  return device_ptr<T>(static_cast<T*>(device_malloc(n * sizeof(T)).get()));
+}
+template <typename T>
+inline void device_free(device_ptr<T> p) {
+  system::hip::detail::throw_on_error(thrust_amd_free(const_cast<void*>(static_cast<const void*>(p.get()))),
+                                      "device_free");
+}
+
+}  // namespace thrust

@@ -1,0 +1,228 @@
+// thrust::device_vector<T>: a resizable array in device memory.
+//
+// The subset of the reference's vector_base that code on the sort / scan / reduce /
+// select / merge path uses (thrust/device_vector.h:54-64, thrust/detail/vector_base.inl):
+// construction from a size, a size and a value, a host range, a std::vector / host_vector
+// or another device_vector; begin/end/data/size/resize/clear/swap; operator[] / front /
+// back through device_reference; assignment across systems.  Elements must be trivially
+// copyable: storage is raw device memory, filled and copied by the device system.
+#pragma once
+#include <cstddef>
+#include <iterator>
+#include <type_traits>
+#include <utility>
+#include <vector>
+
+#include <thrust/device_ptr.h>
+#include <thrust/host_vector.h>
+
+namespace thrust {
+
+template <typename T>
+class device_vector {
+  static_assert(std::is_trivially_copyable<T>::value,
+                "thrust::device_vector: elements must be trivially copyable");
+
+ public:
+  typedef T value_type;
+  typedef std::size_t size_type;
+  typedef std::ptrdiff_t difference_type;
+  typedef device_ptr<T> pointer;
+  typedef device_ptr<const T> const_pointer;
+  typedef device_ptr<T> iterator;
+  typedef device_ptr<const T> const_iterator;
+  typedef device_reference<T> reference;
+  typedef device_reference<const T> const_reference;
+
+  device_vector() : data_(nullptr), size_(0), capacity_(0) {}
+  explicit device_vector(size_type n) : device_vector() { resize(n); }
+  device_vector(size_type n, const T& value) : device_vector() { resize(n, value); }
+  device_vector(const device_vector& o) : device_vector() { assign_device(o.data_, o.size_); }
+  device_vector(device_vector&& o) noexcept : data_(o.data_), size_(o.size_), capacity_(o.capacity_) {
+    o.data_ = nullptr;
+    o.size_ = o.capacity_ = 0;
+  }
+  template <typename A>
+  device_vector(const std::vector<T, A>& h) : device_vector() { assign_host(h.data(), h.size()); }
+  template <typename InputIterator,
+            typename = typename std::iterator_traits<InputIterator>::iterator_category>
+  device_vector(InputIterator first, InputIterator last) : device_vector() { assign(first, last); }
+  ~device_vector() { release(); }
+
+  device_vector& operator=(const device_vector& o) {
+    if (this != &o) assign_device(o.data_, o.size_);
+    return *this;
+  }
+  device_vector& operator=(device_vector&& o) noexcept {
+    swap(o);
+    return *this;
+  }
+  template <typename A>
+  device_vector& operator=(const std::vector<T, A>& h) {
+    assign_host(h.data(), h.size());
+    return *this;
+  }
+
+  template <typename InputIterator>
+  void assign(InputIterator first, InputIterator last) { assign_range(first, last, 0); }
+  void assign(size_type n, const T& value) {
+    size_ = 0;
+    resize(n, value);
+  }
+
+  iterator begin() { return iterator(data_); }
+  iterator end() { return iterator(data_ + size_); }
+  const_iterator begin() const { return const_iterator(data_); }
+  const_iterator end() const { return const_iterator(data_ + size_); }
+  const_iterator cbegin() const { return begin(); }
+  const_iterator cend() const { return end(); }
+  pointer data() { return pointer(data_); }
+  const_pointer data() const { return const_pointer(data_); }
+  size_type size() const { return size_; }
+  size_type capacity() const { return capacity_; }
+  bool empty() const { return size_ == 0; }
+
+  reference operator[](size_type i) { return reference(data_ + i); }
+  const_reference operator[](size_type i) const { return const_reference(data_ + i); }
+  reference front() { return reference(data_); }
+  reference back() { return reference(data_ + size_ - 1); }
+
+  void reserve(size_type n) {
+    if (n <= capacity_) return;
+    T* fresh = allocate(n);
+    if (size_) copy_raw(fresh, data_, size_, THRUST_AMD_D2D);
+    sync();
+    free_raw(data_);
+    data_ = fresh;
+    capacity_ = n;
+  }
+  void resize(size_type n) { resize(n, T()); }
+  void resize(size_type n, const T& value) {
+    if (n > capacity_) reserve(n);
+    if (n > size_) {
+      system::hip::detail::throw_on_error(
+          thrust_amd_fill(data_ + size_, n - size_, sizeof(T), &value, nullptr), "device_vector fill");
+      sync();
+    }
+    size_ = n;
+  }
+  void clear() { size_ = 0; }
+  void shrink_to_fit() {
+    if (size_ == capacity_) return;
+    device_vector tmp(*this);
+    swap(tmp);
+  }
+  void push_back(const T& v) {
+    if (size_ == capacity_) reserve(capacity_ ? 2 * capacity_ : 16);
+    copy_raw(data_ + size_, &v, 1, THRUST_AMD_H2D);
+    ++size_;
+  }
+  void pop_back() { --size_; }
+  iterator erase(iterator first, iterator last) {
+    const size_type tail = end() - last;
+    if (tail && first != last) {
+      // overlapping move towards the front: stage through a copy of the tail
+      device_vector tmp(last, end());
+      copy_raw(first.get(), tmp.data_, tail, THRUST_AMD_D2D);
+      sync();
+    }
+    size_ -= (last - first);
+    return first;
+  }
+  void swap(device_vector& o) noexcept {
+    std::swap(data_, o.data_);
+    std::swap(size_, o.size_);
+    std::swap(capacity_, o.capacity_);
+  }
+
+  // Host copy of the contents.
+  void copy_to_host(T* dst) const {
+    if (size_) copy_raw(dst, data_, size_, THRUST_AMD_D2H);
+  }
+
+ private:
+  template <typename U> friend class device_vector;
+
+  static T* allocate(size_type n) {
+    if (n == 0) return nullptr;
+    if (n > (~size_type(0)) / sizeof(T)) throw system::detail::bad_alloc("device_vector: size overflow");
+    void* p = nullptr;
+    const int rc = thrust_amd_malloc(&p, n * sizeof(T));
+    if (rc != 0) throw system::detail::bad_alloc(thrust_amd_error_string(rc));
+    return static_cast<T*>(p);
+  }
+  static void free_raw(T* p) {
+    if (p) (void)thrust_amd_free(p);
+  }
+  static void sync() {
+    system::hip::detail::throw_on_error(thrust_amd_stream_synchronize(nullptr), "device_vector synchronize");
+  }
+  static void copy_raw(T* dst, const T* src, size_type n, int kind) {
+    system::hip::detail::throw_on_error(thrust_amd_memcpy(dst, src, n * sizeof(T), kind, nullptr),
+                                        "device_vector copy");
+  }
+  void release() {
+    free_raw(data_);
+    data_ = nullptr;
+    size_ = capacity_ = 0;
+  }
+  void assign_host(const T* src, size_type n) {
+    size_ = 0;
+    if (n > capacity_) reserve(n);
+    if (n) copy_raw(data_, src, n, THRUST_AMD_H2D);
+    size_ = n;
+  }
+  void assign_device(const T* src, size_type n) {
+    size_ = 0;
+    if (n > capacity_) reserve(n);
+    if (n) {
+      copy_raw(data_, src, n, THRUST_AMD_D2D);
+      sync();
+    }
+    size_ = n;
+  }
+  // device range
+  template <typename U>
+  void assign_range(device_ptr<U> first, device_ptr<U> last, int) {
+    static_assert(std::is_same<typename std::remove_const<U>::type, T>::value,
+                  "device_vector: element types of a device range must match");
+    assign_device(first.get(), (size_type)(last - first));
+  }
+  // host range (any input iterator)
+  template <typename It>
+  void assign_range(It first, It last, long) {
+    std::vector<T> staged(first, last);
+    assign_host(staged.data(), staged.size());
+  }
+
+  T* data_;
+  size_type size_, capacity_;
+};
+
+template <typename T>
+inline void swap(device_vector<T>& a, device_vector<T>& b) { a.swap(b); }
+
+template <typename T, typename Alloc>
+host_vector<T, Alloc>::host_vector(const device_vector<T>& d) : base(d.size()) {
+  d.copy_to_host(this->data());
+}
+template <typename T, typename Alloc>
+host_vector<T, Alloc>& host_vector<T, Alloc>::operator=(const device_vector<T>& d) {
+  this->resize(d.size());
+  d.copy_to_host(this->data());
+  return *this;
+}
+
+template <typename T>
+inline bool operator==(const device_vector<T>& a, const device_vector<T>& b) {
+  return host_vector<T>(a) == host_vector<T>(b);
+}
+template <typename T, typename A>
+inline bool operator==(const device_vector<T>& a, const std::vector<T, A>& b) {
+  host_vector<T> h(a);
+  return h.size() == b.size() && std::equal(h.begin(), h.end(), b.begin());
+}
+template <typename T, typename A>
+inline bool operator==(const std::vector<T, A>& a, const device_vector<T>& b) { return b == a; }
+
+}  // namespace thrust

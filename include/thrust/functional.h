@@ -1,0 +1,107 @@
+// Function objects of the front end.  For the device system these types are also
+// dispatch keys: the C ABI knows a closed set of operators, and an algorithm reaches
+// its kernel when the functor type is one of the recognised ones below (the reference
+// applies the same idea to sorting, where only exactly less<Key> / greater<Key> take
+// the radix path, thrust/system/cuda/detail/sort.h:1518-1523).
+//   binary operators   plus, minimum, maximum            (reduce, scans, reduce_by_key)
+//   orderings          less, greater                     (sort, merge)
+//   equivalence        equal_to                          (unique, reduce_by_key)
+//   unary predicates   placeholder comparisons (_1 < t), identity / "is true",
+//                      logical_not                       (copy_if, partition)
+#pragma once
+#include <thrust/detail/config.h>
+
+namespace thrust {
+
+template <typename A, typename R> struct unary_function { typedef A argument_type; typedef R result_type; };
+template <typename A1, typename A2, typename R>
+struct binary_function { typedef A1 first_argument_type; typedef A2 second_argument_type; typedef R result_type; };
+
+#define THRUST_AMD_BINARY_FUNCTOR(NAME, RESULT, EXPR)                                   \
+  template <typename T = void>                                                          \
+  struct NAME {                                                                         \
+    typedef T first_argument_type;                                                      \
+    typedef T second_argument_type;                                                     \
+    typedef RESULT result_type;                                                         \
+    constexpr RESULT operator()(const T& lhs, const T& rhs) const { return EXPR; }      \
+  };                                                                                    \
+  template <>                                                                           \
+  struct NAME<void> {                                                                   \
+    template <typename A, typename B>                                                   \
+    constexpr auto operator()(const A& lhs, const B& rhs) const -> decltype(EXPR) { return EXPR; } \
+  };
+
+THRUST_AMD_BINARY_FUNCTOR(plus, T, lhs + rhs)
+THRUST_AMD_BINARY_FUNCTOR(minus, T, lhs - rhs)
+THRUST_AMD_BINARY_FUNCTOR(multiplies, T, lhs * rhs)
+THRUST_AMD_BINARY_FUNCTOR(equal_to, bool, lhs == rhs)
+THRUST_AMD_BINARY_FUNCTOR(not_equal_to, bool, lhs != rhs)
+THRUST_AMD_BINARY_FUNCTOR(less, bool, lhs < rhs)
+THRUST_AMD_BINARY_FUNCTOR(greater, bool, lhs > rhs)
+THRUST_AMD_BINARY_FUNCTOR(less_equal, bool, lhs <= rhs)
+THRUST_AMD_BINARY_FUNCTOR(greater_equal, bool, lhs >= rhs)
+THRUST_AMD_BINARY_FUNCTOR(maximum, T, (lhs < rhs ? rhs : lhs))
+THRUST_AMD_BINARY_FUNCTOR(minimum, T, (lhs < rhs ? lhs : rhs))
+#undef THRUST_AMD_BINARY_FUNCTOR
+
+template <typename T = void>
+struct identity {
+  typedef T argument_type;
+  typedef T result_type;
+  constexpr const T& operator()(const T& x) const { return x; }
+};
+template <>
+struct identity<void> {
+  template <typename A>
+  constexpr const A& operator()(const A& x) const { return x; }
+};
+
+template <typename T = void>
+struct logical_not {
+  typedef T argument_type;
+  typedef bool result_type;
+  constexpr bool operator()(const T& x) const { return !x; }
+};
+template <typename T = void>
+struct negate {
+  typedef T argument_type;
+  typedef T result_type;
+  constexpr T operator()(const T& x) const { return -x; }
+};
+
+namespace detail {
+// `x CMP value` as a unary predicate; CMP is a thrust_amd_cmp code (0 LT .. 5 NE).
+template <int CMP, typename T>
+struct compare_with {
+  T value;
+  constexpr bool operator()(const T& x) const {
+    return CMP == 0 ? x < value : CMP == 1 ? x <= value : CMP == 2 ? x > value
+         : CMP == 3 ? x >= value : CMP == 4 ? x == value : x != value;
+  }
+  template <typename A>
+  constexpr bool operator()(const A& x) const { return (*this)(static_cast<T>(x)); }
+};
+struct placeholder1 {};
+}  // namespace detail
+
+// Placeholder expressions of the form `_1 < t` (and <=, >, >=, ==, !=), the shape the
+// reference's own code uses for simple predicates (thrust/functional.h placeholders).
+namespace placeholders {
+static const thrust::detail::placeholder1 _1;
+}
+namespace detail {
+#define THRUST_AMD_PLACEHOLDER_CMP(OP, CODE, SWAPPED)                                                  \
+  template <typename T>                                                                                \
+  constexpr compare_with<CODE, T> operator OP(placeholder1, const T& v) { return compare_with<CODE, T>{v}; } \
+  template <typename T>                                                                                \
+  constexpr compare_with<SWAPPED, T> operator OP(const T& v, placeholder1) { return compare_with<SWAPPED, T>{v}; }
+THRUST_AMD_PLACEHOLDER_CMP(<, 0, 2)
+THRUST_AMD_PLACEHOLDER_CMP(<=, 1, 3)
+THRUST_AMD_PLACEHOLDER_CMP(>, 2, 0)
+THRUST_AMD_PLACEHOLDER_CMP(>=, 3, 1)
+THRUST_AMD_PLACEHOLDER_CMP(==, 4, 4)
+THRUST_AMD_PLACEHOLDER_CMP(!=, 5, 5)
+#undef THRUST_AMD_PLACEHOLDER_CMP
+}  // namespace detail
+
+}  // namespace thrust

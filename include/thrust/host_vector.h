@@ -1,0 +1,27 @@
+// thrust::host_vector<T>: a std::vector whose iterators belong to the host system.
+#pragma once
+#include <vector>
+
+#include <thrust/detail/config.h>
+
+namespace thrust {
+
+template <typename T> class device_vector;
+
+template <typename T, typename Alloc = std::allocator<T> >
+class host_vector : public std::vector<T, Alloc> {
+  typedef std::vector<T, Alloc> base;
+
+ public:
+  using base::base;
+  host_vector() : base() {}
+  host_vector(const base& v) : base(v) {}
+  host_vector(const host_vector&) = default;
+  host_vector(host_vector&&) = default;
+  host_vector& operator=(const host_vector&) = default;
+  host_vector& operator=(host_vector&&) = default;
+  host_vector(const device_vector<T>& d);             // defined in device_vector.h
+  host_vector& operator=(const device_vector<T>& d);  // defined in device_vector.h
+};
+
+}  // namespace thrust

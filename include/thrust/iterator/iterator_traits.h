@@ -1,0 +1,66 @@
+// iterator_value / iterator_system / contiguous-range helpers used by the dispatch layer.
+#pragma once
+#include <iterator>
+#include <type_traits>
+#include <vector>
+
+#include <thrust/device_ptr.h>
+
+namespace thrust {
+
+template <typename It>
+struct iterator_value { typedef typename std::iterator_traits<It>::value_type type; };
+template <typename It>
+struct iterator_difference { typedef typename std::iterator_traits<It>::difference_type type; };
+
+// The system an iterator belongs to: device_ptr -> device system, anything else -> host.
+template <typename It>
+struct iterator_system { typedef thrust::host_system_tag type; };
+template <typename T>
+struct iterator_system<device_ptr<T> > { typedef thrust::device_system_tag type; };
+
+namespace detail {
+
+template <typename It> struct is_device_iterator : std::false_type {};
+template <typename T> struct is_device_iterator<device_ptr<T> > : std::true_type {};
+
+// Raw address of the element an iterator points at.  Device iterators are device_ptr or,
+// under an explicit device policy, plain pointers; host iterators must be contiguous
+// (pointers, std::vector / host_vector iterators).
+template <typename T> inline T* raw(const device_ptr<T>& p) { return p.get(); }
+template <typename T> inline T* raw(T* p) { return p; }
+template <typename It>
+inline auto raw(It it) -> typename std::enable_if<
+    !std::is_pointer<It>::value && !is_device_iterator<It>::value,
+    typename std::remove_reference<decltype(*it)>::type*>::type {
+  // never dereferences: callers pass begin() of a non-empty contiguous range or use n == 0
+  return std::addressof(*it);
+}
+
+template <typename It>
+struct is_contiguous_host_iterator
+    : std::integral_constant<bool,
+          std::is_pointer<It>::value ||
+          std::is_same<It, typename std::vector<typename std::iterator_traits<It>::value_type>::iterator>::value ||
+          std::is_same<It, typename std::vector<typename std::iterator_traits<It>::value_type>::const_iterator>::value> {};
+
+template <typename T>
+struct is_execution_policy : std::is_base_of<thrust::detail::execution_policy_marker,
+                                             typename std::remove_cv<typename std::remove_reference<T>::type>::type> {};
+
+// The policy a policy-less call uses for iterators of system tag Tag.
+inline thrust::system::hip::tag& default_policy(thrust::device_system_tag) {
+  static thrust::system::hip::tag t;
+  return t;
+}
+inline thrust::system::cpp::tag& default_policy(thrust::host_system_tag) {
+  static thrust::system::cpp::tag t;
+  return t;
+}
+template <typename It>
+inline auto policy_for() -> decltype(default_policy(typename iterator_system<It>::type())) {
+  return default_policy(typename iterator_system<It>::type());
+}
+
+}  // namespace detail
+}  // namespace thrust

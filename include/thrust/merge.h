@@ -1,0 +1,161 @@
+// thrust::merge and thrust::merge_by_key.
+//
+// Stable merge of two sorted ranges; on ties the elements of the first range come first
+// (thrust/system/detail/sequential/merge.inl:40-71,85-146).  The device system supports
+// arithmetic keys ordered by thrust::less (default) or thrust::greater.
+#pragma once
+#include <thrust/functional.h>
+#include <thrust/pair.h>
+#include <thrust/system/hip/detail/backend.h>
+
+namespace thrust {
+
+template <typename D, typename In1, typename In2, typename Out, typename Comp>
+Out merge(const detail::execution_policy_base<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result,
+          Comp comp);
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
+pair<KOut, VOut> merge_by_key(const detail::execution_policy_base<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1,
+                              V2 vf2, KOut ko, VOut vo, Comp comp);
+
+namespace system {
+namespace detail {
+namespace generic {
+template <typename D, typename In1, typename In2, typename Out>
+Out merge(thrust::execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result) {
+  typedef typename iterator_value<In1>::type K;
+  return thrust::merge(exec, first1, last1, first2, last2, result, thrust::less<K>());
+}
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut>
+pair<KOut, VOut> merge_by_key(thrust::execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2,
+                              KOut ko, VOut vo) {
+  typedef typename iterator_value<K1>::type K;
+  return thrust::merge_by_key(exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, thrust::less<K>());
+}
+}  // namespace generic
+}  // namespace detail
+
+namespace cpp {
+template <typename D, typename In1, typename In2, typename Out, typename Comp>
+Out merge(execution_policy<D>&, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+  while (first1 != last1 && first2 != last2) {
+    if (comp(*first2, *first1)) { *result = *first2; ++first2; }
+    else { *result = *first1; ++first1; }
+    ++result;
+  }
+  for (; first1 != last1; ++first1, ++result) *result = *first1;
+  for (; first2 != last2; ++first2, ++result) *result = *first2;
+  return result;
+}
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
+pair<KOut, VOut> merge_by_key(execution_policy<D>&, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko, VOut vo,
+                              Comp comp) {
+  while (kf1 != kl1 && kf2 != kl2) {
+    if (comp(*kf2, *kf1)) { *ko = *kf2; *vo = *vf2; ++kf2; ++vf2; }
+    else { *ko = *kf1; *vo = *vf1; ++kf1; ++vf1; }
+    ++ko; ++vo;
+  }
+  for (; kf1 != kl1; ++kf1, ++vf1, ++ko, ++vo) { *ko = *kf1; *vo = *vf1; }
+  for (; kf2 != kl2; ++kf2, ++vf2, ++ko, ++vo) { *ko = *kf2; *vo = *vf2; }
+  return thrust::make_pair(ko, vo);
+}
+}  // namespace cpp
+
+namespace hip {
+template <typename D, typename In1, typename In2, typename Out, typename Comp>
+Out merge(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp) {
+  typedef typename std::remove_const<typename iterator_value<In1>::type>::type K;
+  static_assert(detail::is_abi_type<K>::value &&
+                    std::is_same<typename std::remove_const<typename iterator_value<In2>::type>::type, K>::value &&
+                    std::is_same<typename iterator_value<Out>::type, K>::value,
+                "merge on the device system needs one arithmetic key type for both inputs and the output");
+  static_assert(detail::order_code<Comp, K>::value >= 0,
+                "merge on the device system supports thrust::less and thrust::greater");
+  void* stream = detail::stream_of(exec);
+  const uint64_t na = (uint64_t)(last1 - first1), nb = (uint64_t)(last2 - first2);
+  if (na + nb == 0) return result;
+  detail::temp_storage temp(stream);
+  detail::run(temp, 0, "merge failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_merge(t, b, na ? thrust::detail::raw(first1) : nullptr, na,
+                            nb ? thrust::detail::raw(first2) : nullptr, nb, thrust::detail::raw(result),
+                            detail::dtype_of<K>::value, detail::order_code<Comp, K>::value, stream);
+  });
+  detail::synchronize(stream, "merge: synchronize");
+  return result + (na + nb);
+}
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
+pair<KOut, VOut> merge_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko,
+                              VOut vo, Comp) {
+  typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<V1>::type>::type V;
+  static_assert(detail::is_abi_type<K>::value &&
+                    std::is_same<typename std::remove_const<typename iterator_value<K2>::type>::type, K>::value &&
+                    std::is_same<typename iterator_value<KOut>::type, K>::value,
+                "merge_by_key on the device system needs one arithmetic key type for both inputs and the output");
+  static_assert(detail::is_abi_item<V>::value &&
+                    std::is_same<typename std::remove_const<typename iterator_value<V2>::type>::type, V>::value &&
+                    std::is_same<typename iterator_value<VOut>::type, V>::value,
+                "merge_by_key on the device system supports values of 1, 2, 4 or 8 bytes, one type throughout");
+  static_assert(detail::order_code<Comp, K>::value >= 0,
+                "merge_by_key on the device system supports thrust::less and thrust::greater");
+  void* stream = detail::stream_of(exec);
+  const uint64_t na = (uint64_t)(kl1 - kf1), nb = (uint64_t)(kl2 - kf2);
+  if (na + nb == 0) return thrust::make_pair(ko, vo);
+  detail::temp_storage temp(stream);
+  detail::run(temp, 0, "merge_by_key failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_merge_by_key(t, b, na ? thrust::detail::raw(kf1) : nullptr, na,
+                                   nb ? thrust::detail::raw(kf2) : nullptr, nb,
+                                   na ? thrust::detail::raw(vf1) : nullptr, nb ? thrust::detail::raw(vf2) : nullptr,
+                                   thrust::detail::raw(ko), thrust::detail::raw(vo), detail::dtype_of<K>::value,
+                                   sizeof(V), detail::order_code<Comp, K>::value, stream);
+  });
+  detail::synchronize(stream, "merge_by_key: synchronize");
+  return thrust::make_pair(ko + (na + nb), vo + (na + nb));
+}
+}  // namespace hip
+}  // namespace system
+
+// ------------------------------------------------------------------ entry points
+template <typename D, typename In1, typename In2, typename Out>
+Out merge(const detail::execution_policy_base<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result) {
+  using thrust::system::detail::generic::merge;
+  return merge(detail::derived_cast(detail::strip_const(exec)), first1, last1, first2, last2, result);
+}
+template <typename D, typename In1, typename In2, typename Out, typename Comp>
+Out merge(const detail::execution_policy_base<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result,
+          Comp comp) {
+  using thrust::system::detail::generic::merge;
+  return merge(detail::derived_cast(detail::strip_const(exec)), first1, last1, first2, last2, result, comp);
+}
+template <typename In1, typename In2, typename Out>
+Out merge(In1 first1, In1 last1, In2 first2, In2 last2, Out result) {
+  return thrust::merge(detail::policy_for<In1>(), first1, last1, first2, last2, result);
+}
+template <typename In1, typename In2, typename Out, typename Comp,
+          typename = typename std::enable_if<!detail::is_execution_policy<In1>::value>::type>
+Out merge(In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+  return thrust::merge(detail::policy_for<In1>(), first1, last1, first2, last2, result, comp);
+}
+
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut>
+pair<KOut, VOut> merge_by_key(const detail::execution_policy_base<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1,
+                              V2 vf2, KOut ko, VOut vo) {
+  using thrust::system::detail::generic::merge_by_key;
+  return merge_by_key(detail::derived_cast(detail::strip_const(exec)), kf1, kl1, kf2, kl2, vf1, vf2, ko, vo);
+}
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
+pair<KOut, VOut> merge_by_key(const detail::execution_policy_base<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1,
+                              V2 vf2, KOut ko, VOut vo, Comp comp) {
+  using thrust::system::detail::generic::merge_by_key;
+  return merge_by_key(detail::derived_cast(detail::strip_const(exec)), kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp);
+}
+template <typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut>
+pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko, VOut vo) {
+  return thrust::merge_by_key(detail::policy_for<K1>(), kf1, kl1, kf2, kl2, vf1, vf2, ko, vo);
+}
+template <typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp,
+          typename = typename std::enable_if<!detail::is_execution_policy<K1>::value>::type>
+pair<KOut, VOut> merge_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko, VOut vo, Comp comp) {
+  return thrust::merge_by_key(detail::policy_for<K1>(), kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp);
+}
+
+}  // namespace thrust

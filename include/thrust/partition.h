@@ -1,0 +1,172 @@
+// thrust::partition, stable_partition, partition_copy, stable_partition_copy (with and
+// without stencil).
+//
+// All four are stable here, as in the reference's generic layer where partition is
+// stable_partition (thrust/system/detail/generic/partition.inl:46-64,103-119,154-160).
+// On the device system the predicate must be one of the recognised forms listed in
+// thrust/functional.h.
+#pragma once
+#include <algorithm>
+#include <vector>
+
+#include <thrust/copy.h>
+#include <thrust/pair.h>
+
+namespace thrust {
+
+namespace system {
+namespace cpp {
+template <typename D, typename It, typename St, typename Pred>
+It stable_partition(execution_policy<D>&, It first, It last, St stencil, Pred pred) {
+  typedef typename iterator_value<It>::type T;
+  std::vector<T> yes, no;
+  for (It it = first; it != last; ++it, ++stencil) (pred(*stencil) ? yes : no).push_back(*it);
+  It mid = std::copy(yes.begin(), yes.end(), first);
+  std::copy(no.begin(), no.end(), mid);
+  return mid;
+}
+template <typename D, typename It, typename Pred>
+It stable_partition(execution_policy<D>& exec, It first, It last, Pred pred) {
+  typedef typename iterator_value<It>::type T;
+  std::vector<T> copy(first, last);
+  return stable_partition(exec, first, last, copy.begin(), pred);
+}
+template <typename D, typename In, typename St, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy(execution_policy<D>&, In first, In last, St stencil, Out1 out_true,
+                                       Out2 out_false, Pred pred) {
+  for (; first != last; ++first, ++stencil) {
+    if (pred(*stencil)) { *out_true = *first; ++out_true; }
+    else { *out_false = *first; ++out_false; }
+  }
+  return thrust::make_pair(out_true, out_false);
+}
+template <typename D, typename In, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In last, Out1 out_true, Out2 out_false,
+                                       Pred pred) {
+  return stable_partition_copy(exec, first, last, first, out_true, out_false, pred);
+}
+}  // namespace cpp
+
+namespace hip {
+template <typename D, typename It, typename Pred>
+It stable_partition(execution_policy<D>& exec, It first, It last, Pred pred) {
+  typedef typename iterator_value<It>::type T;
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return first;
+  const uint64_t cnt = detail::run_selection<T>(stream, pred, "stable_partition failed",
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_stable_partition(t, b, thrust::detail::raw(first), nullptr, d_num, n, sizeof(T),
+                                           detail::dtype_of<T>::value, cmp, thr, stream);
+      });
+  detail::synchronize(stream, "stable_partition: synchronize");
+  return first + cnt;
+}
+template <typename D, typename It, typename St, typename Pred>
+It stable_partition(execution_policy<D>& exec, It first, It last, St stencil, Pred pred) {
+  typedef typename iterator_value<It>::type T;
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  static_assert(detail::is_abi_item<T>::value, "stable_partition on the device system: items of 1, 2, 4 or 8 bytes");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return first;
+  const uint64_t cnt = detail::run_selection<S>(stream, pred, "stable_partition failed",
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_stable_partition(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil), d_num, n,
+                                           sizeof(T), detail::dtype_of<S>::value, cmp, thr, stream);
+      });
+  detail::synchronize(stream, "stable_partition: synchronize");
+  return first + cnt;
+}
+template <typename D, typename In, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In last, Out1 out_true, Out2 out_false,
+                                       Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  static_assert(std::is_same<typename iterator_value<Out1>::type, T>::value &&
+                    std::is_same<typename iterator_value<Out2>::type, T>::value,
+                "partition_copy on the device system: input and output element types must match");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return thrust::make_pair(out_true, out_false);
+  const uint64_t cnt = detail::run_selection<T>(stream, pred, "partition_copy failed",
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_partition_copy(t, b, thrust::detail::raw(first), nullptr, thrust::detail::raw(out_true),
+                                         thrust::detail::raw(out_false), d_num, n, sizeof(T),
+                                         detail::dtype_of<T>::value, cmp, thr, stream);
+      });
+  detail::synchronize(stream, "partition_copy: synchronize");
+  return thrust::make_pair(out_true + cnt, out_false + (n - cnt));
+}
+template <typename D, typename In, typename St, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In last, St stencil, Out1 out_true,
+                                       Out2 out_false, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out1>::type, T>::value &&
+                    std::is_same<typename iterator_value<Out2>::type, T>::value,
+                "partition_copy on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return thrust::make_pair(out_true, out_false);
+  const uint64_t cnt = detail::run_selection<S>(stream, pred, "partition_copy failed",
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_partition_copy(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil),
+                                         thrust::detail::raw(out_true), thrust::detail::raw(out_false), d_num, n,
+                                         sizeof(T), detail::dtype_of<S>::value, cmp, thr, stream);
+      });
+  detail::synchronize(stream, "partition_copy: synchronize");
+  return thrust::make_pair(out_true + cnt, out_false + (n - cnt));
+}
+}  // namespace hip
+}  // namespace system
+
+// ------------------------------------------------------------------ entry points
+// partition == stable_partition, partition_copy == stable_partition_copy
+// (thrust/system/detail/generic/partition.inl:154-160,196-214).
+#define THRUST_AMD_PARTITION_ENTRY(NAME)                                                                        \
+  template <typename D, typename It, typename Pred>                                                             \
+  It NAME(const detail::execution_policy_base<D>& exec, It first, It last, Pred pred) {                         \
+    return stable_partition(detail::derived_cast(detail::strip_const(exec)), first, last, pred);                \
+  }                                                                                                             \
+  template <typename D, typename It, typename St, typename Pred>                                                \
+  It NAME(const detail::execution_policy_base<D>& exec, It first, It last, St stencil, Pred pred) {             \
+    return stable_partition(detail::derived_cast(detail::strip_const(exec)), first, last, stencil, pred);       \
+  }                                                                                                             \
+  template <typename It, typename Pred>                                                                         \
+  It NAME(It first, It last, Pred pred) { return thrust::NAME(detail::policy_for<It>(), first, last, pred); }   \
+  template <typename It, typename St, typename Pred,                                                            \
+            typename = typename std::enable_if<!detail::is_execution_policy<It>::value>::type>                  \
+  It NAME(It first, It last, St stencil, Pred pred) {                                                           \
+    return thrust::NAME(detail::policy_for<It>(), first, last, stencil, pred);                                  \
+  }
+THRUST_AMD_PARTITION_ENTRY(partition)
+THRUST_AMD_PARTITION_ENTRY(stable_partition)
+#undef THRUST_AMD_PARTITION_ENTRY
+
+#define THRUST_AMD_PARTITION_COPY_ENTRY(NAME)                                                                   \
+  template <typename D, typename In, typename Out1, typename Out2, typename Pred>                               \
+  pair<Out1, Out2> NAME(const detail::execution_policy_base<D>& exec, In first, In last, Out1 out_true,         \
+                        Out2 out_false, Pred pred) {                                                            \
+    return stable_partition_copy(detail::derived_cast(detail::strip_const(exec)), first, last, out_true,        \
+                                 out_false, pred);                                                              \
+  }                                                                                                             \
+  template <typename D, typename In, typename St, typename Out1, typename Out2, typename Pred>                  \
+  pair<Out1, Out2> NAME(const detail::execution_policy_base<D>& exec, In first, In last, St stencil,            \
+                        Out1 out_true, Out2 out_false, Pred pred) {                                             \
+    return stable_partition_copy(detail::derived_cast(detail::strip_const(exec)), first, last, stencil,         \
+                                 out_true, out_false, pred);                                                    \
+  }                                                                                                             \
+  template <typename In, typename Out1, typename Out2, typename Pred>                                           \
+  pair<Out1, Out2> NAME(In first, In last, Out1 out_true, Out2 out_false, Pred pred) {                          \
+    return thrust::NAME(detail::policy_for<In>(), first, last, out_true, out_false, pred);                      \
+  }                                                                                                             \
+  template <typename In, typename St, typename Out1, typename Out2, typename Pred,                              \
+            typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>                  \
+  pair<Out1, Out2> NAME(In first, In last, St stencil, Out1 out_true, Out2 out_false, Pred pred) {              \
+    return thrust::NAME(detail::policy_for<In>(), first, last, stencil, out_true, out_false, pred);             \
+  }
+THRUST_AMD_PARTITION_COPY_ENTRY(partition_copy)
+THRUST_AMD_PARTITION_COPY_ENTRY(stable_partition_copy)
+#undef THRUST_AMD_PARTITION_COPY_ENTRY
+
+}  // namespace thrust

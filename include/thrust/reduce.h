@@ -1,0 +1,221 @@
+// thrust::reduce and thrust::reduce_by_key.
+//
+// Overload set as in the reference (thrust/detail/reduce.inl:34-72,141-187 and
+// :75-138,190-274): with and without an execution policy; reduce(first,last) uses
+// init = value_type(0) and plus<value_type>, i.e. an integer sum wraps in the value type
+// (thrust/system/detail/generic/reduce.inl:35-53).
+#pragma once
+#include <thrust/functional.h>
+#include <thrust/pair.h>
+#include <thrust/system/hip/detail/backend.h>
+
+namespace thrust {
+
+// ------------------------------------------------------------------ entry points
+template <typename D, typename It>
+typename iterator_value<It>::type reduce(const detail::execution_policy_base<D>& exec, It first, It last);
+template <typename D, typename It, typename T>
+T reduce(const detail::execution_policy_base<D>& exec, It first, It last, T init);
+template <typename D, typename It, typename T, typename Op>
+T reduce(const detail::execution_policy_base<D>& exec, It first, It last, T init, Op op);
+
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut>
+pair<KOut, VOut> reduce_by_key(const detail::execution_policy_base<D>& exec, KIt keys_first, KIt keys_last,
+                               VIt values_first, KOut keys_output, VOut values_output);
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred>
+pair<KOut, VOut> reduce_by_key(const detail::execution_policy_base<D>& exec, KIt keys_first, KIt keys_last,
+                               VIt values_first, KOut keys_output, VOut values_output, Pred pred);
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key(const detail::execution_policy_base<D>& exec, KIt keys_first, KIt keys_last,
+                               VIt values_first, KOut keys_output, VOut values_output, Pred pred, Op op);
+
+namespace system {
+namespace detail {
+namespace generic {
+// Defaulting chain (thrust/system/detail/generic/reduce.inl:35-53, reduce_by_key.inl:139-190).
+template <typename D, typename It>
+typename iterator_value<It>::type reduce(thrust::execution_policy<D>& exec, It first, It last) {
+  typedef typename iterator_value<It>::type T;
+  return thrust::reduce(exec, first, last, T(0));
+}
+template <typename D, typename It, typename T>
+T reduce(thrust::execution_policy<D>& exec, It first, It last, T init) {
+  return thrust::reduce(exec, first, last, init, thrust::plus<T>());
+}
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut>
+pair<KOut, VOut> reduce_by_key(thrust::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo) {
+  typedef typename iterator_value<KIt>::type K;
+  return thrust::reduce_by_key(exec, kf, kl, vf, ko, vo, thrust::equal_to<K>());
+}
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred>
+pair<KOut, VOut> reduce_by_key(thrust::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo,
+                               Pred pred) {
+  typedef typename iterator_value<VIt>::type V;
+  return thrust::reduce_by_key(exec, kf, kl, vf, ko, vo, pred, thrust::plus<V>());
+}
+}  // namespace generic
+}  // namespace detail
+
+namespace cpp {
+// Sequential host system (thrust/system/detail/sequential/reduce.h:39-66, reduce_by_key.h:36-98).
+template <typename D, typename It, typename T, typename Op>
+T reduce(execution_policy<D>&, It first, It last, T init, Op op) {
+  for (; first != last; ++first) init = op(init, *first);
+  return init;
+}
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred pred, Op op) {
+  typedef typename iterator_value<KIt>::type K;
+  typedef typename iterator_value<VIt>::type V;
+  if (kf == kl) return thrust::make_pair(ko, vo);
+  K run_key = *kf;
+  K prev = run_key;
+  V acc = *vf;
+  for (++kf, ++vf; kf != kl; ++kf, ++vf) {
+    const K k = *kf;
+    if (pred(prev, k)) {
+      acc = op(acc, *vf);
+    } else {
+      *ko = run_key; ++ko;
+      *vo = acc; ++vo;
+      run_key = k;
+      acc = *vf;
+    }
+    prev = k;
+  }
+  *ko = run_key; ++ko;
+  *vo = acc; ++vo;
+  return thrust::make_pair(ko, vo);
+}
+}  // namespace cpp
+
+namespace hip {
+template <typename D, typename It, typename T, typename Op>
+T reduce(execution_policy<D>& exec, It first, It last, T init, Op) {
+  typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
+  static_assert(std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value,
+                "thrust::reduce on the device system needs device_ptr / device_vector iterators or raw device pointers");
+  static_assert(detail::is_abi_type<T>::value && std::is_same<V, T>::value,
+                "thrust::reduce on the device system: init must have the (arithmetic) element type");
+  static_assert(detail::binop_code<Op, T>::value >= 0,
+                "thrust::reduce on the device system supports thrust::plus, thrust::minimum and thrust::maximum");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  const void* in = n ? (const void*)thrust::detail::raw(first) : nullptr;
+  detail::temp_storage temp(stream);
+  void* d_out = nullptr;
+  // the result slot is the `extra` region, which run() only knows after the size query
+  std::size_t need = 0;
+  detail::throw_on_error(thrust_amd_reduce(nullptr, &need, in, n, detail::dtype_of<T>::value,
+                                           detail::binop_code<Op, T>::value, &init, nullptr, stream),
+                         "reduce: temp size query");
+  const std::size_t aligned = (need + 255) / 256 * 256;
+  temp.ensure(aligned + 256);
+  d_out = static_cast<char*>(temp.ptr()) + aligned;
+  std::size_t bytes = aligned;
+  detail::throw_on_error(thrust_amd_reduce(temp.ptr(), &bytes, in, n, detail::dtype_of<T>::value,
+                                           detail::binop_code<Op, T>::value, &init, d_out, stream),
+                         "reduce failed");
+  return detail::read_scalar<T>(d_out, stream, "reduce: result copy");
+}
+
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred, Op) {
+  typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
+  static_assert(detail::is_abi_type<K>::value && detail::is_abi_type<V>::value,
+                "thrust::reduce_by_key on the device system needs arithmetic keys and values");
+  static_assert(std::is_same<typename iterator_value<KOut>::type, K>::value &&
+                    std::is_same<typename iterator_value<VOut>::type, V>::value,
+                "thrust::reduce_by_key on the device system: output element types must equal the input types");
+  static_assert(detail::is_equal_to<Pred, K>::value,
+                "thrust::reduce_by_key on the device system supports thrust::equal_to as key predicate");
+  static_assert(detail::binop_code<Op, V>::value >= 0,
+                "thrust::reduce_by_key on the device system supports thrust::plus, minimum and maximum");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(kl - kf);
+  if (n == 0) return thrust::make_pair(ko, vo);
+  detail::temp_storage temp(stream);
+  uint64_t* d_runs = nullptr;
+  std::size_t need = 0;
+  auto call = [&](void* t, std::size_t* b) {
+    return thrust_amd_reduce_by_key(t, b, thrust::detail::raw(kf), thrust::detail::raw(vf),
+                                    thrust::detail::raw(ko), thrust::detail::raw(vo), d_runs, n,
+                                    detail::dtype_of<K>::value, detail::dtype_of<V>::value,
+                                    detail::binop_code<Op, V>::value, stream);
+  };
+  detail::throw_on_error(call(nullptr, &need), "reduce_by_key: temp size query");
+  const std::size_t aligned = (need + 255) / 256 * 256;
+  temp.ensure(aligned + 256);
+  d_runs = reinterpret_cast<uint64_t*>(static_cast<char*>(temp.ptr()) + aligned);
+  std::size_t bytes = aligned;
+  detail::throw_on_error(call(temp.ptr(), &bytes), "reduce_by_key failed");
+  const uint64_t runs = detail::read_scalar<uint64_t>(d_runs, stream, "reduce_by_key: count copy");
+  return thrust::make_pair(ko + runs, vo + runs);
+}
+}  // namespace hip
+}  // namespace system
+
+// ------------------------------------------------------------------ entry point bodies
+template <typename D, typename It>
+typename iterator_value<It>::type reduce(const detail::execution_policy_base<D>& exec, It first, It last) {
+  using thrust::system::detail::generic::reduce;
+  return reduce(detail::derived_cast(detail::strip_const(exec)), first, last);
+}
+template <typename D, typename It, typename T>
+T reduce(const detail::execution_policy_base<D>& exec, It first, It last, T init) {
+  using thrust::system::detail::generic::reduce;
+  return reduce(detail::derived_cast(detail::strip_const(exec)), first, last, init);
+}
+template <typename D, typename It, typename T, typename Op>
+T reduce(const detail::execution_policy_base<D>& exec, It first, It last, T init, Op op) {
+  using thrust::system::detail::generic::reduce;
+  return reduce(detail::derived_cast(detail::strip_const(exec)), first, last, init, op);
+}
+template <typename It>
+typename iterator_value<It>::type reduce(It first, It last) {
+  return thrust::reduce(detail::policy_for<It>(), first, last);
+}
+template <typename It, typename T>
+T reduce(It first, It last, T init) {
+  return thrust::reduce(detail::policy_for<It>(), first, last, init);
+}
+template <typename It, typename T, typename Op>
+T reduce(It first, It last, T init, Op op) {
+  return thrust::reduce(detail::policy_for<It>(), first, last, init, op);
+}
+
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut>
+pair<KOut, VOut> reduce_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko,
+                               VOut vo) {
+  using thrust::system::detail::generic::reduce_by_key;
+  return reduce_by_key(detail::derived_cast(detail::strip_const(exec)), kf, kl, vf, ko, vo);
+}
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred>
+pair<KOut, VOut> reduce_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko,
+                               VOut vo, Pred pred) {
+  using thrust::system::detail::generic::reduce_by_key;
+  return reduce_by_key(detail::derived_cast(detail::strip_const(exec)), kf, kl, vf, ko, vo, pred);
+}
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko,
+                               VOut vo, Pred pred, Op op) {
+  using thrust::system::detail::generic::reduce_by_key;
+  return reduce_by_key(detail::derived_cast(detail::strip_const(exec)), kf, kl, vf, ko, vo, pred, op);
+}
+template <typename KIt, typename VIt, typename KOut, typename VOut>
+pair<KOut, VOut> reduce_by_key(KIt kf, KIt kl, VIt vf, KOut ko, VOut vo) {
+  return thrust::reduce_by_key(detail::policy_for<KIt>(), kf, kl, vf, ko, vo);
+}
+template <typename KIt, typename VIt, typename KOut, typename VOut, typename Pred,
+          typename = typename std::enable_if<!detail::is_execution_policy<KIt>::value>::type>
+pair<KOut, VOut> reduce_by_key(KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred pred) {
+  return thrust::reduce_by_key(detail::policy_for<KIt>(), kf, kl, vf, ko, vo, pred);
+}
+template <typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op,
+          typename = typename std::enable_if<!detail::is_execution_policy<KIt>::value>::type>
+pair<KOut, VOut> reduce_by_key(KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred pred, Op op) {
+  return thrust::reduce_by_key(detail::policy_for<KIt>(), kf, kl, vf, ko, vo, pred, op);
+}
+
+}  // namespace thrust

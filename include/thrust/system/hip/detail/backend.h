@@ -1,0 +1,142 @@
+// Glue between the templated front end and the C ABI of libthrust_amd:
+//   - element types -> dtype codes, functor types -> operator codes (compile time);
+//     an unsupported combination is a static_assert naming the limitation, the analogue
+//     of the reference's "unimplemented for this system" terminals
+//     (thrust/system/detail/generic/reduce.inl:56-72),
+//   - temp_storage: RAII over the temp arena (the reference allocates a
+//     temporary_array<uint8_t,Derived>, thrust/system/cuda/detail/reduce.h:959-960),
+//   - run(): the two-phase size-query / run protocol plus error conversion.
+#pragma once
+#include <cstdint>
+#include <type_traits>
+
+#include <thrust/detail/execution_policy.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/iterator/iterator_traits.h>
+#include <thrust/system_error.h>
+#include <thrust_amd.h>
+
+namespace thrust {
+namespace system {
+namespace hip {
+namespace detail {
+
+template <typename T, typename Enable = void>
+struct dtype_of { static const int value = -1; };
+template <typename T>
+struct dtype_of<T, typename std::enable_if<std::is_integral<T>::value && !std::is_same<T, bool>::value>::type> {
+  static const int value = sizeof(T) == 1 ? (std::is_signed<T>::value ? THRUST_AMD_I8 : THRUST_AMD_U8)
+                         : sizeof(T) == 2 ? (std::is_signed<T>::value ? THRUST_AMD_I16 : THRUST_AMD_U16)
+                         : sizeof(T) == 4 ? (std::is_signed<T>::value ? THRUST_AMD_I32 : THRUST_AMD_U32)
+                                          : (std::is_signed<T>::value ? THRUST_AMD_I64 : THRUST_AMD_U64);
+};
+template <> struct dtype_of<float> { static const int value = THRUST_AMD_F32; };
+template <> struct dtype_of<double> { static const int value = THRUST_AMD_F64; };
+
+template <typename T>
+struct is_abi_type : std::integral_constant<bool, (dtype_of<T>::value >= 0)> {};
+template <typename T>
+struct is_abi_item : std::integral_constant<bool, std::is_trivially_copyable<T>::value &&
+                                                  (sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8)> {};
+
+// ---- functor types -> codes
+template <typename Op, typename T> struct binop_code { static const int value = -1; };
+template <typename T> struct binop_code<thrust::plus<T>, T> { static const int value = THRUST_AMD_PLUS; };
+template <typename T> struct binop_code<thrust::plus<void>, T> { static const int value = THRUST_AMD_PLUS; };
+template <typename T> struct binop_code<thrust::minimum<T>, T> { static const int value = THRUST_AMD_MIN; };
+template <typename T> struct binop_code<thrust::minimum<void>, T> { static const int value = THRUST_AMD_MIN; };
+template <typename T> struct binop_code<thrust::maximum<T>, T> { static const int value = THRUST_AMD_MAX; };
+template <typename T> struct binop_code<thrust::maximum<void>, T> { static const int value = THRUST_AMD_MAX; };
+
+// 0 ascending (less), 1 descending (greater), -1 not a recognised ordering
+template <typename Comp, typename T> struct order_code { static const int value = -1; };
+template <typename T> struct order_code<thrust::less<T>, T> { static const int value = 0; };
+template <typename T> struct order_code<thrust::less<void>, T> { static const int value = 0; };
+template <typename T> struct order_code<thrust::greater<T>, T> { static const int value = 1; };
+template <typename T> struct order_code<thrust::greater<void>, T> { static const int value = 1; };
+
+template <typename Pred, typename T> struct is_equal_to : std::false_type {};
+template <typename T> struct is_equal_to<thrust::equal_to<T>, T> : std::true_type {};
+template <typename T> struct is_equal_to<thrust::equal_to<void>, T> : std::true_type {};
+
+// Unary predicate -> (cmp code, threshold of the tested type).
+template <typename Pred, typename T>
+struct unary_pred {
+  static const bool supported = false;
+  static int cmp(const Pred&) { return -1; }
+  static T threshold(const Pred&) { return T(); }
+};
+template <int CMP, typename U, typename T>
+struct unary_pred<thrust::detail::compare_with<CMP, U>, T> {
+  // the comparison happens in the tested type, as `x < t` would after the usual
+  // conversion of t when U converts to T without loss for the values in use
+  static const bool supported = std::is_convertible<U, T>::value;
+  static int cmp(const thrust::detail::compare_with<CMP, U>&) { return CMP; }
+  static T threshold(const thrust::detail::compare_with<CMP, U>& p) { return static_cast<T>(p.value); }
+};
+template <typename I, typename T>
+struct unary_pred<thrust::identity<I>, T> {
+  static const bool supported = true;
+  static int cmp(const thrust::identity<I>&) { return THRUST_AMD_NONZERO; }
+  static T threshold(const thrust::identity<I>&) { return T(); }
+};
+template <typename I, typename T>
+struct unary_pred<thrust::logical_not<I>, T> {
+  static const bool supported = true;
+  static int cmp(const thrust::logical_not<I>&) { return THRUST_AMD_EQ; }
+  static T threshold(const thrust::logical_not<I>&) { return T(0); }
+};
+
+// ---- temp storage from the arena, returned when the scope ends
+class temp_storage {
+ public:
+  temp_storage(void* stream) : ptr_(nullptr), stream_(stream), bytes_(0) {}
+  ~temp_storage() {
+    if (ptr_) (void)thrust_amd_temp_release(ptr_, stream_);
+  }
+  void ensure(std::size_t bytes) {
+    bytes_ = bytes;
+    const int rc = thrust_amd_temp_acquire(&ptr_, bytes ? bytes : 1, stream_);
+    if (rc != 0) throw thrust::system::detail::bad_alloc(thrust_amd_error_string(rc));
+  }
+  void* ptr() const { return ptr_; }
+  std::size_t* bytes() { return &bytes_; }
+
+ private:
+  temp_storage(const temp_storage&);
+  temp_storage& operator=(const temp_storage&);
+  void* ptr_;
+  void* stream_;
+  std::size_t bytes_;
+};
+
+// Size query, allocation from the arena with `extra` more bytes at the end (for device
+// scalars such as counts), then the run.  call(temp, &bytes) -> status.  Returns the
+// address of the extra region.
+template <typename Call>
+inline void* run(temp_storage& temp, std::size_t extra, const char* what, Call call) {
+  std::size_t need = 0;
+  throw_on_error(call((void*)nullptr, &need), what);
+  const std::size_t aligned = (need + 255) / 256 * 256;
+  temp.ensure(aligned + extra);
+  *temp.bytes() = aligned;
+  throw_on_error(call(temp.ptr(), temp.bytes()), what);
+  return static_cast<char*>(temp.ptr()) + aligned;
+}
+
+inline void synchronize(void* stream, const char* what) {
+  throw_on_error(thrust_amd_stream_synchronize(stream), what);
+}
+
+template <typename T>
+inline T read_scalar(const void* device_src, void* stream, const char* what) {
+  T v;
+  throw_on_error(thrust_amd_memcpy(&v, device_src, sizeof(T), THRUST_AMD_D2H, stream), what);
+  return v;
+}
+
+}  // namespace detail
+}  // namespace hip
+}  // namespace system
+}  // namespace thrust

@@ -1,0 +1,505 @@
+// Front-end tests: the unchanged thrust:: API on the gfx950 device system.
+//
+// Part 1 replays the literal known-answer vectors of the reference's own unit tests
+// (cited per test) on device_vector.  Part 2 is the reference's differential pattern:
+// the same algorithm on host_vector (sequential host system) and device_vector over the
+// reference's size list, results compared exactly (testing/unittest/testframework.cu:21-31,
+// e.g. testing/reduce.cu:80-95).  Part 3 covers policies, streams, dispatch interception,
+// the memory model and error reporting.
+#include <thrust/copy.h>
+#include <thrust/device_vector.h>
+#include <thrust/execution_policy.h>
+#include <thrust/fill.h>
+#include <thrust/functional.h>
+#include <thrust/host_vector.h>
+#include <thrust/merge.h>
+#include <thrust/partition.h>
+#include <thrust/reduce.h>
+#include <thrust/scan.h>
+#include <thrust/sort.h>
+#include <thrust/unique.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+#include <functional>
+#include <string>
+#include <vector>
+
+static int g_failed = 0, g_checks = 0;
+static const char* g_test = "";
+
+#define ASSERT_TRUE(c)                                                                    \
+  do {                                                                                    \
+    ++g_checks;                                                                           \
+    if (!(c)) { ++g_failed; std::printf("FAIL [%s] %s:%d: %s\n", g_test, __FILE__, __LINE__, #c); } \
+  } while (0)
+
+template <typename A, typename B>
+static bool same(const A& a, const B& b) {
+  if (a.size() != b.size()) return false;
+  for (size_t i = 0; i < a.size(); ++i)
+    if (!(a[i] == b[i])) return false;
+  return true;
+}
+#define ASSERT_EQUAL_VEC(a, b) ASSERT_TRUE(same((a), (b)))
+
+template <typename T>
+static thrust::host_vector<T> hv(std::initializer_list<T> l) { return thrust::host_vector<T>(std::vector<T>(l)); }
+template <typename T>
+static thrust::host_vector<T> to_host(const thrust::device_vector<T>& d) { return thrust::host_vector<T>(d); }
+
+// deterministic inputs: an index hash, in the spirit of testing/unittest/random.h:12-21
+static uint64_t mix(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+template <typename T>
+static thrust::host_vector<T> random_integers(size_t n, uint64_t seed, uint64_t modulus = 0) {
+  thrust::host_vector<T> h(n);
+  for (size_t i = 0; i < n; ++i) {
+    const uint64_t r = mix(seed * 1000003ull + i);
+    h[i] = (T)(modulus ? (r % modulus) : r);
+  }
+  return h;
+}
+
+static const size_t kSizes[] = {0, 1, 2, 3, 4, 5, 8, 10, 13, 16, 17, 19, 27, 30, 31, 32, 33, 35, 42, 53, 58, 63,
+                                64, 65, 72, 97, 100, 127, 128, 129, 142, 183, 192, 201, 240, 255, 256, 257, 302,
+                                511, 512, 513, 687, 900, 1023, 1024, 1025, 1565, 1786, 1973, 2047, 2048, 2049,
+                                3050, 4095, 4096, 4097, 5030, 7791, 10000, 10027, 12345, 16384, 17354, 26255,
+                                32768, 43718, 65533, 65536, 65539};
+
+using namespace thrust::placeholders;
+
+// ================================================================ part 1: known answers
+static void TestReduceSimple() {  // testing/reduce.cu:26-39
+  g_test = "ReduceSimple";
+  thrust::device_vector<int> v(hv<int>({1, -2, 3}));
+  ASSERT_TRUE(thrust::reduce(v.begin(), v.end()) == 2);
+  ASSERT_TRUE(thrust::reduce(v.begin(), v.end(), 10) == 12);
+  ASSERT_TRUE(thrust::reduce(v.begin(), v.end(), 10, thrust::plus<int>()) == 12);
+  ASSERT_TRUE(thrust::reduce(thrust::device, v.begin(), v.end(), 10) == 12);
+  ASSERT_TRUE(thrust::reduce(v.begin(), v.end(), 0, thrust::maximum<int>()) == 3);
+  ASSERT_TRUE(thrust::reduce(v.begin(), v.end(), 0, thrust::minimum<int>()) == -2);
+  ASSERT_TRUE(thrust::reduce(v.begin(), v.begin(), 7) == 7);  // empty range returns init
+}
+
+static void TestReduceWithOperatorTable() {  // the data of testing/reduce.cu:166-192, plain plus here
+  g_test = "ReduceTable";
+  thrust::device_vector<unsigned int> v(hv<unsigned int>({0, 1, 2, 1, 2, 0, 1}));
+  ASSERT_TRUE(thrust::reduce(v.begin(), v.end()) == 7u);
+}
+
+static void TestScanSimple() {  // testing/scan.cu:23-93
+  g_test = "ScanSimple";
+  const thrust::host_vector<int> in = hv<int>({1, 3, -2, 4, -5});
+  thrust::device_vector<int> input(in), output(5, 0);
+  auto it = thrust::inclusive_scan(input.begin(), input.end(), output.begin());
+  ASSERT_TRUE(it - output.begin() == 5);
+  ASSERT_EQUAL_VEC(to_host(input), in);
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({1, 4, 2, 6, 1}));
+  it = thrust::exclusive_scan(input.begin(), input.end(), output.begin(), 0);
+  ASSERT_TRUE(it - output.begin() == 5);
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({0, 1, 4, 2, 6}));
+  thrust::exclusive_scan(input.begin(), input.end(), output.begin(), 3);
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({3, 4, 7, 5, 9}));
+  // inclusive scan with op
+  thrust::inclusive_scan(input.begin(), input.end(), output.begin(), thrust::plus<int>());
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({1, 4, 2, 6, 1}));
+  // exclusive scan with init and op
+  thrust::exclusive_scan(input.begin(), input.end(), output.begin(), 3, thrust::plus<int>());
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({3, 4, 7, 5, 9}));
+  // in-place
+  input = in;
+  thrust::inclusive_scan(input.begin(), input.end(), input.begin(), thrust::plus<int>());
+  ASSERT_EQUAL_VEC(to_host(input), hv<int>({1, 4, 2, 6, 1}));
+  input = in;
+  thrust::exclusive_scan(input.begin(), input.end(), input.begin(), 3, thrust::plus<int>());
+  ASSERT_EQUAL_VEC(to_host(input), hv<int>({3, 4, 7, 5, 9}));
+  // exclusive_scan without init starts from 0
+  input = in;
+  thrust::exclusive_scan(input.begin(), input.end(), output.begin());
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({0, 1, 4, 2, 6}));
+}
+
+static void TestSortSimple() {  // testing/sort.cu:43-76
+  g_test = "SortSimple";
+  thrust::device_vector<int> d(hv<int>({1, 3, 6, 5, 2, 0, 4}));
+  thrust::sort(d.begin(), d.end());
+  ASSERT_EQUAL_VEC(to_host(d), hv<int>({0, 1, 2, 3, 4, 5, 6}));
+  thrust::sort(d.begin(), d.end(), thrust::greater<int>());
+  ASSERT_EQUAL_VEC(to_host(d), hv<int>({6, 5, 4, 3, 2, 1, 0}));
+  thrust::stable_sort(thrust::device, d.begin(), d.end(), thrust::less<int>());
+  ASSERT_EQUAL_VEC(to_host(d), hv<int>({0, 1, 2, 3, 4, 5, 6}));
+}
+
+static void TestSortByKeySimple() {  // testing/sort_by_key.cu:47-85, stable_sort_by_key.cu:51-95
+  g_test = "SortByKeySimple";
+  thrust::device_vector<int> keys(hv<int>({1, 3, 6, 5, 2, 0, 4}));
+  thrust::device_vector<int> vals(hv<int>({0, 1, 2, 3, 4, 5, 6}));
+  thrust::sort_by_key(keys.begin(), keys.end(), vals.begin());
+  ASSERT_EQUAL_VEC(to_host(keys), hv<int>({0, 1, 2, 3, 4, 5, 6}));
+  ASSERT_EQUAL_VEC(to_host(vals), hv<int>({5, 0, 4, 1, 6, 3, 2}));
+  // stability: equal keys keep the order of their values
+  thrust::device_vector<int> k2(hv<int>({2, 1, 2, 1, 2, 1, 0, 0, 1}));
+  thrust::device_vector<int> v2(hv<int>({0, 1, 2, 3, 4, 5, 6, 7, 8}));
+  thrust::stable_sort_by_key(k2.begin(), k2.end(), v2.begin());
+  ASSERT_EQUAL_VEC(to_host(k2), hv<int>({0, 0, 1, 1, 1, 1, 2, 2, 2}));
+  ASSERT_EQUAL_VEC(to_host(v2), hv<int>({6, 7, 1, 3, 5, 8, 0, 2, 4}));
+  thrust::stable_sort_by_key(k2.begin(), k2.end(), v2.begin(), thrust::greater<int>());
+  ASSERT_EQUAL_VEC(to_host(k2), hv<int>({2, 2, 2, 1, 1, 1, 1, 0, 0}));
+  ASSERT_EQUAL_VEC(to_host(v2), hv<int>({0, 2, 4, 1, 3, 5, 8, 6, 7}));
+}
+
+static void TestReduceByKeySimple() {  // testing/reduce_by_key.cu:16-112
+  g_test = "ReduceByKeySimple";
+  thrust::device_vector<int> keys(hv<int>({11, 11, 21, 20, 21, 21, 21, 37, 37}));
+  thrust::device_vector<int> vals(hv<int>({0, 1, 2, 3, 4, 5, 6, 7, 8}));
+  thrust::device_vector<int> ok(9), ov(9);
+  auto ends = thrust::reduce_by_key(keys.begin(), keys.end(), vals.begin(), ok.begin(), ov.begin());
+  ASSERT_TRUE(ends.first - ok.begin() == 5 && ends.second - ov.begin() == 5);
+  ok.resize(5); ov.resize(5);
+  ASSERT_EQUAL_VEC(to_host(ok), hv<int>({11, 21, 20, 21, 37}));
+  ASSERT_EQUAL_VEC(to_host(ov), hv<int>({1, 2, 3, 15, 15}));
+  ok.resize(9); ov.resize(9);
+  ends = thrust::reduce_by_key(keys.begin(), keys.end(), vals.begin(), ok.begin(), ov.begin(),
+                               thrust::equal_to<int>(), thrust::plus<int>());
+  ASSERT_TRUE(ends.first - ok.begin() == 5);
+  ok.resize(5); ov.resize(5);
+  ASSERT_EQUAL_VEC(to_host(ov), hv<int>({1, 2, 3, 15, 15}));
+}
+
+static void TestUniqueSimple() {  // testing/unique.cu:105-142
+  g_test = "UniqueSimple";
+  thrust::device_vector<int> d(hv<int>({11, 11, 12, 20, 29, 21, 21, 31, 31, 37}));
+  auto e = thrust::unique(d.begin(), d.end());
+  ASSERT_TRUE(e - d.begin() == 7);
+  d.resize(7);
+  ASSERT_EQUAL_VEC(to_host(d), hv<int>({11, 12, 20, 29, 21, 31, 37}));
+  thrust::device_vector<int> src(hv<int>({11, 11, 12, 20, 29, 21, 21, 31, 31, 37})), out(10);
+  auto e2 = thrust::unique_copy(src.begin(), src.end(), out.begin());
+  ASSERT_TRUE(e2 - out.begin() == 7);
+}
+
+static void TestUniqueByKeySimple() {  // testing/unique_by_key.cu:160-253
+  g_test = "UniqueByKeySimple";
+  thrust::device_vector<int> keys(hv<int>({11, 11, 21, 20, 21, 21, 21, 37, 37}));
+  thrust::device_vector<int> vals(hv<int>({0, 1, 2, 3, 4, 5, 6, 7, 8}));
+  thrust::device_vector<int> ok(9), ov(9);
+  auto ends = thrust::unique_by_key_copy(keys.begin(), keys.end(), vals.begin(), ok.begin(), ov.begin());
+  ASSERT_TRUE(ends.first - ok.begin() == 5 && ends.second - ov.begin() == 5);
+  ok.resize(5); ov.resize(5);
+  ASSERT_EQUAL_VEC(to_host(ok), hv<int>({11, 21, 20, 21, 37}));
+  ASSERT_EQUAL_VEC(to_host(ov), hv<int>({0, 2, 3, 4, 7}));
+  auto ends2 = thrust::unique_by_key(keys.begin(), keys.end(), vals.begin());
+  ASSERT_TRUE(ends2.first - keys.begin() == 5);
+  keys.resize(5); vals.resize(5);
+  ASSERT_EQUAL_VEC(to_host(keys), hv<int>({11, 21, 20, 21, 37}));
+  ASSERT_EQUAL_VEC(to_host(vals), hv<int>({0, 2, 3, 4, 7}));
+}
+
+static void TestCopyIfSimple() {  // testing/copy.cu:252-269, :378-397
+  g_test = "CopyIfSimple";
+  thrust::device_vector<int> v(hv<int>({0, 1, 2, 3, 4})), dest(5, 10);
+  auto e = thrust::copy_if(v.begin(), v.end(), dest.begin(), thrust::identity<int>());  // "is_true"
+  ASSERT_TRUE(e - dest.begin() == 4);
+  dest.resize(4);
+  ASSERT_EQUAL_VEC(to_host(dest), hv<int>({1, 2, 3, 4}));
+  // stencil form
+  thrust::device_vector<int> st(hv<int>({1, 0, 1, 0, 1})), dest2(5, 0);
+  auto e2 = thrust::copy_if(v.begin(), v.end(), st.begin(), dest2.begin(), thrust::identity<int>());
+  ASSERT_TRUE(e2 - dest2.begin() == 3);
+  dest2.resize(3);
+  ASSERT_EQUAL_VEC(to_host(dest2), hv<int>({0, 2, 4}));
+}
+
+static void TestStablePartitionSimple() {  // testing/partition.cu:158-182 with is_even as a stencil
+  g_test = "StablePartitionSimple";
+  thrust::device_vector<int> data(hv<int>({1, 2, 1, 3, 2}));
+  // is_even(x) expressed through a stencil of parities and "== 0"
+  thrust::device_vector<int> parity(hv<int>({1, 0, 1, 1, 0}));
+  auto mid = thrust::stable_partition(data.begin(), data.end(), parity.begin(), _1 == 0);
+  ASSERT_TRUE(mid - data.begin() == 2);
+  ASSERT_EQUAL_VEC(to_host(data), hv<int>({2, 2, 1, 1, 3}));
+  // predicate on the data itself
+  thrust::device_vector<int> d2(hv<int>({5, 1, 7, 2, 9, 3}));
+  auto m2 = thrust::partition(d2.begin(), d2.end(), _1 < 4);
+  ASSERT_TRUE(m2 - d2.begin() == 3);
+  ASSERT_EQUAL_VEC(to_host(d2), hv<int>({1, 2, 3, 5, 7, 9}));
+  thrust::device_vector<int> src(hv<int>({5, 1, 7, 2, 9, 3})), t(6), f(6);
+  auto ends = thrust::stable_partition_copy(src.begin(), src.end(), t.begin(), f.begin(), _1 >= 5);
+  ASSERT_TRUE(ends.first - t.begin() == 3 && ends.second - f.begin() == 3);
+  t.resize(3); f.resize(3);
+  ASSERT_EQUAL_VEC(to_host(t), hv<int>({5, 7, 9}));
+  ASSERT_EQUAL_VEC(to_host(f), hv<int>({1, 2, 3}));
+}
+
+static void TestMergeSimple() {  // testing/merge.cu:11-38
+  g_test = "MergeSimple";
+  thrust::device_vector<int> a(hv<int>({0, 2, 4})), b(hv<int>({0, 3, 3, 4})), r(7);
+  auto e = thrust::merge(a.begin(), a.end(), b.begin(), b.end(), r.begin());
+  ASSERT_TRUE(e - r.begin() == 7);
+  ASSERT_EQUAL_VEC(to_host(r), hv<int>({0, 0, 2, 3, 3, 4, 4}));
+}
+
+static void TestMergeByKeySimple() {  // testing/merge_by_key.cu:10-45
+  g_test = "MergeByKeySimple";
+  thrust::device_vector<int> ak(hv<int>({0, 2, 4})), av(hv<int>({13, 7, 42}));
+  thrust::device_vector<int> bk(hv<int>({0, 3, 3, 4})), bv(hv<int>({42, 42, 7, 13}));
+  thrust::device_vector<int> rk(7), rv(7);
+  auto ends = thrust::merge_by_key(ak.begin(), ak.end(), bk.begin(), bk.end(), av.begin(), bv.begin(),
+                                   rk.begin(), rv.begin());
+  ASSERT_TRUE(ends.first - rk.begin() == 7 && ends.second - rv.begin() == 7);
+  ASSERT_EQUAL_VEC(to_host(rk), hv<int>({0, 0, 2, 3, 3, 4, 4}));
+  ASSERT_EQUAL_VEC(to_host(rv), hv<int>({13, 42, 7, 42, 7, 42, 13}));  // ties: first range first
+}
+
+// ================================================================ part 2: host vs device
+template <typename T>
+static void DifferentialForType(const char* name) {
+  std::string label = std::string("Differential<") + name + ">";
+  g_test = label.c_str();
+  for (size_t n : kSizes) {
+    thrust::host_vector<T> h = random_integers<T>(n, 7, 0);
+    thrust::device_vector<T> d = h;
+    // reduce (wraps in T on both systems for integers)
+    const T init = (T)13;
+    if (std::is_integral<T>::value) {
+      using U = typename std::conditional<std::is_integral<T>::value, typename std::make_unsigned<
+                typename std::conditional<std::is_integral<T>::value, T, int>::type>::type, T>::type;
+      U acc = (U)init;
+      for (size_t i = 0; i < n; ++i) acc = (U)(acc + (U)h[i]);
+      ASSERT_TRUE(thrust::reduce(d.begin(), d.end(), init) == (T)acc);
+    }
+    // sort / stable_sort
+    thrust::host_vector<T> hs = h;
+    thrust::device_vector<T> ds = d;
+    thrust::sort(hs.begin(), hs.end());
+    thrust::sort(ds.begin(), ds.end());
+    ASSERT_EQUAL_VEC(to_host(ds), hs);
+    hs = h; ds = d;
+    thrust::sort(hs.begin(), hs.end(), thrust::greater<T>());
+    thrust::sort(ds.begin(), ds.end(), thrust::greater<T>());
+    ASSERT_EQUAL_VEC(to_host(ds), hs);
+    // sort_by_key with duplicate-heavy keys: values reveal stability
+    thrust::host_vector<T> hk = random_integers<T>(n, 9, 17);
+    thrust::host_vector<unsigned int> hval(n);
+    for (size_t i = 0; i < n; ++i) hval[i] = (unsigned int)i;
+    thrust::device_vector<T> dk = hk;
+    thrust::device_vector<unsigned int> dval = hval;
+    thrust::stable_sort_by_key(hk.begin(), hk.end(), hval.begin());
+    thrust::stable_sort_by_key(dk.begin(), dk.end(), dval.begin());
+    ASSERT_EQUAL_VEC(to_host(dk), hk);
+    ASSERT_EQUAL_VEC(to_host(dval), hval);
+    // unique / unique_by_key on the sorted keys
+    thrust::host_vector<T> hu = hk;
+    thrust::device_vector<T> du = dk;
+    hu.resize(thrust::unique(hu.begin(), hu.end()) - hu.begin());
+    du.resize(thrust::unique(du.begin(), du.end()) - du.begin());
+    ASSERT_EQUAL_VEC(to_host(du), hu);
+    // reduce_by_key
+    thrust::host_vector<T> hko(n);
+    thrust::host_vector<unsigned int> hvo(n);
+    thrust::device_vector<T> dko(n);
+    thrust::device_vector<unsigned int> dvo(n);
+    auto he = thrust::reduce_by_key(hk.begin(), hk.end(), hval.begin(), hko.begin(), hvo.begin());
+    auto de = thrust::reduce_by_key(dk.begin(), dk.end(), dval.begin(), dko.begin(), dvo.begin());
+    ASSERT_TRUE((he.first - hko.begin()) == (de.first - dko.begin()));
+    hko.resize(he.first - hko.begin()); hvo.resize(hko.size());
+    dko.resize(hko.size()); dvo.resize(hko.size());
+    ASSERT_EQUAL_VEC(to_host(dko), hko);
+    ASSERT_EQUAL_VEC(to_host(dvo), hvo);
+    // scans (integers: exact)
+    if (std::is_integral<T>::value) {
+      thrust::host_vector<T> ho(n);
+      thrust::device_vector<T> dout(n);
+      thrust::inclusive_scan(h.begin(), h.end(), ho.begin());
+      thrust::inclusive_scan(d.begin(), d.end(), dout.begin());
+      ASSERT_EQUAL_VEC(to_host(dout), ho);
+      thrust::exclusive_scan(h.begin(), h.end(), ho.begin(), (T)11);
+      thrust::exclusive_scan(d.begin(), d.end(), dout.begin(), (T)11);
+      ASSERT_EQUAL_VEC(to_host(dout), ho);
+    }
+    // copy_if / stable_partition with a threshold predicate
+    thrust::host_vector<T> hsel = random_integers<T>(n, 21, 100);
+    thrust::device_vector<T> dsel = hsel;
+    thrust::host_vector<T> hc(n);
+    thrust::device_vector<T> dc(n);
+    const T thr = (T)37;
+    hc.resize(thrust::copy_if(hsel.begin(), hsel.end(), hc.begin(), _1 < thr) - hc.begin());
+    dc.resize(thrust::copy_if(dsel.begin(), dsel.end(), dc.begin(), _1 < thr) - dc.begin());
+    ASSERT_EQUAL_VEC(to_host(dc), hc);
+    auto hm = thrust::stable_partition(hsel.begin(), hsel.end(), _1 < thr);
+    auto dm = thrust::stable_partition(dsel.begin(), dsel.end(), _1 < thr);
+    ASSERT_TRUE((hm - hsel.begin()) == (dm - dsel.begin()));
+    ASSERT_EQUAL_VEC(to_host(dsel), hsel);
+    // merge of two sorted ranges
+    thrust::host_vector<T> ha = random_integers<T>(n, 31, 50), hb = random_integers<T>(n / 2 + 1, 33, 50);
+    thrust::sort(ha.begin(), ha.end());
+    thrust::sort(hb.begin(), hb.end());
+    thrust::device_vector<T> da = ha, db = hb;
+    thrust::host_vector<T> hr(ha.size() + hb.size());
+    thrust::device_vector<T> dr(ha.size() + hb.size());
+    thrust::merge(ha.begin(), ha.end(), hb.begin(), hb.end(), hr.begin());
+    thrust::merge(da.begin(), da.end(), db.begin(), db.end(), dr.begin());
+    ASSERT_EQUAL_VEC(to_host(dr), hr);
+  }
+}
+
+static void TestFloatSortTotalOrder() {
+  g_test = "FloatSortTotalOrder";
+  // -0.0 sorts before +0.0 (radix order on the encoded bits), as the reference's
+  // sequential radix sort does (stable_radix_sort.inl:115-125)
+  thrust::device_vector<float> d(hv<float>({0.0f, -0.0f, 1.0f, -1.0f, 0.0f, -0.0f}));
+  thrust::sort(d.begin(), d.end());
+  thrust::host_vector<float> h = d;
+  const uint32_t expect[6] = {0xBF800000u, 0x80000000u, 0x80000000u, 0u, 0u, 0x3F800000u};
+  for (int i = 0; i < 6; ++i) {
+    uint32_t bits;
+    std::memcpy(&bits, &h[i], 4);
+    ASSERT_TRUE(bits == expect[i]);
+  }
+}
+
+// ================================================================ part 3: policies, dispatch, memory
+// A user policy derived from device_execution_policy intercepts an algorithm by overload,
+// as in the reference's examples/minimal_custom_backend.cu:17-37 and
+// testing/unittest/special_types.h:131-166 (my_system / validate_dispatch).
+struct my_system : thrust::device_execution_policy<my_system> {
+  mutable bool dispatched = false;
+};
+template <typename It>
+void sort(my_system& sys, It first, It last) {
+  sys.dispatched = true;
+}
+template <typename It, typename T>
+T reduce(my_system& sys, It, It, T init) {
+  sys.dispatched = true;
+  return init;
+}
+
+static void TestDispatch() {
+  g_test = "Dispatch";
+  thrust::device_vector<int> d(hv<int>({3, 1, 2}));
+  my_system sys;
+  thrust::sort(sys, d.begin(), d.end());
+  ASSERT_TRUE(sys.dispatched);
+  ASSERT_EQUAL_VEC(to_host(d), hv<int>({3, 1, 2}));  // the user's overload ran, not ours
+  my_system sys2;
+  ASSERT_TRUE(thrust::reduce(sys2, d.begin(), d.end(), 42) == 42 && sys2.dispatched);
+  // a derived policy without overloads falls through to the device system
+  my_system sys3;
+  thrust::stable_sort(sys3, d.begin(), d.end());
+  ASSERT_TRUE(!sys3.dispatched);
+  ASSERT_EQUAL_VEC(to_host(d), hv<int>({1, 2, 3}));
+}
+
+static void TestPoliciesAndRawPointers() {
+  g_test = "Policies";
+  thrust::device_vector<int> d(hv<int>({5, 4, 3, 2, 1}));
+  int* raw = thrust::raw_pointer_cast(d.data());
+  // raw device pointers need an explicit device policy
+  thrust::sort(thrust::device, raw, raw + 5);
+  ASSERT_EQUAL_VEC(to_host(d), hv<int>({1, 2, 3, 4, 5}));
+  ASSERT_TRUE(thrust::reduce(thrust::hip::par, raw, raw + 5) == 15);
+  ASSERT_TRUE(thrust::reduce(thrust::hip::par.on(nullptr), d.begin(), d.end(), 1) == 16);
+  // host policies and containers run on the host system
+  std::vector<int> hvec = {3, 1, 2};
+  thrust::sort(thrust::host, hvec.begin(), hvec.end());
+  ASSERT_TRUE(hvec[0] == 1 && hvec[2] == 3);
+  ASSERT_TRUE(thrust::reduce(thrust::seq, hvec.begin(), hvec.end()) == 6);
+  thrust::device_ptr<int> p = thrust::device_pointer_cast(raw);
+  ASSERT_TRUE(thrust::reduce(p, p + 5) == 15);
+}
+
+static void TestDeviceVector() {
+  g_test = "DeviceVector";
+  thrust::device_vector<int> a(4, 7);
+  ASSERT_TRUE(a.size() == 4 && (int)a[0] == 7 && (int)a[3] == 7);
+  a[1] = 42;
+  ASSERT_TRUE((int)a[1] == 42);
+  a[1] += 1;
+  ASSERT_TRUE((int)a[1] == 43);
+  thrust::device_vector<int> b = a;  // device to device
+  b.resize(6);                       // new elements are value-initialised
+  ASSERT_TRUE(b.size() == 6 && (int)b[1] == 43 && (int)b[5] == 0);
+  thrust::host_vector<int> h = b;
+  ASSERT_TRUE(h.size() == 6 && h[0] == 7 && h[1] == 43);
+  thrust::device_vector<int> c(h.begin(), h.end());
+  ASSERT_TRUE(c == b);
+  c.push_back(9);
+  ASSERT_TRUE(c.size() == 7 && (int)c.back() == 9);
+  thrust::fill(c.begin(), c.end(), 3);
+  ASSERT_TRUE(thrust::reduce(c.begin(), c.end()) == 21);
+  thrust::copy(h.begin(), h.end(), c.begin());  // host to device
+  ASSERT_TRUE((int)c[1] == 43);
+  std::vector<int> out(6);
+  thrust::copy(b.begin(), b.end(), out.begin());  // device to host
+  ASSERT_TRUE(out[1] == 43 && out[5] == 0);
+  thrust::device_vector<double> e;
+  ASSERT_TRUE(e.empty() && thrust::reduce(e.begin(), e.end()) == 0.0);
+  thrust::device_vector<int> moved(std::move(c));
+  ASSERT_TRUE(moved.size() == 7 && c.size() == 0);
+  a.swap(b);
+  ASSERT_TRUE(a.size() == 6 && b.size() == 4);
+}
+
+static void TestOutOfMemoryThrows() {  // testing/out_of_memory_recovery.cu:24-34
+  g_test = "OutOfMemory";
+  bool threw = false;
+  try {
+    thrust::device_vector<uint32_t> y(0x00ffffffffffffffull);
+  } catch (const std::bad_alloc&) {
+    threw = true;
+  }
+  ASSERT_TRUE(threw);
+  // the system stays usable afterwards
+  thrust::device_vector<int> ok(hv<int>({2, 1}));
+  thrust::sort(ok.begin(), ok.end());
+  ASSERT_EQUAL_VEC(to_host(ok), hv<int>({1, 2}));
+}
+
+static void TestTempArenaReuse() {
+  g_test = "TempArena";
+  thrust::device_vector<int> d(1 << 20, 1);
+  (void)thrust::reduce(d.begin(), d.end());
+  const size_t held = thrust_amd_temp_bytes_held();
+  for (int i = 0; i < 10; ++i) (void)thrust::reduce(d.begin(), d.end());
+  ASSERT_TRUE(thrust_amd_temp_bytes_held() == held);  // steady state: no new allocations
+  ASSERT_TRUE(thrust_amd_temp_trim() == 0);
+  ASSERT_TRUE(thrust_amd_temp_bytes_held() == 0);
+}
+
+int main() {
+  TestReduceSimple();
+  TestReduceWithOperatorTable();
+  TestScanSimple();
+  TestSortSimple();
+  TestSortByKeySimple();
+  TestReduceByKeySimple();
+  TestUniqueSimple();
+  TestUniqueByKeySimple();
+  TestCopyIfSimple();
+  TestStablePartitionSimple();
+  TestMergeSimple();
+  TestMergeByKeySimple();
+  DifferentialForType<signed char>("signed char");
+  DifferentialForType<short>("short");
+  DifferentialForType<int>("int");
+  DifferentialForType<unsigned int>("unsigned int");
+  DifferentialForType<long long>("long long");
+  DifferentialForType<unsigned long long>("unsigned long long");
+  DifferentialForType<float>("float");
+  DifferentialForType<double>("double");
+  TestFloatSortTotalOrder();
+  TestDispatch();
+  TestPoliciesAndRawPointers();
+  TestDeviceVector();
+  TestOutOfMemoryThrows();
+  TestTempArenaReuse();
+  std::printf("%s: %d checks, %d failed\n", g_failed ? "FAILED" : "PASSED", g_checks, g_failed);
+  return g_failed ? 1 : 0;
+}

@@ -1,0 +1,34 @@
+"""Runs the C++ front-end test programs (the thrust:: API over the C ABI) on the GPU.
+
+The programs are built by tests/cpp/Makefile (driven by __graft_entry__.build) with the
+plain host compiler; they replay the reference's literal known-answer vectors and its
+host-vs-device differential pattern through device_vector.
+"""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "bin")
+
+
+def _run(name, timeout=300):
+    path = os.path.join(BIN, name)
+    assert os.path.exists(path), f"{path} is not built (python -c 'import __graft_entry__ as g; g.build()')"
+    r = subprocess.run([path], capture_output=True, text=True, timeout=timeout)
+    print(r.stdout[-4000:])
+    print(r.stderr[-2000:])
+    assert r.returncode == 0, r.stdout[-4000:]
+    return r.stdout
+
+
+def test_thrust_api_known_answers_and_differential():
+    out = _run("test_thrust_api")
+    assert "PASSED" in out
+
+
+def test_c_abi_from_plain_c():
+    out = _run("test_thrust_c11")
+    assert "PASS" in out
