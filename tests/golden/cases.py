@@ -1,0 +1,90 @@
+"""The seeded cases of the golden fixtures: one function per BASELINE config, returning
+{name: output array} when run on an implementation with the Oracle/Reference interface
+(oracle.cpu) or on the device (tests pass an adapter).  Shared by the fixture writer
+(which runs the REAL reference) and by the tests (which run the restatement / the GPU)."""
+import hashlib
+
+import numpy as np
+
+from thrust_amd import datagen
+
+LT = 0
+SMALL = {"c1": 1 << 14, "c2": 1 << 14, "c3": 1 << 13, "c4": 1 << 15, "c5": 1 << 14}
+LARGE = {"c1": 1 << 22, "c2": 1 << 22, "c3": 1 << 21, "c4": 1 << 22, "c5": 1 << 22}
+
+
+def c1(impl, n):
+    x = datagen.c1_int32(n)
+    x64 = x.astype(np.int64) * 1000003
+    return {
+        "c1.reduce_i32": np.array([impl.reduce(x)], np.int32),
+        "c1.reduce_i32_init7": np.array([impl.reduce(x, init=7)], np.int32),
+        "c1.inclusive_scan_i32": impl.inclusive_scan(x),
+        "c1.exclusive_scan_i32_init5": impl.exclusive_scan(x, 5),
+        "c1.reduce_i64": np.array([impl.reduce(x64)], np.int64),
+        "c1.inclusive_scan_i64": impl.inclusive_scan(x64),
+    }
+
+
+def c2(impl, n):
+    # impl must be the sequential (CPP) system for the float case: the multi-thread OMP
+    # layout of +-0.0 depends on the thread count
+    k = datagen.c2_uint32(n)
+    f = datagen.c2_float32(n)
+    return {
+        "c2.sort_u32": impl.sort_keys(k),
+        "c2.sort_u32_desc": impl.sort_keys(k, descending=True),
+        "c2.sort_f32_bits": impl.sort_keys(f).view(np.uint32),
+        "c2.sort_i32": impl.sort_keys(k.view(np.int32)),
+    }
+
+
+def c3(impl, n):
+    out = {}
+    v = np.arange(n, dtype=np.uint32)
+    for kind in ("full", "low16", "skew90"):
+        k = datagen.c3_uint64(n, kind)
+        ko, vo = impl.sort_pairs(k, v)
+        out[f"c3.{kind}.keys"] = ko
+        out[f"c3.{kind}.values"] = vo
+    return out
+
+
+def c4(impl, n, float_sums=True):
+    out = {}
+    for mean in (8, 1000):
+        k, v = datagen.c4_segments(n, mean)
+        ko, vo = impl.reduce_by_key(k, v)
+        out[f"c4.m{mean}.rbk_keys"] = ko
+        if float_sums:
+            out[f"c4.m{mean}.rbk_sums_f32"] = vo
+        iv = (v * 1000).astype(np.int32)
+        _, io = impl.reduce_by_key(k, iv)
+        out[f"c4.m{mean}.rbk_sums_i32"] = io
+        uk, uv = impl.unique_by_key(k, v)
+        out[f"c4.m{mean}.ubk_keys"] = uk
+        out[f"c4.m{mean}.ubk_values_bits"] = uv.view(np.uint32)
+    return out
+
+
+def c5(impl, n):
+    out = {}
+    x = datagen.c5_float32(n)
+    for t in (0.5, 0.05):
+        out[f"c5.copy_if_lt{t}"] = impl.copy_if(x, LT, t).view(np.uint32)
+        part, split = impl.stable_partition(x, LT, t)
+        out[f"c5.stable_partition_lt{t}"] = part.view(np.uint32)
+        out[f"c5.stable_partition_lt{t}.split"] = np.array([split], np.uint64)
+    (ka, va), (kb, vb) = datagen.c5_merge_inputs(n // 2)
+    ko, vo = impl.merge_by_key(ka, kb, va, vb)
+    out["c5.merge_keys"] = ko
+    out["c5.merge_values"] = vo
+    return out
+
+
+CASES = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5}
+
+
+def digest(a):
+    a = np.ascontiguousarray(a)
+    return hashlib.sha256(a.view(np.uint8).tobytes()).hexdigest()

@@ -1,0 +1,100 @@
+"""GPU parity against the golden fixtures written from the REAL reference
+(tests/golden/make_fixtures.py): every BASELINE config at small N (exact arrays) and at a
+larger N (sha256 of the output bytes).  Bit-exact everywhere except float32 run sums,
+which are compared within 1e-5 relative (tree order on the device, strict left fold in
+the reference)."""
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "golden"))
+
+import cases  # noqa: E402
+
+pytestmark = pytest.mark.gpu
+
+SMALL = np.load(os.path.join(HERE, "golden", "small.npz"))
+DIGESTS = json.load(open(os.path.join(HERE, "golden", "digests.json")))
+
+
+class DeviceImpl:
+    """The oracle's interface implemented by the C ABI on the GPU."""
+
+    def __init__(self, dev):
+        self.dev = dev
+
+    def _d(self, a):
+        return self.dev.DeviceArray.from_numpy(np.ascontiguousarray(a))
+
+    def reduce(self, x, op=0, init=0):
+        return self.dev.reduce(self._d(x), op, init).numpy()[0]
+
+    def inclusive_scan(self, x, op=0):
+        return self.dev.inclusive_scan(self._d(x), op=op).numpy()
+
+    def exclusive_scan(self, x, init=0, op=0):
+        return self.dev.exclusive_scan(self._d(x), init, op=op).numpy()
+
+    def sort_keys(self, k, descending=False):
+        d = self._d(k)
+        self.dev.sort_keys(d, descending=descending)
+        return d.numpy()
+
+    def sort_pairs(self, k, v, descending=False):
+        dk, dv = self._d(k), self._d(v)
+        self.dev.sort_pairs(dk, dv, descending=descending)
+        return dk.numpy(), dv.numpy()
+
+    def reduce_by_key(self, k, v, op=0):
+        ko, vo, runs = self.dev.reduce_by_key(self._d(k), self._d(v), op=op)
+        return ko.numpy(runs), vo.numpy(runs)
+
+    def unique_by_key(self, k, v):
+        ko, vo, cnt = self.dev.unique_by_key(self._d(k), self._d(v))
+        return ko.numpy(cnt), vo.numpy(cnt)
+
+    def copy_if(self, x, cmp, threshold=0, stencil=None):
+        out, cnt = self.dev.copy_if(self._d(x), cmp, threshold,
+                                    stencil=self._d(stencil) if stencil is not None else None)
+        return out.numpy(cnt)
+
+    def stable_partition(self, x, cmp, threshold=0, stencil=None):
+        d = self._d(x)
+        cnt = self.dev.stable_partition(d, cmp, threshold,
+                                        stencil=self._d(stencil) if stencil is not None else None)
+        return d.numpy(), cnt
+
+    def merge_by_key(self, ka, kb, va, vb):
+        ko, vo = self.dev.merge_by_key(self._d(ka), self._d(kb), self._d(va), self._d(vb))
+        return ko.numpy(), vo.numpy()
+
+
+def _bytes_equal(a, b):
+    return np.array_equal(np.ascontiguousarray(a).view(np.uint8), np.ascontiguousarray(b).view(np.uint8))
+
+
+@pytest.mark.parametrize("case", sorted(cases.CASES))
+def test_small_fixtures(dev, case):
+    got = cases.CASES[case](DeviceImpl(dev), cases.SMALL[case])
+    for name, arr in got.items():
+        ref = SMALL[name]
+        if name.endswith("rbk_sums_f32"):
+            assert arr.shape == ref.shape
+            assert np.max(np.abs(arr.astype(np.float64) - ref) / np.abs(ref)) <= 1e-5, name
+        else:
+            assert _bytes_equal(arr, ref), name
+
+
+@pytest.mark.parametrize("case", sorted(cases.CASES))
+def test_large_digests(dev, case):
+    impl = DeviceImpl(dev)
+    if case == "c4":
+        got = cases.c4(impl, cases.LARGE[case], float_sums=False)  # float sums are not bit-exact
+    else:
+        got = cases.CASES[case](impl, cases.LARGE[case])
+    for name, arr in got.items():
+        assert cases.digest(arr) == DIGESTS["sha256"][name], name

@@ -1,0 +1,235 @@
+"""CPU tests that pin the oracle (the C restatement of the reference's OMP / sequential
+device system) -- no GPU involved.
+
+Three independent anchors:
+  1. the literal known-answer vectors of the reference's own unit tests
+     (tests/golden/known_answers.json),
+  2. outputs of the REAL reference on seeded inputs (tests/golden/small.npz, digests.json,
+     written by tests/golden/make_fixtures.py from oracle/_ref), and live against
+     oracle/_ref where that library is present,
+  3. independent definitions: numpy cumsum modulo 2^k, np.sort(kind="stable"),
+     boolean-mask filters, np.add.reduceat in float64, closed forms.
+"""
+import json
+import os
+import sys
+
+import numpy as np
+import pytest
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(HERE, "golden"))
+
+import cases  # noqa: E402
+from oracle import cpu  # noqa: E402
+from thrust_amd import datagen  # noqa: E402
+
+KA = json.load(open(os.path.join(HERE, "golden", "known_answers.json")))
+SMALL = np.load(os.path.join(HERE, "golden", "small.npz"))
+DIGESTS = json.load(open(os.path.join(HERE, "golden", "digests.json")))
+
+I32 = np.int32
+
+
+# ---------------------------------------------------------------- 1. known answers
+def test_known_reduce(oracle):
+    for c in KA["reduce"]:
+        assert oracle.reduce(np.array(c["in"], c["dtype"]), init=c["init"]) == c["out"]
+
+
+def test_known_decompose(oracle):
+    for c in KA["decompose"]:
+        ranges = oracle.decompose(c["n"], c["granularity"], c["max_intervals"])
+        assert [e - b for b, e in ranges] == c["sizes"]
+        assert ranges[0][0] == 0 and ranges[-1][1] == c["n"]
+
+
+def test_known_scans(oracle):
+    for c in KA["inclusive_scan"]:
+        assert oracle.inclusive_scan(np.array(c["in"], c["dtype"])).tolist() == c["out"]
+    for c in KA["exclusive_scan"]:
+        assert oracle.exclusive_scan(np.array(c["in"], c["dtype"]), c["init"]).tolist() == c["out"]
+
+
+def test_known_sorts(oracle, oracle_seq):
+    for o in (oracle, oracle_seq):
+        for c in KA["sort"]:
+            assert o.sort_keys(np.array(c["in"], c["dtype"])).tolist() == c["out"]
+        for c in KA["sort_by_key"]:
+            k, v = o.sort_pairs(np.array(c["keys"], I32), np.array(c["values"], I32))
+            assert k.tolist() == c["keys_out"] and v.tolist() == c["values_out"]
+
+
+def test_known_by_key_and_selection(oracle):
+    for c in KA["reduce_by_key"]:
+        k, v = oracle.reduce_by_key(np.array(c["keys"], I32), np.array(c["values"], I32))
+        assert k.tolist() == c["keys_out"] and v.tolist() == c["values_out"]
+    for c in KA["unique"]:
+        assert oracle.unique(np.array(c["in"], I32)).tolist() == c["out"]
+    for c in KA["unique_by_key"]:
+        k, v = oracle.unique_by_key(np.array(c["keys"], I32), np.array(c["values"], I32))
+        assert k.tolist() == c["keys_out"] and v.tolist() == c["values_out"]
+    for c in KA["copy_if"]:
+        assert oracle.copy_if(np.array(c["in"], I32), cpu.NONZERO).tolist() == c["out"]
+    for c in KA["stable_partition"]:
+        out, split = oracle.stable_partition(np.array(c["in"], I32), cpu.NONZERO,
+                                             stencil=np.array(c["stencil_is_even"], I32))
+        assert out.tolist() == c["out"] and split == c["split"]
+
+
+def test_known_merges(oracle):
+    for c in KA["merge"]:
+        assert oracle.merge(np.array(c["a"], I32), np.array(c["b"], I32)).tolist() == c["out"]
+    for c in KA["merge_by_key"]:
+        k, v = oracle.merge_by_key(np.array(c["a_keys"], I32), np.array(c["b_keys"], I32),
+                                   np.array(c["a_values"], I32), np.array(c["b_values"], I32))
+        assert k.tolist() == c["keys_out"] and v.tolist() == c["values_out"]
+
+
+# ---------------------------------------------------------------- 2. the real reference
+def _bytes_equal(a, b):
+    return np.array_equal(np.ascontiguousarray(a).view(np.uint8), np.ascontiguousarray(b).view(np.uint8))
+
+
+@pytest.mark.parametrize("case", sorted(cases.CASES))
+def test_oracle_reproduces_reference_fixtures(oracle, oracle_seq, case):
+    impl = oracle_seq if case == "c2" else oracle
+    got = cases.CASES[case](impl, cases.SMALL[case])
+    assert got, case
+    for name, arr in got.items():
+        assert _bytes_equal(arr, SMALL[name]), name
+
+
+@pytest.mark.parametrize("case", sorted(cases.CASES))
+def test_oracle_reproduces_reference_digests(oracle, oracle_seq, case):
+    impl = oracle_seq if case == "c2" else oracle
+    got = cases.CASES[case](impl, cases.LARGE[case])
+    for name, arr in got.items():
+        assert cases.digest(arr) == DIGESTS["sha256"][name], name
+
+
+@pytest.mark.skipif(not (cpu.ref_available("omp") and cpu.ref_available("cpp")),
+                    reason="oracle/_ref is built only where the reference tree is present")
+def test_oracle_matches_live_reference_on_ragged_sizes(oracle, oracle_seq):
+    omp, cpp = cpu.Reference("omp"), cpu.Reference("cpp")
+    for n in [0, 1, 2, 7, 8, 9, 63, 1000, 4099, 70001]:
+        x = (datagen.splitmix64(3, n) % np.uint64(1001)).astype(np.int32)
+        assert oracle.reduce(x, init=5) == omp.reduce(x, init=5) == cpp.reduce(x, init=5)
+        assert np.array_equal(oracle.inclusive_scan(x), omp.inclusive_scan(x))
+        assert np.array_equal(oracle.exclusive_scan(x, 3), cpp.exclusive_scan(x, 3))
+        for dt in (np.uint32, np.int64, np.float32, np.float64, np.uint8, np.int16):
+            k = (datagen.splitmix64(5, n) >> np.uint64(11)).astype(dt)
+            if np.dtype(dt).kind == "f":
+                k = (k / dt(3.0) - dt(1e5)).astype(dt)
+                if n > 4:
+                    k[1], k[3] = dt(-0.0), dt(0.0)
+            assert _bytes_equal(oracle_seq.sort_keys(k), cpp.sort_keys(k)), (dt, n)
+            assert _bytes_equal(oracle_seq.sort_keys(k, True), cpp.sort_keys(k, True)), (dt, n)
+            v = np.arange(n, dtype=np.uint32)
+            kk = (k.astype(np.float64) % 7).astype(dt)
+            a, b = oracle.sort_pairs(kk, v), omp.sort_pairs(kk, v)
+            assert _bytes_equal(a[0], b[0]) and np.array_equal(a[1], b[1]), (dt, n)
+            a, b = oracle.sort_pairs(kk, v, True), omp.sort_pairs(kk, v, True)
+            assert _bytes_equal(a[0], b[0]) and np.array_equal(a[1], b[1]), (dt, n)
+        keys = np.sort((datagen.splitmix64(7, n) % np.uint64(50)).astype(np.int32))
+        vals = datagen.u01(9, n)
+        a, b = oracle.reduce_by_key(keys, vals), omp.reduce_by_key(keys, vals)
+        assert np.array_equal(a[0], b[0]) and _bytes_equal(a[1], b[1])
+        for op in (cpu.MIN, cpu.MAX):
+            a, b = oracle.reduce_by_key(keys, vals, op), cpp.reduce_by_key(keys, vals, op)
+            assert np.array_equal(a[0], b[0]) and _bytes_equal(a[1], b[1])
+        a, b = oracle.unique_by_key(keys, vals), omp.unique_by_key(keys, vals)
+        assert np.array_equal(a[0], b[0]) and _bytes_equal(a[1], b[1])
+        assert np.array_equal(oracle.unique(keys), cpp.unique(keys))
+        for cmp in range(6):
+            assert _bytes_equal(oracle.copy_if(vals, cmp, 0.3), omp.copy_if(vals, cmp, 0.3))
+        assert _bytes_equal(oracle.copy_if(vals, cpu.GT, 10, stencil=keys), omp.copy_if(vals, cpu.GT, 10, stencil=keys))
+        a, b = oracle.stable_partition(vals, cpu.LT, 0.5), omp.stable_partition(vals, cpu.LT, 0.5)
+        assert a[1] == b[1] and _bytes_equal(a[0], b[0])
+        a, b = oracle.partition_copy(vals, cpu.LT, 0.5), cpp.partition_copy(vals, cpu.LT, 0.5)
+        assert _bytes_equal(a[0], b[0]) and _bytes_equal(a[1], b[1])
+        kb = np.sort((datagen.splitmix64(11, n // 2 + 1) % np.uint64(50)).astype(np.int32))
+        va, vb = np.arange(n, dtype=np.uint64), np.arange(kb.size, dtype=np.uint64) + 10 ** 9
+        a, b = oracle.merge_by_key(keys, kb, va, vb), omp.merge_by_key(keys, kb, va, vb)
+        assert np.array_equal(a[0], b[0]) and np.array_equal(a[1], b[1])
+
+
+# ---------------------------------------------------------------- 3. independent definitions
+def test_reduce_and_scan_are_sums_modulo_2k(oracle):
+    for dt, bits in ((np.int8, 8), (np.uint16, 16), (np.int32, 32), (np.uint32, 32), (np.int64, 64)):
+        x = (datagen.splitmix64(13, 100003) >> np.uint64(3)).astype(dt)
+        exact = [int(v) for v in x]
+        total = sum(exact)
+        assert (int(oracle.reduce(x)) - total) % (1 << bits) == 0
+        run, ok = 0, True
+        scan = oracle.inclusive_scan(x)
+        for i in (0, 1, 999, 50000, 100002):
+            run = sum(exact[: i + 1])
+            ok = ok and (int(scan[i]) - run) % (1 << bits) == 0
+        assert ok
+        ex = oracle.exclusive_scan(x, 9)
+        assert int(ex[0]) == 9 and (int(ex[-1]) - (9 + total - exact[-1])) % (1 << bits) == 0
+
+
+def test_reduce_is_independent_of_chunk_count_for_integers():
+    x = datagen.c1_int32(100000)
+    vals = {cpu.Oracle(nthreads=p).reduce(x) for p in (1, 2, 3, 7, 8, 64)}
+    assert len(vals) == 1 and int(vals.pop()) == int(np.sum(x.astype(np.int64)))
+
+
+def test_sort_against_numpy_stable_sort(oracle, oracle_seq):
+    n = 200003
+    k = datagen.c2_uint32(n)
+    assert np.array_equal(oracle.sort_keys(k), np.sort(k, kind="stable"))
+    ks = (k % np.uint32(100)).astype(np.uint32)
+    v = np.arange(n, dtype=np.uint32)
+    order = np.argsort(ks, kind="stable")
+    a = oracle.sort_pairs(ks, v)
+    assert np.array_equal(a[0], ks[order]) and np.array_equal(a[1], v[order])
+    f = datagen.c2_float32(n)
+    out = oracle_seq.sort_keys(f)
+    u = out.view(np.uint32)
+    enc = u ^ np.where(u >> 31, np.uint32(0xFFFFFFFF), np.uint32(0x80000000))
+    assert np.all(enc[:-1] <= enc[1:])  # total order on the encoded bits: -0.0 before +0.0
+    assert np.array_equal(np.sort(f), np.sort(out))
+
+
+def test_float_sort_signed_zero_layout_depends_on_thread_count():
+    """Why the parity comparator for float sorts is the sequential system: with several
+    threads the merges compare with operator<, for which -0.0 == +0.0."""
+    f = datagen.c2_float32(1 << 16)
+    seq = cpu.Oracle(nthreads=1).sort_keys(f).view(np.uint32)
+    par = cpu.Oracle(nthreads=8).sort_keys(f).view(np.uint32)
+    assert np.array_equal(np.sort(seq), np.sort(par))  # same multiset of bit patterns
+    assert np.array_equal(seq.view(np.float32), par.view(np.float32))  # equal as values
+
+
+def test_selection_against_boolean_masks(oracle):
+    x = datagen.c5_float32(100003)
+    for t in (0.5, 0.05):
+        m = x < np.float32(t)
+        assert np.array_equal(oracle.copy_if(x, cpu.LT, t), x[m])
+        out, split = oracle.stable_partition(x, cpu.LT, t)
+        assert split == m.sum() and np.array_equal(out, np.r_[x[m], x[~m]])
+
+
+def test_by_key_against_reduceat(oracle):
+    k, v = datagen.c4_segments(100003, 8)
+    starts = np.flatnonzero(np.r_[True, k[1:] != k[:-1]])
+    ko, vo = oracle.reduce_by_key(k, v)
+    assert np.array_equal(ko, k[starts])
+    ref64 = np.add.reduceat(v.astype(np.float64), starts)
+    assert np.max(np.abs(vo - ref64) / ref64) < 1e-5
+    iv = (v * 1000).astype(np.int32)
+    assert np.array_equal(oracle.reduce_by_key(k, iv)[1], np.add.reduceat(iv, starts))
+    uk, uv = oracle.unique_by_key(k, v)
+    assert np.array_equal(uk, k[starts]) and np.array_equal(uv, v[starts])
+
+
+def test_merge_against_stable_sort_of_concatenation(oracle):
+    (ka, va), (kb, vb) = datagen.c5_merge_inputs(50001)
+    ka, kb = ka % np.uint32(1000), kb % np.uint32(1000)
+    ka.sort(), kb.sort()
+    ko, vo = oracle.merge_by_key(ka, kb, va, vb)
+    order = np.argsort(np.r_[ka, kb], kind="stable")
+    assert np.array_equal(ko, np.r_[ka, kb][order]) and np.array_equal(vo, np.r_[va, vb][order])
