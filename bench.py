@@ -27,9 +27,9 @@ N_SORT = 1 << 28
 N_C1 = 1 << 28
 
 # HBM bytes per onesweep pass launch at n = 2^28 uint32, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE, scaled by the same counters on a plain copy kernel of known size (see the
-# profiles/ summary for the sort kernels); None until measured.
-PASS_TRAFFIC_BYTES = None
+# WRITE_SIZE, each scaled by what the same counter reads for kernels of known size in the
+# same run (reduce: 1 GiB read, scan: 1 GiB read + 1 GiB written).
+PASS_TRAFFIC_BYTES = 2.348e9  # profiles/sort_u32_2p28_hbm_traffic.txt
 
 
 def device_random_u32(torch, n, seed):
