@@ -285,9 +285,13 @@ TA_DEVICE uint32_t tile_try_load(const uint64_t* slot, P& payload) {
 // waited on, and those have started, so the spin terminates without assuming any
 // workgroup scheduling order.  `id` must be a true identity of op.  Returns, in all
 // lanes, the fold of all tiles before `tile`.
+#ifndef TA_LOOKBACK_LANES
+#define TA_LOOKBACK_LANES 8
+#endif
 template <typename P, typename Op>
 TA_DEVICE P tile_lookback(const uint64_t* status_base, uint32_t tile, Op op, P id) {
   constexpr int W = TileWords<P>::W;
+  constexpr int WIN = TA_LOOKBACK_LANES;  // descriptors inspected per round (the nearest WIN)
   const int lane = lane_id();
   P running = id;
   int64_t base = (int64_t)tile - 1;
@@ -297,7 +301,10 @@ TA_DEVICE P tile_lookback(const uint64_t* status_base, uint32_t tile, Op op, P i
     uint32_t st;
     uint64_t needed;
     for (;;) {
-      if (idx >= 0) {
+      if (lane < WAVE - WIN) {
+        st = TS_PARTIAL;  // outside the window: contributes nothing
+        val = id;
+      } else if (idx >= 0) {
         st = tile_try_load<P>(status_base + (size_t)idx * W, val);
       } else {
         st = TS_INCLUSIVE;  // before tile 0: an inclusive prefix that contributes nothing
@@ -317,7 +324,7 @@ TA_DEVICE P tile_lookback(const uint64_t* status_base, uint32_t tile, Op op, P i
       }
       __builtin_amdgcn_s_sleep(1);
     }
-    base -= 64;
+    base -= WIN;
   }
 }
 

@@ -88,7 +88,10 @@ __global__ __launch_bounds__(256) void sort_init_kernel(uint32_t* __restrict__ w
 // copy serialise about five-fold on bank conflicts).  Keys are read with 16-byte loads;
 // their order does not matter here.
 constexpr int HIST_BLOCK = 1024;
-constexpr int HIST_UNROLL = 4;  // 16-byte vectors in flight per lane
+#ifndef TA_HIST_UNROLL
+#define TA_HIST_UNROLL 4
+#endif
+constexpr int HIST_UNROLL = TA_HIST_UNROLL;  // 16-byte vectors in flight per lane
 
 template <typename K, int NP>
 __global__ __launch_bounds__(HIST_BLOCK) void sort_histogram_kernel(const K* __restrict__ keys,

@@ -21,7 +21,11 @@ namespace ta {
 // Tile shapes (threads x 16-byte vectors per lane).  The per-tile cost of the ticket
 // (a same-address atomic retires every ~12 ns on MI355X) and of the look-back makes large
 // tiles win once there are enough of them to fill 256 CUs; small inputs use small tiles.
-struct ScanShapeLarge { static constexpr int BLOCK = 1024, CHUNKS = 12; };
+#ifndef TA_SCAN_LARGE_BLOCK
+#define TA_SCAN_LARGE_BLOCK 1024
+#define TA_SCAN_LARGE_CHUNKS 12
+#endif
+struct ScanShapeLarge { static constexpr int BLOCK = TA_SCAN_LARGE_BLOCK, CHUNKS = TA_SCAN_LARGE_CHUNKS; };
 struct ScanShapeSmall { static constexpr int BLOCK = 256, CHUNKS = 4; };
 constexpr uint64_t SCAN_LARGE_MIN_BYTES = (uint64_t)32 << 20;
 
@@ -82,8 +86,9 @@ __global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out,
     }
   }
 
-  // ---- per-lane sums, wave scans chained through the chunks
-  T lane_excl[SCAN_CHUNKS];
+  // ---- wave-local scan in place: every element becomes the fold of the wave's span up to
+  // it (inclusive), or up to but excluding it (exclusive); CHUNKS DPP wave scans chained by
+  // the wave total.  Nothing but x[] and the carry stays live.
   T carry = id;  // fold of this wave's chunks before chunk j
 #pragma unroll
   for (int j = 0; j < SCAN_CHUNKS; ++j) {
@@ -91,8 +96,19 @@ __global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out,
 #pragma unroll
     for (int i = 1; i < VEC; ++i) s = op(s, x[j].v[i]);
     const T incl = wave_inclusive_scan(s, op, id);
-    lane_excl[j] = op(carry, wave_shift_up(incl, id));
+    T run = op(carry, wave_shift_up(incl, id));
     carry = op(carry, readlane(incl, WAVE - 1));
+#pragma unroll
+    for (int i = 0; i < VEC; ++i) {
+      if constexpr (EXCLUSIVE) {
+        const T next = op(run, x[j].v[i]);
+        x[j].v[i] = run;
+        run = next;
+      } else {
+        run = op(run, x[j].v[i]);
+        x[j].v[i] = run;
+      }
+    }
   }
   if (lane == 0) s_wave_agg[wave] = carry;
   __syncthreads();
@@ -123,21 +139,11 @@ __global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out,
   if constexpr (EXCLUSIVE) prefix = (tile == 0) ? init : op(init, prefix);
   prefix = op(prefix, wave_prefix);
 
-  // ---- apply and store
+  // ---- apply the prefix of everything before this wave and store
 #pragma unroll
   for (int j = 0; j < SCAN_CHUNKS; ++j) {
-    T run = op(prefix, lane_excl[j]);
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      if constexpr (EXCLUSIVE) {
-        const T next = op(run, x[j].v[i]);
-        x[j].v[i] = run;
-        run = next;
-      } else {
-        run = op(run, x[j].v[i]);
-        x[j].v[i] = run;
-      }
-    }
+    for (int i = 0; i < VEC; ++i) x[j].v[i] = op(prefix, x[j].v[i]);
   }
   if (valid == TILE) {
 #pragma unroll
