@@ -88,10 +88,7 @@ __global__ __launch_bounds__(256) void sort_init_kernel(uint32_t* __restrict__ w
 // copy serialise about five-fold on bank conflicts).  Keys are read with 16-byte loads;
 // their order does not matter here.
 constexpr int HIST_BLOCK = 1024;
-#ifndef TA_HIST_UNROLL
-#define TA_HIST_UNROLL 4
-#endif
-constexpr int HIST_UNROLL = TA_HIST_UNROLL;  // 16-byte vectors in flight per lane
+constexpr int HIST_UNROLL = 2;  // 16-byte vectors in flight per lane
 
 template <typename K, int NP>
 __global__ __launch_bounds__(HIST_BLOCK) void sort_histogram_kernel(const K* __restrict__ keys,
@@ -208,19 +205,6 @@ __global__ __launch_bounds__(RADIX_SIZE) void sort_scan_kernel(uint32_t* __restr
 }
 
 // ------------------------------------------------------------------ onesweep pass
-#ifdef TA_DBG_PHASES
-__device__ unsigned long long g_phase[16384 * 16];
-#define TA_PHASE(i)                                                                   \
-  do {                                                                                \
-    if (threadIdx.x == TA_DBG_PHASE_THREAD) {                                         \
-      const unsigned long long _now = __builtin_readcyclecounter();                   \
-      g_phase[blockIdx.x * 16 + (i)] += _now - _t_prev;                                         \
-      _t_prev = _now;                                                                 \
-    }                                                                                 \
-  } while (0)
-#else
-#define TA_PHASE(i)
-#endif
 // f(a, b, c) = a & ~(b ^ c): truth table index = a*4 + b*2 + c.
 constexpr int BITOP_AND_XNOR = 0x90;
 
@@ -234,20 +218,11 @@ struct PassShape {
   static constexpr size_t UNION_BYTES = EXCH_BYTES > CNT_BYTES ? EXCH_BYTES : CNT_BYTES;
 };
 
-#ifndef TA_RANK_VARIANT
-#define TA_RANK_VARIANT 1
-#endif
-#ifndef TA_BFE_ASM
-#define TA_BFE_ASM 1
-#endif
-#ifndef TA_RANK_GROUP
-#define TA_RANK_GROUP 2
-#endif
-#ifndef TA_SORT_MIN_WAVES
-#define TA_SORT_MIN_WAVES 1
-#endif
+// Tile descriptors fetched together per look-back round by each digit thread.
+constexpr int LOOKBACK_WINDOW = 4;
+
 template <typename K, typename V, bool HAS_VALUES, int BLOCK, int ITEMS>
-__global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel(
+__global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     K* __restrict__ keys_a, K* __restrict__ keys_b, V* __restrict__ vals_a, V* __restrict__ vals_b,
     uint32_t n, int pass, SortGeometry geo, KeyCodec<K> codec,
     const uint32_t* __restrict__ bin_base,  // [RADIX_SIZE] global digit offsets of this pass
@@ -259,9 +234,6 @@ __global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel
   static_assert(BLOCK >= RADIX_SIZE, "one thread per digit is required");
 
   if (ctl->skip[pass]) return;
-#ifdef TA_DBG_PHASES
-  unsigned long long _t_prev = __builtin_readcyclecounter();
-#endif
   const bool from_alt = ctl->src_alt[pass] != 0;
   const K* __restrict__ keys_in = from_alt ? keys_b : keys_a;
   K* __restrict__ keys_out = from_alt ? keys_a : keys_b;
@@ -276,14 +248,11 @@ __global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel
   K* s_keys = reinterpret_cast<K*>(s_union);
   V* s_vals = reinterpret_cast<V*>(s_union);
 
-#ifdef TA_DBG_NOTICKET
-  if (threadIdx.x == 0) s_tile = blockIdx.x;
-#else
-  if (threadIdx.x == 0) s_tile = atomicAdd(ticket, 1u);
-#endif
+  if (threadIdx.x == 0) {
+    s_tile = atomicAdd(ticket, 1u);
+  }
   for (int i = threadIdx.x; i < WAVES * RADIX_SIZE; i += BLOCK) s_cnt[i] = 0;
   __syncthreads();
-  TA_PHASE(0);
   const uint32_t tile = s_tile;
   const uint32_t tile_base = tile * (uint32_t)TILE;
   const uint32_t valid = (n - tile_base < (uint32_t)TILE) ? (n - tile_base) : (uint32_t)TILE;
@@ -312,7 +281,6 @@ __global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel
     }
   }
 
-  TA_PHASE(1);
   // ---- rank inside the wave by digit
   // Per digit bit: v_bfe_i32 (lane's bit as 0 / -1), one ballot, and two v_bitop3 folding
   // "same bit as mine" into the 64-bit peer mask.  The wave-private counter is read, then
@@ -329,45 +297,25 @@ __global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel
 #pragma unroll
     for (int b = 0; b < RADIX_BITS; ++b) {
       int sb;
-#if TA_BFE_ASM
       // opaque to the optimiser so that the compare below is made on sb itself
       asm volatile("v_bfe_i32 %0, %1, %2, 1" : "=v"(sb) : "v"(d), "n"(b));
-#else
-      sb = __builtin_amdgcn_sbfe(d, b, 1);
-#endif
       const uint64_t m = __builtin_amdgcn_ballot_w64(sb != 0);
       peers_lo = __builtin_amdgcn_bitop3_b32(peers_lo, (uint32_t)m, (uint32_t)sb, BITOP_AND_XNOR);
       peers_hi = __builtin_amdgcn_bitop3_b32(peers_hi, (uint32_t)(m >> 32), (uint32_t)sb, BITOP_AND_XNOR);
     }
     const uint32_t below = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
-#if TA_RANK_VARIANT == 3
-    const uint32_t old = 0; (void)my_cnt;
-#elif TA_RANK_VARIANT == 2
-    const uint32_t total = __builtin_popcount(peers_lo) + __builtin_popcount(peers_hi);
-    const uint32_t old = my_cnt[d];
-    if (below == total - 1) my_cnt[d] = old + total;
-#elif TA_RANK_VARIANT == 4
-    const uint32_t total = __builtin_popcount(peers_lo) + __builtin_popcount(peers_hi);
-    const uint32_t old = my_cnt[d];
-    my_cnt[d] = old + total;
-#else
     const uint32_t old = my_cnt[d];
     __hip_atomic_fetch_add(&my_cnt[d], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-#endif
     if (r % 2 == 0) rank2[r / 2] = old + below;
     else rank2[r / 2] |= (old + below) << 16;
     // pin the packed rank here: otherwise the add is sunk past the barrier and `old` and
     // `below` of every round stay live
     asm volatile("" : "+v"(rank2[r / 2]));
-#if TA_RANK_GROUP > 0
     // keep the scheduler from computing all peer masks first (two live registers per
-    // round): rounds are finished in groups
-    if (r % TA_RANK_GROUP == TA_RANK_GROUP - 1) __builtin_amdgcn_sched_barrier(0);
-#endif
+    // round): rounds are finished in pairs
+    if (r % 2 == 1) __builtin_amdgcn_sched_barrier(0);
   }
-  TA_PHASE(2);
   __syncthreads();
-  TA_PHASE(3);
 
   // ---- per digit: offsets of the waves, tile count; publish the tile's partial counts
   uint32_t digit_count = 0;
@@ -404,7 +352,6 @@ __global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel
   }
   __syncthreads();
 
-  TA_PHASE(4);
   // ---- final position of every key inside the tile
 #pragma unroll
   for (int r = 0; r < ITEMS; ++r) {
@@ -416,8 +363,11 @@ __global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel
 #pragma unroll
   for (int r = 0; r < ITEMS; ++r) s_keys[(rank2[r / 2] >> (16 * (r % 2))) & 0xffffu] = e[r];
 
-  TA_PHASE(5);
   // ---- look-back: global offset of each digit run of this tile
+  // Windowed: the descriptors of the LOOKBACK_WINDOW nearest unread predecessors are
+  // fetched together (one memory round trip instead of one per tile), then folded nearest
+  // first up to the first inclusive one.  A descriptor not yet published stops the fold;
+  // the next window starts at that tile.
   if (threadIdx.x < RADIX_SIZE) {
     const int d = threadIdx.x;
     uint32_t excl;
@@ -425,21 +375,32 @@ __global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel
       excl = bin_base[d];
     } else {
       uint32_t acc = 0;
-      int64_t t = (int64_t)tile - 1;
-#ifdef TA_DBG_NOLOOKBACK
-      if (false)
-#endif
+      int t = (int)tile - 1;  // tile counts stay below 2^16
+      const uint32_t* my_col = status + d;
       for (;;) {
-        const uint32_t s = __hip_atomic_load(status + (size_t)t * RADIX_SIZE + d, __ATOMIC_RELAXED,
-                                             __HIP_MEMORY_SCOPE_AGENT);
-        const uint32_t flag = s & ~ST_VALUE_MASK;
-        if (flag == 0) {
-          __builtin_amdgcn_s_sleep(1);
-          continue;
+        uint32_t s[LOOKBACK_WINDOW];
+#pragma unroll
+        for (int k = 0; k < LOOKBACK_WINDOW; ++k) {
+          const uint32_t tk = (uint32_t)((t - k) > 0 ? (t - k) : 0);  // tile 0 is always inclusive
+          s[k] = __hip_atomic_load(my_col + (size_t)tk * RADIX_SIZE, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
         }
-        acc += s & ST_VALUE_MASK;
-        if (flag == ST_INCLUSIVE) break;
-        --t;
+        __builtin_amdgcn_sched_barrier(0);  // all loads are in flight before the first is used
+        bool done = false;
+        int used = 0;
+#pragma unroll
+        for (int k = 0; k < LOOKBACK_WINDOW; ++k) {
+          const uint32_t flag = s[k] & ~ST_VALUE_MASK;
+          const bool take = !done && used == k && flag != 0;
+          if (take) {
+            acc += s[k] & ST_VALUE_MASK;
+            used = k + 1;
+            done = flag == ST_INCLUSIVE;
+          }
+        }
+        if (done) break;
+        t -= used;
+        if (used < LOOKBACK_WINDOW) __builtin_amdgcn_s_sleep(1);
       }
       excl = acc;
     }
@@ -447,9 +408,7 @@ __global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel
                        __HIP_MEMORY_SCOPE_AGENT);
     s_scatter_base[d] = excl - local_base;
   }
-  TA_PHASE(6);
   __syncthreads();
-  TA_PHASE(7);
 
   // ---- keys leave in tile-sorted order: consecutive lanes write consecutive addresses
   // Batched so that the 2*ITEMS LDS reads are independent and in flight together.
@@ -474,7 +433,6 @@ __global__ __launch_bounds__(BLOCK, TA_SORT_MIN_WAVES) void onesweep_pass_kernel
         if ((uint32_t)k * BLOCK + threadIdx.x < valid) keys_out[gpos[k]] = ek[k];
     }
   }
-  TA_PHASE(8);
   if constexpr (HAS_VALUES) {
     V v[ITEMS];
 #pragma unroll
@@ -526,15 +484,13 @@ static KeyCodec<K> make_codec(int dtype, int descending) {
 
 template <typename K, typename V, bool HAS_VALUES>
 struct SortPlan {
-  // 16384-key tiles for 4-byte keys keep the ticket rate (one same-address atomic per
-  // tile) far below what a pass needs; 8-byte keys halve the tile to fit LDS.
-#if defined(TA_SORT_BLOCK)
-  static constexpr int BLOCK = TA_SORT_BLOCK;
-  static constexpr int ITEMS = TA_SORT_ITEMS;
-#else
+  // Large tiles (16K-18K keys of 4 bytes) keep the number of tiles in flight, and with it
+  // the length of every look-back, small; two blocks of 1024 threads fill a CU (64 VGPRs,
+  // 80 KB of LDS each).  8-byte keys or values halve the tile to fit LDS.
   static constexpr int BLOCK = 1024;
-  static constexpr int ITEMS = (sizeof(K) == 8 || (HAS_VALUES && sizeof(V) == 8)) ? 8 : 16;
-#endif
+  static constexpr int ITEMS = (sizeof(K) == 8 || (HAS_VALUES && sizeof(V) == 8)) ? 8
+                               : (sizeof(K) == 4 && !HAS_VALUES)                 ? 18
+                                                                                 : 16;
   static constexpr int TILE = BLOCK * ITEMS;
 };
 
