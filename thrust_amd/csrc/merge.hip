@@ -56,13 +56,19 @@ __global__ __launch_bounds__(256) void merge_partition_kernel(const T* __restric
   a_split[t] = merge_path<T>(a, na, b, nb, diag, descending != 0);
 }
 
+// Slot of output element e in the LDS exchange buffer: one spare slot after every
+// MERGE_ITEMS keeps both access patterns off the same banks (lane t writes its run
+// t*ITEMS .. t*ITEMS+ITEMS-1, i.e. slots t*(ITEMS+1)+o; the write-out reads consecutive e).
+TA_DEVICE uint32_t merge_slot(uint32_t e) { return e + e / MERGE_ITEMS; }
+constexpr int MERGE_SLOTS = MERGE_TILE + MERGE_TILE / MERGE_ITEMS + 1;
+
 template <typename T, typename V, bool HAS_VALUES>
 __global__ __launch_bounds__(MERGE_BLOCK) void merge_kernel(
     const T* __restrict__ a, uint64_t na, const T* __restrict__ b, uint64_t nb,
     const V* __restrict__ va, const V* __restrict__ vb, T* __restrict__ out, V* __restrict__ vout,
     int descending_i, const uint64_t* __restrict__ a_split) {
   constexpr size_t ITEM = (HAS_VALUES && sizeof(V) > sizeof(T)) ? sizeof(V) : sizeof(T);
-  __shared__ __attribute__((aligned(16))) unsigned char s_raw[(size_t)(MERGE_TILE + 1) * ITEM];
+  __shared__ __attribute__((aligned(16))) unsigned char s_raw[(size_t)MERGE_SLOTS * ITEM];
   T* s_keys = reinterpret_cast<T*>(s_raw);
   V* s_vals = reinterpret_cast<V*>(s_raw);
   const bool descending = descending_i != 0;
@@ -77,55 +83,76 @@ __global__ __launch_bounds__(MERGE_BLOCK) void merge_kernel(
   const uint32_t count = ca + cb;  // == d1 - d0
 
   // ---- stage the keys: A's part first, then B's
+  {
+    T in[MERGE_ITEMS];
 #pragma unroll
-  for (int i = 0; i < MERGE_ITEMS; ++i) {
-    const uint32_t e = i * MERGE_BLOCK + threadIdx.x;
-    if (e < ca) s_keys[e] = a[a0 + e];
-    else if (e < count) s_keys[e] = b[b0 + (e - ca)];
+    for (int q = 0; q < MERGE_ITEMS; ++q) {
+      const uint32_t e = q * MERGE_BLOCK + threadIdx.x;
+      in[q] = (e < ca) ? a[a0 + e] : (e < count) ? b[b0 + (e - ca)] : T{};
+    }
+#pragma unroll
+    for (int q = 0; q < MERGE_ITEMS; ++q) s_keys[q * MERGE_BLOCK + threadIdx.x] = in[q];
   }
   __syncthreads();
 
   // ---- this lane's start on the path, then a serial merge of ITEMS elements
-  const uint32_t diag = (threadIdx.x * MERGE_ITEMS < count) ? threadIdx.x * MERGE_ITEMS : count;
+  const uint32_t run0 = threadIdx.x * MERGE_ITEMS;
+  const uint32_t diag = run0 < count ? run0 : count;
   uint32_t i = (uint32_t)merge_path<T>(s_keys, (uint64_t)ca, s_keys + ca, (uint64_t)cb, (uint64_t)diag,
                                        descending);
-  uint32_t j = diag - i;  // index into B's part
+  uint32_t j = ca + (diag - i);  // slot of the next element of B's part
   T k[MERGE_ITEMS];
   uint32_t src[MERGE_ITEMS];
-  T ka = (i < ca) ? s_keys[i] : T{};
-  T kb = (j < cb) ? s_keys[ca + j] : T{};
+  // slots past the parts hold staged padding (or the one slack slot): reads stay in bounds
+  T ka = s_keys[i];
+  T kb = s_keys[j];
 #pragma unroll
   for (int o = 0; o < MERGE_ITEMS; ++o) {
-    const bool take_b = (j < cb) && (i >= ca || merge_comp(kb, ka, descending));
+    const bool take_b = (j < count) && (i >= ca || merge_comp(kb, ka, descending));
     k[o] = take_b ? kb : ka;
-    src[o] = take_b ? ca + j : i;
-    if (take_b) {
-      ++j;
-      kb = s_keys[ca + j];  // one slot of slack behind the tile keeps this read in bounds
-    } else {
-      ++i;
-      ka = s_keys[i];
-    }
+    src[o] = take_b ? j : i;
+    const uint32_t next = take_b ? ++j : ++i;
+    const T nk = s_keys[next];  // next <= count <= MERGE_TILE
+    if (take_b) kb = nk;
+    else ka = nk;
+  }
+  __syncthreads();  // all keys have been read from the staging area
+
+  // ---- keys leave through LDS so that consecutive lanes write consecutive addresses
+#pragma unroll
+  for (int o = 0; o < MERGE_ITEMS; ++o) s_keys[merge_slot(run0 + o)] = k[o];
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < MERGE_ITEMS; ++q) {
+    const uint32_t e = q * MERGE_BLOCK + threadIdx.x;
+    if (e < count) out[d0 + e] = s_keys[merge_slot(e)];
   }
 
-  // ---- keys out
-  const uint64_t obase = d0 + (uint64_t)threadIdx.x * MERGE_ITEMS;
-#pragma unroll
-  for (int o = 0; o < MERGE_ITEMS; ++o)
-    if (threadIdx.x * MERGE_ITEMS + o < count) out[obase + o] = k[o];
-
   if constexpr (HAS_VALUES) {
-    __syncthreads();  // everyone is done reading keys from LDS
+    __syncthreads();  // key write-out has read the exchange buffer
+    {
+      V in[MERGE_ITEMS];
+#pragma unroll
+      for (int q = 0; q < MERGE_ITEMS; ++q) {
+        const uint32_t e = q * MERGE_BLOCK + threadIdx.x;
+        in[q] = (e < ca) ? va[a0 + e] : (e < count) ? vb[b0 + (e - ca)] : V{};
+      }
+#pragma unroll
+      for (int q = 0; q < MERGE_ITEMS; ++q) s_vals[q * MERGE_BLOCK + threadIdx.x] = in[q];
+    }
+    __syncthreads();
+    V v[MERGE_ITEMS];
+#pragma unroll
+    for (int o = 0; o < MERGE_ITEMS; ++o) v[o] = s_vals[src[o]];  // src[o] < count for valid outputs
+    __syncthreads();
+#pragma unroll
+    for (int o = 0; o < MERGE_ITEMS; ++o) s_vals[merge_slot(run0 + o)] = v[o];
+    __syncthreads();
 #pragma unroll
     for (int q = 0; q < MERGE_ITEMS; ++q) {
       const uint32_t e = q * MERGE_BLOCK + threadIdx.x;
-      if (e < ca) s_vals[e] = va[a0 + e];
-      else if (e < count) s_vals[e] = vb[b0 + (e - ca)];
+      if (e < count) vout[d0 + e] = s_vals[merge_slot(e)];
     }
-    __syncthreads();
-#pragma unroll
-    for (int o = 0; o < MERGE_ITEMS; ++o)
-      if (threadIdx.x * MERGE_ITEMS + o < count) vout[obase + o] = s_vals[src[o]];
   }
 }
 
