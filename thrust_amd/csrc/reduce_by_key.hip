@@ -21,29 +21,18 @@
 
 namespace ta {
 
-constexpr int RBK_BLOCK = 1024;
-constexpr int RBK_ITEMS = 16;  // elements per lane
-
-// Operator chosen at run time (uniform across the grid).
-struct RtOp {
-  int op;
-  template <typename T>
-  TA_DEVICE T operator()(T a, T b) const {
-    switch (op) {
-      case THRUST_AMD_PLUS: return OpPlus{}(a, b);
-      case THRUST_AMD_MIN: return OpMin{}(a, b);
-      default: return OpMax{}(a, b);
-    }
-  }
-  template <typename T>
-  TA_HOST_DEVICE T identity_value() const {
-    switch (op) {
-      case THRUST_AMD_PLUS: return OpPlus::identity<T>();
-      case THRUST_AMD_MIN: return OpMin::identity<T>();
-      default: return OpMax::identity<T>();
-    }
-  }
-};
+#ifndef TA_RBK_BLOCK
+#define TA_RBK_BLOCK 1024
+#endif
+constexpr int RBK_BLOCK = TA_RBK_BLOCK;
+#ifndef TA_RBK_ITEMS
+#define TA_RBK_ITEMS 16
+#endif
+#ifndef TA_RBK_MIN_WAVES
+#define TA_RBK_MIN_WAVES 4
+#endif
+constexpr int RBK_ITEMS = TA_RBK_ITEMS;  // elements per lane
+constexpr int RBK_MIN_WAVES = TA_RBK_MIN_WAVES;
 
 template <typename V>
 struct alignas(sizeof(V) >= 8 ? 8 : 4) SegPair {
@@ -57,9 +46,9 @@ template <> struct SegValue<uint8_t> { using type = uint32_t; };
 template <> struct SegValue<int16_t> { using type = int32_t; };
 template <> struct SegValue<uint16_t> { using type = uint32_t; };
 
-template <typename V>
+template <typename V, typename Op>
 struct SegOp {
-  RtOp op;
+  Op op;
   // value folds are done in the storage type V and widened only for transport
   using WV = typename SegValue<V>::type;
   TA_DEVICE SegPair<WV> operator()(const SegPair<WV>& a, const SegPair<WV>& b) const {
@@ -78,7 +67,6 @@ struct RbkArgs {
   V* values_out;
   uint64_t* d_num_runs;
   uint64_t n;
-  RtOp op;
   uint64_t* status;
   uint32_t* ticket;
   uint32_t aligned;
@@ -102,8 +90,8 @@ __global__ __launch_bounds__(256) void rbk_init_kernel(uint64_t* __restrict__ wo
 
 // K is the key's comparison class: an unsigned integer type of the key's size (integer
 // keys are equal iff their bits are) or float / double (operator==).
-template <typename K, typename V>
-__global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
+template <typename K, typename V, typename Op>
+__global__ __launch_bounds__(RBK_BLOCK, RBK_MIN_WAVES) void rbk_kernel(RbkArgs<K, V> a) {
   constexpr int VEC = Vec16<K>::N;
   constexpr int CHUNKS = RBK_ITEMS / VEC >= 1 ? RBK_ITEMS / VEC : 1;
   constexpr int WAVES = RBK_BLOCK / WAVE;
@@ -112,8 +100,8 @@ __global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
   using WV = typename SegValue<V>::type;
   using Pair = SegPair<WV>;
   using VV = RbkValueVec<V, VEC>;
-  const SegOp<V> sop{a.op};
-  const V vid = a.op.template identity_value<V>();
+  const SegOp<V, Op> sop{Op{}};
+  const V vid = Op::template identity<V>();
   const Pair pid{0u, (WV)vid};
 
   __shared__ uint32_t s_tile;
@@ -234,9 +222,9 @@ __global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
   }
 }
 
-template <typename K, typename V>
+template <typename K, typename V, typename Op>
 static int rbk_run(void* temp, size_t* temp_bytes, const void* keys_in, const void* values_in,
-                   void* keys_out, void* values_out, uint64_t* d_num_runs, uint64_t n, int op,
+                   void* keys_out, void* values_out, uint64_t* d_num_runs, uint64_t n,
                    hipStream_t stream) {
   constexpr int VEC = Vec16<K>::N;
   constexpr int CHUNKS = RBK_ITEMS / VEC >= 1 ? RBK_ITEMS / VEC : 1;
@@ -262,7 +250,6 @@ static int rbk_run(void* temp, size_t* temp_bytes, const void* keys_in, const vo
   a.values_out = static_cast<V*>(values_out);
   a.d_num_runs = d_num_runs;
   a.n = n;
-  a.op = RtOp{op};
   a.ticket = reinterpret_cast<uint32_t*>(base + off_ticket);
   a.status = reinterpret_cast<uint64_t*>(base + off_status);
   a.aligned = is_aligned16(keys_in) &&
@@ -273,7 +260,7 @@ static int rbk_run(void* temp, size_t* temp_bytes, const void* keys_in, const vo
             a.status, words, a.ticket, d_num_runs);
   TA_CHECK_LAUNCH();
   if (n == 0) return 0;
-  TA_LAUNCH("reduce_by_key", stream, (rbk_kernel<K, V>), dim3((uint32_t)tiles), dim3(RBK_BLOCK), a);
+  TA_LAUNCH("reduce_by_key", stream, (rbk_kernel<K, V, Op>), dim3((uint32_t)tiles), dim3(RBK_BLOCK), a);
   TA_CHECK_LAUNCH();
   return 0;
 }
@@ -291,8 +278,10 @@ TA_EXPORT int thrust_amd_reduce_by_key(void* temp, size_t* temp_bytes, const voi
     using K = typename decltype(kt)::type;
     return with_dtype(value_dtype, [&](auto vt) {
       using V = typename decltype(vt)::type;
-      return rbk_run<K, V>(temp, temp_bytes, keys_in, values_in, keys_out, values_out, d_num_runs, n,
-                           op, (hipStream_t)stream);
+      return with_binop(op, [&](auto o) {
+        return rbk_run<K, V, decltype(o)>(temp, temp_bytes, keys_in, values_in, keys_out, values_out,
+                                          d_num_runs, n, (hipStream_t)stream);
+      });
     });
   };
   if (key_dtype == THRUST_AMD_F32) return by_value(TypeTag<float>{});
