@@ -29,7 +29,7 @@ N_C1 = 1 << 28
 # HBM bytes per onesweep pass launch at n = 2^28 uint32, from rocprofv3 --pmc FETCH_SIZE /
 # WRITE_SIZE, each scaled by what the same counter reads for kernels of known size in the
 # same run (reduce: 1 GiB read, scan: 1 GiB read + 1 GiB written).
-PASS_TRAFFIC_BYTES = 2.348e9  # profiles/sort_u32_2p28_hbm_traffic.txt
+PASS_TRAFFIC_BYTES = 2.318e9  # profiles/sort_u32_2p28_hbm_traffic.txt
 
 
 def device_random_u32(torch, n, seed):

@@ -239,9 +239,9 @@ int thrust_amd_reduce_by_key(void* temp, size_t* temp_bytes, const void* keys_in
 
 /* -------------------------------------------------------------------- merge */
 
-/* Stable merge of two ranges sorted in the radix-encoding order of dtype (ascending, or
- * descending when descending != 0) into out (na + nb elements).  Ties: every equal
- * element of `a` precedes those of `b`
+/* Stable merge of two ranges sorted by operator< of dtype (ascending; by operator> when
+ * descending != 0) into out (na + nb elements).  Keys are compared by value: for floats
+ * -0.0 and +0.0 are equal.  Ties: every equal element of `a` precedes those of `b`
  * (thrust/system/detail/sequential/merge.inl:56-65).  out must not alias a or b.
  * Replaces cuda_cub::__merge::merge keys-only (thrust/system/cuda/detail/merge.h:785-853). */
 int thrust_amd_merge(void* temp, size_t* temp_bytes, const void* a, uint64_t na, const void* b,
