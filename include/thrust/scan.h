@@ -4,6 +4,11 @@
 // P0571): inclusive scans accumulate in the input's value type, exclusive scans in the
 // type of init; exclusive_scan(first,last,result) uses init = value_type(0); the default
 // operator is plus (thrust/system/detail/generic/scan.inl:39-81).  In-place is allowed.
+//
+// thrust::inclusive_scan_by_key and thrust::exclusive_scan_by_key scan every run of
+// consecutive equal keys on its own (thrust/system/detail/generic/scan_by_key.inl:62-238):
+// default key predicate equal_to, default operator plus, default init value_type{}; the
+// exclusive form yields init at the first element of every run.
 #pragma once
 #include <thrust/functional.h>
 #include <thrust/system/hip/detail/backend.h>
@@ -21,9 +26,48 @@ Out exclusive_scan(const detail::execution_policy_base<D>& exec, In first, In la
 template <typename D, typename In, typename Out, typename T, typename Op>
 Out exclusive_scan(const detail::execution_policy_base<D>& exec, In first, In last, Out result, T init, Op op);
 
+template <typename D, typename KIt, typename VIt, typename Out>
+Out inclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, Out result);
+template <typename D, typename KIt, typename VIt, typename Out, typename Pred>
+Out inclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred pred);
+template <typename D, typename KIt, typename VIt, typename Out, typename Pred, typename Op>
+Out inclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred pred,
+                          Op op);
+template <typename D, typename KIt, typename VIt, typename Out>
+Out exclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, Out result);
+template <typename D, typename KIt, typename VIt, typename Out, typename T>
+Out exclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init);
+template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred>
+Out exclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init,
+                          Pred pred);
+template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
+Out exclusive_scan_by_key(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init,
+                          Pred pred, Op op);
+
 namespace system {
 namespace detail {
 namespace generic {
+template <typename D, typename KIt, typename VIt, typename Out>
+Out inclusive_scan_by_key(thrust::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result) {
+  return thrust::inclusive_scan_by_key(exec, kf, kl, vf, result, thrust::equal_to<>());
+}
+template <typename D, typename KIt, typename VIt, typename Out, typename Pred>
+Out inclusive_scan_by_key(thrust::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred pred) {
+  return thrust::inclusive_scan_by_key(exec, kf, kl, vf, result, pred, thrust::plus<>());
+}
+template <typename D, typename KIt, typename VIt, typename Out>
+Out exclusive_scan_by_key(thrust::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result) {
+  typedef typename iterator_value<VIt>::type T;
+  return thrust::exclusive_scan_by_key(exec, kf, kl, vf, result, T());
+}
+template <typename D, typename KIt, typename VIt, typename Out, typename T>
+Out exclusive_scan_by_key(thrust::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init) {
+  return thrust::exclusive_scan_by_key(exec, kf, kl, vf, result, init, thrust::equal_to<>());
+}
+template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred>
+Out exclusive_scan_by_key(thrust::execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init, Pred pred) {
+  return thrust::exclusive_scan_by_key(exec, kf, kl, vf, result, init, pred, thrust::plus<>());
+}
 template <typename D, typename In, typename Out>
 Out inclusive_scan(thrust::execution_policy<D>& exec, In first, In last, Out result) {
   return thrust::inclusive_scan(exec, first, last, result, thrust::plus<>());
@@ -62,6 +106,44 @@ Out exclusive_scan(execution_policy<D>&, In first, In last, Out result, T init, 
       tmp = *first;
       *result = sum;
       sum = op(sum, tmp);
+    }
+  }
+  return result;
+}
+// Sequential segmented scans (thrust/system/detail/sequential/scan_by_key.h:38-145).
+template <typename D, typename KIt, typename VIt, typename Out, typename Pred, typename Op>
+Out inclusive_scan_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, Out result, Pred pred, Op op) {
+  typedef typename iterator_value<KIt>::type K;
+  typedef typename iterator_value<VIt>::type V;
+  if (kf != kl) {
+    K prev_key = *kf;
+    V prev_value = *vf;
+    *result = prev_value;
+    for (++kf, ++vf, ++result; kf != kl; ++kf, ++vf, ++result) {
+      const K key = *kf;
+      if (pred(prev_key, key)) *result = prev_value = op(prev_value, *vf);
+      else *result = prev_value = *vf;
+      prev_key = key;
+    }
+  }
+  return result;
+}
+template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
+Out exclusive_scan_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, Out result, T init, Pred pred, Op op) {
+  typedef typename iterator_value<KIt>::type K;
+  if (kf != kl) {
+    K temp_key = *kf;
+    T temp_value = *vf;
+    T next = init;
+    *result = next;
+    next = op(next, temp_value);
+    for (++kf, ++vf, ++result; kf != kl; ++kf, ++vf, ++result) {
+      const K key = *kf;
+      temp_value = *vf;  // read before the write: in place is allowed
+      if (!pred(temp_key, key)) next = init;
+      *result = next;
+      next = op(next, temp_value);
+      temp_key = key;
     }
   }
   return result;
@@ -115,6 +197,72 @@ Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T i
   detail::synchronize(stream, "exclusive_scan: synchronize");
   return result + n;
 }
+
+namespace detail {
+template <typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
+struct scan_by_key_checks {
+  typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
+  static_assert((std::is_pointer<KIt>::value || thrust::detail::is_device_iterator<KIt>::value) &&
+                    (std::is_pointer<VIt>::value || thrust::detail::is_device_iterator<VIt>::value) &&
+                    (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value),
+                "scan_by_key on the device system needs device_ptr / device_vector iterators or raw device pointers");
+  static_assert(is_abi_type<K>::value && is_abi_type<V>::value && std::is_same<V, T>::value &&
+                    std::is_same<typename iterator_value<Out>::type, V>::value,
+                "scan_by_key on the device system: arithmetic keys; values, output and init share one arithmetic type");
+  static_assert(is_equal_to<Pred, K>::value,
+                "scan_by_key on the device system supports thrust::equal_to as key predicate");
+  static_assert(binop_code<Op, V>::value >= 0,
+                "scan_by_key on the device system supports thrust::plus, thrust::minimum and thrust::maximum");
+};
+}  // namespace detail
+
+template <typename D, typename KIt, typename VIt, typename Out, typename Pred, typename Op>
+Out inclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred, Op) {
+  typedef detail::scan_by_key_checks<KIt, VIt, Out, typename std::remove_const<typename iterator_value<VIt>::type>::type, Pred, Op> C;
+  typedef typename C::K K;
+  typedef typename C::V V;
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(kl - kf);
+  if (n == 0) return result;
+  detail::temp_storage temp(stream);
+  detail::run(temp, 0, "inclusive_scan_by_key failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_inclusive_scan_by_key(t, b, thrust::detail::raw(kf), thrust::detail::raw(vf),
+                                            thrust::detail::raw(result), n, detail::dtype_of<K>::value,
+                                            detail::dtype_of<V>::value, detail::binop_code<Op, V>::value, stream);
+  });
+  detail::synchronize(stream, "inclusive_scan_by_key: synchronize");
+  return result + n;
+}
+
+template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
+Out exclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init, Pred, Op) {
+  typedef detail::scan_by_key_checks<KIt, VIt, Out, T, Pred, Op> C;
+  typedef typename C::K K;
+  typedef typename C::V V;
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(kl - kf);
+  if (n == 0) return result;
+  const void* values = thrust::detail::raw(vf);
+  void* out = thrust::detail::raw(result);
+  // the device entry point reads values[i-1] while other tiles write: an in-place call
+  // scans from a copy of the values
+  detail::temp_storage copy(stream);
+  if (values == out) {
+    copy.ensure(n * sizeof(V));
+    detail::throw_on_error(thrust_amd_memcpy(copy.ptr(), values, n * sizeof(V), THRUST_AMD_D2D, stream),
+                           "exclusive_scan_by_key: copy of the values");
+    values = copy.ptr();
+  }
+  detail::temp_storage temp(stream);
+  detail::run(temp, 0, "exclusive_scan_by_key failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_exclusive_scan_by_key(t, b, thrust::detail::raw(kf), values, out, n,
+                                            detail::dtype_of<K>::value, detail::dtype_of<V>::value,
+                                            detail::binop_code<Op, V>::value, &init, stream);
+  });
+  detail::synchronize(stream, "exclusive_scan_by_key: synchronize");
+  return result + n;
+}
 }  // namespace hip
 }  // namespace system
 
@@ -166,6 +314,69 @@ template <typename In, typename Out, typename T, typename Op,
           typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>
 Out exclusive_scan(In first, In last, Out result, T init, Op op) {
   return thrust::exclusive_scan(detail::policy_for<In>(), first, last, result, init, op);
+}
+
+
+#define THRUST_AMD_SCAN_BY_KEY_ENTRY(NAME, TPARAMS, PARAMS, ARGS)                                                  \
+  template <typename D, typename KIt, typename VIt, typename Out TPARAMS>                                          \
+  Out NAME(const detail::execution_policy_base<D>& exec, KIt kf, KIt kl, VIt vf, Out result PARAMS) {              \
+    using thrust::system::detail::generic::NAME;                                                                   \
+    return NAME(detail::derived_cast(detail::strip_const(exec)), kf, kl, vf, result ARGS);                         \
+  }
+#define THRUST_AMD_COMMA ,
+THRUST_AMD_SCAN_BY_KEY_ENTRY(inclusive_scan_by_key, , , )
+THRUST_AMD_SCAN_BY_KEY_ENTRY(inclusive_scan_by_key, THRUST_AMD_COMMA typename Pred, THRUST_AMD_COMMA Pred pred,
+                             THRUST_AMD_COMMA pred)
+THRUST_AMD_SCAN_BY_KEY_ENTRY(inclusive_scan_by_key, THRUST_AMD_COMMA typename Pred THRUST_AMD_COMMA typename Op,
+                             THRUST_AMD_COMMA Pred pred THRUST_AMD_COMMA Op op,
+                             THRUST_AMD_COMMA pred THRUST_AMD_COMMA op)
+THRUST_AMD_SCAN_BY_KEY_ENTRY(exclusive_scan_by_key, , , )
+THRUST_AMD_SCAN_BY_KEY_ENTRY(exclusive_scan_by_key, THRUST_AMD_COMMA typename T, THRUST_AMD_COMMA T init,
+                             THRUST_AMD_COMMA init)
+THRUST_AMD_SCAN_BY_KEY_ENTRY(exclusive_scan_by_key, THRUST_AMD_COMMA typename T THRUST_AMD_COMMA typename Pred,
+                             THRUST_AMD_COMMA T init THRUST_AMD_COMMA Pred pred,
+                             THRUST_AMD_COMMA init THRUST_AMD_COMMA pred)
+THRUST_AMD_SCAN_BY_KEY_ENTRY(exclusive_scan_by_key,
+                             THRUST_AMD_COMMA typename T THRUST_AMD_COMMA typename Pred THRUST_AMD_COMMA typename Op,
+                             THRUST_AMD_COMMA T init THRUST_AMD_COMMA Pred pred THRUST_AMD_COMMA Op op,
+                             THRUST_AMD_COMMA init THRUST_AMD_COMMA pred THRUST_AMD_COMMA op)
+#undef THRUST_AMD_SCAN_BY_KEY_ENTRY
+
+// without a policy: the system of the key iterator
+template <typename KIt, typename VIt, typename Out,
+          typename = typename std::enable_if<!detail::is_execution_policy<KIt>::value>::type>
+Out inclusive_scan_by_key(KIt kf, KIt kl, VIt vf, Out result) {
+  return thrust::inclusive_scan_by_key(detail::policy_for<KIt>(), kf, kl, vf, result);
+}
+template <typename KIt, typename VIt, typename Out, typename Pred,
+          typename = typename std::enable_if<!detail::is_execution_policy<KIt>::value>::type>
+Out inclusive_scan_by_key(KIt kf, KIt kl, VIt vf, Out result, Pred pred) {
+  return thrust::inclusive_scan_by_key(detail::policy_for<KIt>(), kf, kl, vf, result, pred);
+}
+template <typename KIt, typename VIt, typename Out, typename Pred, typename Op,
+          typename = typename std::enable_if<!detail::is_execution_policy<KIt>::value>::type>
+Out inclusive_scan_by_key(KIt kf, KIt kl, VIt vf, Out result, Pred pred, Op op) {
+  return thrust::inclusive_scan_by_key(detail::policy_for<KIt>(), kf, kl, vf, result, pred, op);
+}
+template <typename KIt, typename VIt, typename Out,
+          typename = typename std::enable_if<!detail::is_execution_policy<KIt>::value>::type>
+Out exclusive_scan_by_key(KIt kf, KIt kl, VIt vf, Out result) {
+  return thrust::exclusive_scan_by_key(detail::policy_for<KIt>(), kf, kl, vf, result);
+}
+template <typename KIt, typename VIt, typename Out, typename T,
+          typename = typename std::enable_if<!detail::is_execution_policy<KIt>::value>::type>
+Out exclusive_scan_by_key(KIt kf, KIt kl, VIt vf, Out result, T init) {
+  return thrust::exclusive_scan_by_key(detail::policy_for<KIt>(), kf, kl, vf, result, init);
+}
+template <typename KIt, typename VIt, typename Out, typename T, typename Pred,
+          typename = typename std::enable_if<!detail::is_execution_policy<KIt>::value>::type>
+Out exclusive_scan_by_key(KIt kf, KIt kl, VIt vf, Out result, T init, Pred pred) {
+  return thrust::exclusive_scan_by_key(detail::policy_for<KIt>(), kf, kl, vf, result, init, pred);
+}
+template <typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op,
+          typename = typename std::enable_if<!detail::is_execution_policy<KIt>::value>::type>
+Out exclusive_scan_by_key(KIt kf, KIt kl, VIt vf, Out result, T init, Pred pred, Op op) {
+  return thrust::exclusive_scan_by_key(detail::policy_for<KIt>(), kf, kl, vf, result, init, pred, op);
 }
 
 }  // namespace thrust

@@ -146,6 +146,23 @@ int thrust_amd_profile_collect(char* text, size_t capacity, size_t* needed);
 int thrust_amd_reduce(void* temp, size_t* temp_bytes, const void* in, uint64_t n, int dtype,
                       int op, const void* init, void* d_out, void* stream);
 
+/* *d_count (uint64 on device) = number of elements with (in[i] CMP *threshold); cmp is a
+ * thrust_amd_cmp code, `threshold` a host pointer to one dtype element (ignored for
+ * THRUST_AMD_NONZERO).
+ * Replaces cuda_cub::count_if -> reduce_n over a 0/1 transform
+ * (thrust/system/cuda/detail/count.h:43-62; generic form
+ * thrust/system/detail/generic/count.inl:64-74). */
+int thrust_amd_count_if(void* temp, size_t* temp_bytes, const void* in, uint64_t n, int dtype,
+                        int cmp, const void* threshold, uint64_t* d_count, void* stream);
+
+/* *d_out = init + a[0]*b[0] + ... + a[n-1]*b[n-1]; products and sums are made in dtype
+ * (integers wrap modulo 2^bits).  `init` is a host pointer to one dtype element.
+ * Replaces cuda_cub::inner_product -> transform_reduce over the zipped ranges
+ * (thrust/system/cuda/detail/inner_product.h:46-70; generic form
+ * thrust/system/detail/generic/inner_product.inl:33-65). */
+int thrust_amd_inner_product(void* temp, size_t* temp_bytes, const void* a, const void* b,
+                             uint64_t n, int dtype, const void* init, void* d_out, void* stream);
+
 /* --------------------------------------------------------------------- scan */
 
 /* out[i] = in[0] OP ... OP in[i]; accumulator type = dtype; out == in allowed.
@@ -159,6 +176,25 @@ int thrust_amd_inclusive_scan(void* temp, size_t* temp_bytes, const void* in, vo
  * Replaces cuda_cub::exclusive_scan_n (thrust/system/cuda/detail/scan.h:132-200). */
 int thrust_amd_exclusive_scan(void* temp, size_t* temp_bytes, const void* in, void* out,
                               uint64_t n, int dtype, int op, const void* init, void* stream);
+
+/* Segmented scans: a segment is a run of equal consecutive keys (compared like
+ * reduce_by_key: integers by value, floats with ==).  out[i] = the OP-fold of the segment's
+ * values up to and including i.  out may alias values.  Accumulator = value_dtype;
+ * floating-point folds use a tree order inside a segment.
+ * Replaces cuda_cub::inclusive_scan_by_key (thrust/system/cuda/detail/scan_by_key.h:795-880;
+ * generic form thrust/system/detail/generic/scan_by_key.inl:96-135). */
+int thrust_amd_inclusive_scan_by_key(void* temp, size_t* temp_bytes, const void* keys,
+                                     const void* values, void* out, uint64_t n, int key_dtype,
+                                     int value_dtype, int op, void* stream);
+
+/* out[i] = *init at the first element of a segment, else init OP (the segment's values
+ * before i).  `init` is a host pointer to one value_dtype element.  out must not alias
+ * values.
+ * Replaces cuda_cub::exclusive_scan_by_key (thrust/system/cuda/detail/scan_by_key.h:885-1000;
+ * generic form thrust/system/detail/generic/scan_by_key.inl:190-238). */
+int thrust_amd_exclusive_scan_by_key(void* temp, size_t* temp_bytes, const void* keys,
+                                     const void* values, void* out, uint64_t n, int key_dtype,
+                                     int value_dtype, int op, const void* init, void* stream);
 
 /* --------------------------------------------------------------------- sort */
 

@@ -187,6 +187,38 @@ class _Base:
                  "reduce_by_key")
         return ko[: num.value].copy(), vo[: num.value].copy()
 
+    def count_if(self, x, cmp, threshold=0):
+        x = _c(x)
+        num = ctypes.c_uint64(0)
+        tv = np.array([threshold], x.dtype)
+        self._ok(self._fn("count_if")(_p(x), ctypes.c_uint64(x.size), _code(x), cmp, _p(tv),
+                                       ctypes.byref(num), *self._extra()), "count_if")
+        return num.value
+
+    def inner_product(self, a, b, init=0):
+        a, b = _c(a), _c(b)
+        out = np.zeros(1, a.dtype)
+        iv = np.array([init], a.dtype)
+        self._ok(self._fn("inner_product")(_p(a), _p(b), ctypes.c_uint64(a.size), _code(a), _p(iv),
+                                            _p(out), *self._extra()), "inner_product")
+        return out[0]
+
+    def inclusive_scan_by_key(self, keys, values, op=PLUS):
+        k, v = _c(keys), _c(values)
+        out = np.empty_like(v)
+        self._ok(self._fn("inclusive_scan_by_key")(_p(k), _p(v), _p(out), ctypes.c_uint64(k.size),
+                                                    _code(k), _code(v), op), "inclusive_scan_by_key")
+        return out
+
+    def exclusive_scan_by_key(self, keys, values, init=0, op=PLUS):
+        k, v = _c(keys), _c(values)
+        out = np.empty_like(v)
+        iv = np.array([init], v.dtype)
+        self._ok(self._fn("exclusive_scan_by_key")(_p(k), _p(v), _p(out), ctypes.c_uint64(k.size),
+                                                    _code(k), _code(v), op, _p(iv)),
+                 "exclusive_scan_by_key")
+        return out
+
 
 class Oracle(_Base):
     """The C restatement.  `nthreads` (0 = all cores) sets the OMP shape; 1 = CPP system."""

@@ -8,9 +8,11 @@
 // real thing and write golden vectors, and the benchmark can time the reference's
 // OMP path as CPU baseline.  Built only into oracle/_ref/, which is not committed.
 #include <thrust/copy.h>
+#include <thrust/count.h>
 #include <thrust/device_ptr.h>
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
+#include <thrust/inner_product.h>
 #include <thrust/merge.h>
 #include <thrust/partition.h>
 #include <thrust/reduce.h>
@@ -295,4 +297,71 @@ REF_API int ref_reduce_by_key(const void* keys_in, const void* values_in, void* 
     case THRUST_AMD_F32: return by_value((float)0);
     default: return -1;
   }
+}
+
+REF_API int ref_count_if(const void* in, uint64_t n, int dtype, int cmp, const void* threshold,
+                         uint64_t* count) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    *count = (uint64_t)thrust::count_if(thrust::device, dp<T>(in), dp<T>(in) + n, make_pred<T>(cmp, threshold));
+    return 0;
+  });
+}
+
+REF_API int ref_inner_product(const void* a, const void* b, uint64_t n, int dtype, const void* init,
+                              void* out) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    *(T*)out = thrust::inner_product(thrust::device, dp<T>(a), dp<T>(a) + n, dp<T>(b), *(const T*)init);
+    return 0;
+  });
+}
+
+namespace {
+template <typename F>
+int with_key_value(int key_dtype, int value_dtype, F&& run) {
+  auto by_value = [&](auto kz) {
+    switch (value_dtype) {
+      case THRUST_AMD_I32: return run(kz, (int32_t)0);
+      case THRUST_AMD_I64: return run(kz, (int64_t)0);
+      case THRUST_AMD_F32: return run(kz, (float)0);
+      case THRUST_AMD_F64: return run(kz, (double)0);
+      default: return -1;
+    }
+  };
+  switch (key_dtype) {
+    case THRUST_AMD_I32: return by_value((int32_t)0);
+    case THRUST_AMD_U32: return by_value((uint32_t)0);
+    case THRUST_AMD_I64: return by_value((int64_t)0);
+    case THRUST_AMD_U64: return by_value((uint64_t)0);
+    case THRUST_AMD_F32: return by_value((float)0);
+    default: return -1;
+  }
+}
+}  // namespace
+
+REF_API int ref_inclusive_scan_by_key(const void* keys, const void* values, void* out, uint64_t n,
+                                      int key_dtype, int value_dtype, int op) {
+  return with_key_value(key_dtype, value_dtype, [&](auto kz, auto vz) {
+    using K = decltype(kz);
+    using V = decltype(vz);
+    return with_op<V>(op, [&](auto o) {
+      thrust::inclusive_scan_by_key(thrust::device, dp<K>(keys), dp<K>(keys) + n, dp<V>(values), dp<V>(out),
+                                    thrust::equal_to<K>(), o);
+      return 0;
+    });
+  });
+}
+
+REF_API int ref_exclusive_scan_by_key(const void* keys, const void* values, void* out, uint64_t n,
+                                      int key_dtype, int value_dtype, int op, const void* init) {
+  return with_key_value(key_dtype, value_dtype, [&](auto kz, auto vz) {
+    using K = decltype(kz);
+    using V = decltype(vz);
+    return with_op<V>(op, [&](auto o) {
+      thrust::exclusive_scan_by_key(thrust::device, dp<K>(keys), dp<K>(keys) + n, dp<V>(values), dp<V>(out),
+                                    *(const V*)init, thrust::equal_to<K>(), o);
+      return 0;
+    });
+  });
 }

@@ -426,3 +426,63 @@ ORACLE_API int oracle_reduce_by_key(const void* keys_in, const void* values_in, 
   *num_runs = runs;
   return runs == runs2 ? 0 : -2;
 }
+
+/* generic::count_if (generic/count.inl:64-74): transform_reduce of pred(x) ? 1 : 0 in the
+ * iterator's difference type with plus; the transform is the same 0/1 map copy_if uses. */
+ORACLE_API int oracle_count_if(const void* in, uint64_t n, int dtype, int cmp, const void* threshold,
+                               uint64_t* count, int nprocs) {
+  const long P = nprocs > 0 ? nprocs : omp_get_num_procs();
+  unsigned* flags = (unsigned*)malloc((n ? n : 1) * sizeof(unsigned));
+#define BODY(S, T) \
+  pred_flags_##S((const T*)in, (size_t)n, cmp, threshold ? *(const T*)threshold : (T)0, flags);
+  DISPATCH(dtype, BODY)
+#undef BODY
+  int64_t* ones = (int64_t*)malloc((n ? n : 1) * sizeof(int64_t));
+  for (uint64_t i = 0; i < n; i++) ones[i] = flags[i] ? 1 : 0;
+  *count = (uint64_t)reduce_i64(ones, (size_t)n, 0, THRUST_AMD_PLUS, P);
+  free(ones);
+  free(flags);
+  return 0;
+}
+
+ORACLE_API int oracle_inner_product(const void* a, const void* b, uint64_t n, int dtype,
+                                    const void* init, void* out, int nprocs) {
+  const long P = nprocs > 0 ? nprocs : omp_get_num_procs();
+#define BODY(S, T) \
+  *(T*)out = inner_product_##S((const T*)a, (const T*)b, (size_t)n, *(const T*)init, P);
+  DISPATCH(dtype, BODY)
+#undef BODY
+  return 0;
+}
+
+/* generic::inclusive_scan_by_key / exclusive_scan_by_key with equal_to on the keys
+ * (generic/scan_by_key.inl:62-238); head flags as in reduce_by_key. */
+ORACLE_API int oracle_inclusive_scan_by_key(const void* keys, const void* values, void* out,
+                                            uint64_t n, int key_dtype, int value_dtype, int op) {
+  if (n == 0) return 0;
+  unsigned* flags = (unsigned*)malloc(n * sizeof(unsigned));
+#define BODY(S, T) head_flags_##S((const T*)keys, (size_t)n, flags);
+  DISPATCH(key_dtype, BODY)
+#undef BODY
+#define BODY(S, T) inclusive_scan_by_flags_##S(flags, (const T*)values, (T*)out, (size_t)n, op);
+  DISPATCH(value_dtype, BODY)
+#undef BODY
+  free(flags);
+  return 0;
+}
+
+ORACLE_API int oracle_exclusive_scan_by_key(const void* keys, const void* values, void* out,
+                                            uint64_t n, int key_dtype, int value_dtype, int op,
+                                            const void* init) {
+  if (n == 0) return 0;
+  unsigned* flags = (unsigned*)malloc(n * sizeof(unsigned));
+#define BODY(S, T) head_flags_##S((const T*)keys, (size_t)n, flags);
+  DISPATCH(key_dtype, BODY)
+#undef BODY
+#define BODY(S, T) \
+  exclusive_scan_by_flags_##S(flags, (const T*)values, (T*)out, (size_t)n, op, *(const T*)init);
+  DISPATCH(value_dtype, BODY)
+#undef BODY
+  free(flags);
+  return 0;
+}

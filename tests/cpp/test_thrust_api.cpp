@@ -7,11 +7,13 @@
 // e.g. testing/reduce.cu:80-95).  Part 3 covers policies, streams, dispatch interception,
 // the memory model and error reporting.
 #include <thrust/copy.h>
+#include <thrust/count.h>
 #include <thrust/device_vector.h>
 #include <thrust/execution_policy.h>
 #include <thrust/fill.h>
 #include <thrust/functional.h>
 #include <thrust/host_vector.h>
+#include <thrust/inner_product.h>
 #include <thrust/merge.h>
 #include <thrust/partition.h>
 #include <thrust/reduce.h>
@@ -123,6 +125,66 @@ static void TestScanSimple() {  // testing/scan.cu:23-93
   input = in;
   thrust::exclusive_scan(input.begin(), input.end(), output.begin());
   ASSERT_EQUAL_VEC(to_host(output), hv<int>({0, 1, 4, 2, 6}));
+}
+
+static void TestScanByKeySimple() {  // testing/scan_by_key.cu:9-60 and :121-180
+  g_test = "ScanByKeySimple";
+  thrust::device_vector<int> keys(hv<int>({0, 1, 1, 1, 2, 3, 3})), vals(hv<int>({1, 2, 3, 4, 5, 6, 7})), output(7, 0);
+  auto it = thrust::inclusive_scan_by_key(keys.begin(), keys.end(), vals.begin(), output.begin());
+  ASSERT_TRUE(it - output.begin() == 7);
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({1, 2, 5, 9, 5, 6, 13}));
+  thrust::inclusive_scan_by_key(keys.begin(), keys.end(), vals.begin(), output.begin(), thrust::equal_to<int>());
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({1, 2, 5, 9, 5, 6, 13}));
+  thrust::inclusive_scan_by_key(keys.begin(), keys.end(), vals.begin(), output.begin(), thrust::equal_to<int>(),
+                                thrust::maximum<int>());
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({1, 2, 3, 4, 5, 6, 7}));
+  it = thrust::exclusive_scan_by_key(keys.begin(), keys.end(), vals.begin(), output.begin());
+  ASSERT_TRUE(it - output.begin() == 7);
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({0, 0, 2, 5, 0, 0, 6}));
+  thrust::exclusive_scan_by_key(keys.begin(), keys.end(), vals.begin(), output.begin(), 10);
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({10, 10, 12, 15, 10, 10, 16}));
+  thrust::exclusive_scan_by_key(keys.begin(), keys.end(), vals.begin(), output.begin(), 10, thrust::equal_to<int>());
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({10, 10, 12, 15, 10, 10, 16}));
+  thrust::exclusive_scan_by_key(thrust::device, keys.begin(), keys.end(), vals.begin(), output.begin(), 10,
+                                thrust::equal_to<int>(), thrust::plus<int>());
+  ASSERT_EQUAL_VEC(to_host(output), hv<int>({10, 10, 12, 15, 10, 10, 16}));
+  // in place, both forms
+  thrust::device_vector<int> v2 = vals;
+  thrust::inclusive_scan_by_key(keys.begin(), keys.end(), v2.begin(), v2.begin());
+  ASSERT_EQUAL_VEC(to_host(v2), hv<int>({1, 2, 5, 9, 5, 6, 13}));
+  v2 = vals;
+  thrust::exclusive_scan_by_key(keys.begin(), keys.end(), v2.begin(), v2.begin(), 10);
+  ASSERT_EQUAL_VEC(to_host(v2), hv<int>({10, 10, 12, 15, 10, 10, 16}));
+  // the host system gives the same answers
+  thrust::host_vector<int> hk = to_host(keys), hvals = to_host(vals), ho(7);
+  thrust::inclusive_scan_by_key(hk.begin(), hk.end(), hvals.begin(), ho.begin());
+  ASSERT_EQUAL_VEC(ho, hv<int>({1, 2, 5, 9, 5, 6, 13}));
+  thrust::exclusive_scan_by_key(hk.begin(), hk.end(), hvals.begin(), ho.begin(), 10);
+  ASSERT_EQUAL_VEC(ho, hv<int>({10, 10, 12, 15, 10, 10, 16}));
+}
+
+static void TestCountSimple() {  // testing/count.cu:5-14 and :40-49
+  g_test = "CountSimple";
+  thrust::device_vector<int> data(hv<int>({1, 1, 0, 0, 1}));
+  ASSERT_TRUE(thrust::count(data.begin(), data.end(), 0) == 2);
+  ASSERT_TRUE(thrust::count(data.begin(), data.end(), 1) == 3);
+  ASSERT_TRUE(thrust::count(data.begin(), data.end(), 2) == 0);
+  thrust::device_vector<int> d2(hv<int>({1, 6, 1, 9, 2}));
+  ASSERT_TRUE(thrust::count_if(d2.begin(), d2.end(), _1 > 5) == 2);
+  ASSERT_TRUE(thrust::count_if(thrust::device, d2.begin(), d2.end(), _1 > 5) == 2);
+  thrust::host_vector<int> h2 = to_host(d2);
+  ASSERT_TRUE(thrust::count_if(h2.begin(), h2.end(), _1 > 5) == 2);
+  ASSERT_TRUE(thrust::count(h2.begin(), h2.end(), 1) == 2);
+}
+
+static void TestInnerProductSimple() {  // testing/inner_product.cu:10-24
+  g_test = "InnerProductSimple";
+  thrust::device_vector<int> v1(hv<int>({1, -2, 3})), v2(hv<int>({-4, 5, 6}));
+  ASSERT_TRUE(thrust::inner_product(v1.begin(), v1.end(), v2.begin(), 3) == 7);
+  ASSERT_TRUE(thrust::inner_product(thrust::device, v1.begin(), v1.end(), v2.begin(), 3) == 7);
+  ASSERT_TRUE(thrust::inner_product(v1.begin(), v1.end(), v2.begin(), 3, thrust::plus<int>(), thrust::multiplies<int>()) == 7);
+  thrust::host_vector<int> h1 = to_host(v1), h2 = to_host(v2);
+  ASSERT_TRUE(thrust::inner_product(h1.begin(), h1.end(), h2.begin(), 3) == 7);
 }
 
 static void TestSortSimple() {  // testing/sort.cu:43-76
@@ -323,6 +385,25 @@ static void DifferentialForType(const char* name) {
       thrust::exclusive_scan(d.begin(), d.end(), dout.begin(), (T)11);
       ASSERT_EQUAL_VEC(to_host(dout), ho);
     }
+    // scan_by_key, count_if, inner_product (integers: exact)
+    if (std::is_integral<T>::value) {
+      thrust::host_vector<T> hsv = random_integers<T>(n, 41, 0), hso(n);
+      thrust::device_vector<T> dsv = hsv, dso(n);
+      thrust::inclusive_scan_by_key(hk.begin(), hk.end(), hsv.begin(), hso.begin());
+      thrust::inclusive_scan_by_key(dk.begin(), dk.end(), dsv.begin(), dso.begin());
+      ASSERT_EQUAL_VEC(to_host(dso), hso);
+      thrust::exclusive_scan_by_key(hk.begin(), hk.end(), hsv.begin(), hso.begin(), (T)5);
+      thrust::exclusive_scan_by_key(dk.begin(), dk.end(), dsv.begin(), dso.begin(), (T)5);
+      ASSERT_EQUAL_VEC(to_host(dso), hso);
+      ASSERT_TRUE(thrust::count_if(hk.begin(), hk.end(), _1 < (T)9) == thrust::count_if(dk.begin(), dk.end(), _1 < (T)9));
+      ASSERT_TRUE(thrust::count(hk.begin(), hk.end(), (T)3) == thrust::count(dk.begin(), dk.end(), (T)3));
+      {  // expected value in unsigned arithmetic (wraps without undefined behaviour)
+        using U = typename std::make_unsigned<typename std::conditional<std::is_integral<T>::value, T, int>::type>::type;
+        U dot = (U)3;
+        for (size_t i = 0; i < n; ++i) dot = (U)(dot + (U)((U)h[i] * (U)hsv[i]));
+        ASSERT_TRUE(thrust::inner_product(d.begin(), d.end(), dsv.begin(), (T)3) == (T)dot);
+      }
+    }
     // copy_if / stable_partition with a threshold predicate
     thrust::host_vector<T> hsel = random_integers<T>(n, 21, 100);
     thrust::device_vector<T> dsel = hsel;
@@ -477,6 +558,9 @@ int main() {
   TestReduceSimple();
   TestReduceWithOperatorTable();
   TestScanSimple();
+  TestScanByKeySimple();
+  TestCountSimple();
+  TestInnerProductSimple();
   TestSortSimple();
   TestSortByKeySimple();
   TestReduceByKeySimple();

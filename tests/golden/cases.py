@@ -9,8 +9,8 @@ import numpy as np
 from thrust_amd import datagen
 
 LT = 0
-SMALL = {"c1": 1 << 14, "c2": 1 << 14, "c3": 1 << 13, "c4": 1 << 15, "c5": 1 << 14}
-LARGE = {"c1": 1 << 22, "c2": 1 << 22, "c3": 1 << 21, "c4": 1 << 22, "c5": 1 << 22}
+SMALL = {"c1": 1 << 14, "c2": 1 << 14, "c3": 1 << 13, "c4": 1 << 15, "c5": 1 << 14, "c6": 1 << 15}
+LARGE = {"c1": 1 << 22, "c2": 1 << 22, "c3": 1 << 21, "c4": 1 << 22, "c5": 1 << 22, "c6": 1 << 22}
 
 
 def c1(impl, n):
@@ -82,7 +82,24 @@ def c5(impl, n):
     return out
 
 
-CASES = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5}
+def c6(impl, n):
+    """Callers on either side of the path: count_if, inner_product, scan_by_key (integer
+    values, so every association order gives the same bits)."""
+    x = datagen.c1_int32(n)
+    y = datagen.c2_uint32(n).view(np.int32)
+    out = {
+        "c6.count_if_lt500": np.array([impl.count_if(x, LT, 500)], np.uint64),
+        "c6.inner_product_i32_init11": np.array([impl.inner_product(x, y, init=11)], np.int32),
+    }
+    for mean in (8, 1000):
+        k, v = datagen.c4_segments(n, mean)
+        iv = (v * 1000).astype(np.int32)
+        out[f"c6.m{mean}.inclusive_scan_by_key_i32"] = impl.inclusive_scan_by_key(k, iv)
+        out[f"c6.m{mean}.exclusive_scan_by_key_i32_init9"] = impl.exclusive_scan_by_key(k, iv, init=9)
+    return out
+
+
+CASES = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5, "c6": c6}
 
 
 def digest(a):

@@ -68,6 +68,18 @@ class DeviceImpl:
                                         stencil=self._d(stencil) if stencil is not None else None)
         return d.numpy(), cnt
 
+    def count_if(self, x, cmp, threshold=0):
+        return self.dev.count_if(self._d(x), cmp, threshold)
+
+    def inner_product(self, a, b, init=0):
+        return self.dev.inner_product(self._d(a), self._d(b), init=init).numpy()[0]
+
+    def inclusive_scan_by_key(self, k, v, op=0):
+        return self.dev.inclusive_scan_by_key(self._d(k), self._d(v), op=op).numpy()
+
+    def exclusive_scan_by_key(self, k, v, init=0, op=0):
+        return self.dev.exclusive_scan_by_key(self._d(k), self._d(v), init=init, op=op).numpy()
+
     def merge_by_key(self, ka, kb, va, vb):
         ko, vo = self.dev.merge_by_key(self._d(ka), self._d(kb), self._d(va), self._d(vb))
         return ko.numpy(), vo.numpy()

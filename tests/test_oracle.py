@@ -77,6 +77,20 @@ def test_known_by_key_and_selection(oracle):
         assert out.tolist() == c["out"] and split == c["split"]
 
 
+def test_known_scan_by_key_count_inner_product(oracle):
+    for c in KA["inclusive_scan_by_key"]:
+        got = oracle.inclusive_scan_by_key(np.array(c["keys"], I32), np.array(c["values"], I32))
+        assert got.tolist() == c["out"]
+    for c in KA["exclusive_scan_by_key"]:
+        got = oracle.exclusive_scan_by_key(np.array(c["keys"], I32), np.array(c["values"], I32), init=c["init"])
+        assert got.tolist() == c["out"]
+    codes = {"gt": cpu.GT, "eq": cpu.EQ}
+    for c in KA["count_if"]:
+        assert oracle.count_if(np.array(c["in"], I32), codes[c["cmp"]], c["threshold"]) == c["out"]
+    for c in KA["inner_product"]:
+        assert oracle.inner_product(np.array(c["a"], I32), np.array(c["b"], I32), init=c["init"]) == c["out"]
+
+
 def test_known_merges(oracle):
     for c in KA["merge"]:
         assert oracle.merge(np.array(c["a"], I32), np.array(c["b"], I32)).tolist() == c["out"]
@@ -233,3 +247,34 @@ def test_merge_against_stable_sort_of_concatenation(oracle):
     ko, vo = oracle.merge_by_key(ka, kb, va, vb)
     order = np.argsort(np.r_[ka, kb], kind="stable")
     assert np.array_equal(ko, np.r_[ka, kb][order]) and np.array_equal(vo, np.r_[va, vb][order])
+
+
+def test_scan_by_key_count_inner_product_against_numpy(oracle):
+    """Independent definitions: per-segment cumulative sums (float64 / modulo 2^32), boolean
+    masks, and the dot product modulo 2^k."""
+    n = 100003
+    k, v = datagen.c4_segments(n, 8)
+    iv = (v * 1000).astype(np.int32)
+    head = np.r_[True, k[1:] != k[:-1]]
+    starts = np.flatnonzero(head)
+    seg = np.cumsum(head) - 1
+    c = np.cumsum(iv.astype(np.int64))
+    incl = c - np.r_[0, c[:-1]][starts][seg]
+    assert np.array_equal(oracle.inclusive_scan_by_key(k, iv), incl.astype(np.int32))
+    assert np.array_equal(oracle.exclusive_scan_by_key(k, iv, init=9), (incl - iv + 9).astype(np.int32))
+    # min / max: running extrema restart at every head
+    mx = oracle.inclusive_scan_by_key(k, iv, op=cpu.MAX)
+    assert np.array_equal(mx[starts], iv[starts]) and np.all(mx >= iv)
+    assert np.array_equal(np.maximum.reduceat(iv, starts), mx[np.r_[starts[1:] - 1, n - 1]])
+    x = datagen.c1_int32(n)
+    for cmp, mask in ((cpu.LT, x < 500), (cpu.GE, x >= 500), (cpu.EQ, x == 500), (cpu.NONZERO, x != 0)):
+        assert oracle.count_if(x, cmp, 500) == int(mask.sum())
+    for dtype in (np.int8, np.uint16, np.int32, np.uint64):
+        a = (datagen.splitmix64(1, n) >> np.uint64(5)).astype(dtype)
+        b = (datagen.splitmix64(2, n) >> np.uint64(11)).astype(dtype)
+        bits = 8 * np.dtype(dtype).itemsize
+        exact = (sum(int(p) * int(q) for p, q in zip(a[:2000].tolist(), b[:2000].tolist())) + 3) % (1 << bits)
+        got = int(oracle.inner_product(a[:2000], b[:2000], init=3)) % (1 << bits)
+        assert got == exact, dtype
+    f = datagen.u01(7, n)
+    assert abs(float(oracle.inner_product(f, f, init=1.0)) - (float(np.dot(f.astype(np.float64), f)) + 1.0)) < 1e-3 * n * 1e-4

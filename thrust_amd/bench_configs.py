@@ -10,9 +10,11 @@ with the algorithmic bytes of the call and the resulting fraction of the 8 TB/s 
   C4  reduce_by_key and unique_by_key over 2^28 (int32 key, float32 value), mean run 8 / 1000
   C5  copy_if and stable_partition of 2^28 float32 at 50 % / 5 % selectivity,
       merge and merge_by_key of two sorted ranges of 2^27 uint32 (+ uint32 values)
+  C6  callers on either side of the path: count_if and inner_product over 2^28 int32 /
+      float32, inclusive and exclusive scan_by_key over 2^28 (int32 key, float32 value)
 
 Inputs are generated on the device from a seeded generator.  Usage:
-  python3 thrust_amd/bench_configs.py [c2] [c3] [c4] [c5]
+  python3 thrust_amd/bench_configs.py [c2] [c3] [c4] [c5] [c6]
 """
 import os
 import sys
@@ -31,7 +33,7 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench_configs.py needs a GPU")
     capi.load()
-    which = [a.lower() for a in sys.argv[1:]] or ["c2", "c3", "c4", "c5"]
+    which = [a.lower() for a in sys.argv[1:]] or ["c2", "c3", "c4", "c5", "c6"]
     g = torch.Generator(device="cuda")
     g.manual_seed(1)
 
@@ -126,6 +128,26 @@ def main():
         run("C5 merge_by_key 2 x 2^27 u32+u32",
             lambda: capi.merge_by_key(*a, temp=t, keys_out=ko, values_out=vo), 16 * 2 * m)
         run("C5 merge 2 x 2^27 u32", lambda: capi.merge(a[0], a[1], out=ko, temp=t2), 8 * 2 * m)
+        del ka, kb, va, vb, a, ko, vo, t, t2
+    if "c6" in which:
+        x = torch.randint(0, 1001, (n,), dtype=torch.int32, device="cuda", generator=g)
+        dx, t = dev(x, capi.I32), capi.Temp()
+        run("C6 count_if i32 x<500", lambda: capi.count_if(dx, capi.LT, 500, temp=t), 4 * n)
+        f1 = torch.rand(n, device="cuda", generator=g)
+        f2 = torch.rand(n, device="cuda", generator=g)
+        d1, d2, t2, out1 = dev(f1, capi.F32), dev(f2, capi.F32), capi.Temp(), capi.DeviceArray(1, capi.F32)
+        run("C6 inner_product f32", lambda: capi.inner_product(d1, d2, init=0.0, temp=t2, out=out1), 8 * n)
+        del x, dx, f1, f2, d1, d2, t, t2
+        mean = 8
+        nseg = int(n / mean * 1.2) + 1000
+        u = torch.rand(nseg, device="cuda", generator=g, dtype=torch.float64).clamp_(1e-12, 1.0)
+        lens = (torch.floor(torch.log(u) / np.log1p(-1.0 / mean)) + 1).long()
+        keys = torch.repeat_interleave(torch.arange(nseg, device="cuda", dtype=torch.int32), lens)[:n].contiguous()
+        vals = torch.rand(n, device="cuda", generator=g)
+        dk, dv, vo, t = dev(keys, capi.I32), dev(vals, capi.F32), capi.DeviceArray(n, capi.F32), capi.Temp()
+        run("C6 inclusive_scan_by_key mean run 8", lambda: capi.inclusive_scan_by_key(dk, dv, out=vo, temp=t), 12 * n)
+        run("C6 exclusive_scan_by_key mean run 8",
+            lambda: capi.exclusive_scan_by_key(dk, dv, init=0.0, out=vo, temp=t), 12 * n)
 
 
 if __name__ == "__main__":

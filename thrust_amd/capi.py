@@ -49,8 +49,12 @@ SIGNATURES = {
     "thrust_amd_profile_enable": (_int, [_int]),
     "thrust_amd_profile_collect": (_int, [_c.c_char_p, _sz, _szp]),
     "thrust_amd_reduce": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp, _vp, _vp]),
+    "thrust_amd_count_if": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp, _vp, _vp]),
+    "thrust_amd_inner_product": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _vp, _vp, _vp]),
     "thrust_amd_inclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _vp]),
     "thrust_amd_exclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _vp, _vp]),
+    "thrust_amd_inclusive_scan_by_key": (_int, [_vp, _szp, _vp, _vp, _vp, _u64, _int, _int, _int, _vp]),
+    "thrust_amd_exclusive_scan_by_key": (_int, [_vp, _szp, _vp, _vp, _vp, _u64, _int, _int, _int, _vp, _vp]),
     "thrust_amd_sort_keys": (_int, [_vp, _szp, _vp, _u64, _int, _int, _int, _int, _vp]),
     "thrust_amd_sort_pairs": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _sz, _int, _int, _int, _vp]),
     "thrust_amd_copy_if": (_int, [_vp, _szp, _vp, _vp, _vp, _vp, _u64, _sz, _int, _int, _vp, _vp]),
@@ -195,6 +199,22 @@ def reduce(x, op=PLUS, init=0, temp=None, out=None):
     return out
 
 
+def count_if(x, cmp, threshold=0, temp=None):
+    num = DeviceArray(1, U64)
+    tv = _scalar(x.dtype, threshold)
+    _run("thrust_amd_count_if", temp, lambda fn, t, b: fn(
+        t, b, x.ptr, x.n, x.dtype, cmp, tv.ctypes.data, num.ptr, stream_ptr()))
+    return _count(num)
+
+
+def inner_product(a, b_, init=0, temp=None, out=None):
+    out = out or DeviceArray(1, a.dtype)
+    iv = _scalar(a.dtype, init)
+    _run("thrust_amd_inner_product", temp, lambda fn, t, b: fn(
+        t, b, a.ptr, b_.ptr, a.n, a.dtype, iv.ctypes.data, out.ptr, stream_ptr()))
+    return out
+
+
 def inclusive_scan(x, out=None, op=PLUS, temp=None):
     out = out or DeviceArray(x.n, x.dtype)
     _run("thrust_amd_inclusive_scan", temp, lambda fn, t, b: fn(
@@ -207,6 +227,22 @@ def exclusive_scan(x, init=0, out=None, op=PLUS, temp=None):
     iv = _scalar(x.dtype, init)
     _run("thrust_amd_exclusive_scan", temp, lambda fn, t, b: fn(
         t, b, x.ptr, out.ptr, x.n, x.dtype, op, iv.ctypes.data, stream_ptr()))
+    return out
+
+
+def inclusive_scan_by_key(keys, values, op=PLUS, out=None, temp=None):
+    out = out or DeviceArray(values.n, values.dtype)
+    _run("thrust_amd_inclusive_scan_by_key", temp, lambda fn, t, b: fn(
+        t, b, keys.ptr, values.ptr, out.ptr, keys.n, keys.dtype, values.dtype, op, stream_ptr()))
+    return out
+
+
+def exclusive_scan_by_key(keys, values, init=0, op=PLUS, out=None, temp=None):
+    out = out or DeviceArray(values.n, values.dtype)
+    iv = _scalar(values.dtype, init)
+    _run("thrust_amd_exclusive_scan_by_key", temp, lambda fn, t, b: fn(
+        t, b, keys.ptr, values.ptr, out.ptr, keys.n, keys.dtype, values.dtype, op, iv.ctypes.data,
+        stream_ptr()))
     return out
 
 

@@ -233,6 +233,20 @@ TA_DEVICE T wave_inclusive_scan(T v, Op op) {
 
 TA_DEVICE int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
 
+// Comparison against a threshold chosen at run time (thrust_amd_cmp codes).
+template <typename T>
+TA_DEVICE bool apply_cmp(int cmp, T x, T t) {
+  switch (cmp) {
+    case THRUST_AMD_LT: return x < t;
+    case THRUST_AMD_LE: return x <= t;
+    case THRUST_AMD_GT: return x > t;
+    case THRUST_AMD_GE: return x >= t;
+    case THRUST_AMD_EQ: return x == t;
+    case THRUST_AMD_NE: return x != t;
+    default: return x != (T)0;
+  }
+}
+
 // ------------------------------------------------------------------ tile status
 // A tile publishes W 32-bit payload words, each inside its own 64-bit word together
 // with the status, using relaxed agent-scope atomics.  A reader accepts a descriptor
@@ -279,19 +293,18 @@ TA_DEVICE uint32_t tile_try_load(const uint64_t* slot, P& payload) {
 
 // Decoupled look-back run by one full wave (all 64 lanes active, uniform control flow).
 // Tile `tile` (> 0) has already published its own PARTIAL descriptor.  In each round
-// lane l inspects tile (base - 63 + l), so lane order equals tile order and lane 63 is
-// the nearest predecessor; the wave folds, oldest to newest, everything from the
+// lane l of the highest WIN lanes inspects tile (base - 63 + l), so lane order equals tile
+// order and lane 63 is the nearest predecessor; the wave folds, oldest to newest, everything from the
 // nearest INCLUSIVE descriptor up to tile - 1.  Only tiles with a smaller ticket are
 // waited on, and those have started, so the spin terminates without assuming any
 // workgroup scheduling order.  `id` must be a true identity of op.  Returns, in all
 // lanes, the fold of all tiles before `tile`.
-#ifndef TA_LOOKBACK_LANES
-#define TA_LOOKBACK_LANES 8
-#endif
 template <typename P, typename Op>
 TA_DEVICE P tile_lookback(const uint64_t* status_base, uint32_t tile, Op op, P id) {
   constexpr int W = TileWords<P>::W;
-  constexpr int WIN = TA_LOOKBACK_LANES;  // descriptors inspected per round (the nearest WIN)
+  // Descriptors inspected per round: the nearest 8.  A wider window reads more cache lines
+  // per round and, with many tiles in flight, costs more than it saves.
+  constexpr int WIN = 8;
   const int lane = lane_id();
   P running = id;
   int64_t base = (int64_t)tile - 1;

@@ -18,46 +18,9 @@
 #include "common.hpp"
 #include "dispatch.hpp"
 #include "launch.hpp"
+#include "segmented.hpp"
 
 namespace ta {
-
-#ifndef TA_RBK_BLOCK
-#define TA_RBK_BLOCK 1024
-#endif
-constexpr int RBK_BLOCK = TA_RBK_BLOCK;
-#ifndef TA_RBK_ITEMS
-#define TA_RBK_ITEMS 16
-#endif
-#ifndef TA_RBK_MIN_WAVES
-#define TA_RBK_MIN_WAVES 4
-#endif
-constexpr int RBK_ITEMS = TA_RBK_ITEMS;  // elements per lane
-constexpr int RBK_MIN_WAVES = TA_RBK_MIN_WAVES;
-
-template <typename V>
-struct alignas(sizeof(V) >= 8 ? 8 : 4) SegPair {
-  uint32_t heads;
-  V value;
-};
-// 1- and 2-byte values are widened so that the pair is a whole number of 32-bit words.
-template <typename V> struct SegValue { using type = V; };
-template <> struct SegValue<int8_t> { using type = int32_t; };
-template <> struct SegValue<uint8_t> { using type = uint32_t; };
-template <> struct SegValue<int16_t> { using type = int32_t; };
-template <> struct SegValue<uint16_t> { using type = uint32_t; };
-
-template <typename V, typename Op>
-struct SegOp {
-  Op op;
-  // value folds are done in the storage type V and widened only for transport
-  using WV = typename SegValue<V>::type;
-  TA_DEVICE SegPair<WV> operator()(const SegPair<WV>& a, const SegPair<WV>& b) const {
-    SegPair<WV> r;
-    r.heads = a.heads + b.heads;
-    r.value = b.heads ? b.value : (WV)op((V)a.value, (V)b.value);
-    return r;
-  }
-};
 
 template <typename K, typename V>
 struct RbkArgs {
@@ -70,11 +33,6 @@ struct RbkArgs {
   uint64_t* status;
   uint32_t* ticket;
   uint32_t aligned;
-};
-
-template <typename V, int VEC>
-struct alignas((VEC * sizeof(V)) >= 16 ? 16 : VEC * sizeof(V)) RbkValueVec {
-  V v[VEC];
 };
 
 __global__ __launch_bounds__(256) void rbk_init_kernel(uint64_t* __restrict__ words, uint64_t count,
@@ -91,7 +49,7 @@ __global__ __launch_bounds__(256) void rbk_init_kernel(uint64_t* __restrict__ wo
 // K is the key's comparison class: an unsigned integer type of the key's size (integer
 // keys are equal iff their bits are) or float / double (operator==).
 template <typename K, typename V, typename Op>
-__global__ __launch_bounds__(RBK_BLOCK, RBK_MIN_WAVES) void rbk_kernel(RbkArgs<K, V> a) {
+__global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
   constexpr int VEC = Vec16<K>::N;
   constexpr int CHUNKS = RBK_ITEMS / VEC >= 1 ? RBK_ITEMS / VEC : 1;
   constexpr int WAVES = RBK_BLOCK / WAVE;

@@ -1,0 +1,44 @@
+// Pieces shared by the segmented single-pass kernels (reduce_by_key, scan_by_key): the
+// (heads, value) pair, its associative operator, the value vector that travels with a
+// 16-byte vector of keys, and the tile shape.
+#pragma once
+#include "common.hpp"
+
+namespace ta {
+
+// 1024 threads x 16 elements: large tiles keep the number of tiles in flight (and the
+// look-back) small; the pair scan needs ~110 VGPRs, so one workgroup fills a CU.
+constexpr int RBK_BLOCK = 1024;
+constexpr int RBK_ITEMS = 16;  // elements per lane
+
+template <typename V>
+struct alignas(sizeof(V) >= 8 ? 8 : 4) SegPair {
+  uint32_t heads;
+  V value;
+};
+// 1- and 2-byte values are widened so that the pair is a whole number of 32-bit words.
+template <typename V> struct SegValue { using type = V; };
+template <> struct SegValue<int8_t> { using type = int32_t; };
+template <> struct SegValue<uint8_t> { using type = uint32_t; };
+template <> struct SegValue<int16_t> { using type = int32_t; };
+template <> struct SegValue<uint16_t> { using type = uint32_t; };
+
+template <typename V, typename Op>
+struct SegOp {
+  Op op;
+  // value folds are done in the storage type V and widened only for transport
+  using WV = typename SegValue<V>::type;
+  TA_DEVICE SegPair<WV> operator()(const SegPair<WV>& a, const SegPair<WV>& b) const {
+    SegPair<WV> r;
+    r.heads = a.heads + b.heads;
+    r.value = b.heads ? b.value : (WV)op((V)a.value, (V)b.value);
+    return r;
+  }
+};
+
+template <typename V, int VEC>
+struct alignas((VEC * sizeof(V)) >= 16 ? 16 : VEC * sizeof(V)) RbkValueVec {
+  V v[VEC];
+};
+
+}  // namespace ta

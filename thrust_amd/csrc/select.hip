@@ -49,19 +49,6 @@ struct SelectArgs {
   uint32_t aligned;     // tested (and payload) pointers allow whole-vector loads
 };
 
-template <typename T>
-TA_DEVICE bool apply_cmp(int cmp, T x, T t) {
-  switch (cmp) {
-    case THRUST_AMD_LT: return x < t;
-    case THRUST_AMD_LE: return x <= t;
-    case THRUST_AMD_GT: return x > t;
-    case THRUST_AMD_GE: return x >= t;
-    case THRUST_AMD_EQ: return x == t;
-    case THRUST_AMD_NE: return x != t;
-    default: return x != (T)0;
-  }
-}
-
 // VEC elements of U that belong to one 16-byte vector of T.
 template <typename U, int VEC>
 struct alignas((VEC * sizeof(U)) >= 16 ? 16 : VEC * sizeof(U)) PayloadVec {
