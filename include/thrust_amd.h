@@ -203,7 +203,8 @@ int thrust_amd_exclusive_scan_by_key(void* temp, size_t* temp_bytes, const void*
  * (-0.0 before +0.0, NaNs by bit pattern), the reference's encoders
  * (thrust/system/detail/sequential/stable_radix_sort.inl:41-138).  Only key bits
  * [begin_bit, end_bit) take part (0 and 8*sizeof(key) sort fully).  descending != 0
- * yields the order thrust::greater<Key> gives, still stable.
+ * yields the order thrust::greater<Key> gives, still stable.  n <= 2^32 - 1 per call
+ * (hipErrorInvalidValue beyond).
  * Replaces cuda_cub::__radix_sort::dispatch -> cub::DeviceRadixSort::SortKeys[Descending]
  * (thrust/system/cuda/detail/sort.h:1326-1429,1438-1508). */
 int thrust_amd_sort_keys(void* temp, size_t* temp_bytes, void* keys, uint64_t n, int key_dtype,

@@ -143,3 +143,41 @@ def test_config2_full_size_properties(dev):
         assert int(np.bitwise_xor.reduce(b_in)) == int(np.bitwise_xor.reduce(b_out))
         assert np.array_equal(np.bincount(b_in >> 20, minlength=4096),
                               np.bincount(b_out >> 20, minlength=4096))
+
+
+def test_sort_beyond_2p30_keys_properties(dev):
+    """More than 2^30 keys take the 64-bit tile descriptors: sortedness, a 64-bit sum / xor
+    checksum and a byte histogram of the keys, and stability through the values, all checked
+    on the device (keys generated there from a seeded generator)."""
+    import torch
+    n = (1 << 30) + 12345
+    g = torch.Generator(device="cuda")
+    g.manual_seed(7)
+    src = torch.randint(-(1 << 31), 1 << 31, (n,), dtype=torch.int32, device="cuda", generator=g)
+
+    def u32(t):  # int32 bits as non-negative int64
+        return t.to(torch.int64) & 0xFFFFFFFF
+
+    s_sum = int(u32(src).sum().item())
+    s_hist = torch.bincount((u32(src) >> 24).to(torch.int64), minlength=256)
+    d = dev.DeviceArray(n, dev.U32, src.view(torch.uint8).clone())
+    dev.sort_keys(d)
+    out = d.storage.view(torch.int32)
+    o = u32(out)
+    assert bool((o[1:] >= o[:-1]).all().item())
+    assert int(o.sum().item()) == s_sum
+    assert torch.equal(torch.bincount((o >> 24).to(torch.int64), minlength=256), s_hist)
+    del o, d, out
+    # pairs with only 8 significant key bits: one pass, and the values of equal keys must
+    # stay in their input order
+    keys = (src & 0xFF).to(torch.int32)
+    vals = torch.arange(n, dtype=torch.int32, device="cuda")
+    dk = dev.DeviceArray(n, dev.U32, keys.view(torch.uint8).clone())
+    dv = dev.DeviceArray(n, dev.U32, vals.view(torch.uint8))
+    dev.sort_pairs(dk, dv)
+    ko = dk.storage.view(torch.int32)
+    vo = dv.storage.view(torch.int32)
+    assert bool((ko[1:] >= ko[:-1]).all().item())
+    same = ko[1:] == ko[:-1]
+    assert bool((vo[1:][same] > vo[:-1][same]).all().item())  # ascending inside every key: stable
+    assert bool((keys[vo.to(torch.int64)] == ko).all().item())  # every value still carries its key

@@ -19,8 +19,9 @@
 // are contiguous per digit run.
 //
 // Tile order is a dynamic ticket, so the look-back only waits for tiles that have
-// started.  Tile descriptors are one 32-bit word per (tile, digit): 2 status bits and a
-// 30-bit count, which limits one call to n < 2^30 keys.
+// started.  Tile descriptors are one word per (tile, digit): 2 status bits above a count,
+// 32-bit words for n < 2^30 keys and 64-bit words up to the limit of 2^32 - 1 keys per call
+// (positions and histogram counts are 32-bit).
 //
 // Algorithmic HBM traffic for K-byte keys, V-byte values, P = K passes:
 // K*n (histogram) + P * 2*(K+V)*n.  Replaces cub::DeviceRadixSort as called from
@@ -34,12 +35,18 @@ namespace ta {
 constexpr int RADIX_BITS = 8;
 constexpr int RADIX_SIZE = 1 << RADIX_BITS;
 constexpr int MAX_PASSES = 8;
-constexpr uint64_t SORT_MAX_N = (1ull << 30) - 1;
+constexpr uint64_t SORT_MAX_N = (1ull << 32) - 1;       // positions and counts are 32-bit
+constexpr uint64_t SORT_MAX_N_NARROW = (1ull << 30) - 1;  // ... and fit 30 bits up to here
 
-constexpr uint32_t ST_FLAG_SHIFT = 30;
-constexpr uint32_t ST_VALUE_MASK = (1u << ST_FLAG_SHIFT) - 1;
-constexpr uint32_t ST_PARTIAL = 1u << ST_FLAG_SHIFT;
-constexpr uint32_t ST_INCLUSIVE = 2u << ST_FLAG_SHIFT;
+// Tile descriptor word: 2 status bits above a count.  32-bit words (30-bit counts) serve
+// sorts of fewer than 2^30 keys, 64-bit words the larger ones.
+template <typename D>
+struct Descriptor {
+  static constexpr int SHIFT = (int)sizeof(D) * 8 - 2;
+  static constexpr D VALUE_MASK = ((D)1 << SHIFT) - 1;
+  static constexpr D PARTIAL = (D)1 << SHIFT;
+  static constexpr D INCLUSIVE = (D)2 << SHIFT;
+};
 
 // Key <-> radix encoding, decided at run time (uniform across the grid).
 //   sign:   sign bit for signed integers and floats, else 0
@@ -221,14 +228,15 @@ struct PassShape {
 // Tile descriptors fetched together per look-back round by each digit thread.
 constexpr int LOOKBACK_WINDOW = 4;
 
-template <typename K, typename V, bool HAS_VALUES, int BLOCK, int ITEMS>
+template <typename K, typename V, bool HAS_VALUES, int BLOCK, int ITEMS, typename D>
 __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     K* __restrict__ keys_a, K* __restrict__ keys_b, V* __restrict__ vals_a, V* __restrict__ vals_b,
     uint32_t n, int pass, SortGeometry geo, KeyCodec<K> codec,
     const uint32_t* __restrict__ bin_base,  // [RADIX_SIZE] global digit offsets of this pass
-    uint32_t* __restrict__ status,          // [tiles][RADIX_SIZE]
+    D* __restrict__ status,                 // [tiles][RADIX_SIZE]
     uint32_t* __restrict__ ticket, const SortCtl* __restrict__ ctl) {
   using Shape = PassShape<K, V, HAS_VALUES, BLOCK, ITEMS>;
+  using Desc = Descriptor<D>;
   constexpr int WAVES = Shape::WAVES;
   constexpr int TILE = Shape::TILE;
   static_assert(BLOCK >= RADIX_SIZE, "one thread per digit is required");
@@ -319,7 +327,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
 
   // ---- per digit: offsets of the waves, tile count; publish the tile's partial counts
   uint32_t digit_count = 0;
-  uint32_t* my_status = status + (size_t)tile * RADIX_SIZE;
+  D* my_status = status + (size_t)tile * RADIX_SIZE;
   if (threadIdx.x < RADIX_SIZE) {
     const int d = threadIdx.x;
     uint32_t sum = 0;
@@ -333,7 +341,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     // padding slots carry the all-ones key and must not be counted
     if (d == (int)dmask) digit_count -= ((uint32_t)TILE - valid);
     if (tile != 0)
-      __hip_atomic_store(my_status + d, ST_PARTIAL | digit_count, __ATOMIC_RELAXED,
+      __hip_atomic_store(my_status + d, (D)(Desc::PARTIAL | digit_count), __ATOMIC_RELAXED,
                          __HIP_MEMORY_SCOPE_AGENT);
     // exclusive scan of the (padded) counts over the digits -> local run offsets;
     // the part inside this wave of 64 digits now, the preceding waves after the barrier
@@ -375,10 +383,10 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
       excl = bin_base[d];
     } else {
       uint32_t acc = 0;
-      int t = (int)tile - 1;  // tile counts stay below 2^16
-      const uint32_t* my_col = status + d;
+      int t = (int)tile - 1;  // tile counts stay below 2^20
+      const D* my_col = status + d;
       for (;;) {
-        uint32_t s[LOOKBACK_WINDOW];
+        D s[LOOKBACK_WINDOW];
 #pragma unroll
         for (int k = 0; k < LOOKBACK_WINDOW; ++k) {
           const uint32_t tk = (uint32_t)((t - k) > 0 ? (t - k) : 0);  // tile 0 is always inclusive
@@ -390,12 +398,12 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
         int used = 0;
 #pragma unroll
         for (int k = 0; k < LOOKBACK_WINDOW; ++k) {
-          const uint32_t flag = s[k] & ~ST_VALUE_MASK;
+          const D flag = s[k] & ~Desc::VALUE_MASK;
           const bool take = !done && used == k && flag != 0;
           if (take) {
-            acc += s[k] & ST_VALUE_MASK;
+            acc += (uint32_t)(s[k] & Desc::VALUE_MASK);
             used = k + 1;
-            done = flag == ST_INCLUSIVE;
+            done = flag == Desc::INCLUSIVE;
           }
         }
         if (done) break;
@@ -404,7 +412,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
       }
       excl = acc;
     }
-    __hip_atomic_store(my_status + d, ST_INCLUSIVE | (excl + digit_count), __ATOMIC_RELAXED,
+    __hip_atomic_store(my_status + d, (D)(Desc::INCLUSIVE | (D)(uint32_t)(excl + digit_count)), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
     s_scatter_base[d] = excl - local_base;
   }
@@ -510,8 +518,9 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
   TempLayout lay;
   const size_t off_ctl = lay.add(sizeof(SortCtl));
   // contiguous zero-initialised region: tickets, histograms, tile descriptors
+  const bool wide = n > SORT_MAX_N_NARROW;  // prefixes need more than 30 bits: 64-bit descriptors
   const size_t zero_words = (size_t)MAX_PASSES + (size_t)MAX_PASSES * RADIX_SIZE +
-                            (size_t)geo.passes * tiles * RADIX_SIZE;
+                            (size_t)geo.passes * tiles * RADIX_SIZE * (wide ? 2 : 1);
   const size_t off_zero = lay.add(zero_words * sizeof(uint32_t));
   const size_t off_keys = lay.add((size_t)n * sizeof(K));
   const size_t off_vals = lay.add(HAS_VALUES ? (size_t)n * sizeof(V) : 0);
@@ -551,7 +560,12 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
   TA_LAUNCH("sort_scan", stream, sort_scan_kernel, dim3(1), dim3(RADIX_SIZE), hist, (uint32_t)n, geo, ctl);
   TA_CHECK_LAUNCH();
   for (int p = 0; p < geo.passes; ++p) {
-    TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + (size_t)p * tiles * RADIX_SIZE, tickets + p, (const SortCtl*)ctl);
+    const size_t status_off = (size_t)p * tiles * RADIX_SIZE;  // in descriptor words
+    if (wide) {
+      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint64_t>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, reinterpret_cast<uint64_t*>(status) + status_off, tickets + p, (const SortCtl*)ctl);
+    } else {
+      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint32_t>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + status_off, tickets + p, (const SortCtl*)ctl);
+    }
     TA_CHECK_LAUNCH();
   }
   {
