@@ -1,5 +1,5 @@
 #!/usr/bin/env python3
-"""Headline benchmark: thrust::sort of 2^28 uint32 keys (BASELINE.json configs[1]) on one MI355X,
+"""Headline benchmark: thrust::sort of 2^28 uint32 keys (the configuration the headline metric is quoted on) on one MI355X,
 with thrust::reduce / inclusive_scan over 2^28 int32 measured beside it.
 
 One step = one full radix sort of a device-resident, never-before-sorted copy of the seeded

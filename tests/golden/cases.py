@@ -1,4 +1,4 @@
-"""The seeded cases of the golden fixtures: one function per BASELINE config, returning
+"""The seeded cases of the golden fixtures: one function per benchmark configuration, returning
 {name: output array} when run on an implementation with the Oracle/Reference interface
 (oracle.cpu) or on the device (tests pass an adapter).  Shared by the fixture writer
 (which runs the REAL reference) and by the tests (which run the restatement / the GPU)."""

@@ -1,5 +1,5 @@
 """GPU parity against the golden fixtures written from the REAL reference
-(tests/golden/make_fixtures.py): every BASELINE config at small N (exact arrays) and at a
+(tests/golden/make_fixtures.py): every benchmark configuration at small N (exact arrays) and at a
 larger N (sha256 of the output bytes).  Bit-exact everywhere except float32 run sums,
 which are compared within 1e-5 relative (tree order on the device, strict left fold in
 the reference)."""

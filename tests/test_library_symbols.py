@@ -64,6 +64,7 @@ def test_size_queries_and_argument_errors_need_no_gpu(lib):
     assert lib.thrust_amd_reduce(None, ctypes.byref(n), None, 10, 99, 0, None, None, None) != 0   # bad dtype
     assert lib.thrust_amd_reduce(None, ctypes.byref(n), None, 10, 4, 99, None, None, None) != 0   # bad op
     assert lib.thrust_amd_sort_keys(None, ctypes.byref(n), None, 10, 5, 0, 8, 40, None) != 0       # bad bit range
-    assert lib.thrust_amd_sort_keys(None, ctypes.byref(n), None, 1 << 31, 5, 0, 0, 32, None) != 0  # n too large
+    assert lib.thrust_amd_sort_keys(None, ctypes.byref(n), None, 1 << 31, 5, 0, 0, 32, None) == 0  # wide descriptors
+    assert lib.thrust_amd_sort_keys(None, ctypes.byref(n), None, 1 << 32, 5, 0, 0, 32, None) != 0  # n too large
     assert lib.thrust_amd_copy_if(None, ctypes.byref(n), None, None, None, None, 10, 3, 8, 0, None, None) != 0  # item size
     assert lib.thrust_amd_reduce(None, None, None, 10, 4, 0, None, None, None) != 0                # no size slot
