@@ -94,10 +94,13 @@ __global__ __launch_bounds__(256) void sort_init_kernel(uint32_t* __restrict__ w
 // atomic fall on 32 distinct banks whatever the digits are (random digits on a single
 // copy serialise about five-fold on bank conflicts).  Keys are read with 16-byte loads;
 // their order does not matter here.
+// WHOLE_BYTES: the keys need no encoding and the sorted bits are NP whole bytes starting
+// at bit 0 (the usual full-range sort of unsigned keys), so every digit is a bit-field
+// extract at a constant position.
 constexpr int HIST_BLOCK = 1024;
-constexpr int HIST_UNROLL = 2;  // 16-byte vectors in flight per lane
+constexpr int HIST_UNROLL = 4;  // 16-byte vectors in flight per lane
 
-template <typename K, int NP>
+template <typename K, int NP, bool WHOLE_BYTES>
 __global__ __launch_bounds__(HIST_BLOCK) void sort_histogram_kernel(const K* __restrict__ keys,
                                                                      uint64_t n, KeyCodec<K> codec,
                                                                      SortGeometry geo,
@@ -111,11 +114,11 @@ __global__ __launch_bounds__(HIST_BLOCK) void sort_histogram_kernel(const K* __r
   uint32_t* my_copy = s_hist + (threadIdx.x % COPIES);
 
   auto count = [&](K k) {
-    const K e = codec.plain ? k : codec.encode(k);
+    const K e = (WHOLE_BYTES || codec.plain) ? k : codec.encode(k);
 #pragma unroll
     for (int p = 0; p < NP; ++p) {
-      const int lo = geo.begin_bit + p * RADIX_BITS;
-      const int nb = (p == NP - 1) ? (geo.end_bit - lo) : RADIX_BITS;
+      const int lo = WHOLE_BYTES ? p * RADIX_BITS : geo.begin_bit + p * RADIX_BITS;
+      const int nb = (WHOLE_BYTES || p < NP - 1) ? RADIX_BITS : (geo.end_bit - lo);
       const uint32_t d = (uint32_t)(e >> lo) & ((1u << nb) - 1u);
       __hip_atomic_fetch_add(my_copy + (p * RADIX_SIZE + d) * COPIES, 1u, __ATOMIC_RELAXED,
                              __HIP_MEMORY_SCOPE_WORKGROUP);
@@ -133,22 +136,50 @@ __global__ __launch_bounds__(HIST_BLOCK) void sort_histogram_kernel(const K* __r
   }
   const Vec16<K>* body = reinterpret_cast<const Vec16<K>*>(keys + head);
   constexpr uint64_t TILE_VECS = (uint64_t)HIST_BLOCK * HIST_UNROLL;
-  const uint64_t tiles = (vecs + TILE_VECS - 1) / TILE_VECS;
-  for (uint64_t tile = blockIdx.x; tile < tiles; tile += gridDim.x) {
-    const uint64_t base = tile * TILE_VECS + threadIdx.x;
-    Vec16<K> x[HIST_UNROLL];
-    bool ok[HIST_UNROLL];
+  // Whole tiles: no predicates, and the next tile's vectors are in flight while this
+  // tile's are counted (two register buffers in turn; the loop body always loads, so
+  // the waits before counting only cover the older buffer).
+  const uint64_t whole_tiles = vecs / TILE_VECS;
+  const uint64_t step = gridDim.x;
+  uint64_t tile = blockIdx.x;
+  Vec16<K> buf_a[HIST_UNROLL], buf_b[HIST_UNROLL];
+  auto load_tile = [&](Vec16<K>(&x)[HIST_UNROLL], uint64_t t) {
+#pragma unroll
+    for (int u = 0; u < HIST_UNROLL; ++u) x[u] = body[t * TILE_VECS + threadIdx.x + (uint64_t)u * HIST_BLOCK];
+  };
+  auto count_tile = [&](const Vec16<K>(&x)[HIST_UNROLL]) {
 #pragma unroll
     for (int u = 0; u < HIST_UNROLL; ++u) {
-      const uint64_t i = base + (uint64_t)u * HIST_BLOCK;
-      ok[u] = i < vecs;
-      if (ok[u]) x[u] = body[i];
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) count(x[u].v[i]);
     }
+  };
+  if (tile < whole_tiles) load_tile(buf_a, tile);
+  while (tile + 2 * step < whole_tiles) {
+    load_tile(buf_b, tile + step);
+    count_tile(buf_a);
+    load_tile(buf_a, tile + 2 * step);
+    count_tile(buf_b);
+    tile += 2 * step;
+  }
+  if (tile < whole_tiles) {
+    if (tile + step < whole_tiles) {
+      load_tile(buf_b, tile + step);
+      count_tile(buf_a);
+      count_tile(buf_b);
+    } else {
+      count_tile(buf_a);
+    }
+  }
+  // the ragged tile after them, if any, goes to the workgroup whose turn it would be
+  if (whole_tiles * TILE_VECS < vecs && whole_tiles % gridDim.x == blockIdx.x) {
 #pragma unroll
     for (int u = 0; u < HIST_UNROLL; ++u) {
-      if (ok[u]) {
+      const uint64_t i = whole_tiles * TILE_VECS + threadIdx.x + (uint64_t)u * HIST_BLOCK;
+      if (i < vecs) {
+        const Vec16<K> x = body[i];
 #pragma unroll
-        for (int i = 0; i < VEC; ++i) count(x[u].v[i]);
+        for (int j = 0; j < VEC; ++j) count(x.v[j]);
       }
     }
   }
@@ -166,10 +197,15 @@ template <typename K>
 static void launch_histogram(int passes, uint32_t blocks, hipStream_t stream, const K* keys,
                              uint64_t n, const KeyCodec<K>& codec, const SortGeometry& geo,
                              uint32_t* hist) {
+  const bool whole = codec.plain && geo.begin_bit == 0 && geo.end_bit == passes * RADIX_BITS;
 #define TA_HIST_CASE(NP)                                                                       \
   case NP:                                                                                     \
-    TA_LAUNCH("sort_histogram", \
-                       stream, (sort_histogram_kernel<K, NP>), dim3(blocks), dim3(HIST_BLOCK), keys, n, codec, geo, hist);                                     \
+    if (whole)                                                                                 \
+      TA_LAUNCH("sort_histogram", stream, (sort_histogram_kernel<K, NP, true>), dim3(blocks),  \
+                dim3(HIST_BLOCK), keys, n, codec, geo, hist);                                  \
+    else                                                                                       \
+      TA_LAUNCH("sort_histogram", stream, (sort_histogram_kernel<K, NP, false>), dim3(blocks), \
+                dim3(HIST_BLOCK), keys, n, codec, geo, hist);                                  \
     break;
   switch (passes) {
     TA_HIST_CASE(1) TA_HIST_CASE(2) TA_HIST_CASE(3) TA_HIST_CASE(4)
