@@ -96,14 +96,27 @@ Out copy(execution_policy<D>& exec, In first, In last, Out result) {
 namespace detail {
 // Shared by copy_if and the partition family: runs `entry` (one of the three selection
 // entry points bound by the caller) and returns the number of selected elements.
+// `negate` selects the elements the predicate rejects (remove_if is copy_if of not1(pred),
+// thrust/system/cuda/detail/remove.h:40-66): every comparison code has its complement.
+inline int negated_cmp(int cmp) {
+  switch (cmp) {
+    case THRUST_AMD_LT: return THRUST_AMD_GE;
+    case THRUST_AMD_LE: return THRUST_AMD_GT;
+    case THRUST_AMD_GT: return THRUST_AMD_LE;
+    case THRUST_AMD_GE: return THRUST_AMD_LT;
+    case THRUST_AMD_EQ: return THRUST_AMD_NE;
+    case THRUST_AMD_NE: return THRUST_AMD_EQ;
+    default: return THRUST_AMD_EQ;  // "is non-zero" -> equal to the zero threshold it carries
+  }
+}
 template <typename Tested, typename Pred, typename Call>
-inline uint64_t run_selection(void* stream, const Pred& pred, const char* what, Call call) {
+inline uint64_t run_selection(void* stream, const Pred& pred, const char* what, Call call, bool negate = false) {
   static_assert(is_abi_type<Tested>::value,
                 "selection on the device system needs an arithmetic type to test");
   static_assert(unary_pred<Pred, Tested>::supported,
                 "selection on the device system supports placeholder comparisons (_1 < t, ...), "
                 "thrust::identity and thrust::logical_not as predicate");
-  const int cmp = unary_pred<Pred, Tested>::cmp(pred);
+  const int cmp = negate ? negated_cmp(unary_pred<Pred, Tested>::cmp(pred)) : unary_pred<Pred, Tested>::cmp(pred);
   const Tested thr = unary_pred<Pred, Tested>::threshold(pred);
   temp_storage temp(stream);
   std::size_t need = 0;

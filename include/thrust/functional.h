@@ -7,7 +7,8 @@
 //   orderings          less, greater                     (sort, merge)
 //   equivalence        equal_to                          (unique, reduce_by_key)
 //   unary predicates   placeholder comparisons (_1 < t), identity / "is true",
-//                      logical_not                       (copy_if, partition)
+//                      logical_not                       (copy_if, partition, remove_if, count_if)
+//   unary transforms   identity, negate, square          (transform_reduce, transform scans)
 #pragma once
 #include <thrust/detail/config.h>
 
@@ -67,6 +68,23 @@ struct negate {
   typedef T argument_type;
   typedef T result_type;
   constexpr T operator()(const T& x) const { return -x; }
+};
+
+template <typename T = void>
+struct square {
+  typedef T argument_type;
+  typedef T result_type;
+  constexpr T operator()(const T& x) const { return x * x; }
+};
+template <>
+struct negate<void> {
+  template <typename A>
+  constexpr auto operator()(const A& x) const -> decltype(-x) { return -x; }
+};
+template <>
+struct square<void> {
+  template <typename A>
+  constexpr auto operator()(const A& x) const -> decltype(x * x) { return x * x; }
 };
 
 namespace detail {

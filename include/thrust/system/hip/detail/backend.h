@@ -49,6 +49,15 @@ template <typename T> struct binop_code<thrust::minimum<void>, T> { static const
 template <typename T> struct binop_code<thrust::maximum<T>, T> { static const int value = THRUST_AMD_MAX; };
 template <typename T> struct binop_code<thrust::maximum<void>, T> { static const int value = THRUST_AMD_MAX; };
 
+// thrust_amd_unary code of a transform whose argument and result are T, or -1
+template <typename Fn, typename T> struct unary_code { static const int value = -1; };
+template <typename T> struct unary_code<thrust::identity<T>, T> { static const int value = THRUST_AMD_IDENTITY; };
+template <typename T> struct unary_code<thrust::identity<void>, T> { static const int value = THRUST_AMD_IDENTITY; };
+template <typename T> struct unary_code<thrust::negate<T>, T> { static const int value = THRUST_AMD_NEGATE; };
+template <typename T> struct unary_code<thrust::negate<void>, T> { static const int value = THRUST_AMD_NEGATE; };
+template <typename T> struct unary_code<thrust::square<T>, T> { static const int value = THRUST_AMD_SQUARE; };
+template <typename T> struct unary_code<thrust::square<void>, T> { static const int value = THRUST_AMD_SQUARE; };
+
 // 0 ascending (less), 1 descending (greater), -1 not a recognised ordering
 template <typename Comp, typename T> struct order_code { static const int value = -1; };
 template <typename T> struct order_code<thrust::less<T>, T> { static const int value = 0; };

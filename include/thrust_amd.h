@@ -73,6 +73,16 @@ typedef enum thrust_amd_cmp {
   THRUST_AMD_CMP_COUNT = 7
 } thrust_amd_cmp;
 
+/* Unary transforms applied to every input element by the transform_* entry points: the
+ * closed set the front end maps thrust::identity / negate / square to
+ * (thrust/functional.h:523-600, 1224-1240).  Integers negate and square modulo 2^bits. */
+typedef enum thrust_amd_unary {
+  THRUST_AMD_IDENTITY = 0,
+  THRUST_AMD_NEGATE = 1,
+  THRUST_AMD_SQUARE = 2,
+  THRUST_AMD_UNARY_COUNT = 3
+} thrust_amd_unary;
+
 typedef enum thrust_amd_memcpy_kind {
   THRUST_AMD_H2D = 1,
   THRUST_AMD_D2H = 2,
@@ -163,6 +173,15 @@ int thrust_amd_count_if(void* temp, size_t* temp_bytes, const void* in, uint64_t
 int thrust_amd_inner_product(void* temp, size_t* temp_bytes, const void* a, const void* b,
                              uint64_t n, int dtype, const void* init, void* d_out, void* stream);
 
+/* *d_out = init OP f(in[0]) OP ... OP f(in[n-1]) with f a thrust_amd_unary code; f's result
+ * and the accumulator have type dtype.  `init` is a host pointer to one dtype element.
+ * Replaces cuda_cub::transform_reduce -> reduce_n over a transform iterator
+ * (thrust/system/cuda/detail/transform_reduce.h:39-64; generic form
+ * thrust/system/detail/generic/transform_reduce.inl:30-48). */
+int thrust_amd_transform_reduce(void* temp, size_t* temp_bytes, const void* in, uint64_t n,
+                                int dtype, int unary, int op, const void* init, void* d_out,
+                                void* stream);
+
 /* --------------------------------------------------------------------- scan */
 
 /* out[i] = in[0] OP ... OP in[i]; accumulator type = dtype; out == in allowed.
@@ -176,6 +195,17 @@ int thrust_amd_inclusive_scan(void* temp, size_t* temp_bytes, const void* in, vo
  * Replaces cuda_cub::exclusive_scan_n (thrust/system/cuda/detail/scan.h:132-200). */
 int thrust_amd_exclusive_scan(void* temp, size_t* temp_bytes, const void* in, void* out,
                               uint64_t n, int dtype, int op, const void* init, void* stream);
+
+/* The two scans above over f(in[i]) instead of in[i], f a thrust_amd_unary code with result
+ * type dtype; out == in allowed.
+ * Replace cuda_cub::transform_inclusive_scan / transform_exclusive_scan -> the scans over a
+ * transform iterator (thrust/system/cuda/detail/transform_scan.h:39-115; generic forms
+ * thrust/system/detail/generic/transform_scan.inl:37-97). */
+int thrust_amd_transform_inclusive_scan(void* temp, size_t* temp_bytes, const void* in, void* out,
+                                        uint64_t n, int dtype, int unary, int op, void* stream);
+int thrust_amd_transform_exclusive_scan(void* temp, size_t* temp_bytes, const void* in, void* out,
+                                        uint64_t n, int dtype, int unary, int op, const void* init,
+                                        void* stream);
 
 /* Segmented scans: a segment is a run of equal consecutive keys (compared like
  * reduce_by_key: integers by value, floats with ==).  out[i] = the OP-fold of the segment's

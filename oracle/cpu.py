@@ -25,6 +25,7 @@ NP_DTYPES = {I8: np.int8, U8: np.uint8, I16: np.int16, U16: np.uint16, I32: np.i
 DTYPE_OF_NP = {np.dtype(v): k for k, v in NP_DTYPES.items()}
 PLUS, MIN, MAX = range(3)
 LT, LE, GT, GE, EQ, NE, NONZERO = range(7)
+IDENTITY, NEGATE, SQUARE = range(3)
 
 
 def build(with_ref=True):
@@ -202,6 +203,30 @@ class _Base:
         self._ok(self._fn("inner_product")(_p(a), _p(b), ctypes.c_uint64(a.size), _code(a), _p(iv),
                                             _p(out), *self._extra()), "inner_product")
         return out[0]
+
+    def transform_reduce(self, x, unary, op=PLUS, init=0):
+        x = _c(x)
+        out = np.zeros(1, x.dtype)
+        iv = np.array([init], x.dtype)
+        self._ok(self._fn("transform_reduce")(_p(x), ctypes.c_uint64(x.size), _code(x), unary, op,
+                                               _p(iv), _p(out), *self._extra()), "transform_reduce")
+        return out[0]
+
+    def transform_inclusive_scan(self, x, unary, op=PLUS):
+        x = _c(x)
+        out = np.empty_like(x)
+        self._ok(self._fn("transform_inclusive_scan")(_p(x), _p(out), ctypes.c_uint64(x.size),
+                                                       _code(x), unary, op), "transform_inclusive_scan")
+        return out
+
+    def transform_exclusive_scan(self, x, unary, init=0, op=PLUS):
+        x = _c(x)
+        out = np.empty_like(x)
+        iv = np.array([init], x.dtype)
+        self._ok(self._fn("transform_exclusive_scan")(_p(x), _p(out), ctypes.c_uint64(x.size),
+                                                       _code(x), unary, op, _p(iv)),
+                 "transform_exclusive_scan")
+        return out
 
     def inclusive_scan_by_key(self, keys, values, op=PLUS):
         k, v = _c(keys), _c(values)

@@ -18,6 +18,8 @@
 #include <thrust/reduce.h>
 #include <thrust/scan.h>
 #include <thrust/sort.h>
+#include <thrust/transform_reduce.h>
+#include <thrust/transform_scan.h>
 #include <thrust/unique.h>
 
 #include <cstdint>
@@ -314,6 +316,57 @@ REF_API int ref_inner_product(const void* a, const void* b, uint64_t n, int dtyp
     using T = decltype(z);
     *(T*)out = thrust::inner_product(thrust::device, dp<T>(a), dp<T>(a) + n, dp<T>(b), *(const T*)init);
     return 0;
+  });
+}
+
+namespace {
+template <typename T, typename F>
+int with_unary(int unary, F&& f) {
+  switch (unary) {
+    case THRUST_AMD_IDENTITY: return f(thrust::identity<T>());
+    case THRUST_AMD_NEGATE: return f(thrust::negate<T>());
+    case THRUST_AMD_SQUARE: return f(thrust::square<T>());
+    default: return -1;
+  }
+}
+}  // namespace
+
+REF_API int ref_transform_reduce(const void* in, uint64_t n, int dtype, int unary, int op,
+                                 const void* init, void* out) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    return with_unary<T>(unary, [&](auto u) {
+      return with_op<T>(op, [&](auto o) {
+        *(T*)out = thrust::transform_reduce(thrust::device, dp<T>(in), dp<T>(in) + n, u, *(const T*)init, o);
+        return 0;
+      });
+    });
+  });
+}
+
+REF_API int ref_transform_inclusive_scan(const void* in, void* out, uint64_t n, int dtype, int unary,
+                                         int op) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    return with_unary<T>(unary, [&](auto u) {
+      return with_op<T>(op, [&](auto o) {
+        thrust::transform_inclusive_scan(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), u, o);
+        return 0;
+      });
+    });
+  });
+}
+
+REF_API int ref_transform_exclusive_scan(const void* in, void* out, uint64_t n, int dtype, int unary,
+                                         int op, const void* init) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    return with_unary<T>(unary, [&](auto u) {
+      return with_op<T>(op, [&](auto o) {
+        thrust::transform_exclusive_scan(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), u, *(const T*)init, o);
+        return 0;
+      });
+    });
   });
 }
 

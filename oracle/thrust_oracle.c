@@ -445,6 +445,43 @@ ORACLE_API int oracle_count_if(const void* in, uint64_t n, int dtype, int cmp, c
   return 0;
 }
 
+/* generic::transform_reduce (generic/transform_reduce.inl:30-48): the system's reduce over
+ * the transformed range; generic::transform_inclusive_scan / transform_exclusive_scan
+ * (generic/transform_scan.inl:37-97): the system's scans over it. */
+ORACLE_API int oracle_transform_reduce(const void* in, uint64_t n, int dtype, int unary, int op,
+                                       const void* init, void* out, int nprocs) {
+  const long P = nprocs > 0 ? nprocs : omp_get_num_procs();
+#define BODY(S, T)                                                     \
+  T* f = transformed_##S((const T*)in, (size_t)n, unary);              \
+  *(T*)out = reduce_##S(f, (size_t)n, *(const T*)init, op, P);         \
+  free(f);
+  DISPATCH(dtype, BODY)
+#undef BODY
+  return 0;
+}
+
+ORACLE_API int oracle_transform_inclusive_scan(const void* in, void* out, uint64_t n, int dtype,
+                                               int unary, int op) {
+#define BODY(S, T)                                            \
+  T* f = transformed_##S((const T*)in, (size_t)n, unary);     \
+  inclusive_scan_##S(f, (T*)out, (size_t)n, op);              \
+  free(f);
+  DISPATCH(dtype, BODY)
+#undef BODY
+  return 0;
+}
+
+ORACLE_API int oracle_transform_exclusive_scan(const void* in, void* out, uint64_t n, int dtype,
+                                               int unary, int op, const void* init) {
+#define BODY(S, T)                                                   \
+  T* f = transformed_##S((const T*)in, (size_t)n, unary);            \
+  exclusive_scan_##S(f, (T*)out, (size_t)n, op, *(const T*)init);    \
+  free(f);
+  DISPATCH(dtype, BODY)
+#undef BODY
+  return 0;
+}
+
 ORACLE_API int oracle_inner_product(const void* a, const void* b, uint64_t n, int dtype,
                                     const void* init, void* out, int nprocs) {
   const long P = nprocs > 0 ? nprocs : omp_get_num_procs();

@@ -17,8 +17,11 @@
 #include <thrust/merge.h>
 #include <thrust/partition.h>
 #include <thrust/reduce.h>
+#include <thrust/remove.h>
 #include <thrust/scan.h>
 #include <thrust/sort.h>
+#include <thrust/transform_reduce.h>
+#include <thrust/transform_scan.h>
 #include <thrust/unique.h>
 
 #include <cstdint>
@@ -185,6 +188,82 @@ static void TestInnerProductSimple() {  // testing/inner_product.cu:10-24
   ASSERT_TRUE(thrust::inner_product(v1.begin(), v1.end(), v2.begin(), 3, thrust::plus<int>(), thrust::multiplies<int>()) == 7);
   thrust::host_vector<int> h1 = to_host(v1), h2 = to_host(v2);
   ASSERT_TRUE(thrust::inner_product(h1.begin(), h1.end(), h2.begin(), 3) == 7);
+}
+
+static void TestTransformReduceAndScanSimple() {  // testing/transform_reduce.cu:70-83, transform_scan.cu:140-190,355-399
+  g_test = "TransformReduceAndScanSimple";
+  thrust::device_vector<int> data(hv<int>({1, -2, 3}));
+  ASSERT_TRUE(thrust::transform_reduce(data.begin(), data.end(), thrust::negate<int>(), 10, thrust::plus<int>()) == 8);
+  ASSERT_TRUE(thrust::transform_reduce(thrust::device, data.begin(), data.end(), thrust::square<int>(), 1, thrust::plus<int>()) == 15);
+  thrust::host_vector<int> hdata = to_host(data);
+  ASSERT_TRUE(thrust::transform_reduce(hdata.begin(), hdata.end(), thrust::negate<int>(), 10, thrust::plus<int>()) == 8);
+  thrust::device_vector<int> in(hv<int>({1, 3, -2, 4, -5})), out(5);
+  auto it = thrust::transform_inclusive_scan(in.begin(), in.end(), out.begin(), thrust::negate<int>(), thrust::plus<int>());
+  ASSERT_TRUE(it - out.begin() == 5);
+  ASSERT_EQUAL_VEC(to_host(out), hv<int>({-1, -4, -2, -6, -1}));
+  ASSERT_EQUAL_VEC(to_host(in), hv<int>({1, 3, -2, 4, -5}));
+  thrust::transform_exclusive_scan(in.begin(), in.end(), out.begin(), thrust::negate<int>(), 0, thrust::plus<int>());
+  ASSERT_EQUAL_VEC(to_host(out), hv<int>({0, -1, -4, -2, -6}));
+  thrust::transform_exclusive_scan(thrust::device, in.begin(), in.end(), out.begin(), thrust::negate<int>(), 3, thrust::plus<int>());
+  ASSERT_EQUAL_VEC(to_host(out), hv<int>({3, 2, -1, 1, -3}));
+  thrust::device_vector<int> inplace = in;  // in place
+  thrust::transform_inclusive_scan(inplace.begin(), inplace.end(), inplace.begin(), thrust::negate<int>(), thrust::plus<int>());
+  ASSERT_EQUAL_VEC(to_host(inplace), hv<int>({-1, -4, -2, -6, -1}));
+  inplace = in;
+  thrust::transform_exclusive_scan(inplace.begin(), inplace.end(), inplace.begin(), thrust::negate<int>(), 3, thrust::plus<int>());
+  ASSERT_EQUAL_VEC(to_host(inplace), hv<int>({3, 2, -1, 1, -3}));
+  thrust::host_vector<int> hin = to_host(in), hout(5);
+  thrust::transform_inclusive_scan(hin.begin(), hin.end(), hout.begin(), thrust::negate<int>(), thrust::plus<int>());
+  ASSERT_EQUAL_VEC(hout, hv<int>({-1, -4, -2, -6, -1}));
+  thrust::device_vector<int> vec(hv<int>({5, 0, 5, 8, 6, 7, 5, 3, 0, 9}));
+  thrust::transform_inclusive_scan(thrust::device, vec.cbegin(), vec.cend(), vec.begin(), thrust::identity<>{}, thrust::maximum<>{});
+  ASSERT_EQUAL_VEC(to_host(vec), hv<int>({5, 5, 5, 8, 8, 8, 8, 8, 8, 9}));
+  vec = thrust::device_vector<int>(hv<int>({5, 0, 5, 8, 6, 7, 5, 3, 0, 9}));
+  thrust::transform_exclusive_scan(thrust::device, vec.cbegin(), vec.cend(), vec.begin(), thrust::identity<>{}, int{}, thrust::maximum<>{});
+  ASSERT_EQUAL_VEC(to_host(vec), hv<int>({0, 5, 5, 5, 8, 8, 8, 8, 8, 8}));
+}
+
+static void TestRemoveSimple() {  // testing/remove.cu:28-47,100-122,184-203,256-283,345-367,429-460
+  g_test = "RemoveSimple";
+  const thrust::host_vector<int> src = hv<int>({1, 2, 1, 3, 2});
+  const thrust::host_vector<int> kept = hv<int>({1, 1, 3});
+  thrust::device_vector<int> data(src);
+  auto end = thrust::remove(data.begin(), data.end(), 2);
+  ASSERT_TRUE(end - data.begin() == 3);
+  data.resize(3);
+  ASSERT_EQUAL_VEC(to_host(data), kept);
+  data = thrust::device_vector<int>(src);
+  thrust::device_vector<int> result(5);
+  auto rend = thrust::remove_copy(data.begin(), data.end(), result.begin(), 2);
+  ASSERT_TRUE(rend - result.begin() == 3);
+  result.resize(3);
+  ASSERT_EQUAL_VEC(to_host(result), kept);
+  ASSERT_EQUAL_VEC(to_host(data), src);
+  end = thrust::remove_if(data.begin(), data.end(), _1 == 2);
+  ASSERT_TRUE(end - data.begin() == 3);
+  data.resize(3);
+  ASSERT_EQUAL_VEC(to_host(data), kept);
+  data = thrust::device_vector<int>(src);
+  thrust::device_vector<int> stencil(hv<int>({0, 1, 0, 0, 1}));
+  end = thrust::remove_if(thrust::device, data.begin(), data.end(), stencil.begin(), thrust::identity<int>());
+  ASSERT_TRUE(end - data.begin() == 3);
+  data.resize(3);
+  ASSERT_EQUAL_VEC(to_host(data), kept);
+  data = thrust::device_vector<int>(src);
+  result = thrust::device_vector<int>(5);
+  rend = thrust::remove_copy_if(data.begin(), data.end(), result.begin(), _1 == 2);
+  ASSERT_TRUE(rend - result.begin() == 3);
+  rend = thrust::remove_copy_if(data.begin(), data.end(), stencil.begin(), result.begin(), thrust::identity<int>());
+  ASSERT_TRUE(rend - result.begin() == 3);
+  result.resize(3);
+  ASSERT_EQUAL_VEC(to_host(result), kept);
+  thrust::host_vector<int> h = src;  // the host system
+  h.resize(thrust::remove(h.begin(), h.end(), 2) - h.begin());
+  ASSERT_EQUAL_VEC(h, kept);
+  h = src;
+  thrust::host_vector<int> hst = hv<int>({0, 1, 0, 0, 1});
+  h.resize(thrust::remove_if(h.begin(), h.end(), hst.begin(), thrust::identity<int>()) - h.begin());
+  ASSERT_EQUAL_VEC(h, kept);
 }
 
 static void TestSortSimple() {  // testing/sort.cu:43-76
@@ -402,7 +481,35 @@ static void DifferentialForType(const char* name) {
         U dot = (U)3;
         for (size_t i = 0; i < n; ++i) dot = (U)(dot + (U)((U)h[i] * (U)hsv[i]));
         ASSERT_TRUE(thrust::inner_product(d.begin(), d.end(), dsv.begin(), (T)3) == (T)dot);
+        // transform_reduce / transform scans: negate with plus (testing/transform_scan.cu:253-279)
+        U neg = (U)13;
+        for (size_t i = 0; i < n; ++i) neg = (U)(neg - (U)h[i]);
+        ASSERT_TRUE(thrust::transform_reduce(d.begin(), d.end(), thrust::negate<T>(), (T)13, thrust::plus<T>()) == (T)neg);
+        thrust::host_vector<T> hts(n);
+        thrust::device_vector<T> dts(n);
+        U run = 0;
+        for (size_t i = 0; i < n; ++i) { run = (U)(run - (U)h[i]); hts[i] = (T)run; }
+        thrust::transform_inclusive_scan(d.begin(), d.end(), dts.begin(), thrust::negate<T>(), thrust::plus<T>());
+        ASSERT_EQUAL_VEC(to_host(dts), hts);
+        run = (U)11;
+        for (size_t i = 0; i < n; ++i) { hts[i] = (T)run; run = (U)(run + (U)((U)h[i] * (U)h[i])); }
+        thrust::transform_exclusive_scan(d.begin(), d.end(), dts.begin(), thrust::square<T>(), (T)11, thrust::plus<T>());
+        ASSERT_EQUAL_VEC(to_host(dts), hts);
       }
+    }
+    // remove_if / remove_copy_if / remove against the host system
+    {
+      thrust::host_vector<T> hr = random_integers<T>(n, 23, 100), hro(n);
+      thrust::device_vector<T> dr = hr, dro(n);
+      hro.resize(thrust::remove_copy_if(hr.begin(), hr.end(), hro.begin(), _1 >= (T)50) - hro.begin());
+      dro.resize(thrust::remove_copy_if(dr.begin(), dr.end(), dro.begin(), _1 >= (T)50) - dro.begin());
+      ASSERT_EQUAL_VEC(to_host(dro), hro);
+      hr.resize(thrust::remove_if(hr.begin(), hr.end(), _1 < (T)30) - hr.begin());
+      dr.resize(thrust::remove_if(dr.begin(), dr.end(), _1 < (T)30) - dr.begin());
+      ASSERT_EQUAL_VEC(to_host(dr), hr);
+      hr.resize(thrust::remove(hr.begin(), hr.end(), (T)77) - hr.begin());
+      dr.resize(thrust::remove(dr.begin(), dr.end(), (T)77) - dr.begin());
+      ASSERT_EQUAL_VEC(to_host(dr), hr);
     }
     // copy_if / stable_partition with a threshold predicate
     thrust::host_vector<T> hsel = random_integers<T>(n, 21, 100);
@@ -561,6 +668,8 @@ int main() {
   TestScanByKeySimple();
   TestCountSimple();
   TestInnerProductSimple();
+  TestTransformReduceAndScanSimple();
+  TestRemoveSimple();
   TestSortSimple();
   TestSortByKeySimple();
   TestReduceByKeySimple();

@@ -83,14 +83,20 @@ def c5(impl, n):
 
 
 def c6(impl, n):
-    """Callers on either side of the path: count_if, inner_product, scan_by_key (integer
-    values, so every association order gives the same bits)."""
+    """Callers on either side of the path: count_if, inner_product, transform_reduce, the
+    transform scans and scan_by_key (integer values, so every association order gives the
+    same bits)."""
     x = datagen.c1_int32(n)
     y = datagen.c2_uint32(n).view(np.int32)
     out = {
         "c6.count_if_lt500": np.array([impl.count_if(x, LT, 500)], np.uint64),
         "c6.inner_product_i32_init11": np.array([impl.inner_product(x, y, init=11)], np.int32),
     }
+    NEGATE, SQUARE, MAX = 1, 2, 2
+    out["c6.transform_reduce_square_i32_init3"] = np.array([impl.transform_reduce(y, SQUARE, init=3)], np.int32)
+    out["c6.transform_reduce_negate_max_i32"] = np.array([impl.transform_reduce(x, NEGATE, MAX, init=-2000)], np.int32)
+    out["c6.transform_inclusive_scan_negate_i32"] = impl.transform_inclusive_scan(x, NEGATE)
+    out["c6.transform_exclusive_scan_square_i32_init5"] = impl.transform_exclusive_scan(y, SQUARE, init=5)
     for mean in (8, 1000):
         k, v = datagen.c4_segments(n, mean)
         iv = (v * 1000).astype(np.int32)

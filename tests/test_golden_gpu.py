@@ -74,6 +74,15 @@ class DeviceImpl:
     def inner_product(self, a, b, init=0):
         return self.dev.inner_product(self._d(a), self._d(b), init=init).numpy()[0]
 
+    def transform_reduce(self, x, unary, op=0, init=0):
+        return self.dev.transform_reduce(self._d(x), unary, op=op, init=init).numpy()[0]
+
+    def transform_inclusive_scan(self, x, unary, op=0):
+        return self.dev.transform_inclusive_scan(self._d(x), unary, op=op).numpy()
+
+    def transform_exclusive_scan(self, x, unary, init=0, op=0):
+        return self.dev.transform_exclusive_scan(self._d(x), unary, init=init, op=op).numpy()
+
     def inclusive_scan_by_key(self, k, v, op=0):
         return self.dev.inclusive_scan_by_key(self._d(k), self._d(v), op=op).numpy()
 

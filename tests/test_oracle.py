@@ -91,6 +91,19 @@ def test_known_scan_by_key_count_inner_product(oracle):
         assert oracle.inner_product(np.array(c["a"], I32), np.array(c["b"], I32), init=c["init"]) == c["out"]
 
 
+def test_known_transform_reduce_and_scans(oracle):
+    un = {"identity": cpu.IDENTITY, "negate": cpu.NEGATE, "square": cpu.SQUARE}
+    ops = {"plus": cpu.PLUS, "min": cpu.MIN, "max": cpu.MAX}
+    for c in KA["transform_reduce"]:
+        assert oracle.transform_reduce(np.array(c["in"], I32), un[c["unary"]], ops[c["op"]], c["init"]) == c["out"]
+    for c in KA["transform_inclusive_scan"]:
+        got = oracle.transform_inclusive_scan(np.array(c["in"], I32), un[c["unary"]], ops[c["op"]])
+        assert got.tolist() == c["out"]
+    for c in KA["transform_exclusive_scan"]:
+        got = oracle.transform_exclusive_scan(np.array(c["in"], I32), un[c["unary"]], c["init"], ops[c["op"]])
+        assert got.tolist() == c["out"]
+
+
 def test_known_merges(oracle):
     for c in KA["merge"]:
         assert oracle.merge(np.array(c["a"], I32), np.array(c["b"], I32)).tolist() == c["out"]
@@ -145,6 +158,13 @@ def test_oracle_matches_live_reference_on_ragged_sizes(oracle, oracle_seq):
             assert _bytes_equal(a[0], b[0]) and np.array_equal(a[1], b[1]), (dt, n)
             a, b = oracle.sort_pairs(kk, v, True), omp.sort_pairs(kk, v, True)
             assert _bytes_equal(a[0], b[0]) and np.array_equal(a[1], b[1]), (dt, n)
+        for dt in (np.int8, np.uint16, np.int32, np.uint64, np.float32, np.float64):
+            t = ((datagen.splitmix64(15, n) % np.uint64(200)).astype(np.int64) - 100).astype(dt)
+            for un in (cpu.NEGATE, cpu.SQUARE):
+                for op in (cpu.PLUS, cpu.MIN, cpu.MAX):
+                    assert _bytes_equal(oracle.transform_reduce(t, un, op, 3), omp.transform_reduce(t, un, op, 3)), (dt, n)
+                    assert _bytes_equal(oracle.transform_inclusive_scan(t, un, op), cpp.transform_inclusive_scan(t, un, op))
+                    assert _bytes_equal(oracle.transform_exclusive_scan(t, un, 3, op), omp.transform_exclusive_scan(t, un, 3, op))
         keys = np.sort((datagen.splitmix64(7, n) % np.uint64(50)).astype(np.int32))
         vals = datagen.u01(9, n)
         a, b = oracle.reduce_by_key(keys, vals), omp.reduce_by_key(keys, vals)
@@ -276,5 +296,20 @@ def test_scan_by_key_count_inner_product_against_numpy(oracle):
         exact = (sum(int(p) * int(q) for p, q in zip(a[:2000].tolist(), b[:2000].tolist())) + 3) % (1 << bits)
         got = int(oracle.inner_product(a[:2000], b[:2000], init=3)) % (1 << bits)
         assert got == exact, dtype
+    # transform_reduce / transform scans: negate and square against numpy, modulo 2^bits
+    for dtype in (np.int8, np.uint16, np.int32, np.uint64):
+        bits = 8 * np.dtype(dtype).itemsize
+        a = (datagen.splitmix64(4, 3000) >> np.uint64(9)).astype(dtype)
+        ints = [int(v) for v in a]
+        assert (int(oracle.transform_reduce(a, cpu.SQUARE, init=1)) - (sum(v * v for v in ints) + 1)) % (1 << bits) == 0
+        assert (int(oracle.transform_reduce(a, cpu.NEGATE, init=1)) - (1 - sum(ints))) % (1 << bits) == 0
+        sq = np.cumsum(np.array([(v * v) % (1 << bits) for v in ints], dtype=object))
+        got = oracle.transform_inclusive_scan(a, cpu.SQUARE)
+        assert all((int(g) - int(e)) % (1 << bits) == 0 for g, e in zip(got[::97], sq[::97]))
+        ex = oracle.transform_exclusive_scan(a, cpu.NEGATE, init=7)
+        assert int(ex[0]) % (1 << bits) == 7 and (int(ex[-1]) - (7 - sum(ints[:-1]))) % (1 << bits) == 0
+    g = datagen.u01(8, 5000) - 0.5
+    assert np.array_equal(oracle.transform_inclusive_scan(g, cpu.NEGATE, cpu.MAX), np.maximum.accumulate(-g))
+    assert oracle.transform_reduce(g, cpu.SQUARE, cpu.MIN, init=9.0) == np.min(g * g)
     f = datagen.u01(7, n)
     assert abs(float(oracle.inner_product(f, f, init=1.0)) - (float(np.dot(f.astype(np.float64), f)) + 1.0)) < 1e-3 * n * 1e-4

@@ -69,6 +69,25 @@ def test_copy_if_stencil(dev, oracle, item, sdtype):
         assert cnt == ref.size and np.array_equal(out.numpy(cnt), ref)
 
 
+@pytest.mark.parametrize("dtype", [np.float32, np.uint8, np.uint64])
+def test_copy_if_in_place(dev, oracle, dtype):
+    """out aliases in, the form remove_if uses (thrust/system/cuda/detail/remove.h:54-66): a
+    tile is written only after every earlier tile has been read."""
+    thr = 0.5 if np.dtype(dtype).kind == "f" else 100
+    for n in [1, 777, 16384, 16385, 70001, (1 << 22) + 11]:
+        x = _vals(n, dtype, 17)
+        for cmp in (dev.GE, dev.LT):
+            d = dev.DeviceArray.from_numpy(x)
+            _, cnt = dev.copy_if(d, cmp, thr, out=d)
+            ref = oracle.copy_if(x, cmp, thr)
+            assert cnt == ref.size and np.array_equal(d.numpy()[:cnt], ref), (dtype, n, cmp)
+        st = _vals(n, np.int32, 19)
+        d, ds = dev.DeviceArray.from_numpy(x), dev.DeviceArray.from_numpy(st)
+        _, cnt = dev.copy_if(d, dev.EQ, 0, stencil=ds, out=d)
+        ref = oracle.copy_if(x, dev.EQ, 0, stencil=st)
+        assert cnt == ref.size and np.array_equal(d.numpy()[:cnt], ref), (dtype, n, "stencil")
+
+
 def test_copy_if_unaligned(dev, oracle):
     x = _vals(40003, np.float32, 13)
     d = dev.DeviceArray.from_numpy(x)

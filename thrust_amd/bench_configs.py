@@ -10,8 +10,9 @@ with the algorithmic bytes of the call and the resulting fraction of the 8 TB/s 
   C4  reduce_by_key and unique_by_key over 2^28 (int32 key, float32 value), mean run 8 / 1000
   C5  copy_if and stable_partition of 2^28 float32 at 50 % / 5 % selectivity,
       merge and merge_by_key of two sorted ranges of 2^27 uint32 (+ uint32 values)
-  C6  callers on either side of the path: count_if and inner_product over 2^28 int32 /
-      float32, inclusive and exclusive scan_by_key over 2^28 (int32 key, float32 value)
+  C6  callers on either side of the path: count_if, inner_product, transform_reduce and
+      the transform scans over 2^28 int32 / float32, inclusive and exclusive scan_by_key
+      over 2^28 (int32 key, float32 value)
 
 Inputs are generated on the device from a seeded generator.  Usage:
   python3 thrust_amd/bench_configs.py [c2] [c3] [c4] [c5] [c6]
@@ -137,7 +138,14 @@ def main():
         f2 = torch.rand(n, device="cuda", generator=g)
         d1, d2, t2, out1 = dev(f1, capi.F32), dev(f2, capi.F32), capi.Temp(), capi.DeviceArray(1, capi.F32)
         run("C6 inner_product f32", lambda: capi.inner_product(d1, d2, init=0.0, temp=t2, out=out1), 8 * n)
-        del x, dx, f1, f2, d1, d2, t, t2
+        t3, t4, so, so_i = capi.Temp(), capi.Temp(), capi.DeviceArray(n, capi.F32), capi.DeviceArray(n, capi.I32)
+        run("C6 transform_reduce f32 square, plus",
+            lambda: capi.transform_reduce(d1, capi.SQUARE, init=0.0, temp=t3, out=out1), 4 * n)
+        run("C6 transform_inclusive_scan f32 negate, plus",
+            lambda: capi.transform_inclusive_scan(d1, capi.NEGATE, out=so, temp=t4), 8 * n)
+        run("C6 transform_exclusive_scan i32 square, plus",
+            lambda: capi.transform_exclusive_scan(dx, capi.SQUARE, init=3, out=so_i, temp=t4), 8 * n)
+        del x, dx, f1, f2, d1, d2, t, t2, t3, t4, so, so_i
         mean = 8
         nseg = int(n / mean * 1.2) + 1000
         u = torch.rand(nseg, device="cuda", generator=g, dtype=torch.float64).clamp_(1e-12, 1.0)

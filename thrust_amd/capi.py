@@ -26,6 +26,7 @@ DTYPE_NAMES = {I8: "i8", U8: "u8", I16: "i16", U16: "u16", I32: "i32", U32: "u32
 PLUS, MIN, MAX = range(3)
 # thrust_amd_cmp
 LT, LE, GT, GE, EQ, NE, NONZERO = range(7)
+IDENTITY, NEGATE, SQUARE = range(3)
 H2D, D2H, D2D = 1, 2, 3
 
 _c = ctypes
@@ -49,10 +50,13 @@ SIGNATURES = {
     "thrust_amd_profile_enable": (_int, [_int]),
     "thrust_amd_profile_collect": (_int, [_c.c_char_p, _sz, _szp]),
     "thrust_amd_reduce": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp, _vp, _vp]),
+    "thrust_amd_transform_reduce": (_int, [_vp, _szp, _vp, _u64, _int, _int, _int, _vp, _vp, _vp]),
     "thrust_amd_count_if": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp, _vp, _vp]),
     "thrust_amd_inner_product": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _vp, _vp, _vp]),
     "thrust_amd_inclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _vp]),
     "thrust_amd_exclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _vp, _vp]),
+    "thrust_amd_transform_inclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _int, _vp]),
+    "thrust_amd_transform_exclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _int, _vp, _vp]),
     "thrust_amd_inclusive_scan_by_key": (_int, [_vp, _szp, _vp, _vp, _vp, _u64, _int, _int, _int, _vp]),
     "thrust_amd_exclusive_scan_by_key": (_int, [_vp, _szp, _vp, _vp, _vp, _u64, _int, _int, _int, _vp, _vp]),
     "thrust_amd_sort_keys": (_int, [_vp, _szp, _vp, _u64, _int, _int, _int, _int, _vp]),
@@ -199,6 +203,14 @@ def reduce(x, op=PLUS, init=0, temp=None, out=None):
     return out
 
 
+def transform_reduce(x, unary, op=PLUS, init=0, temp=None, out=None):
+    out = out or DeviceArray(1, x.dtype)
+    iv = _scalar(x.dtype, init)
+    _run("thrust_amd_transform_reduce", temp, lambda fn, t, b: fn(
+        t, b, x.ptr, x.n, x.dtype, unary, op, iv.ctypes.data, out.ptr, stream_ptr()))
+    return out
+
+
 def count_if(x, cmp, threshold=0, temp=None):
     num = DeviceArray(1, U64)
     tv = _scalar(x.dtype, threshold)
@@ -227,6 +239,21 @@ def exclusive_scan(x, init=0, out=None, op=PLUS, temp=None):
     iv = _scalar(x.dtype, init)
     _run("thrust_amd_exclusive_scan", temp, lambda fn, t, b: fn(
         t, b, x.ptr, out.ptr, x.n, x.dtype, op, iv.ctypes.data, stream_ptr()))
+    return out
+
+
+def transform_inclusive_scan(x, unary, out=None, op=PLUS, temp=None):
+    out = out or DeviceArray(x.n, x.dtype)
+    _run("thrust_amd_transform_inclusive_scan", temp, lambda fn, t, b: fn(
+        t, b, x.ptr, out.ptr, x.n, x.dtype, unary, op, stream_ptr()))
+    return out
+
+
+def transform_exclusive_scan(x, unary, init=0, out=None, op=PLUS, temp=None):
+    out = out or DeviceArray(x.n, x.dtype)
+    iv = _scalar(x.dtype, init)
+    _run("thrust_amd_transform_exclusive_scan", temp, lambda fn, t, b: fn(
+        t, b, x.ptr, out.ptr, x.n, x.dtype, unary, op, iv.ctypes.data, stream_ptr()))
     return out
 
 

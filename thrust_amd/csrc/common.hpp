@@ -109,6 +109,46 @@ struct OpPlus {
   }
 };
 
+// a * b in T; integers multiply on the unsigned representation (wraps, no overflow UB).
+template <typename T>
+TA_DEVICE T mul_wrap(T a, T b) {
+  if constexpr (std::is_integral<T>::value && sizeof(T) < 4) {
+    // 8- and 16-bit products are made in a 32-bit register of their own; the empty asm
+    // keeps them from being packed into byte vectors, which this compiler cannot select
+    uint32_t p = (uint32_t)(int32_t)a * (uint32_t)(int32_t)b;
+    asm volatile("" : "+v"(p));
+    return (T)p;
+  } else if constexpr (std::is_integral<T>::value) {
+    using U = typename std::make_unsigned<T>::type;
+    return (T)(U)((U)a * (U)b);
+  } else {
+    return a * b;
+  }
+}
+
+// Unary transforms of the transform_* entry points: thrust::identity, thrust::negate and
+// thrust::square (thrust/functional.h:523-600, 1224-1240).  Integers negate and square on
+// the unsigned representation (wrap modulo 2^bits).
+struct UnIdentity {
+  template <typename T>
+  TA_DEVICE T operator()(T x) const { return x; }
+};
+struct UnNegate {
+  template <typename T>
+  TA_DEVICE T operator()(T x) const {
+    if constexpr (std::is_integral<T>::value) {
+      using U = typename std::make_unsigned<T>::type;
+      return (T)(U)((U)0 - (U)x);
+    } else {
+      return -x;
+    }
+  }
+};
+struct UnSquare {
+  template <typename T>
+  TA_DEVICE T operator()(T x) const { return mul_wrap(x, x); }
+};
+
 template <typename T> struct Limits;
 #define TA_LIMITS(T, LO, HI)                                   \
   template <> struct Limits<T> {                               \

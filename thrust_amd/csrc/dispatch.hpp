@@ -7,6 +7,7 @@ namespace ta {
 inline bool valid_dtype(int d) { return d >= 0 && d < THRUST_AMD_DTYPE_COUNT; }
 inline bool valid_binop(int o) { return o >= 0 && o < THRUST_AMD_BINOP_COUNT; }
 inline bool valid_cmp(int c) { return c >= 0 && c < THRUST_AMD_CMP_COUNT; }
+inline bool valid_unary(int u) { return u >= 0 && u < THRUST_AMD_UNARY_COUNT; }
 inline bool valid_item_bytes(size_t b) { return b == 1 || b == 2 || b == 4 || b == 8; }
 
 template <typename T> struct TypeTag { using type = T; };
@@ -47,6 +48,16 @@ inline int with_binop(int op, F&& f) {
     case THRUST_AMD_PLUS: return f(OpPlus{});
     case THRUST_AMD_MIN: return f(OpMin{});
     case THRUST_AMD_MAX: return f(OpMax{});
+    default: return (int)hipErrorInvalidValue;
+  }
+}
+
+// The transforms other than the identity (callers route the identity to the plain kernels).
+template <typename F>
+inline int with_transform(int unary, F&& f) {
+  switch (unary) {
+    case THRUST_AMD_NEGATE: return f(UnNegate{});
+    case THRUST_AMD_SQUARE: return f(UnSquare{});
     default: return (int)hipErrorInvalidValue;
   }
 }

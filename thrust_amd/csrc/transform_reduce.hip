@@ -1,14 +1,17 @@
-// thrust_amd_count_if / thrust_amd_inner_product: reductions of a value computed on the
-// fly from one or two input streams, with the two-kernel tree of thrust_amd_reduce.
+// thrust_amd_transform_reduce / thrust_amd_count_if / thrust_amd_inner_product: reductions
+// of a value computed on the fly from one or two input streams, with the two-kernel tree
+// of thrust_amd_reduce.
 //
-//   count_if       number of elements with (x CMP threshold), as a 64-bit count
-//   inner_product  init + sum of a[i] * b[i], products and sums in the element type
-//                  (integers wrap modulo 2^bits)
+//   transform_reduce  init OP f(x[0]) OP ... with f one of identity / negate / square
+//   count_if          number of elements with (x CMP threshold), as a 64-bit count
+//   inner_product     init + sum of a[i] * b[i], products and sums in the element type
+//                     (integers wrap modulo 2^bits)
 //
-// The reference builds both on transform_reduce: count_if maps each element to 0/1 of
-// the difference type and adds (thrust/system/detail/generic/count.inl:45-67), and
-// inner_product multiplies with multiplies<T> and adds with plus<T>, T being the type of
-// init (thrust/system/detail/generic/inner_product.inl:33-72); on the device both end in
+// The reference builds the other two on transform_reduce (reduce over a transform
+// iterator, thrust/system/detail/generic/transform_reduce.inl:30-48): count_if maps each
+// element to 0/1 of the difference type and adds (thrust/system/detail/generic/count.inl:45-67),
+// and inner_product multiplies with multiplies<T> and adds with plus<T>, T being the type of
+// init (thrust/system/detail/generic/inner_product.inl:33-72); on the device all three end in
 // reduce_n (thrust/system/cuda/detail/transform_reduce.h, inner_product.h).
 //
 // HBM traffic: every input element is read once; a few KB of partials are written.
@@ -18,23 +21,6 @@
 #include "reduce_common.hpp"
 
 namespace ta {
-
-// a * b in T; integers multiply on the unsigned representation (wraps, no overflow UB).
-template <typename T>
-TA_DEVICE T mul_wrap(T a, T b) {
-  if constexpr (std::is_integral<T>::value && sizeof(T) < 4) {
-    // 8- and 16-bit products are made in a 32-bit register of their own; the empty asm
-    // keeps them from being packed into byte vectors, which this compiler cannot select
-    uint32_t p = (uint32_t)(int32_t)a * (uint32_t)(int32_t)b;
-    asm volatile("" : "+v"(p));
-    return (T)p;
-  } else if constexpr (std::is_integral<T>::value) {
-    using U = typename std::make_unsigned<T>::type;
-    return (T)(U)((U)a * (U)b);
-  } else {
-    return a * b;
-  }
-}
 
 // The comparison is a template parameter: one kernel per (type, comparison), so that the
 // inner loop is a single compare and add.
@@ -81,6 +67,39 @@ __global__ __launch_bounds__(REDUCE_BLOCK) void count_if_partials_kernel(const T
   if (threadIdx.x == 0) partials[blockIdx.x] = r;
 }
 
+// reduce_partials_kernel of thrust_amd_reduce with `un` applied to every element first.
+template <typename T, typename Un, typename Op, bool ALIGNED>
+__global__ __launch_bounds__(REDUCE_BLOCK) void transform_reduce_partials_kernel(const T* __restrict__ in,
+                                                                                 uint64_t n,
+                                                                                 T* __restrict__ partials) {
+  constexpr int VEC = Vec16<T>::N;
+  constexpr uint64_t TILE = (uint64_t)REDUCE_BLOCK * VEC * REDUCE_UNROLL;
+  const Op op;
+  const Un un;
+  T acc = Op::template identity<T>();
+  const uint64_t full_tiles = n / TILE;
+  for (uint64_t tile = blockIdx.x; tile < full_tiles; tile += gridDim.x) {
+    const T* base = in + tile * TILE + (uint64_t)threadIdx.x * VEC;
+    Vec16<T> x[REDUCE_UNROLL];
+#pragma unroll
+    for (int u = 0; u < REDUCE_UNROLL; ++u)
+      x[u] = load_vec<ALIGNED>(base + (uint64_t)u * REDUCE_BLOCK * VEC);
+#pragma unroll
+    for (int u = 0; u < REDUCE_UNROLL; ++u) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) acc = op(acc, un(x[u].v[i]));
+    }
+  }
+  const uint64_t tail_begin = full_tiles * TILE;
+  for (uint64_t i = tail_begin + (uint64_t)blockIdx.x * REDUCE_BLOCK + threadIdx.x; i < n;
+       i += (uint64_t)gridDim.x * REDUCE_BLOCK)
+    acc = op(acc, un(in[i]));
+
+  __shared__ T lds[REDUCE_BLOCK / WAVE];
+  const T r = block_reduce<REDUCE_BLOCK>(acc, op, lds);
+  if (threadIdx.x == 0) partials[blockIdx.x] = r;
+}
+
 template <typename T, bool ALIGNED>
 __global__ __launch_bounds__(REDUCE_BLOCK) void inner_product_partials_kernel(const T* __restrict__ a,
                                                                               const T* __restrict__ b,
@@ -121,6 +140,48 @@ static size_t transform_reduce_temp(size_t elem) {
 }
 
 }  // namespace ta
+
+TA_EXPORT int thrust_amd_transform_reduce(void* temp, size_t* temp_bytes, const void* in, uint64_t n,
+                                          int dtype, int unary, int op, const void* init,
+                                          void* d_out, void* stream_v) {
+  using namespace ta;
+  if (!temp_bytes || !valid_dtype(dtype) || !valid_unary(unary) || !valid_binop(op))
+    return (int)hipErrorInvalidValue;
+  if (unary == THRUST_AMD_IDENTITY)
+    return thrust_amd_reduce(temp, temp_bytes, in, n, dtype, op, init, d_out, stream_v);
+  const size_t need = transform_reduce_temp(thrust_amd_dtype_size(dtype));
+  if (temp == nullptr) {
+    *temp_bytes = need;
+    return 0;
+  }
+  if (*temp_bytes < need || !init || !d_out || (n && !in)) return (int)hipErrorInvalidValue;
+  hipStream_t stream = (hipStream_t)stream_v;
+  return with_dtype(dtype, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    return with_transform(unary, [&](auto un) {
+      using Un = decltype(un);
+      return with_binop(op, [&](auto o) {
+        using Op = decltype(o);
+        T init_v;
+        __builtin_memcpy(&init_v, init, sizeof(T));
+        T* partials = static_cast<T*>(temp);
+        uint32_t grid = 0;
+        if (n) {
+          grid = reduce_grid(n, sizeof(T));
+          const T* src = static_cast<const T*>(in);
+          if (is_aligned16(in))
+            TA_LAUNCH("transform_reduce_partials", stream, (transform_reduce_partials_kernel<T, Un, Op, true>), dim3(grid), dim3(REDUCE_BLOCK), src, n, partials);
+          else
+            TA_LAUNCH("transform_reduce_partials", stream, (transform_reduce_partials_kernel<T, Un, Op, false>), dim3(grid), dim3(REDUCE_BLOCK), src, n, partials);
+          TA_CHECK_LAUNCH();
+        }
+        TA_LAUNCH("reduce_final", stream, (reduce_final_kernel<T, Op>), dim3(1), dim3(REDUCE_BLOCK), (const T*)partials, grid, init_v, static_cast<T*>(d_out));
+        TA_CHECK_LAUNCH();
+        return 0;
+      });
+    });
+  });
+}
 
 TA_EXPORT int thrust_amd_count_if(void* temp, size_t* temp_bytes, const void* in, uint64_t n, int dtype,
                                   int cmp, const void* threshold, uint64_t* d_count, void* stream_v) {
