@@ -110,7 +110,8 @@ inline int negated_cmp(int cmp) {
   }
 }
 template <typename Tested, typename Pred, typename Call>
-inline uint64_t run_selection(void* stream, const Pred& pred, const char* what, Call call, bool negate = false) {
+inline uint64_t run_selection(void* stream, const temp_source& source, const Pred& pred, const char* what, Call call,
+                              bool negate = false) {
   static_assert(is_abi_type<Tested>::value,
                 "selection on the device system needs an arithmetic type to test");
   static_assert(unary_pred<Pred, Tested>::supported,
@@ -118,7 +119,7 @@ inline uint64_t run_selection(void* stream, const Pred& pred, const char* what, 
                 "thrust::identity and thrust::logical_not as predicate");
   const int cmp = negate ? negated_cmp(unary_pred<Pred, Tested>::cmp(pred)) : unary_pred<Pred, Tested>::cmp(pred);
   const Tested thr = unary_pred<Pred, Tested>::threshold(pred);
-  temp_storage temp(stream);
+  temp_storage temp(stream, source);
   std::size_t need = 0;
   uint64_t* d_num = nullptr;
   throw_on_error(call((void*)nullptr, &need, d_num, cmp, (const void*)&thr), what);
@@ -139,7 +140,7 @@ Out copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred)
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  const uint64_t cnt = detail::run_selection<T>(stream, pred, "copy_if failed",
+  const uint64_t cnt = detail::run_selection<T>(stream, detail::temp_source_of(exec), pred, "copy_if failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
         return thrust_amd_copy_if(t, b, thrust::detail::raw(first), nullptr, thrust::detail::raw(result), d_num, n,
                                   sizeof(T), detail::dtype_of<T>::value, cmp, thr, stream);
@@ -155,7 +156,7 @@ Out copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  const uint64_t cnt = detail::run_selection<S>(stream, pred, "copy_if failed",
+  const uint64_t cnt = detail::run_selection<S>(stream, detail::temp_source_of(exec), pred, "copy_if failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
         return thrust_amd_copy_if(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil),
                                   thrust::detail::raw(result), d_num, n, sizeof(T), detail::dtype_of<S>::value, cmp,

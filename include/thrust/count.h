@@ -54,7 +54,7 @@ std::ptrdiff_t count_if(execution_policy<D>& exec, It first, It last, Pred pred)
   if (n == 0) return 0;
   const V threshold = detail::unary_pred<Pred, V>::threshold(pred);
   const int cmp = detail::unary_pred<Pred, V>::cmp(pred);
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   uint64_t* d_count = nullptr;
   std::size_t need = 0;
   auto call = [&](void* t, std::size_t* b) {

@@ -8,6 +8,8 @@
 //   - the system's overload taking hip::execution_policy<Derived>& or
 //     cpp::execution_policy<Derived>&, a nearer base than execution_policy_base.
 #pragma once
+#include <cstddef>
+
 #include <thrust/detail/config.h>
 
 namespace thrust {
@@ -53,6 +55,22 @@ struct execution_policy : thrust::execution_policy<Derived> {};
 struct tag : execution_policy<tag> {};
 template <typename Derived>
 inline void* get_stream(const execution_policy<Derived>&) { return nullptr; }
+
+// get_temp_source(policy) says where an algorithm's temporary storage comes from: the
+// library's arena (all members null, the default) or an allocator the caller attached
+// with par(alloc) (the reference: thrust/detail/allocator_aware_execution_policy.h:37-100
+// and temporary_array, thrust/detail/temporary_array.h).
+namespace detail {
+struct temp_source {
+  void* ctx;
+  void* (*acquire)(void* ctx, std::size_t bytes);
+  void (*release)(void* ctx, void* p, std::size_t bytes);
+};
+}  // namespace detail
+template <typename Derived>
+inline detail::temp_source get_temp_source(const execution_policy<Derived>&) {
+  return detail::temp_source{nullptr, nullptr, nullptr};
+}
 }  // namespace hip
 }  // namespace system
 

@@ -1,5 +1,9 @@
-// thrust::host, thrust::device, thrust::seq, thrust::hip::par, par.on(stream).
+// thrust::host, thrust::device, thrust::seq, thrust::hip::par, par.on(stream), par(alloc),
+// par(alloc).on(stream).
 #pragma once
+#include <cstddef>
+#include <utility>
+
 #include <thrust/detail/execution_policy.h>
 
 namespace thrust {
@@ -23,9 +27,50 @@ struct stream_policy : execution_policy<stream_policy> {
 };
 inline void* get_stream(const stream_policy& p) { return p.stream; }
 
+// Policy carrying a user allocator for temporary storage: thrust::hip::par(alloc), optionally
+// .on(stream).  Every algorithm then takes its scratch memory from alloc.allocate(n) (n in
+// units of Alloc::value_type; the result may be a raw device pointer or a device_ptr) and
+// returns it with alloc.deallocate(p, n) before it returns -- the contract of the
+// reference's examples/cuda/custom_temporary_allocation.cu:44-140.  The allocator is held
+// by reference and must outlive the call.
+template <typename Alloc>
+struct allocator_policy : execution_policy<allocator_policy<Alloc> > {
+  Alloc* alloc;
+  void* stream;
+  explicit allocator_policy(Alloc& a, void* s = nullptr) : alloc(&a), stream(s) {}
+  allocator_policy on(void* s) const { return allocator_policy(*alloc, s); }
+};
+template <typename Alloc>
+inline void* get_stream(const allocator_policy<Alloc>& p) { return p.stream; }
+
+namespace detail {
+template <typename Alloc>
+struct allocator_thunks {
+  typedef typename Alloc::value_type value_type;
+  typedef decltype(std::declval<Alloc&>().allocate(std::size_t())) pointer;
+  static std::size_t count(std::size_t bytes) { return (bytes + sizeof(value_type) - 1) / sizeof(value_type); }
+  static value_type* to_raw(value_type* p) { return p; }
+  template <typename P>
+  static value_type* to_raw(const P& p) { return p.get(); }
+  static void* acquire(void* ctx, std::size_t bytes) {
+    return to_raw(static_cast<Alloc*>(ctx)->allocate(count(bytes)));
+  }
+  static void release(void* ctx, void* p, std::size_t bytes) {
+    static_cast<Alloc*>(ctx)->deallocate(pointer(static_cast<value_type*>(p)), count(bytes));
+  }
+};
+}  // namespace detail
+template <typename Alloc>
+inline detail::temp_source get_temp_source(const allocator_policy<Alloc>& p) {
+  return detail::temp_source{p.alloc, &detail::allocator_thunks<Alloc>::acquire,
+                             &detail::allocator_thunks<Alloc>::release};
+}
+
 struct par_t : execution_policy<par_t> {
   // `stream` is a hipStream_t; it is taken as void* so that user code needs no HIP headers.
   stream_policy on(void* stream) const { return stream_policy(stream); }
+  template <typename Alloc>
+  allocator_policy<Alloc> operator()(Alloc& alloc) const { return allocator_policy<Alloc>(alloc); }
 };
 static const par_t par;
 
@@ -34,6 +79,10 @@ namespace detail {
 template <typename Derived>
 inline void* stream_of(execution_policy<Derived>& p) {
   return get_stream(thrust::detail::derived_cast(p));
+}
+template <typename Derived>
+inline temp_source temp_source_of(execution_policy<Derived>& p) {
+  return get_temp_source(thrust::detail::derived_cast(p));
 }
 }  // namespace detail
 

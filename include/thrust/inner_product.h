@@ -50,7 +50,7 @@ T inner_product(execution_policy<D>& exec, It1 first1, It1 last1, It2 first2, T 
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last1 - first1);
   if (n == 0) return init;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   void* d_out = nullptr;
   std::size_t need = 0;
   auto call = [&](void* t, std::size_t* b) {

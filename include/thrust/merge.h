@@ -73,7 +73,7 @@ Out merge(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last
   void* stream = detail::stream_of(exec);
   const uint64_t na = (uint64_t)(last1 - first1), nb = (uint64_t)(last2 - first2);
   if (na + nb == 0) return result;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "merge failed", [&](void* t, std::size_t* b) {
     return thrust_amd_merge(t, b, na ? thrust::detail::raw(first1) : nullptr, na,
                             nb ? thrust::detail::raw(first2) : nullptr, nb, thrust::detail::raw(result),
@@ -100,7 +100,7 @@ pair<KOut, VOut> merge_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2,
   void* stream = detail::stream_of(exec);
   const uint64_t na = (uint64_t)(kl1 - kf1), nb = (uint64_t)(kl2 - kf2);
   if (na + nb == 0) return thrust::make_pair(ko, vo);
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "merge_by_key failed", [&](void* t, std::size_t* b) {
     return thrust_amd_merge_by_key(t, b, na ? thrust::detail::raw(kf1) : nullptr, na,
                                    nb ? thrust::detail::raw(kf2) : nullptr, nb,

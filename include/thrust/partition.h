@@ -54,7 +54,7 @@ It stable_partition(execution_policy<D>& exec, It first, It last, Pred pred) {
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return first;
-  const uint64_t cnt = detail::run_selection<T>(stream, pred, "stable_partition failed",
+  const uint64_t cnt = detail::run_selection<T>(stream, detail::temp_source_of(exec), pred, "stable_partition failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
         return thrust_amd_stable_partition(t, b, thrust::detail::raw(first), nullptr, d_num, n, sizeof(T),
                                            detail::dtype_of<T>::value, cmp, thr, stream);
@@ -70,7 +70,7 @@ It stable_partition(execution_policy<D>& exec, It first, It last, St stencil, Pr
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return first;
-  const uint64_t cnt = detail::run_selection<S>(stream, pred, "stable_partition failed",
+  const uint64_t cnt = detail::run_selection<S>(stream, detail::temp_source_of(exec), pred, "stable_partition failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
         return thrust_amd_stable_partition(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil), d_num, n,
                                            sizeof(T), detail::dtype_of<S>::value, cmp, thr, stream);
@@ -88,7 +88,7 @@ pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In l
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return thrust::make_pair(out_true, out_false);
-  const uint64_t cnt = detail::run_selection<T>(stream, pred, "partition_copy failed",
+  const uint64_t cnt = detail::run_selection<T>(stream, detail::temp_source_of(exec), pred, "partition_copy failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
         return thrust_amd_partition_copy(t, b, thrust::detail::raw(first), nullptr, thrust::detail::raw(out_true),
                                          thrust::detail::raw(out_false), d_num, n, sizeof(T),
@@ -108,7 +108,7 @@ pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In l
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return thrust::make_pair(out_true, out_false);
-  const uint64_t cnt = detail::run_selection<S>(stream, pred, "partition_copy failed",
+  const uint64_t cnt = detail::run_selection<S>(stream, detail::temp_source_of(exec), pred, "partition_copy failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
         return thrust_amd_partition_copy(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil),
                                          thrust::detail::raw(out_true), thrust::detail::raw(out_false), d_num, n,

@@ -102,7 +102,7 @@ T reduce(execution_policy<D>& exec, It first, It last, T init, Op) {
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   const void* in = n ? (const void*)thrust::detail::raw(first) : nullptr;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   void* d_out = nullptr;
   // the result slot is the `extra` region, which run() only knows after the size query
   std::size_t need = 0;
@@ -135,7 +135,7 @@ pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n == 0) return thrust::make_pair(ko, vo);
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   uint64_t* d_runs = nullptr;
   std::size_t need = 0;
   auto call = [&](void* t, std::size_t* b) {

@@ -72,7 +72,7 @@ Out remove_copy_if(execution_policy<D>& exec, In first, In last, Out result, Pre
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  const uint64_t cnt = detail::run_selection<T>(stream, pred, "remove_copy_if failed",
+  const uint64_t cnt = detail::run_selection<T>(stream, detail::temp_source_of(exec), pred, "remove_copy_if failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
         return thrust_amd_copy_if(t, b, thrust::detail::raw(first), nullptr, thrust::detail::raw(result), d_num, n,
                                   sizeof(T), detail::dtype_of<T>::value, cmp, thr, stream);
@@ -88,7 +88,7 @@ Out remove_copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  const uint64_t cnt = detail::run_selection<S>(stream, pred, "remove_copy_if failed",
+  const uint64_t cnt = detail::run_selection<S>(stream, detail::temp_source_of(exec), pred, "remove_copy_if failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
         return thrust_amd_copy_if(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil),
                                   thrust::detail::raw(result), d_num, n, sizeof(T), detail::dtype_of<S>::value, cmp,

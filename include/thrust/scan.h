@@ -173,7 +173,7 @@ Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op)
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "inclusive_scan failed", [&](void* t, std::size_t* b) {
     return thrust_amd_inclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
                                      detail::dtype_of<V>::value, detail::binop_code<Op, V>::value, stream);
@@ -189,7 +189,7 @@ Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T i
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "exclusive_scan failed", [&](void* t, std::size_t* b) {
     return thrust_amd_exclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
                                      detail::dtype_of<V>::value, detail::binop_code<Op, V>::value, &init, stream);
@@ -225,7 +225,7 @@ Out inclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n == 0) return result;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "inclusive_scan_by_key failed", [&](void* t, std::size_t* b) {
     return thrust_amd_inclusive_scan_by_key(t, b, thrust::detail::raw(kf), thrust::detail::raw(vf),
                                             thrust::detail::raw(result), n, detail::dtype_of<K>::value,
@@ -247,14 +247,14 @@ Out exclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out
   void* out = thrust::detail::raw(result);
   // the device entry point reads values[i-1] while other tiles write: an in-place call
   // scans from a copy of the values
-  detail::temp_storage copy(stream);
+  detail::temp_storage copy(stream, detail::temp_source_of(exec));
   if (values == out) {
     copy.ensure(n * sizeof(V));
     detail::throw_on_error(thrust_amd_memcpy(copy.ptr(), values, n * sizeof(V), THRUST_AMD_D2D, stream),
                            "exclusive_scan_by_key: copy of the values");
     values = copy.ptr();
   }
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "exclusive_scan_by_key failed", [&](void* t, std::size_t* b) {
     return thrust_amd_exclusive_scan_by_key(t, b, thrust::detail::raw(kf), values, out, n,
                                             detail::dtype_of<K>::value, detail::dtype_of<V>::value,

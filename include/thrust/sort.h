@@ -88,7 +88,7 @@ void stable_sort(execution_policy<D>& exec, It first, It last, Comp) {
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n < 2) return;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "sort failed", [&](void* t, std::size_t* b) {
     return thrust_amd_sort_keys(t, b, thrust::detail::raw(first), n, detail::dtype_of<K>::value,
                                 detail::order_code<Comp, K>::value, 0, (int)sizeof(K) * 8, stream);
@@ -106,7 +106,7 @@ void stable_sort_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Comp)
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n < 2) return;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "sort_by_key failed", [&](void* t, std::size_t* b) {
     return thrust_amd_sort_pairs(t, b, thrust::detail::raw(kf), thrust::detail::raw(vf), n,
                                  detail::dtype_of<K>::value, sizeof(V), detail::order_code<Comp, K>::value, 0,

@@ -97,17 +97,35 @@ struct unary_pred<thrust::logical_not<I>, T> {
   static T threshold(const thrust::logical_not<I>&) { return T(0); }
 };
 
-// ---- temp storage from the arena, returned when the scope ends
+// ---- temp storage, returned when the scope ends: from the library's arena, or from the
+// allocator of a par(alloc) policy.  A user allocator may hand out memory of any
+// alignment, so 256 more bytes are requested and the pointer is rounded up; its memory
+// goes back only after the stream has drained (the arena's release is stream-ordered).
 class temp_storage {
  public:
-  temp_storage(void* stream) : ptr_(nullptr), stream_(stream), bytes_(0) {}
+  temp_storage(void* stream, const temp_source& source)
+      : ptr_(nullptr), raw_(nullptr), stream_(stream), bytes_(0), raw_bytes_(0), source_(source) {}
   ~temp_storage() {
-    if (ptr_) (void)thrust_amd_temp_release(ptr_, stream_);
+    if (!raw_) return;
+    if (source_.acquire) {
+      (void)thrust_amd_stream_synchronize(stream_);
+      source_.release(source_.ctx, raw_, raw_bytes_);
+    } else {
+      (void)thrust_amd_temp_release(raw_, stream_);
+    }
   }
   void ensure(std::size_t bytes) {
     bytes_ = bytes;
-    const int rc = thrust_amd_temp_acquire(&ptr_, bytes ? bytes : 1, stream_);
+    if (source_.acquire) {
+      raw_bytes_ = (bytes ? bytes : 1) + 256;
+      raw_ = source_.acquire(source_.ctx, raw_bytes_);
+      if (!raw_) throw thrust::system::detail::bad_alloc("the policy's allocator returned a null pointer");
+      ptr_ = reinterpret_cast<void*>((reinterpret_cast<std::uintptr_t>(raw_) + 255) / 256 * 256);
+      return;
+    }
+    const int rc = thrust_amd_temp_acquire(&raw_, bytes ? bytes : 1, stream_);
     if (rc != 0) throw thrust::system::detail::bad_alloc(thrust_amd_error_string(rc));
+    ptr_ = raw_;
   }
   void* ptr() const { return ptr_; }
   std::size_t* bytes() { return &bytes_; }
@@ -116,8 +134,10 @@ class temp_storage {
   temp_storage(const temp_storage&);
   temp_storage& operator=(const temp_storage&);
   void* ptr_;
+  void* raw_;
   void* stream_;
-  std::size_t bytes_;
+  std::size_t bytes_, raw_bytes_;
+  temp_source source_;
 };
 
 // Size query, allocation from the arena with `extra` more bytes at the end (for device

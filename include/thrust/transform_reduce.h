@@ -38,7 +38,7 @@ T transform_reduce(execution_policy<D>& exec, It first, It last, Fn, T init, Op)
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   const void* in = n ? (const void*)thrust::detail::raw(first) : nullptr;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   void* d_out = nullptr;
   std::size_t need = 0;
   auto call = [&](void* t, std::size_t* b) {

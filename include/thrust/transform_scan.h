@@ -73,7 +73,7 @@ Out transform_inclusive_scan(execution_policy<D>& exec, In first, In last, Out r
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "transform_inclusive_scan failed", [&](void* t, std::size_t* b) {
     return thrust_amd_transform_inclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
                                                detail::dtype_of<V>::value, detail::unary_code<Fn, V>::value,
@@ -90,7 +90,7 @@ Out transform_exclusive_scan(execution_policy<D>& exec, In first, In last, Out r
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "transform_exclusive_scan failed", [&](void* t, std::size_t* b) {
     return thrust_amd_transform_exclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
                                                detail::dtype_of<V>::value, detail::unary_code<Fn, V>::value,

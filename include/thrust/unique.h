@@ -92,7 +92,7 @@ Out unique_copy(execution_policy<D>& exec, In first, In last, Out result, Pred) 
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   uint64_t* d_num = nullptr;
   auto call = [&](void* t, std::size_t* b) {
     return thrust_amd_unique(t, b, thrust::detail::raw(first), thrust::detail::raw(result), d_num, n,
@@ -119,7 +119,7 @@ pair<KOut, VOut> unique_by_key_copy(execution_policy<D>& exec, KIn kf, KIn kl, V
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n == 0) return thrust::make_pair(ko, vo);
-  detail::temp_storage temp(stream);
+  detail::temp_storage temp(stream, detail::temp_source_of(exec));
   uint64_t* d_num = nullptr;
   auto call = [&](void* t, std::size_t* b) {
     return thrust_amd_unique_by_key(t, b, thrust::detail::raw(kf), thrust::detail::raw(vf), thrust::detail::raw(ko),

@@ -6,6 +6,9 @@
 // reference's size list, results compared exactly (testing/unittest/testframework.cu:21-31,
 // e.g. testing/reduce.cu:80-95).  Part 3 covers policies, streams, dispatch interception,
 // the memory model and error reporting.
+#include <map>
+#include <stdexcept>
+
 #include <thrust/copy.h>
 #include <thrust/count.h>
 #include <thrust/device_vector.h>
@@ -661,6 +664,110 @@ static void TestTempArenaReuse() {
   ASSERT_TRUE(thrust_amd_temp_bytes_held() == 0);
 }
 
+// A block cache in the role of the reference's examples/cuda/custom_temporary_allocation.cu:
+// freed blocks are kept by size and handed out again.  `skew` shifts every pointer it returns,
+// to show that the library does not rely on the allocator's alignment.
+struct CachingTempAllocator {
+  typedef char value_type;
+  std::multimap<std::ptrdiff_t, char*> free_blocks;
+  std::map<char*, std::ptrdiff_t> live;
+  int fresh = 0, reused = 0, returned = 0;
+  std::ptrdiff_t skew = 0;
+  char* allocate(std::ptrdiff_t n) {
+    char* block = nullptr;
+    auto hit = free_blocks.find(n);
+    if (hit != free_blocks.end()) {
+      block = hit->second;
+      free_blocks.erase(hit);
+      ++reused;
+    } else {
+      block = thrust::device_malloc<char>((std::size_t)(n + skew)).get();
+      ++fresh;
+    }
+    live[block + skew] = n;
+    return block + skew;
+  }
+  void deallocate(char* p, std::size_t n) {
+    auto it = live.find(p);
+    if (it == live.end() || it->second != (std::ptrdiff_t)n) throw std::runtime_error("not a live block of this allocator");
+    live.erase(it);
+    free_blocks.insert(std::make_pair((std::ptrdiff_t)n, p - skew));
+    ++returned;
+  }
+  ~CachingTempAllocator() {
+    for (auto& b : free_blocks) thrust::device_free(thrust::device_pointer_cast(b.second));
+  }
+};
+
+// The same interface handing out device_ptr<char>, as an allocator built on thrust::device_malloc would.
+struct FancyPointerAllocator {
+  typedef char value_type;
+  int calls = 0;
+  thrust::device_ptr<char> allocate(std::size_t n) { ++calls; return thrust::device_malloc<char>(n); }
+  void deallocate(thrust::device_ptr<char> p, std::size_t) { --calls; thrust::device_free(p); }
+};
+
+struct FailingAllocator {
+  typedef char value_type;
+  char* allocate(std::size_t) { throw std::bad_alloc(); }
+  void deallocate(char*, std::size_t) {}
+};
+
+static void TestCustomTemporaryAllocation() {  // examples/cuda/custom_temporary_allocation.cu:142-186
+  g_test = "CustomTemporaryAllocation";
+  const size_t n = 1 << 16;
+  thrust::host_vector<int> h = random_integers<int>(n, 3, 0);
+  thrust::host_vector<int> sorted = h;
+  thrust::sort(sorted.begin(), sorted.end());
+  for (std::ptrdiff_t skew : {0, 8}) {
+    CachingTempAllocator alloc;
+    alloc.skew = skew;
+    ASSERT_TRUE(thrust_amd_temp_trim() == 0);
+    for (int round = 0; round < 3; ++round) {
+      thrust::device_vector<int> d = h;
+      thrust::sort(thrust::hip::par(alloc), d.begin(), d.end());
+      ASSERT_EQUAL_VEC(to_host(d), sorted);
+    }
+    ASSERT_TRUE(alloc.fresh == 1 && alloc.reused == 2 && alloc.returned == 3 && alloc.live.empty());
+    ASSERT_TRUE(thrust_amd_temp_bytes_held() == 0);  // the library's own arena was not touched
+    // other algorithms through the same policy, also bound to a stream
+    thrust::device_vector<int> d = h, out(n);
+    long long total = 0;
+    for (size_t i = 0; i < n; ++i) total += h[i];
+    ASSERT_TRUE(thrust::reduce(thrust::hip::par(alloc).on(nullptr), d.begin(), d.end(), 0) == (int)total);
+    thrust::inclusive_scan(thrust::hip::par(alloc), d.begin(), d.end(), out.begin());
+    thrust::host_vector<int> hs(n);
+    thrust::inclusive_scan(h.begin(), h.end(), hs.begin());
+    ASSERT_EQUAL_VEC(to_host(out), hs);
+    thrust::host_vector<int> hc(n);
+    hc.resize(thrust::copy_if(h.begin(), h.end(), hc.begin(), _1 < 1000) - hc.begin());
+    out.resize(thrust::copy_if(thrust::hip::par(alloc), d.begin(), d.end(), out.begin(), _1 < 1000) - out.begin());
+    ASSERT_EQUAL_VEC(to_host(out), hc);
+    thrust::device_vector<int> keys = h, vals(n, 1), ko(n), vo(n);
+    thrust::sort_by_key(thrust::hip::par(alloc), keys.begin(), keys.end(), vals.begin());
+    auto ends = thrust::reduce_by_key(thrust::hip::par(alloc), keys.begin(), keys.end(), vals.begin(), ko.begin(), vo.begin());
+    ASSERT_TRUE(thrust::reduce(thrust::hip::par(alloc), vo.begin(), ends.second, 0) == (int)n);
+    ASSERT_TRUE(alloc.live.empty() && alloc.returned == alloc.fresh + alloc.reused);
+    ASSERT_TRUE(thrust_amd_temp_bytes_held() == 0);
+  }
+  FancyPointerAllocator fancy;
+  thrust::device_vector<int> d = h;
+  thrust::sort(thrust::hip::par(fancy), d.begin(), d.end());
+  ASSERT_EQUAL_VEC(to_host(d), sorted);
+  ASSERT_TRUE(fancy.calls == 0);
+  // an allocator that throws: the exception reaches the caller and the data is untouched
+  FailingAllocator failing;
+  d = h;
+  bool threw = false;
+  try {
+    thrust::sort(thrust::hip::par(failing), d.begin(), d.end());
+  } catch (const std::bad_alloc&) {
+    threw = true;
+  }
+  ASSERT_TRUE(threw);
+  ASSERT_EQUAL_VEC(to_host(d), h);
+}
+
 int main() {
   TestReduceSimple();
   TestReduceWithOperatorTable();
@@ -693,6 +800,7 @@ int main() {
   TestDeviceVector();
   TestOutOfMemoryThrows();
   TestTempArenaReuse();
+  TestCustomTemporaryAllocation();
   std::printf("%s: %d checks, %d failed\n", g_failed ? "FAILED" : "PASSED", g_checks, g_failed);
   return g_failed ? 1 : 0;
 }
