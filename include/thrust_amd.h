@@ -83,6 +83,16 @@ typedef enum thrust_amd_unary {
   THRUST_AMD_UNARY_COUNT = 3
 } thrust_amd_unary;
 
+/* The four set operations on sorted ranges (multiset semantics,
+ * thrust/system/detail/sequential/set_operations.h:42-215). */
+typedef enum thrust_amd_set_op {
+  THRUST_AMD_SET_DIFFERENCE = 0,
+  THRUST_AMD_SET_INTERSECTION = 1,
+  THRUST_AMD_SET_SYMMETRIC_DIFFERENCE = 2,
+  THRUST_AMD_SET_UNION = 3,
+  THRUST_AMD_SET_OP_COUNT = 4
+} thrust_amd_set_op;
+
 typedef enum thrust_amd_memcpy_kind {
   THRUST_AMD_H2D = 1,
   THRUST_AMD_D2H = 2,
@@ -246,6 +256,32 @@ int thrust_amd_sort_keys(void* temp, size_t* temp_bytes, void* keys, uint64_t n,
 int thrust_amd_sort_pairs(void* temp, size_t* temp_bytes, void* keys, void* values, uint64_t n,
                           int key_dtype, size_t value_bytes, int descending, int begin_bit,
                           int end_bit, void* stream);
+
+/* ---------------------------------------------------------- set operations */
+
+/* out = a OP b for two ranges sorted by operator< (descending != 0: by operator>), OP a
+ * thrust_amd_set_op code.  A key that occurs m times in a and n times in b appears
+ * max(m-n,0) times (difference, the last copies of a), min(m,n) times (intersection, the
+ * first copies of a), |m-n| times (symmetric difference, the last copies of the longer
+ * side) or max(m,n) times (union: all of a, then the last n-m copies of b); the result is
+ * sorted and stable.  *d_num_out (uint64 on device) receives its length; out must hold
+ * na + nb elements for union and symmetric difference, na for difference, min(na, nb) for
+ * intersection, and must not overlap a or b.  na + nb < 2^43.
+ * Replaces cuda_cub::set_difference / set_intersection / set_symmetric_difference /
+ * set_union (thrust/system/cuda/detail/set_operations.h:1480-1960). */
+int thrust_amd_set_operation(void* temp, size_t* temp_bytes, int op, const void* a, uint64_t na,
+                             const void* b, uint64_t nb, void* out, uint64_t* d_num_out, int dtype,
+                             int descending, void* stream);
+
+/* Same on keys, with one value (opaque item of value_bytes = 1, 2, 4 or 8) travelling with
+ * every kept key from the range the key came from.  values_b is read only by union and
+ * symmetric difference and may be NULL otherwise.
+ * Replaces the *_by_key forms (thrust/system/cuda/detail/set_operations.h:1480-1960). */
+int thrust_amd_set_operation_by_key(void* temp, size_t* temp_bytes, int op, const void* keys_a,
+                                    uint64_t na, const void* keys_b, uint64_t nb,
+                                    const void* values_a, const void* values_b, void* keys_out,
+                                    void* values_out, uint64_t* d_num_out, int key_dtype,
+                                    size_t value_bytes, int descending, void* stream);
 
 /* ----------------------------------------------------- selection / partition */
 

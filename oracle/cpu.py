@@ -26,6 +26,7 @@ DTYPE_OF_NP = {np.dtype(v): k for k, v in NP_DTYPES.items()}
 PLUS, MIN, MAX = range(3)
 LT, LE, GT, GE, EQ, NE, NONZERO = range(7)
 IDENTITY, NEGATE, SQUARE = range(3)
+SET_DIFFERENCE, SET_INTERSECTION, SET_SYMMETRIC_DIFFERENCE, SET_UNION = range(4)
 
 
 def build(with_ref=True):
@@ -203,6 +204,26 @@ class _Base:
         self._ok(self._fn("inner_product")(_p(a), _p(b), ctypes.c_uint64(a.size), _code(a), _p(iv),
                                             _p(out), *self._extra()), "inner_product")
         return out[0]
+
+    def set_operation(self, op, a, b, descending=False):
+        a, b = _c(a), _c(b)
+        out = np.empty(a.size + b.size, a.dtype)
+        num = ctypes.c_uint64(0)
+        self._ok(self._fn("set_operation")(op, _p(a), ctypes.c_uint64(a.size), _p(b), ctypes.c_uint64(b.size),
+                                            _p(out), ctypes.byref(num), _code(a), int(descending)),
+                 "set_operation")
+        return out[: num.value].copy()
+
+    def set_operation_by_key(self, op, ka, kb, va, vb, descending=False):
+        ka, kb, va, vb = _c(ka), _c(kb), _c(va), _c(vb)
+        ko = np.empty(ka.size + kb.size, ka.dtype)
+        vo = np.empty(ka.size + kb.size, va.dtype)
+        num = ctypes.c_uint64(0)
+        self._ok(self._fn("set_operation_by_key")(op, _p(ka), ctypes.c_uint64(ka.size), _p(kb),
+                                                   ctypes.c_uint64(kb.size), _p(va), _p(vb), _p(ko), _p(vo),
+                                                   ctypes.byref(num), _code(ka), ctypes.c_uint64(va.itemsize),
+                                                   int(descending)), "set_operation_by_key")
+        return ko[: num.value].copy(), vo[: num.value].copy()
 
     def transform_reduce(self, x, unary, op=PLUS, init=0):
         x = _c(x)

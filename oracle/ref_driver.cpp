@@ -17,6 +17,7 @@
 #include <thrust/partition.h>
 #include <thrust/reduce.h>
 #include <thrust/scan.h>
+#include <thrust/set_operations.h>
 #include <thrust/sort.h>
 #include <thrust/transform_reduce.h>
 #include <thrust/transform_scan.h>
@@ -317,6 +318,76 @@ REF_API int ref_inner_product(const void* a, const void* b, uint64_t n, int dtyp
     *(T*)out = thrust::inner_product(thrust::device, dp<T>(a), dp<T>(a) + n, dp<T>(b), *(const T*)init);
     return 0;
   });
+}
+
+namespace {
+// The real set operations; C is thrust::less<K> or thrust::greater<K>.
+template <typename K, typename C>
+uint64_t run_set_operation(int op, const void* a, uint64_t na, const void* b, uint64_t nb, void* out, C comp) {
+  auto a0 = dp<K>(a), b0 = dp<K>(b);
+  auto o0 = dp<K>(out);
+  switch (op) {
+    case THRUST_AMD_SET_DIFFERENCE: return thrust::set_difference(thrust::device, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
+    case THRUST_AMD_SET_INTERSECTION: return thrust::set_intersection(thrust::device, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
+    case THRUST_AMD_SET_SYMMETRIC_DIFFERENCE:
+      return thrust::set_symmetric_difference(thrust::device, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
+    default: return thrust::set_union(thrust::device, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
+  }
+}
+template <typename K, typename V, typename C>
+uint64_t run_set_operation_by_key(int op, const void* ka, uint64_t na, const void* kb, uint64_t nb, const void* va,
+                                  const void* vb, void* kout, void* vout, C comp) {
+  auto a0 = dp<K>(ka), b0 = dp<K>(kb);
+  auto v1 = dp<V>(va), v2 = dp<V>(vb);
+  auto ko = dp<K>(kout);
+  auto vo = dp<V>(vout);
+  switch (op) {
+    case THRUST_AMD_SET_DIFFERENCE:
+      return thrust::set_difference_by_key(thrust::device, a0, a0 + na, b0, b0 + nb, v1, v2, ko, vo, comp).first - ko;
+    case THRUST_AMD_SET_INTERSECTION:
+      return thrust::set_intersection_by_key(thrust::device, a0, a0 + na, b0, b0 + nb, v1, ko, vo, comp).first - ko;
+    case THRUST_AMD_SET_SYMMETRIC_DIFFERENCE:
+      return thrust::set_symmetric_difference_by_key(thrust::device, a0, a0 + na, b0, b0 + nb, v1, v2, ko, vo, comp).first - ko;
+    default: return thrust::set_union_by_key(thrust::device, a0, a0 + na, b0, b0 + nb, v1, v2, ko, vo, comp).first - ko;
+  }
+}
+}  // namespace
+
+REF_API int ref_set_operation(int op, const void* a, uint64_t na, const void* b, uint64_t nb, void* out,
+                              uint64_t* num, int dtype, int descending) {
+  return with_dtype(dtype, [&](auto z) {
+    using K = decltype(z);
+    *num = descending ? run_set_operation<K>(op, a, na, b, nb, out, thrust::greater<K>())
+                      : run_set_operation<K>(op, a, na, b, nb, out, thrust::less<K>());
+    return 0;
+  });
+}
+
+// Keys of the types the fixtures use; values as opaque 4- or 8-byte items.
+REF_API int ref_set_operation_by_key(int op, const void* ka, uint64_t na, const void* kb, uint64_t nb,
+                                     const void* va, const void* vb, void* kout, void* vout, uint64_t* num,
+                                     int dtype, uint64_t value_bytes, int descending) {
+  auto run = [&](auto kz, auto vz) {
+    using K = decltype(kz);
+    using V = decltype(vz);
+    *num = descending ? run_set_operation_by_key<K, V>(op, ka, na, kb, nb, va, vb, kout, vout, thrust::greater<K>())
+                      : run_set_operation_by_key<K, V>(op, ka, na, kb, nb, va, vb, kout, vout, thrust::less<K>());
+    return 0;
+  };
+  auto by_value = [&](auto kz) {
+    switch (value_bytes) {
+      case 4: return run(kz, (uint32_t)0);
+      case 8: return run(kz, (uint64_t)0);
+      default: return -1;
+    }
+  };
+  switch (dtype) {
+    case THRUST_AMD_I32: return by_value((int32_t)0);
+    case THRUST_AMD_U32: return by_value((uint32_t)0);
+    case THRUST_AMD_U64: return by_value((uint64_t)0);
+    case THRUST_AMD_F32: return by_value((float)0);
+    default: return -1;
+  }
 }
 
 namespace {

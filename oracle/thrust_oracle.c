@@ -445,6 +445,47 @@ ORACLE_API int oracle_count_if(const void* in, uint64_t n, int dtype, int cmp, c
   return 0;
 }
 
+/* The four set operations and their by-key forms; values are opaque items of value_bytes
+ * that travel with the key the reference's tuple loop emits. */
+static int set_operation_impl(int op, const void* ka, uint64_t na, const void* kb, uint64_t nb,
+                              const void* va, const void* vb, void* kout, void* vout, uint64_t* num,
+                              int dtype, uint64_t value_bytes, int descending) {
+  if (op < 0 || op >= THRUST_AMD_SET_OP_COUNT) return -1;
+  const size_t cap = (size_t)(na + nb) + 1;
+  unsigned char* side = (unsigned char*)malloc(cap);
+  size_t* idx = (size_t*)malloc(cap * sizeof(size_t));
+  size_t k = 0;
+#define BODY(S, T) \
+  k = set_operation_##S(op, (const T*)ka, (size_t)na, (const T*)kb, (size_t)nb, descending, side, idx);
+  DISPATCH(dtype, BODY)
+#undef BODY
+  const size_t kbytes = dtype_size(dtype);
+  for (size_t o = 0; o < k; o++) {
+    const char* ksrc = side[o] ? (const char*)kb : (const char*)ka;
+    memcpy((char*)kout + o * kbytes, ksrc + idx[o] * kbytes, kbytes);
+    if (vout) {
+      const char* vsrc = side[o] ? (const char*)vb : (const char*)va;
+      memcpy((char*)vout + o * value_bytes, vsrc + idx[o] * value_bytes, value_bytes);
+    }
+  }
+  free(side);
+  free(idx);
+  *num = k;
+  return 0;
+}
+
+ORACLE_API int oracle_set_operation(int op, const void* a, uint64_t na, const void* b, uint64_t nb,
+                                    void* out, uint64_t* num, int dtype, int descending) {
+  return set_operation_impl(op, a, na, b, nb, NULL, NULL, out, NULL, num, dtype, 0, descending);
+}
+
+ORACLE_API int oracle_set_operation_by_key(int op, const void* ka, uint64_t na, const void* kb,
+                                           uint64_t nb, const void* va, const void* vb, void* kout,
+                                           void* vout, uint64_t* num, int dtype, uint64_t value_bytes,
+                                           int descending) {
+  return set_operation_impl(op, ka, na, kb, nb, va, vb, kout, vout, num, dtype, value_bytes, descending);
+}
+
 /* generic::transform_reduce (generic/transform_reduce.inl:30-48): the system's reduce over
  * the transformed range; generic::transform_inclusive_scan / transform_exclusive_scan
  * (generic/transform_scan.inl:37-97): the system's scans over it. */

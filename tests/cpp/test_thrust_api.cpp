@@ -22,6 +22,7 @@
 #include <thrust/reduce.h>
 #include <thrust/remove.h>
 #include <thrust/scan.h>
+#include <thrust/set_operations.h>
 #include <thrust/sort.h>
 #include <thrust/transform_reduce.h>
 #include <thrust/transform_scan.h>
@@ -267,6 +268,74 @@ static void TestRemoveSimple() {  // testing/remove.cu:28-47,100-122,184-203,256
   thrust::host_vector<int> hst = hv<int>({0, 1, 0, 0, 1});
   h.resize(thrust::remove_if(h.begin(), h.end(), hst.begin(), thrust::identity<int>()) - h.begin());
   ASSERT_EQUAL_VEC(h, kept);
+}
+
+static void TestSetOperationsSimple() {
+  // testing/set_difference.cu:70-80, set_intersection.cu:71-81, set_symmetric_difference.cu:70-80,
+  // set_union.cu:71-106, set_union_descending.cu:7-18 and the *_by_key.cu simple tests
+  g_test = "SetOperationsSimple";
+  {
+    thrust::device_vector<int> a(hv<int>({0, 2, 4, 5})), b(hv<int>({0, 3, 3, 4, 6})), r(9);
+    r.resize(thrust::set_difference(a.begin(), a.end(), b.begin(), b.end(), r.begin()) - r.begin());
+    ASSERT_EQUAL_VEC(to_host(r), hv<int>({2, 5}));
+  }
+  {
+    thrust::device_vector<int> a(hv<int>({0, 2, 4})), b(hv<int>({0, 3, 3, 4})), r(7);
+    r.resize(thrust::set_intersection(thrust::device, a.begin(), a.end(), b.begin(), b.end(), r.begin()) - r.begin());
+    ASSERT_EQUAL_VEC(to_host(r), hv<int>({0, 4}));
+    r.resize(7);
+    r.resize(thrust::set_union(a.begin(), a.end(), b.begin(), b.end(), r.begin()) - r.begin());
+    ASSERT_EQUAL_VEC(to_host(r), hv<int>({0, 2, 3, 3, 4}));
+    thrust::host_vector<int> ha = to_host(a), hb = to_host(b), hr(7);
+    hr.resize(thrust::set_union(ha.begin(), ha.end(), hb.begin(), hb.end(), hr.begin()) - hr.begin());
+    ASSERT_EQUAL_VEC(hr, hv<int>({0, 2, 3, 3, 4}));
+  }
+  {
+    thrust::device_vector<int> a(hv<int>({0, 2, 2})), b(hv<int>({0, 2, 2, 2, 3})), r(8);
+    r.resize(thrust::set_union(a.begin(), a.end(), b.begin(), b.end(), r.begin()) - r.begin());
+    ASSERT_EQUAL_VEC(to_host(r), hv<int>({0, 2, 2, 2, 3}));
+  }
+  {
+    thrust::device_vector<int> a(hv<int>({0, 2, 4, 6})), b(hv<int>({0, 3, 3, 4, 7})), r(9);
+    r.resize(thrust::set_symmetric_difference(a.begin(), a.end(), b.begin(), b.end(), r.begin()) - r.begin());
+    ASSERT_EQUAL_VEC(to_host(r), hv<int>({2, 3, 3, 6, 7}));
+  }
+  {
+    thrust::device_vector<int> a(hv<int>({4, 2, 0})), b(hv<int>({4, 3, 3, 0})), r(7);
+    r.resize(thrust::set_union(a.begin(), a.end(), b.begin(), b.end(), r.begin(), thrust::greater<int>()) - r.begin());
+    ASSERT_EQUAL_VEC(to_host(r), hv<int>({4, 3, 3, 2, 0}));
+  }
+  {
+    thrust::device_vector<int> ak(hv<int>({0, 2, 4})), av(hv<int>({0, 0, 0}));
+    thrust::device_vector<int> bk(hv<int>({0, 3, 3, 4})), bv(hv<int>({1, 1, 1, 1})), rk(7), rv(7);
+    auto e = thrust::set_union_by_key(ak.begin(), ak.end(), bk.begin(), bk.end(), av.begin(), bv.begin(), rk.begin(), rv.begin());
+    ASSERT_TRUE(e.first - rk.begin() == 5 && e.second - rv.begin() == 5);
+    rk.resize(5); rv.resize(5);
+    ASSERT_EQUAL_VEC(to_host(rk), hv<int>({0, 2, 3, 3, 4}));
+    ASSERT_EQUAL_VEC(to_host(rv), hv<int>({0, 0, 1, 1, 0}));
+    rk.resize(7); rv.resize(7);
+    e = thrust::set_intersection_by_key(ak.begin(), ak.end(), bk.begin(), bk.end(), av.begin(), rk.begin(), rv.begin());
+    ASSERT_TRUE(e.first - rk.begin() == 2);
+    rk.resize(2); rv.resize(2);
+    ASSERT_EQUAL_VEC(to_host(rk), hv<int>({0, 4}));
+    ASSERT_EQUAL_VEC(to_host(rv), hv<int>({0, 0}));
+  }
+  {
+    thrust::device_vector<int> ak(hv<int>({6, 4, 2, 0})), av(hv<int>({0, 0, 0, 0}));
+    thrust::device_vector<int> bk(hv<int>({7, 4, 3, 3, 0})), bv(hv<int>({1, 1, 1, 1, 1})), rk(9), rv(9);
+    auto e = thrust::set_symmetric_difference_by_key(thrust::device, ak.begin(), ak.end(), bk.begin(), bk.end(), av.begin(),
+                                                     bv.begin(), rk.begin(), rv.begin(), thrust::greater<int>());
+    ASSERT_TRUE(e.first - rk.begin() == 5);
+    rk.resize(5); rv.resize(5);
+    ASSERT_EQUAL_VEC(to_host(rk), hv<int>({7, 6, 3, 3, 2}));
+    ASSERT_EQUAL_VEC(to_host(rv), hv<int>({1, 0, 1, 1, 0}));
+    rk.resize(9); rv.resize(9);
+    e = thrust::set_difference_by_key(ak.begin(), ak.end(), bk.begin(), bk.end(), av.begin(), bv.begin(), rk.begin(),
+                                      rv.begin(), thrust::greater<int>());
+    ASSERT_TRUE(e.first - rk.begin() == 2);
+    rk.resize(2);
+    ASSERT_EQUAL_VEC(to_host(rk), hv<int>({6, 2}));
+  }
 }
 
 static void TestSortSimple() {  // testing/sort.cu:43-76
@@ -537,6 +606,48 @@ static void DifferentialForType(const char* name) {
     thrust::merge(ha.begin(), ha.end(), hb.begin(), hb.end(), hr.begin());
     thrust::merge(da.begin(), da.end(), db.begin(), db.end(), dr.begin());
     ASSERT_EQUAL_VEC(to_host(dr), hr);
+    // the four set operations on the same sorted ranges (values drawn from 50 keys: long runs)
+    {
+      thrust::host_vector<T> hs(ha.size() + hb.size());
+      thrust::device_vector<T> ds(ha.size() + hb.size());
+      size_t hn = thrust::set_difference(ha.begin(), ha.end(), hb.begin(), hb.end(), hs.begin()) - hs.begin();
+      size_t dn = thrust::set_difference(da.begin(), da.end(), db.begin(), db.end(), ds.begin()) - ds.begin();
+      ASSERT_TRUE(hn == dn);
+      ASSERT_TRUE(std::equal(hs.begin(), hs.begin() + hn, to_host(ds).begin()));
+      hn = thrust::set_intersection(ha.begin(), ha.end(), hb.begin(), hb.end(), hs.begin()) - hs.begin();
+      dn = thrust::set_intersection(da.begin(), da.end(), db.begin(), db.end(), ds.begin()) - ds.begin();
+      ASSERT_TRUE(hn == dn);
+      ASSERT_TRUE(std::equal(hs.begin(), hs.begin() + hn, to_host(ds).begin()));
+      hn = thrust::set_symmetric_difference(ha.begin(), ha.end(), hb.begin(), hb.end(), hs.begin()) - hs.begin();
+      dn = thrust::set_symmetric_difference(da.begin(), da.end(), db.begin(), db.end(), ds.begin()) - ds.begin();
+      ASSERT_TRUE(hn == dn);
+      ASSERT_TRUE(std::equal(hs.begin(), hs.begin() + hn, to_host(ds).begin()));
+      hn = thrust::set_union(ha.begin(), ha.end(), hb.begin(), hb.end(), hs.begin()) - hs.begin();
+      dn = thrust::set_union(da.begin(), da.end(), db.begin(), db.end(), ds.begin()) - ds.begin();
+      ASSERT_TRUE(hn == dn);
+      ASSERT_TRUE(std::equal(hs.begin(), hs.begin() + hn, to_host(ds).begin()));
+      // by key: the values name the side and the index of every kept element
+      thrust::host_vector<int> hva(ha.size()), hvb(hb.size()), hvo(ha.size() + hb.size());
+      for (size_t i = 0; i < hva.size(); ++i) hva[i] = (int)i;
+      for (size_t i = 0; i < hvb.size(); ++i) hvb[i] = -(int)i - 1;
+      thrust::device_vector<int> dva = hva, dvb = hvb, dvo(ha.size() + hb.size());
+      auto he = thrust::set_union_by_key(ha.begin(), ha.end(), hb.begin(), hb.end(), hva.begin(), hvb.begin(), hs.begin(), hvo.begin());
+      auto de = thrust::set_union_by_key(da.begin(), da.end(), db.begin(), db.end(), dva.begin(), dvb.begin(), ds.begin(), dvo.begin());
+      ASSERT_TRUE((he.first - hs.begin()) == (de.first - ds.begin()));
+      ASSERT_TRUE(std::equal(hvo.begin(), hvo.begin() + (he.second - hvo.begin()), to_host(dvo).begin()));
+      he = thrust::set_symmetric_difference_by_key(ha.begin(), ha.end(), hb.begin(), hb.end(), hva.begin(), hvb.begin(), hs.begin(), hvo.begin());
+      de = thrust::set_symmetric_difference_by_key(da.begin(), da.end(), db.begin(), db.end(), dva.begin(), dvb.begin(), ds.begin(), dvo.begin());
+      ASSERT_TRUE((he.first - hs.begin()) == (de.first - ds.begin()));
+      ASSERT_TRUE(std::equal(hvo.begin(), hvo.begin() + (he.second - hvo.begin()), to_host(dvo).begin()));
+      he = thrust::set_intersection_by_key(ha.begin(), ha.end(), hb.begin(), hb.end(), hva.begin(), hs.begin(), hvo.begin());
+      de = thrust::set_intersection_by_key(da.begin(), da.end(), db.begin(), db.end(), dva.begin(), ds.begin(), dvo.begin());
+      ASSERT_TRUE((he.first - hs.begin()) == (de.first - ds.begin()));
+      ASSERT_TRUE(std::equal(hvo.begin(), hvo.begin() + (he.second - hvo.begin()), to_host(dvo).begin()));
+      he = thrust::set_difference_by_key(ha.begin(), ha.end(), hb.begin(), hb.end(), hva.begin(), hvb.begin(), hs.begin(), hvo.begin());
+      de = thrust::set_difference_by_key(da.begin(), da.end(), db.begin(), db.end(), dva.begin(), dvb.begin(), ds.begin(), dvo.begin());
+      ASSERT_TRUE((he.first - hs.begin()) == (de.first - ds.begin()));
+      ASSERT_TRUE(std::equal(hvo.begin(), hvo.begin() + (he.second - hvo.begin()), to_host(dvo).begin()));
+    }
   }
 }
 
@@ -777,6 +888,7 @@ int main() {
   TestInnerProductSimple();
   TestTransformReduceAndScanSimple();
   TestRemoveSimple();
+  TestSetOperationsSimple();
   TestSortSimple();
   TestSortByKeySimple();
   TestReduceByKeySimple();

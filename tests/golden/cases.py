@@ -9,8 +9,8 @@ import numpy as np
 from thrust_amd import datagen
 
 LT = 0
-SMALL = {"c1": 1 << 14, "c2": 1 << 14, "c3": 1 << 13, "c4": 1 << 15, "c5": 1 << 14, "c6": 1 << 15}
-LARGE = {"c1": 1 << 22, "c2": 1 << 22, "c3": 1 << 21, "c4": 1 << 22, "c5": 1 << 22, "c6": 1 << 22}
+SMALL = {"c1": 1 << 14, "c2": 1 << 14, "c3": 1 << 13, "c4": 1 << 15, "c5": 1 << 14, "c6": 1 << 15, "c7": 1 << 14}
+LARGE = {"c1": 1 << 22, "c2": 1 << 22, "c3": 1 << 21, "c4": 1 << 22, "c5": 1 << 22, "c6": 1 << 22, "c7": 1 << 22}
 
 
 def c1(impl, n):
@@ -105,7 +105,24 @@ def c6(impl, n):
     return out
 
 
-CASES = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5, "c6": c6}
+def c7(impl, n):
+    """The four set operations on two sorted uint32 ranges with many repeated keys, and their
+    by-key forms with the original index as value."""
+    def sorted_with_index(count, seed, distinct):
+        k = datagen.c2_uint32(count, seed) % np.uint32(distinct)
+        order = np.argsort(k, kind="stable").astype(np.uint32)
+        return k[order], order
+    ka, va = sorted_with_index(n // 2, 8, n // 8 + 1)   # runs of about four equal keys
+    kb, vb = sorted_with_index(n // 2, 9, n // 4 + 1)   # runs of about two, half the keys unmatched
+    out = {}
+    for op, name in enumerate(("difference", "intersection", "symmetric_difference", "union")):
+        out[f"c7.set_{name}"] = impl.set_operation(op, ka, kb)
+        k, v = impl.set_operation_by_key(op, ka, kb, va, vb)
+        out[f"c7.set_{name}_by_key.values"] = v
+    return out
+
+
+CASES = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5, "c6": c6, "c7": c7}
 
 
 def digest(a):

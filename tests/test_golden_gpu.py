@@ -74,6 +74,14 @@ class DeviceImpl:
     def inner_product(self, a, b, init=0):
         return self.dev.inner_product(self._d(a), self._d(b), init=init).numpy()[0]
 
+    def set_operation(self, op, a, b, descending=False):
+        out, cnt = self.dev.set_operation(op, self._d(a), self._d(b), descending)
+        return out.numpy()[:cnt]
+
+    def set_operation_by_key(self, op, ka, kb, va, vb, descending=False):
+        ko, vo, cnt = self.dev.set_operation_by_key(op, self._d(ka), self._d(kb), self._d(va), self._d(vb), descending)
+        return ko.numpy()[:cnt], vo.numpy()[:cnt]
+
     def transform_reduce(self, x, unary, op=0, init=0):
         return self.dev.transform_reduce(self._d(x), unary, op=op, init=init).numpy()[0]
 

@@ -104,6 +104,58 @@ def test_known_transform_reduce_and_scans(oracle):
         assert got.tolist() == c["out"]
 
 
+def test_known_set_operations(oracle):
+    codes = {"difference": cpu.SET_DIFFERENCE, "intersection": cpu.SET_INTERSECTION,
+             "symmetric_difference": cpu.SET_SYMMETRIC_DIFFERENCE, "union": cpu.SET_UNION}
+    for c in KA["set_operation"]:
+        got = oracle.set_operation(codes[c["op"]], np.array(c["a"], I32), np.array(c["b"], I32), c.get("descending", False))
+        assert got.tolist() == c["out"], c["source"]
+    for c in KA["set_operation_by_key"]:
+        k, v = oracle.set_operation_by_key(codes[c["op"]], np.array(c["a_keys"], I32), np.array(c["b_keys"], I32),
+                                           np.array(c["a_values"], np.uint32), np.array(c["b_values"], np.uint32),
+                                           c.get("descending", False))
+        assert k.tolist() == c["keys_out"] and v.tolist() == c["values_out"], c["source"]
+
+
+def test_set_operations_against_multiset_definition(oracle):
+    """Independent definition: with h_a, h_b the histograms of the two ranges, the result's
+    histogram is max(h_a - h_b, 0), min, |h_a - h_b| and max; the result is sorted; and the
+    by-key values name the side and the copies the two-pointer loop keeps (for a key with m
+    copies in A and n in B: A's first min(m, n) for intersection, A's last m - n for
+    difference, all of A then B's last n - m for union)."""
+    n = 20000
+    a = np.sort((datagen.splitmix64(21, n) % np.uint64(3000)).astype(np.int32))
+    b = np.sort((datagen.splitmix64(22, n // 2) % np.uint64(3000)).astype(np.int32))
+    ha, hb = np.bincount(a, minlength=3000), np.bincount(b, minlength=3000)
+    want = {cpu.SET_DIFFERENCE: np.maximum(ha - hb, 0), cpu.SET_INTERSECTION: np.minimum(ha, hb),
+            cpu.SET_SYMMETRIC_DIFFERENCE: np.abs(ha - hb), cpu.SET_UNION: np.maximum(ha, hb)}
+    va, vb = np.arange(a.size, dtype=np.uint32), np.arange(b.size, dtype=np.uint32) + np.uint32(1 << 20)
+    first_a = np.searchsorted(a, np.arange(3000))
+    first_b = np.searchsorted(b, np.arange(3000))
+    for op, hist in want.items():
+        got = oracle.set_operation(op, a, b)
+        assert np.all(got[1:] >= got[:-1]) and np.array_equal(np.bincount(got, minlength=3000), hist)
+        k, v = oracle.set_operation_by_key(op, a, b, va, vb)
+        assert np.array_equal(k, got)
+        expect = []
+        for x in range(3000):
+            m, nn = int(ha[x]), int(hb[x])
+            ia, ib = int(first_a[x]), int(first_b[x]) + (1 << 20)
+            if op == cpu.SET_INTERSECTION:
+                expect += range(ia, ia + min(m, nn))
+            elif op == cpu.SET_DIFFERENCE:
+                expect += range(ia + min(m, nn), ia + m)
+            elif op == cpu.SET_UNION:
+                expect += list(range(ia, ia + m)) + list(range(ib + min(m, nn), ib + nn))
+            else:
+                expect += list(range(ia + min(m, nn), ia + m)) + list(range(ib + min(m, nn), ib + nn))
+        assert v.tolist() == expect, op
+    # descending inputs mirror the ascending result
+    ad, bd = a[::-1].copy(), b[::-1].copy()
+    for op in want:
+        assert np.array_equal(np.bincount(oracle.set_operation(op, ad, bd, True), minlength=3000), want[op])
+
+
 def test_known_merges(oracle):
     for c in KA["merge"]:
         assert oracle.merge(np.array(c["a"], I32), np.array(c["b"], I32)).tolist() == c["out"]
@@ -165,6 +217,16 @@ def test_oracle_matches_live_reference_on_ragged_sizes(oracle, oracle_seq):
                     assert _bytes_equal(oracle.transform_reduce(t, un, op, 3), omp.transform_reduce(t, un, op, 3)), (dt, n)
                     assert _bytes_equal(oracle.transform_inclusive_scan(t, un, op), cpp.transform_inclusive_scan(t, un, op))
                     assert _bytes_equal(oracle.transform_exclusive_scan(t, un, 3, op), omp.transform_exclusive_scan(t, un, 3, op))
+        for dt in (np.int32, np.uint64, np.float32):
+            sa = np.sort((datagen.splitmix64(17, n) % np.uint64(n // 3 + 2)).astype(dt))
+            sb = np.sort((datagen.splitmix64(19, n // 2 + 1) % np.uint64(n // 3 + 2)).astype(dt))
+            wa, wb = np.arange(sa.size, dtype=np.uint32), np.arange(sb.size, dtype=np.uint32) + np.uint32(1 << 30)
+            for op in range(4):
+                assert _bytes_equal(oracle.set_operation(op, sa, sb), omp.set_operation(op, sa, sb)), (dt, n, op)
+                assert _bytes_equal(oracle.set_operation(op, sa[::-1].copy(), sb[::-1].copy(), True),
+                                    cpp.set_operation(op, sa[::-1].copy(), sb[::-1].copy(), True)), (dt, n, op)
+                x, y = oracle.set_operation_by_key(op, sa, sb, wa, wb), omp.set_operation_by_key(op, sa, sb, wa, wb)
+                assert _bytes_equal(x[0], y[0]) and np.array_equal(x[1], y[1]), (dt, n, op)
         keys = np.sort((datagen.splitmix64(7, n) % np.uint64(50)).astype(np.int32))
         vals = datagen.u01(9, n)
         a, b = oracle.reduce_by_key(keys, vals), omp.reduce_by_key(keys, vals)

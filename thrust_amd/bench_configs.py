@@ -14,8 +14,11 @@ with the algorithmic bytes of the call and the resulting fraction of the 8 TB/s 
       the transform scans over 2^28 int32 / float32, inclusive and exclusive scan_by_key
       over 2^28 (int32 key, float32 value)
 
+  C7  the four set operations on two sorted ranges of 2^27 uint32 with runs of about four
+      and two equal keys (bytes: both inputs read, the result written)
+
 Inputs are generated on the device from a seeded generator.  Usage:
-  python3 thrust_amd/bench_configs.py [c2] [c3] [c4] [c5] [c6]
+  python3 thrust_amd/bench_configs.py [c2] [c3] [c4] [c5] [c6] [c7]
 """
 import os
 import sys
@@ -34,7 +37,7 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench_configs.py needs a GPU")
     capi.load()
-    which = [a.lower() for a in sys.argv[1:]] or ["c2", "c3", "c4", "c5", "c6"]
+    which = [a.lower() for a in sys.argv[1:]] or ["c2", "c3", "c4", "c5", "c6", "c7"]
     g = torch.Generator(device="cuda")
     g.manual_seed(1)
 
@@ -156,6 +159,26 @@ def main():
         run("C6 inclusive_scan_by_key mean run 8", lambda: capi.inclusive_scan_by_key(dk, dv, out=vo, temp=t), 12 * n)
         run("C6 exclusive_scan_by_key mean run 8",
             lambda: capi.exclusive_scan_by_key(dk, dv, init=0.0, out=vo, temp=t), 12 * n)
+    if "c7" in which:
+        m = 1 << 27
+
+        def sorted_keys(distinct):
+            r = torch.randint(0, distinct, (m,), dtype=torch.int32, device="cuda", generator=g)
+            return torch.sort(r)[0]
+        ka, kb = sorted_keys(m // 4), sorted_keys(m // 2)
+        da, db = dev(ka, capi.U32), dev(kb, capi.U32)
+        out, t = capi.DeviceArray(2 * m, capi.U32), capi.Temp()
+        names = ("set_difference", "set_intersection", "set_symmetric_difference", "set_union")
+        for op, name in enumerate(names):
+            _, cnt = capi.set_operation(op, da, db, out=out, temp=t)
+            run(f"C7 {name} 2 x 2^27 u32", lambda: capi.set_operation(op, da, db, out=out, temp=t),
+                4 * (2 * m + cnt), extra=f"{cnt} out")
+        va = torch.arange(m, dtype=torch.int32, device="cuda")
+        dva, dvb, vo, t2 = dev(va, capi.U32), dev(va + m, capi.U32), capi.DeviceArray(2 * m, capi.U32), capi.Temp()
+        _, _, cnt = capi.set_operation_by_key(3, da, db, dva, dvb, keys_out=out, values_out=vo, temp=t2)
+        run("C7 set_union_by_key 2 x 2^27 u32+u32",
+            lambda: capi.set_operation_by_key(3, da, db, dva, dvb, keys_out=out, values_out=vo, temp=t2),
+            4 * (2 * m + cnt) + 8 * cnt, extra=f"{cnt} out")
 
 
 if __name__ == "__main__":

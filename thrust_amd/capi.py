@@ -27,6 +27,7 @@ PLUS, MIN, MAX = range(3)
 # thrust_amd_cmp
 LT, LE, GT, GE, EQ, NE, NONZERO = range(7)
 IDENTITY, NEGATE, SQUARE = range(3)
+SET_DIFFERENCE, SET_INTERSECTION, SET_SYMMETRIC_DIFFERENCE, SET_UNION = range(4)
 H2D, D2H, D2D = 1, 2, 3
 
 _c = ctypes
@@ -59,6 +60,9 @@ SIGNATURES = {
     "thrust_amd_transform_exclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _int, _vp, _vp]),
     "thrust_amd_inclusive_scan_by_key": (_int, [_vp, _szp, _vp, _vp, _vp, _u64, _int, _int, _int, _vp]),
     "thrust_amd_exclusive_scan_by_key": (_int, [_vp, _szp, _vp, _vp, _vp, _u64, _int, _int, _int, _vp, _vp]),
+    "thrust_amd_set_operation": (_int, [_vp, _szp, _int, _vp, _u64, _vp, _u64, _vp, _vp, _int, _int, _vp]),
+    "thrust_amd_set_operation_by_key": (_int, [_vp, _szp, _int, _vp, _u64, _vp, _u64, _vp, _vp, _vp, _vp, _vp,
+                                               _int, _sz, _int, _vp]),
     "thrust_amd_sort_keys": (_int, [_vp, _szp, _vp, _u64, _int, _int, _int, _int, _vp]),
     "thrust_amd_sort_pairs": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _sz, _int, _int, _int, _vp]),
     "thrust_amd_copy_if": (_int, [_vp, _szp, _vp, _vp, _vp, _vp, _u64, _sz, _int, _int, _vp, _vp]),
@@ -355,6 +359,25 @@ def merge(a, b_, descending=False, out=None, temp=None):
     _run("thrust_amd_merge", temp, lambda fn, t, b: fn(
         t, b, a.ptr, a.n, b_.ptr, b_.n, out.ptr, a.dtype, int(descending), stream_ptr()))
     return out
+
+
+def set_operation(op, a, b_, descending=False, out=None, temp=None):
+    """Returns (out, length); out holds a.n + b.n elements unless the caller passes one."""
+    out = out or DeviceArray(a.n + b_.n, a.dtype)
+    num = DeviceArray(1, U64)
+    _run("thrust_amd_set_operation", temp, lambda fn, t, b: fn(
+        t, b, op, a.ptr, a.n, b_.ptr, b_.n, out.ptr, num.ptr, a.dtype, int(descending), stream_ptr()))
+    return out, _count(num)
+
+
+def set_operation_by_key(op, ka, kb, va, vb, descending=False, temp=None, keys_out=None, values_out=None):
+    keys_out = keys_out or DeviceArray(ka.n + kb.n, ka.dtype)
+    values_out = values_out or DeviceArray(ka.n + kb.n, va.dtype)
+    num = DeviceArray(1, U64)
+    _run("thrust_amd_set_operation_by_key", temp, lambda fn, t, b: fn(
+        t, b, op, ka.ptr, ka.n, kb.ptr, kb.n, va.ptr, vb.ptr if vb is not None else None, keys_out.ptr,
+        values_out.ptr, num.ptr, ka.dtype, va.itemsize, int(descending), stream_ptr()))
+    return keys_out, values_out, _count(num)
 
 
 def merge_by_key(ka, kb, va, vb, descending=False, temp=None, keys_out=None, values_out=None):
