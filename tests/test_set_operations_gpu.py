@@ -66,14 +66,17 @@ def test_set_operation_descending(dev, oracle, op):
 
 @pytest.mark.parametrize("op", OPS)
 def test_set_operation_long_runs_across_tiles(dev, oracle, op):
-    """Runs of equal keys much longer than a tile (4096 merged elements), in one range, in
-    both, and ending exactly on tile borders."""
+    """Runs of equal keys much longer than a tile (8192 merged elements for 4-byte keys), in
+    one range, in both, and ending exactly on tile borders."""
     shapes = [
         (np.zeros(20000, np.int32), np.zeros(9000, np.int32)),
         (np.zeros(9000, np.int32), np.zeros(20000, np.int32)),
         (np.repeat(np.arange(4, dtype=np.int32), 4096), np.repeat(np.arange(4, dtype=np.int32), 4096)),
         (np.repeat(np.arange(3, dtype=np.int32), [5000, 1, 7000]), np.repeat(np.arange(1, 4, dtype=np.int32), [3000, 6000, 2])),
         (np.r_[np.zeros(4096, np.int32), np.ones(100, np.int32)], np.r_[np.ones(4096, np.int32), np.full(3, 2, np.int32)]),
+        (np.repeat(np.arange(4, dtype=np.int32), 8192), np.repeat(np.arange(4, dtype=np.int32), 8192)),
+        (np.r_[np.zeros(8192, np.int32), np.ones(100, np.int32)], np.r_[np.ones(8192, np.int32), np.full(3, 2, np.int32)]),
+        (np.repeat(np.arange(3, dtype=np.int32), [30000, 1, 17000]), np.repeat(np.arange(1, 4, dtype=np.int32), [9000, 26000, 2])),
         (np.arange(12288, dtype=np.int32), np.arange(12288, dtype=np.int32)),
         (np.arange(0, 24576, 2, dtype=np.int32), np.arange(1, 24576, 2, dtype=np.int32)),
     ]

@@ -35,10 +35,16 @@
 
 namespace ta {
 
-constexpr int SET_BLOCK = 256;
+// Tile = BLOCK threads x 16 merged elements each.  Tiles take dynamic tickets (a same-address
+// atomic retires about every 12 ns) and chain their counts, so they are made as large as
+// LDS allows: 16384 elements for keys and values of up to 4 bytes, 8192 for 8-byte items.
 constexpr int SET_ITEMS = 16;
-constexpr int SET_TILE = SET_BLOCK * SET_ITEMS;
-constexpr int SET_WAVES = SET_BLOCK / WAVE;
+template <typename T, typename V, bool HAS_VALUES>
+struct SetShape {
+  static constexpr size_t ITEM = (HAS_VALUES && sizeof(V) > sizeof(T)) ? sizeof(V) : sizeof(T);
+  static constexpr int BLOCK = ITEM > 4 ? 256 : 512;
+  static constexpr int TILE = BLOCK * SET_ITEMS;
+};
 
 template <typename T>
 TA_DEVICE bool set_comp(const T& x, const T& y, bool descending) {
@@ -81,13 +87,14 @@ TA_DEVICE uint64_t set_upper_bound(const T* p, uint64_t n, T x, bool descending)
 }
 
 // Per tile boundary t (t = 0 .. tiles): split[t] = elements of A before merged position
-// t * TILE; for boundaries inside the merged order, key[t] = the element at that position
+// t * tile_size; for boundaries inside the merged order, key[t] = the element at that position
 // and run[3t .. 3t+2] = merged positions where its run starts, where the run's B part
 // starts, and where the run ends.
 template <typename T>
 __global__ __launch_bounds__(256) void set_partition_kernel(const T* __restrict__ a, uint64_t na,
                                                             const T* __restrict__ b, uint64_t nb,
-                                                            uint64_t tiles, int descending_i,
+                                                            uint64_t tiles, uint32_t tile_size,
+                                                            int descending_i,
                                                             uint64_t* __restrict__ split,
                                                             uint64_t* __restrict__ run,
                                                             T* __restrict__ key) {
@@ -95,7 +102,7 @@ __global__ __launch_bounds__(256) void set_partition_kernel(const T* __restrict_
   if (t > tiles) return;
   const bool descending = descending_i != 0;
   const uint64_t total = na + nb;
-  uint64_t diag = t * SET_TILE;
+  uint64_t diag = t * tile_size;
   if (diag > total) diag = total;
   const uint64_t as = set_merge_path<T>(a, na, b, nb, diag, descending);
   split[t] = as;
@@ -134,9 +141,9 @@ struct OpMaxPair {
   }
 };
 
-// Fold of the values of all threads before this one (`id` for thread 0), 256 threads.
-// `buf` holds SET_WAVES values; the caller separates uses of it with a barrier.
-template <typename V, typename Op>
+// Fold of the values of all threads before this one (`id` for thread 0) in a workgroup of
+// WAVES waves.  `buf` holds WAVES values; the caller separates uses of it with a barrier.
+template <int WAVES, typename V, typename Op>
 TA_DEVICE V set_block_exclusive(V v, Op op, V id, V* buf, V* total) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const V incl = wave_inclusive_scan(v, op, id);
@@ -144,7 +151,7 @@ TA_DEVICE V set_block_exclusive(V v, Op op, V id, V* buf, V* total) {
   __syncthreads();
   V prefix = id, all = id;
 #pragma unroll
-  for (int w = 0; w < SET_WAVES; ++w) {
+  for (int w = 0; w < WAVES; ++w) {
     if (w == wave) prefix = all;
     all = op(all, buf[w]);
   }
@@ -174,9 +181,16 @@ struct SetArgs {
 };
 
 template <typename T, typename V, bool HAS_VALUES>
-__global__ __launch_bounds__(SET_BLOCK) void set_op_kernel(SetArgs<T, V, HAS_VALUES> g) {
-  __shared__ __attribute__((aligned(16))) T s_keys[SET_TILE + 1];
-  __shared__ uint16_t s_src[SET_TILE];
+__global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), 4) void set_op_kernel(SetArgs<T, V, HAS_VALUES> g) {
+  using Shape = SetShape<T, V, HAS_VALUES>;
+  constexpr int SET_BLOCK = Shape::BLOCK;
+  constexpr int SET_TILE = Shape::TILE;
+  constexpr int SET_WAVES = SET_BLOCK / WAVE;
+  // one buffer for the staged keys, the compacted keys and (later) the staged values
+  __shared__ __attribute__((aligned(16))) unsigned char s_raw[(size_t)(SET_TILE + 1) * Shape::ITEM];
+  T* s_keys = reinterpret_cast<T*>(s_raw);
+  V* s_vals = reinterpret_cast<V*>(s_raw);
+  __shared__ uint16_t s_src[HAS_VALUES ? SET_TILE : 1];
   __shared__ T s_edge_key[SET_BLOCK];
   __shared__ uint8_t s_edge_b[SET_BLOCK];
   __shared__ uint64_t s_pair[SET_BLOCK];
@@ -197,17 +211,29 @@ __global__ __launch_bounds__(SET_BLOCK) void set_op_kernel(SetArgs<T, V, HAS_VAL
   const uint32_t ca = (uint32_t)(a1 - a0), cb = (uint32_t)(b1 - b0);
   const uint32_t count = ca + cb;  // == d1 - d0, 1 .. SET_TILE
 
-  // the run the tile starts in, and the run the next tile starts in
+  // The run the tile starts in, and the run the next tile starts in (the only runs that can
+  // reach outside the tile).  With rs / rm / re the merged positions where such a run
+  // starts, where its B part starts and where it ends, its element at merged position P
+  // has rank P - rs >= (re - rm) [A] or P - rm >= (rm - rs) [B] exactly when its tile-local
+  // position is at or past a threshold that is the same for the whole tile.
   const T f0_key = g.key[tile];
-  const uint64_t f0_start = g.run[3 * tile], f0_mid = g.run[3 * tile + 1], f0_end = g.run[3 * tile + 2];
   const bool f1_valid = d1 < total;
-  T f1_key = f0_key;
-  uint64_t f1_start = 0, f1_mid = 0, f1_end = 0;
+  const T f1_key = f1_valid ? g.key[tile + 1] : f0_key;
+  auto local_threshold = [&](uint64_t global_pos) -> uint32_t {
+    if (global_pos <= d0) return 0u;
+    const uint64_t rel = global_pos - d0;
+    return rel > (uint64_t)SET_TILE ? (uint32_t)SET_TILE + 1u : (uint32_t)rel;
+  };
+  uint32_t thr_a0, thr_b0, thr_a1 = 0, thr_b1 = 0;
+  {
+    const uint64_t rs = g.run[3 * tile], rm = g.run[3 * tile + 1], re = g.run[3 * tile + 2];
+    thr_a0 = local_threshold(rs + (re - rm));
+    thr_b0 = local_threshold(rm + (rm - rs));
+  }
   if (f1_valid) {
-    f1_key = g.key[tile + 1];
-    f1_start = g.run[3 * (tile + 1)];
-    f1_mid = g.run[3 * (tile + 1) + 1];
-    f1_end = g.run[3 * (tile + 1) + 2];
+    const uint64_t rs = g.run[3 * (tile + 1)], rm = g.run[3 * (tile + 1) + 1], re = g.run[3 * (tile + 1) + 2];
+    thr_a1 = local_threshold(rs + (re - rm));
+    thr_b1 = local_threshold(rm + (rm - rs));
   }
 
   // ---- stage the keys: A's part first, then B's
@@ -251,122 +277,115 @@ __global__ __launch_bounds__(SET_BLOCK) void set_op_kernel(SetArgs<T, V, HAS_VAL
   // valid elements of this lane: merged positions run0 + o < count
   const uint32_t live = (run0 >= count) ? 0u : ((count - run0 >= (uint32_t)SET_ITEMS) ? 0xffffu : ((1u << (count - run0)) - 1u));
 
-  // ---- head flags on the merged order: bit o set when element o starts a run (local
-  // position 0 and every position past the end count as starts); e2: first B of a run
+  // does the tile's last run go on in the next tile?  (the last merged key is the later of
+  // the two parts' last keys; only its equivalence class matters)
+  bool tail_continues = false;
+  if (f1_valid) {
+    const T last_a = s_keys[ca ? ca - 1 : 0], last_b = s_keys[count - 1];
+    const T last = (cb == 0) ? last_a : (ca == 0) ? last_b : (set_comp(last_b, last_a, descending) ? last_a : last_b);
+    tail_continues = !set_comp(last, f1_key, descending);
+  }
+
+  // ---- head flags on the merged order: bit o set when valid element o starts a run (local
+  // position 0 counts as a start); e2: first B of a run
   s_edge_key[threadIdx.x] = k[SET_ITEMS - 1];
   s_edge_b[threadIdx.x] = (uint8_t)((is_b >> (SET_ITEMS - 1)) & 1u);
   __syncthreads();
-  uint32_t head = 0, e2 = 0;
+  uint32_t head = 0;
   {
     T prev = (threadIdx.x > 0) ? s_edge_key[threadIdx.x - 1] : k[0];
-    bool prev_b = (threadIdx.x > 0) ? (s_edge_b[threadIdx.x - 1] != 0) : false;
 #pragma unroll
     for (int o = 0; o < SET_ITEMS; ++o) {
-      const bool valid = (live >> o) & 1u;
-      bool h = set_comp(prev, k[o], descending);
-      if ((threadIdx.x == 0 && o == 0) || !valid) h = true;
-      const bool bo = (is_b >> o) & 1u;
-      const bool first_b = valid && bo && (h || !prev_b);
-      head |= (uint32_t)h << o;
-      e2 |= (uint32_t)first_b << o;
+      head |= (uint32_t)set_comp(prev, k[o], descending) << o;
       prev = k[o];
-      prev_b = bo;
     }
+    if (threadIdx.x == 0) head |= 1u;
+    head &= live;
   }
+  // first B of a run: a B whose predecessor is an A, or that starts a run
+  const uint32_t prev_b_bits = (is_b << 1) | ((threadIdx.x > 0) ? (uint32_t)s_edge_b[threadIdx.x - 1] : 0u);
+  const uint32_t e2 = is_b & (head | ~prev_b_bits) & live;
 
-  // ---- last run start / B-part start at or before each element (forward), next ones
-  // after it (backward).  Positions are stored +1 so that 0 means "none" in the forward
+  // ---- last run start / B-part start at or before each element (forward scan), next ones
+  // after it (backward scan).  Positions are stored +1 so that 0 means "none" in the forward
   // scan; the backward scan runs over mirrored positions (SET_TILE - p) and mirrored lanes.
-  uint64_t fwd_in, bwd_in;
+  uint64_t fwd_in, bwd_in, fwd_all, bwd_all;
   {
-    uint32_t last_h = 0, last_e2 = 0, first_h = 0, first_e2 = 0;  // forward: p + 1; mirrored: SET_TILE - p
-#pragma unroll
-    for (int o = 0; o < SET_ITEMS; ++o) {
-      const uint32_t p = run0 + o;
-      if ((head >> o) & 1u) last_h = p + 1;
-      if ((e2 >> o) & 1u) last_e2 = p + 1;
-    }
-#pragma unroll
-    for (int o = SET_ITEMS - 1; o >= 0; --o) {
-      const uint32_t p = run0 + o;
-      if ((head >> o) & 1u) first_h = SET_TILE - p;
-      if ((e2 >> o) & 1u) first_e2 = SET_TILE - p;
-    }
-    fwd_in = set_block_exclusive<uint64_t>(((uint64_t)last_h << 32) | last_e2, OpMaxPair{}, (uint64_t)0, s_scan64,
-                                           (uint64_t*)nullptr);
-    // mirrored lanes: thread t contributes as thread 255 - t
+    const uint32_t head_after0 = (threadIdx.x == 0) ? (head & ~1u) : head;  // position 0 is never "next"
+    const uint32_t last_h = head ? run0 + (31 - __builtin_clz(head)) + 1 : 0u;
+    const uint32_t last_e2 = e2 ? run0 + (31 - __builtin_clz(e2)) + 1 : 0u;
+    const uint32_t first_h = head_after0 ? SET_TILE - (run0 + __builtin_ctz(head_after0)) : 0u;
+    const uint32_t first_e2 = e2 ? SET_TILE - (run0 + __builtin_ctz(e2)) : 0u;
+    fwd_in = set_block_exclusive<SET_WAVES, uint64_t>(((uint64_t)last_h << 32) | last_e2, OpMaxPair{}, (uint64_t)0,
+                                                      s_scan64, &fwd_all);
+    // mirrored lanes: thread t contributes as thread BLOCK - 1 - t
     s_pair[SET_BLOCK - 1 - threadIdx.x] = ((uint64_t)first_h << 32) | first_e2;
     __syncthreads();
     const uint64_t mirrored = s_pair[threadIdx.x];
     __syncthreads();  // s_scan64 and s_pair are reused below
-    const uint64_t r = set_block_exclusive<uint64_t>(mirrored, OpMaxPair{}, (uint64_t)0, s_scan64, (uint64_t*)nullptr);
+    const uint64_t r = set_block_exclusive<SET_WAVES, uint64_t>(mirrored, OpMaxPair{}, (uint64_t)0, s_scan64, &bwd_all);
     s_pair[SET_BLOCK - 1 - threadIdx.x] = r;
     __syncthreads();
     bwd_in = s_pair[threadIdx.x];
   }
+  // the first run of the tile ends where the first later run starts; the last run starts at
+  // the last run start (position 0 is one, so there always is one)
+  const uint32_t first_end = (uint32_t)(bwd_all >> 32) ? SET_TILE - (uint32_t)(bwd_all >> 32) : count;
+  const uint32_t last_start = (uint32_t)(fwd_all >> 32) - 1u;
 
   // ---- decide every element
-  // backward pass: next run start and next B-part start strictly after each element
-  uint16_t nxt_h[SET_ITEMS], nxt_e2[SET_ITEMS];
+  // backward pass: the number of B elements of the element's run that lie after it (for an
+  // element of A that is the size of the run's B part, because all of them follow it);
+  // two 16-bit counts per register
+  uint32_t b_after[SET_ITEMS / 2];
   {
     // mirrored value v = SET_TILE - p, 0 = none  ->  position, `count` when there is none
-    uint32_t nh = (uint32_t)(bwd_in >> 32), ne = (uint32_t)bwd_in;
-    uint32_t cur_h = nh ? SET_TILE - nh : count;
-    uint32_t cur_e = ne ? SET_TILE - ne : count;
-    if (cur_h > count) cur_h = count;
-    if (cur_e > count) cur_e = count;
+    const uint32_t nh = (uint32_t)(bwd_in >> 32), ne = (uint32_t)bwd_in;
+    uint32_t cur_h = nh ? SET_TILE - nh : count;  // next run start after this element
+    uint32_t cur_e = ne ? SET_TILE - ne : count;  // next B-part start after this element
 #pragma unroll
     for (int o = SET_ITEMS - 1; o >= 0; --o) {
-      nxt_h[o] = (uint16_t)cur_h;
-      nxt_e2[o] = (uint16_t)cur_e;
+      const uint32_t nb_run = (cur_e < cur_h) ? cur_h - cur_e : 0u;
+      if (o & 1) b_after[o / 2] = nb_run << 16;
+      else b_after[o / 2] |= nb_run;
       const uint32_t p = run0 + o;
-      if (((head >> o) & 1u) && p < count) cur_h = p;
+      if ((head >> o) & 1u) cur_h = p;
       if ((e2 >> o) & 1u) cur_e = p;
     }
   }
+  // what is kept, by side and by "rank inside the own part >= size of the other part"
+  const bool a_ge = g.op != THRUST_AMD_SET_INTERSECTION;                                  // A, rank >= |B part|
+  const bool a_lt = g.op == THRUST_AMD_SET_INTERSECTION || g.op == THRUST_AMD_SET_UNION;  // A, rank <  |B part|
+  const bool b_ge = g.op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE || g.op == THRUST_AMD_SET_UNION;
   uint32_t keep = 0;
   {
-    uint32_t cur_h = (uint32_t)(fwd_in >> 32);  // p + 1 of the last start before this lane, 0 = none
-    uint32_t cur_e = (uint32_t)fwd_in;
+    uint32_t cur_h = (uint32_t)(fwd_in >> 32);  // p + 1 of the last run start at or before the element
+    uint32_t cur_e = (uint32_t)fwd_in;          // p + 1 of the last B-part start at or before it
 #pragma unroll
     for (int o = 0; o < SET_ITEMS; ++o) {
       const uint32_t p = run0 + o;
       if ((head >> o) & 1u) cur_h = p + 1;
       if ((e2 >> o) & 1u) cur_e = p + 1;
-      if (!((live >> o) & 1u)) continue;
       const bool bo = (is_b >> o) & 1u;
-      const uint64_t gp = d0 + p;  // position on the whole merge path
-      uint64_t rs, rm, re;         // run start, B-part start, run end
-      if (!set_comp(f0_key, k[o], descending)) {
-        rs = f0_start; rm = f0_mid; re = f0_end;
-      } else if (f1_valid && !set_comp(k[o], f1_key, descending)) {
-        rs = f1_start; rm = f1_mid; re = f1_end;
-      } else {
-        const uint32_t ps = cur_h - 1;  // an interior run starts inside the tile: cur_h >= 1
-        const uint32_t pe = nxt_h[o];
-        uint32_t pm;
-        if (bo) pm = cur_e - 1;  // the first B of this run is at or before p
-        else pm = (nxt_e2[o] < pe) ? nxt_e2[o] : pe;
-        rs = d0 + ps; rm = d0 + pm; re = d0 + pe;
-      }
-      const uint64_t m = rm - rs, n = re - rm;
-      const uint64_t r = bo ? gp - rm : gp - rs;
-      bool kp;
-      switch (g.op) {
-        case THRUST_AMD_SET_DIFFERENCE: kp = !bo && r >= n; break;
-        case THRUST_AMD_SET_INTERSECTION: kp = !bo && r < n; break;
-        case THRUST_AMD_SET_SYMMETRIC_DIFFERENCE: kp = bo ? (r >= m) : (r >= n); break;
-        default: kp = bo ? (r >= m) : true; break;
-      }
+      // an interior run starts inside the tile (cur_h >= 1); for a B, the run's first B is at or before p
+      const uint32_t n_b = (o & 1) ? (b_after[o / 2] >> 16) : (b_after[o / 2] & 0xffffu);
+      const uint32_t own_start = (bo ? cur_e : cur_h) - 1u;
+      const uint32_t other = bo ? cur_e - cur_h : n_b;
+      const bool ge_local = p - own_start >= other;
+      const bool ge_first = p >= (bo ? thr_b0 : thr_a0);
+      const bool ge_next = p >= (bo ? thr_b1 : thr_a1);
+      const bool ge = (p < first_end) ? ge_first : ((tail_continues && p >= last_start) ? ge_next : ge_local);
+      const bool kp = bo ? (b_ge && ge) : (ge ? a_ge : a_lt);
       keep |= (uint32_t)kp << o;
     }
+    keep &= live;
   }
 
   // ---- ranks inside the tile, then the tile's place in the output
   uint32_t tile_cnt = 0;
   __syncthreads();  // s_scan32 is fresh, but s_keys is about to be overwritten: all merges are done
   const uint32_t mine = __builtin_popcount(keep);
-  const uint32_t excl = set_block_exclusive<uint32_t>(mine, OpPlus{}, 0u, s_scan32, &tile_cnt);
+  const uint32_t excl = set_block_exclusive<SET_WAVES, uint32_t>(mine, OpPlus{}, 0u, s_scan32, &tile_cnt);
 
   constexpr int W = TileWords<uint64_t>::W;
   uint64_t* my_slot = g.status + (size_t)tile * W;
@@ -403,12 +422,28 @@ __global__ __launch_bounds__(SET_BLOCK) void set_op_kernel(SetArgs<T, V, HAS_VAL
 #pragma unroll
   for (int q = 0; q < SET_ITEMS; ++q) {
     const uint32_t e = q * SET_BLOCK + threadIdx.x;
-    if (e < tile_cnt) {
-      g.out[base + e] = s_keys[e];
-      if constexpr (HAS_VALUES) {
-        const uint32_t s = s_src[e];
-        g.vout[base + e] = (s < ca) ? g.va[a0 + s] : g.vb[b0 + (s - ca)];
+    if (e < tile_cnt) g.out[base + e] = s_keys[e];
+  }
+  if constexpr (HAS_VALUES) {
+    // values: the two sub-ranges are staged like the keys were (A's part, then B's, so a
+    // key's staging slot is its value's), then gathered by slot in output order
+    const bool keeps_b = g.op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE || g.op == THRUST_AMD_SET_UNION;
+    __syncthreads();  // the compacted keys have been read
+    {
+      V in[SET_ITEMS];
+#pragma unroll
+      for (int q = 0; q < SET_ITEMS; ++q) {
+        const uint32_t e = q * SET_BLOCK + threadIdx.x;
+        in[q] = (e < ca) ? g.va[a0 + e] : (keeps_b && e < count) ? g.vb[b0 + (e - ca)] : V{};
       }
+#pragma unroll
+      for (int q = 0; q < SET_ITEMS; ++q) s_vals[q * SET_BLOCK + threadIdx.x] = in[q];
+    }
+    __syncthreads();
+#pragma unroll
+    for (int q = 0; q < SET_ITEMS; ++q) {
+      const uint32_t e = q * SET_BLOCK + threadIdx.x;
+      if (e < tile_cnt) g.vout[base + e] = s_vals[s_src[e]];  // s_src[e] < count
     }
   }
 }
@@ -417,6 +452,8 @@ template <typename T, typename V, bool HAS_VALUES>
 static int set_run(void* temp, size_t* temp_bytes, int op, const void* a, uint64_t na, const void* b,
                    uint64_t nb, const void* va, const void* vb, void* out, void* vout,
                    uint64_t* d_num, int descending, hipStream_t stream) {
+  using Shape = SetShape<T, V, HAS_VALUES>;
+  constexpr uint32_t SET_TILE = Shape::TILE;
   const uint64_t total = na + nb;
   const uint64_t tiles = (total + SET_TILE - 1) / SET_TILE;
   if (tiles > 0x7fffffffull) return (int)hipErrorInvalidValue;
@@ -449,8 +486,8 @@ static int set_run(void* temp, size_t* temp_bytes, int op, const void* a, uint64
   TA_CHECK_LAUNCH();
   if (total == 0) return 0;
   TA_LAUNCH("set_partition", stream, (set_partition_kernel<T>), dim3((uint32_t)((tiles + 1 + 255) / 256)),
-            dim3(256), static_cast<const T*>(a), na, static_cast<const T*>(b), nb, tiles, descending, split,
-            run, key);
+            dim3(256), static_cast<const T*>(a), na, static_cast<const T*>(b), nb, tiles, SET_TILE, descending,
+            split, run, key);
   TA_CHECK_LAUNCH();
   SetArgs<T, V, HAS_VALUES> g;
   g.a = static_cast<const T*>(a);
@@ -470,7 +507,7 @@ static int set_run(void* temp, size_t* temp_bytes, int op, const void* a, uint64
   g.tiles = tiles;
   g.op = op;
   g.descending = descending;
-  TA_LAUNCH("set_operation", stream, (set_op_kernel<T, V, HAS_VALUES>), dim3((uint32_t)tiles), dim3(SET_BLOCK), g);
+  TA_LAUNCH("set_operation", stream, (set_op_kernel<T, V, HAS_VALUES>), dim3((uint32_t)tiles), dim3(Shape::BLOCK), g);
   TA_CHECK_LAUNCH();
   return 0;
 }
