@@ -35,9 +35,11 @@
 
 namespace ta {
 
-// Tile = BLOCK threads x 16 merged elements each.  Tiles take dynamic tickets (a same-address
-// atomic retires about every 12 ns) and chain their counts, so they are made as large as
-// LDS allows: 16384 elements for keys and values of up to 4 bytes, 8192 for 8-byte items.
+// Tile = BLOCK threads x 16 merged elements each: 8192 elements for keys and values of up
+// to 4 bytes, 4096 for 8-byte items.  Tiles take dynamic tickets (a same-address atomic
+// retires about every 12 ns) and chain their counts, which favours large tiles; two
+// workgroups per CU hide each other's barriers, which caps them (16384-element tiles of
+// 1024 threads measured slower than these).
 constexpr int SET_ITEMS = 16;
 template <typename T, typename V, bool HAS_VALUES>
 struct SetShape {
@@ -64,32 +66,10 @@ TA_DEVICE uint64_t set_merge_path(PA a, uint64_t na, PB b, uint64_t nb, uint64_t
   return lo;
 }
 
-// First index whose element is not before x / is after x.
-template <typename T>
-TA_DEVICE uint64_t set_lower_bound(const T* p, uint64_t n, T x, bool descending) {
-  uint64_t lo = 0, hi = n;
-  while (lo < hi) {
-    const uint64_t mid = (lo + hi) >> 1;
-    if (set_comp(p[mid], x, descending)) lo = mid + 1;
-    else hi = mid;
-  }
-  return lo;
-}
-template <typename T>
-TA_DEVICE uint64_t set_upper_bound(const T* p, uint64_t n, T x, bool descending) {
-  uint64_t lo = 0, hi = n;
-  while (lo < hi) {
-    const uint64_t mid = (lo + hi) >> 1;
-    if (!set_comp(x, p[mid], descending)) lo = mid + 1;
-    else hi = mid;
-  }
-  return lo;
-}
-
-// Per tile boundary t (t = 0 .. tiles): split[t] = elements of A before merged position
-// t * tile_size; for boundaries inside the merged order, key[t] = the element at that position
-// and run[3t .. 3t+2] = merged positions where its run starts, where the run's B part
-// starts, and where the run ends.
+// Per tile boundary t (t = 0 .. tiles), found by one thread: split[t] = elements of A before
+// merged position t * tile_size; for boundaries inside the merged order, key[t] = the
+// element at that position and run[3t .. 3t+2] = merged positions where its run starts,
+// where the run's B part starts, and where the run ends.
 template <typename T>
 __global__ __launch_bounds__(256) void set_partition_kernel(const T* __restrict__ a, uint64_t na,
                                                             const T* __restrict__ b, uint64_t nb,
@@ -104,17 +84,20 @@ __global__ __launch_bounds__(256) void set_partition_kernel(const T* __restrict_
   const uint64_t total = na + nb;
   uint64_t diag = t * tile_size;
   if (diag > total) diag = total;
-  const uint64_t as = set_merge_path<T>(a, na, b, nb, diag, descending);
+  const uint64_t as = partition_point(diag > nb ? diag - nb : 0, diag < na ? diag : na, [&](uint64_t mid) {
+    return !set_comp(b[diag - 1 - mid], a[mid], descending);
+  });
   split[t] = as;
   if (diag >= total) return;
   const uint64_t bs = diag - as;
   T x;
   if (as < na && (bs >= nb || !set_comp(b[bs], a[as], descending))) x = a[as];
   else x = b[bs];
-  const uint64_t lb_a = set_lower_bound(a, na, x, descending);
-  const uint64_t ub_a = set_upper_bound(a, na, x, descending);
-  const uint64_t lb_b = set_lower_bound(b, nb, x, descending);
-  const uint64_t ub_b = set_upper_bound(b, nb, x, descending);
+  // first index whose element is not before x / is after x, in each range
+  const uint64_t lb_a = partition_point(0, na, [&](uint64_t i) { return set_comp(a[i], x, descending); });
+  const uint64_t ub_a = partition_point(lb_a, na, [&](uint64_t i) { return !set_comp(x, a[i], descending); });
+  const uint64_t lb_b = partition_point(0, nb, [&](uint64_t i) { return set_comp(b[i], x, descending); });
+  const uint64_t ub_b = partition_point(lb_b, nb, [&](uint64_t i) { return !set_comp(x, b[i], descending); });
   key[t] = x;
   run[3 * t + 0] = lb_a + lb_b;
   run[3 * t + 1] = ub_a + lb_b;
