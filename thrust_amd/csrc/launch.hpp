@@ -10,17 +10,20 @@
 namespace ta {
 
 bool profile_on();
-void profile_mark(const char* label, hipStream_t stream, bool begin);
+// Records an event on the stream and returns it (null on failure).
+hipEvent_t profile_begin(hipStream_t stream);
+// Records the closing event and files the pair under the label.
+void profile_end(const char* label, hipStream_t stream, hipEvent_t begin);
 
+// The opening event lives in the timer object, so launches from several host threads do
+// not mix their brackets.
 struct LaunchTimer {
   const char* label;
   hipStream_t stream;
-  bool on;
-  LaunchTimer(const char* l, hipStream_t s) : label(l), stream(s), on(profile_on()) {
-    if (on) profile_mark(label, stream, true);
-  }
+  hipEvent_t begin;
+  LaunchTimer(const char* l, hipStream_t s) : label(l), stream(s), begin(profile_on() ? profile_begin(s) : nullptr) {}
   ~LaunchTimer() {
-    if (on) profile_mark(label, stream, false);
+    if (begin) profile_end(label, stream, begin);
   }
 };
 

@@ -5,8 +5,6 @@
 #include "dispatch.hpp"
 #include "launch.hpp"
 
-#include "launch.hpp"
-
 #include <atomic>
 #include <cstdio>
 #include <cstring>
@@ -254,7 +252,6 @@ struct ProfileRecord {
 struct Profile {
   std::mutex mu;
   std::vector<ProfileRecord> records;
-  hipEvent_t pending = nullptr;
 };
 
 static std::atomic<int> g_profile_on{0};
@@ -265,18 +262,26 @@ static Profile& profile() {
 
 bool profile_on() { return g_profile_on.load(std::memory_order_relaxed) != 0; }
 
-void profile_mark(const char* label, hipStream_t stream, bool begin) {
+hipEvent_t profile_begin(hipStream_t stream) {
+  hipEvent_t ev = nullptr;
+  if (hipEventCreate(&ev) != hipSuccess) return nullptr;
+  if (hipEventRecord(ev, stream) != hipSuccess) {
+    (void)hipEventDestroy(ev);
+    return nullptr;
+  }
+  return ev;
+}
+
+void profile_end(const char* label, hipStream_t stream, hipEvent_t begin) {
+  hipEvent_t ev = nullptr;
+  if (hipEventCreate(&ev) != hipSuccess || hipEventRecord(ev, stream) != hipSuccess) {
+    if (ev) (void)hipEventDestroy(ev);
+    (void)hipEventDestroy(begin);
+    return;
+  }
   Profile& p = profile();
   std::lock_guard<std::mutex> g(p.mu);
-  hipEvent_t ev = nullptr;
-  if (hipEventCreate(&ev) != hipSuccess) return;
-  (void)hipEventRecord(ev, stream);
-  if (begin) {
-    p.pending = ev;
-  } else {
-    p.records.push_back(ProfileRecord{label, p.pending, ev});
-    p.pending = nullptr;
-  }
+  p.records.push_back(ProfileRecord{label, begin, ev});
 }
 
 }  // namespace ta
