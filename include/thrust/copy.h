@@ -17,14 +17,15 @@ namespace thrust {
 namespace detail {
 // Copy n elements between any two of {host, device} given raw element addresses.
 template <typename T>
-inline void copy_raw(const T* src, bool src_device, T* dst, bool dst_device, std::size_t n, void* stream) {
+inline void copy_raw(const T* src, bool src_device, T* dst, bool dst_device, std::size_t n, void* stream,
+                     bool blocking = true) {
   if (n == 0) return;
   using thrust::system::hip::detail::throw_on_error;
   if (!src_device && !dst_device) {
     std::copy(src, src + n, dst);
   } else if (src_device && dst_device) {
     throw_on_error(thrust_amd_memcpy(dst, src, n * sizeof(T), THRUST_AMD_D2D, stream), "copy (device to device)");
-    throw_on_error(thrust_amd_stream_synchronize(stream), "copy: synchronize");
+    if (blocking) throw_on_error(thrust_amd_stream_synchronize(stream), "copy: synchronize");
   } else {
     throw_on_error(thrust_amd_memcpy(dst, src, n * sizeof(T), src_device ? THRUST_AMD_D2H : THRUST_AMD_H2D, stream),
                    "copy (across systems)");
@@ -32,7 +33,8 @@ inline void copy_raw(const T* src, bool src_device, T* dst, bool dst_device, std
 }
 
 template <typename In, typename Out>
-inline Out copy_dispatch(In first, In last, Out result, bool in_device, bool out_device, void* stream) {
+inline Out copy_dispatch(In first, In last, Out result, bool in_device, bool out_device, void* stream,
+                         bool blocking = true) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
   typedef typename iterator_value<Out>::type U;
   const std::size_t n = (std::size_t)std::distance(first, last);
@@ -41,7 +43,7 @@ inline Out copy_dispatch(In first, In last, Out result, bool in_device, bool out
   static_assert(std::is_trivially_copyable<T>::value, "thrust::copy involving the device needs trivially copyable elements");
   if (std::is_same<T, U>::value && (in_device || is_contiguous_host_iterator<In>::value) &&
       (out_device || is_contiguous_host_iterator<Out>::value)) {
-    copy_raw<T>(raw(first), in_device, reinterpret_cast<T*>(raw(result)), out_device, n, stream);
+    copy_raw<T>(raw(first), in_device, reinterpret_cast<T*>(raw(result)), out_device, n, stream, blocking);
   } else if (in_device) {
     // device -> host with conversion or a non-contiguous destination: stage on the host
     std::vector<T> staged(n);

@@ -9,21 +9,23 @@
 namespace thrust {
 namespace detail {
 struct host_t : thrust::host_execution_policy<host_t> {};
-struct device_t : thrust::device_execution_policy<device_t> {};
 struct seq_t : thrust::system::cpp::execution_policy<seq_t> {};
 }  // namespace detail
 
 static const detail::host_t host;
-static const detail::device_t device;
 static const detail::seq_t seq;
 
 namespace system {
 namespace hip {
 
+struct after_policy;  // thrust/future.h: a policy with dependencies, for the asynchronous algorithms
+
 // Policy bound to a stream: thrust::hip::par.on(stream).
 struct stream_policy : execution_policy<stream_policy> {
   void* stream;
   explicit stream_policy(void* s) : stream(s) {}
+  template <typename... Events>
+  after_policy after(const Events&... events) const;  // defined in thrust/future.h
 };
 inline void* get_stream(const stream_policy& p) { return p.stream; }
 
@@ -71,6 +73,8 @@ struct par_t : execution_policy<par_t> {
   stream_policy on(void* stream) const { return stream_policy(stream); }
   template <typename Alloc>
   allocator_policy<Alloc> operator()(Alloc& alloc) const { return allocator_policy<Alloc>(alloc); }
+  template <typename... Events>
+  after_policy after(const Events&... events) const;  // defined in thrust/future.h
 };
 static const par_t par;
 
@@ -88,6 +92,18 @@ inline temp_source temp_source_of(execution_policy<Derived>& p) {
 
 }  // namespace hip
 }  // namespace system
+
+namespace detail {
+// thrust::device: the device system's default policy, with the same builders as hip::par.
+struct device_t : thrust::device_execution_policy<device_t> {
+  system::hip::stream_policy on(void* stream) const { return system::hip::stream_policy(stream); }
+  template <typename Alloc>
+  system::hip::allocator_policy<Alloc> operator()(Alloc& alloc) const { return system::hip::allocator_policy<Alloc>(alloc); }
+  template <typename... Events>
+  system::hip::after_policy after(const Events&... events) const;  // defined in thrust/future.h
+};
+}  // namespace detail
+static const detail::device_t device;
 
 namespace hip = system::hip;
 namespace cpp {

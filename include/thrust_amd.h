@@ -128,6 +128,21 @@ int thrust_amd_memcpy(void* dst, const void* src, size_t bytes, int kind, void* 
  * cuda_cub::synchronize (thrust/system/cuda/detail/util.h:75-104). */
 int thrust_amd_stream_synchronize(void* stream);
 
+/* Streams and events for callers that overlap work (the asynchronous algorithms of the
+ * front end).  A stream created here is independent of the null stream; an event is
+ * recorded on one stream and another stream can be made to wait for it without blocking
+ * the host.  *done = 1 when everything enqueued on the stream has finished.  Streams keep
+ * the default priority.  Replace the unique_stream / event machinery of
+ * thrust/system/cuda/detail/future.inl:60-260 (cudaStreamCreateWithFlags, cudaEventRecord,
+ * cudaStreamWaitEvent, cudaStreamQuery). */
+int thrust_amd_stream_create(void** stream);
+int thrust_amd_stream_destroy(void* stream);
+int thrust_amd_stream_query(void* stream, int* done);
+int thrust_amd_event_create(void** event);
+int thrust_amd_event_record(void* event, void* stream);
+int thrust_amd_stream_wait_event(void* stream, void* event);
+int thrust_amd_event_destroy(void* event);
+
 /* Fill n elements of `elem_bytes` (1, 2, 4 or 8) with the host value *value.  Replaces
  * cuda_cub::fill_n (thrust/system/cuda/detail/fill.h) as used by
  * device_vector(n, value) (thrust/detail/vector_base.inl:214-234). */

@@ -9,12 +9,17 @@
 #include <map>
 #include <stdexcept>
 
+#include <thrust/async/copy.h>
+#include <thrust/async/reduce.h>
+#include <thrust/async/scan.h>
+#include <thrust/async/sort.h>
 #include <thrust/copy.h>
 #include <thrust/count.h>
 #include <thrust/device_vector.h>
 #include <thrust/execution_policy.h>
 #include <thrust/fill.h>
 #include <thrust/functional.h>
+#include <thrust/future.h>
 #include <thrust/host_vector.h>
 #include <thrust/inner_product.h>
 #include <thrust/merge.h>
@@ -879,6 +884,103 @@ static void TestCustomTemporaryAllocation() {  // examples/cuda/custom_temporary
   ASSERT_EQUAL_VEC(to_host(d), h);
 }
 
+// thrust::async: results equal the synchronous algorithms; the stream of the result follows
+// .on(stream) / .after(...) as testing/async_reduce.cu:773-990 checks; independent work
+// overlaps on streams of its own (testing/async_sort.cu, async_copy.cu, async/inclusive_scan).
+static void TestAsyncAlgorithms() {
+  g_test = "AsyncAlgorithms";
+  const size_t n = (1 << 20) + 17;
+  thrust::host_vector<int> h = random_integers<int>(n, 5, 0);
+  thrust::device_vector<int> d0 = h, d1 = h, d2 = h, d3 = h;
+  long long total = 0;
+  for (size_t i = 0; i < n; ++i) total += h[i];
+  const int expect = (int)total;
+
+  // four independent reductions in flight, each on a stream of its own
+  auto f0a = thrust::async::reduce(d0.begin(), d0.end());
+  auto f0b = thrust::async::reduce(thrust::device, d1.begin(), d1.end());
+  auto f0c = thrust::async::reduce(thrust::device, d2.begin(), d2.end(), 0);
+  auto f0d = thrust::async::reduce(thrust::device, d3.begin(), d3.end(), 7, thrust::plus<int>());
+  ASSERT_TRUE(f0a.valid_stream() && f0b.valid_stream() && f0a.valid_content());
+  ASSERT_TRUE(f0a.stream().native_handle() != f0b.stream().native_handle());
+  ASSERT_TRUE(f0a.get() == expect && f0b.get() == expect && f0c.get() == expect && f0d.get() == expect + 7);
+  ASSERT_TRUE(f0a.ready());
+  ASSERT_TRUE(f0a.extract() == expect);  // the value stays available
+
+  // .after: runs on the first dependency's stream once every dependency has finished
+  auto g0 = thrust::async::reduce(d0.begin(), d0.end());
+  void* g0_stream = g0.stream().native_handle();
+  auto g1 = thrust::async::reduce(thrust::device.after(g0), d0.begin(), d0.end());
+  ASSERT_TRUE(g1.stream().native_handle() == g0_stream);
+  auto g2 = thrust::async::reduce(thrust::device.after(g1, f0b), d0.begin(), d0.end());
+  ASSERT_TRUE(g2.stream().native_handle() == g0_stream);
+  ASSERT_TRUE(g2.get() == expect && g0.get() == expect);
+
+  // .on(stream) wins over the dependencies' streams
+  void* user_stream = nullptr;
+  ASSERT_TRUE(thrust_amd_stream_create(&user_stream) == 0);
+  auto k0 = thrust::async::reduce(thrust::device.on(user_stream), d0.begin(), d0.end());
+  ASSERT_TRUE(k0.stream().native_handle() == user_stream);
+  auto k1 = thrust::async::reduce(thrust::device.on(user_stream).after(g2), d0.begin(), d0.end());
+  ASSERT_TRUE(k1.stream().native_handle() == user_stream);
+  ASSERT_TRUE(k0.get() == expect && k1.get() == expect);
+
+  // a chain on one stream: sort, then scan into another vector, then reduce the scan's last run
+  thrust::device_vector<int> sorted = h, scanned(n), slot(1);
+  thrust::host_vector<int> hs = h, hscan(n);
+  thrust::sort(hs.begin(), hs.end());
+  thrust::inclusive_scan(hs.begin(), hs.end(), hscan.begin());
+  auto e0 = thrust::async::sort(thrust::device.on(user_stream), sorted.begin(), sorted.end());
+  auto e1 = thrust::async::inclusive_scan(thrust::device.after(e0), sorted.begin(), sorted.end(), scanned.begin());
+  ASSERT_TRUE(e1.stream().native_handle() == user_stream);
+  auto e2 = thrust::async::reduce_into(thrust::device.after(e1), sorted.begin(), sorted.end(), slot.begin(), 3, thrust::plus<int>());
+  e2.wait();
+  ASSERT_EQUAL_VEC(to_host(sorted), hs);
+  ASSERT_EQUAL_VEC(to_host(scanned), hscan);
+  ASSERT_TRUE((int)slot[0] == expect + 3);
+
+  // work on another stream that depends on the chain: descending sort of the scan, exclusive scan, copy
+  thrust::device_vector<int> desc(n), copied(n);
+  auto c0 = thrust::async::copy(thrust::device.after(e1), scanned.begin(), scanned.end(), desc.begin());
+  auto c1 = thrust::async::sort(thrust::device.after(c0), desc.begin(), desc.end(), thrust::greater<int>());
+  auto c2 = thrust::async::exclusive_scan(thrust::device.after(c1), desc.begin(), desc.end(), copied.begin(), 11);
+  thrust::when_all_wait(c2, e2);
+  thrust::host_vector<int> hdesc = hscan, hex(n);
+  thrust::sort(hdesc.begin(), hdesc.end(), thrust::greater<int>());
+  thrust::exclusive_scan(hdesc.begin(), hdesc.end(), hex.begin(), 11);
+  ASSERT_EQUAL_VEC(to_host(desc), hdesc);
+  ASSERT_EQUAL_VEC(to_host(copied), hex);
+
+  // host <-> device copies complete before they return; the event is ready
+  thrust::device_vector<int> up(n);
+  auto u0 = thrust::async::copy(h.begin(), h.end(), up.begin());
+  ASSERT_EQUAL_VEC(to_host(up), h);
+  u0.wait();
+
+  // a synchronous algorithm accepts the same policies and waits for the dependencies itself
+  auto s0 = thrust::async::reduce(d1.begin(), d1.end());
+  ASSERT_TRUE(thrust::reduce(thrust::device.after(s0), d1.begin(), d1.end()) == expect);
+
+  // with a caller's allocator: the temporary storage goes back when the future dies
+  {
+    CachingTempAllocator alloc;
+    {
+      auto a0 = thrust::async::reduce(thrust::device(alloc), d2.begin(), d2.end());
+      ASSERT_TRUE(a0.get() == expect && alloc.live.size() == 1);
+    }
+    ASSERT_TRUE(alloc.live.empty() && alloc.returned == 1);
+  }
+  // empty range: the value is init
+  auto z = thrust::async::reduce(d0.begin(), d0.begin(), 42);
+  ASSERT_TRUE(z.get() == 42);
+  k0 = thrust::device_future<int>();  // futures let go of the user's stream before it is destroyed
+  k1 = thrust::device_future<int>();
+  e0 = thrust::device_event(); e1 = thrust::device_event(); e2 = thrust::device_event();
+  c0 = thrust::device_event(); c1 = thrust::device_event(); c2 = thrust::device_event();
+  ASSERT_TRUE(thrust_amd_stream_synchronize(user_stream) == 0);
+  ASSERT_TRUE(thrust_amd_stream_destroy(user_stream) == 0);
+}
+
 int main() {
   TestReduceSimple();
   TestReduceWithOperatorTable();
@@ -913,6 +1015,7 @@ int main() {
   TestOutOfMemoryThrows();
   TestTempArenaReuse();
   TestCustomTemporaryAllocation();
+  TestAsyncAlgorithms();
   std::printf("%s: %d checks, %d failed\n", g_failed ? "FAILED" : "PASSED", g_checks, g_failed);
   return g_failed ? 1 : 0;
 }

@@ -50,6 +50,13 @@ SIGNATURES = {
     "thrust_amd_temp_bytes_held": (_sz, []),
     "thrust_amd_profile_enable": (_int, [_int]),
     "thrust_amd_profile_collect": (_int, [_c.c_char_p, _sz, _szp]),
+    "thrust_amd_stream_create": (_int, [ctypes.POINTER(_vp)]),
+    "thrust_amd_stream_destroy": (_int, [_vp]),
+    "thrust_amd_stream_query": (_int, [_vp, ctypes.POINTER(_int)]),
+    "thrust_amd_event_create": (_int, [ctypes.POINTER(_vp)]),
+    "thrust_amd_event_record": (_int, [_vp, _vp]),
+    "thrust_amd_stream_wait_event": (_int, [_vp, _vp]),
+    "thrust_amd_event_destroy": (_int, [_vp]),
     "thrust_amd_reduce": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp, _vp, _vp]),
     "thrust_amd_transform_reduce": (_int, [_vp, _szp, _vp, _u64, _int, _int, _int, _vp, _vp, _vp]),
     "thrust_amd_count_if": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp, _vp, _vp]),

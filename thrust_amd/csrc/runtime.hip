@@ -68,6 +68,54 @@ TA_EXPORT int thrust_amd_stream_synchronize(void* stream) {
   return (int)hipStreamSynchronize((hipStream_t)stream);
 }
 
+TA_EXPORT int thrust_amd_stream_create(void** stream) {
+  if (!stream) return (int)hipErrorInvalidValue;
+  hipStream_t s = nullptr;
+  const hipError_t e = hipStreamCreateWithFlags(&s, hipStreamNonBlocking);
+  *stream = (e == hipSuccess) ? (void*)s : nullptr;
+  return (int)e;
+}
+
+TA_EXPORT int thrust_amd_stream_destroy(void* stream) {
+  if (!stream) return 0;
+  return (int)hipStreamDestroy((hipStream_t)stream);
+}
+
+TA_EXPORT int thrust_amd_stream_query(void* stream, int* done) {
+  if (!done) return (int)hipErrorInvalidValue;
+  const hipError_t e = hipStreamQuery((hipStream_t)stream);
+  if (e == hipErrorNotReady) {
+    (void)hipGetLastError();  // "not ready" is an answer, not a failure to leave behind
+    *done = 0;
+    return 0;
+  }
+  *done = (e == hipSuccess) ? 1 : 0;
+  return (int)e;
+}
+
+TA_EXPORT int thrust_amd_event_create(void** event) {
+  if (!event) return (int)hipErrorInvalidValue;
+  hipEvent_t ev = nullptr;
+  const hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+  *event = (e == hipSuccess) ? (void*)ev : nullptr;
+  return (int)e;
+}
+
+TA_EXPORT int thrust_amd_event_record(void* event, void* stream) {
+  if (!event) return (int)hipErrorInvalidValue;
+  return (int)hipEventRecord((hipEvent_t)event, (hipStream_t)stream);
+}
+
+TA_EXPORT int thrust_amd_stream_wait_event(void* stream, void* event) {
+  if (!event) return (int)hipErrorInvalidValue;
+  return (int)hipStreamWaitEvent((hipStream_t)stream, (hipEvent_t)event, 0);
+}
+
+TA_EXPORT int thrust_amd_event_destroy(void* event) {
+  if (!event) return 0;
+  return (int)hipEventDestroy((hipEvent_t)event);
+}
+
 namespace ta {
 
 template <typename U>
