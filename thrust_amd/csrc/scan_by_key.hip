@@ -45,10 +45,10 @@ __global__ __launch_bounds__(256) void sbk_init_kernel(uint64_t* __restrict__ wo
 // K is the key's comparison class: an unsigned integer type of the key's size (integer
 // keys are equal iff their bits are) or float / double (operator==).
 template <typename K, typename V, typename Op>
-__global__ __launch_bounds__(RBK_BLOCK, 4) void sbk_kernel(SbkArgs<K, V> a) {
+__global__ __launch_bounds__(SBK_BLOCK, 4) void sbk_kernel(SbkArgs<K, V> a) {
   constexpr int VEC = Vec16<K>::N;
   constexpr int CHUNKS = RBK_ITEMS / VEC >= 1 ? RBK_ITEMS / VEC : 1;
-  constexpr int WAVES = RBK_BLOCK / WAVE;
+  constexpr int WAVES = SBK_BLOCK / WAVE;
   constexpr uint32_t WAVE_SPAN = WAVE * CHUNKS * VEC;
   constexpr uint32_t TILE = WAVES * WAVE_SPAN;
   using WV = typename SegValue<V>::type;
@@ -190,7 +190,7 @@ static int sbk_run(void* temp, size_t* temp_bytes, const void* keys, const void*
                    uint64_t n, bool exclusive, const void* init, hipStream_t stream) {
   constexpr int VEC = Vec16<K>::N;
   constexpr int CHUNKS = RBK_ITEMS / VEC >= 1 ? RBK_ITEMS / VEC : 1;
-  constexpr uint64_t TILE = (uint64_t)RBK_BLOCK * CHUNKS * VEC;
+  constexpr uint64_t TILE = (uint64_t)SBK_BLOCK * CHUNKS * VEC;
   using Pair = SegPair<typename SegValue<V>::type>;
   constexpr int W = TileWords<Pair>::W;
   const uint64_t tiles = (n + TILE - 1) / TILE;
@@ -224,7 +224,7 @@ static int sbk_run(void* temp, size_t* temp_bytes, const void* keys, const void*
   TA_LAUNCH("sbk_init", stream, sbk_init_kernel, dim3((uint32_t)((words + 255) / 256)), dim3(256), a.status,
             words, a.ticket);
   TA_CHECK_LAUNCH();
-  TA_LAUNCH("scan_by_key", stream, (sbk_kernel<K, V, Op>), dim3((uint32_t)tiles), dim3(RBK_BLOCK), a);
+  TA_LAUNCH("scan_by_key", stream, (sbk_kernel<K, V, Op>), dim3((uint32_t)tiles), dim3(SBK_BLOCK), a);
   TA_CHECK_LAUNCH();
   return 0;
 }

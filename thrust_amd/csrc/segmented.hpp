@@ -6,9 +6,13 @@
 
 namespace ta {
 
-// 1024 threads x 16 elements: large tiles keep the number of tiles in flight (and the
-// look-back) small; the pair scan needs ~110 VGPRs, so one workgroup fills a CU.
+// 16 elements per lane; the pair scan needs ~110 VGPRs, so a CU holds 16 waves.  For
+// reduce_by_key one workgroup of 1024 threads measured best (large tiles keep the number of
+// tiles in flight, and the look-back, small: 0.73 against 0.77 ms with 512 threads at 2^28
+// pairs); scan_by_key, which also writes every element, prefers two workgroups of 512 that
+// overlap each other's load, scan and store phases (0.71 against 0.79 ms).
 constexpr int RBK_BLOCK = 1024;
+constexpr int SBK_BLOCK = 512;
 constexpr int RBK_ITEMS = 16;  // elements per lane
 
 template <typename V>
