@@ -1,11 +1,14 @@
-// thrust::device_vector<T>: a resizable array in device memory.
+// thrust::device_vector<T, Alloc>: a resizable array in device memory.
 //
 // The subset of the reference's vector_base that code on the sort / scan / reduce /
 // select / merge path uses (thrust/device_vector.h:54-64, thrust/detail/vector_base.inl):
 // construction from a size, a size and a value, a host range, a std::vector / host_vector
 // or another device_vector; begin/end/data/size/resize/clear/swap; operator[] / front /
 // back through device_reference; assignment across systems.  Elements must be trivially
-// copyable: storage is raw device memory, filled and copied by the device system.
+// copyable: storage is raw device memory, filled and copied by the device system.  Storage
+// comes from Alloc (default thrust::device_allocator<T>: the device system's malloc); any
+// allocator whose allocate(n) yields a device_ptr<T> or a raw device pointer will do, e.g.
+// thrust::mr::allocator<T, Pool> over a pool resource (thrust/mr/pool.h).
 #pragma once
 #include <cstddef>
 #include <iterator>
@@ -13,18 +16,20 @@
 #include <utility>
 #include <vector>
 
+#include <thrust/device_allocator.h>
 #include <thrust/device_ptr.h>
 #include <thrust/host_vector.h>
 
 namespace thrust {
 
-template <typename T>
+template <typename T, typename Alloc = device_allocator<T> >
 class device_vector {
   static_assert(std::is_trivially_copyable<T>::value,
                 "thrust::device_vector: elements must be trivially copyable");
 
  public:
   typedef T value_type;
+  typedef Alloc allocator_type;
   typedef std::size_t size_type;
   typedef std::ptrdiff_t difference_type;
   typedef device_ptr<T> pointer;
@@ -34,19 +39,29 @@ class device_vector {
   typedef device_reference<T> reference;
   typedef device_reference<const T> const_reference;
 
-  device_vector() : data_(nullptr), size_(0), capacity_(0) {}
-  explicit device_vector(size_type n) : device_vector() { resize(n); }
-  device_vector(size_type n, const T& value) : device_vector() { resize(n, value); }
-  device_vector(const device_vector& o) : device_vector() { assign_device(o.data_, o.size_); }
-  device_vector(device_vector&& o) noexcept : data_(o.data_), size_(o.size_), capacity_(o.capacity_) {
+  device_vector() : data_(nullptr), size_(0), capacity_(0), alloc_() {}
+  explicit device_vector(const Alloc& alloc) : data_(nullptr), size_(0), capacity_(0), alloc_(alloc) {}
+  explicit device_vector(size_type n, const Alloc& alloc = Alloc()) : device_vector(alloc) { resize(n); }
+  device_vector(size_type n, const T& value, const Alloc& alloc = Alloc()) : device_vector(alloc) { resize(n, value); }
+  device_vector(const device_vector& o) : device_vector(o.alloc_) { assign_device(o.data_, o.size_); }
+  template <typename A2>
+  device_vector(const device_vector<T, A2>& o, const Alloc& alloc = Alloc()) : device_vector(alloc) {
+    assign_device(o.data_, o.size_);
+  }
+  device_vector(device_vector&& o) noexcept
+      : data_(o.data_), size_(o.size_), capacity_(o.capacity_), alloc_(o.alloc_) {
     o.data_ = nullptr;
     o.size_ = o.capacity_ = 0;
   }
   template <typename A>
-  device_vector(const std::vector<T, A>& h) : device_vector() { assign_host(h.data(), h.size()); }
+  device_vector(const std::vector<T, A>& h, const Alloc& alloc = Alloc()) : device_vector(alloc) {
+    assign_host(h.data(), h.size());
+  }
   template <typename InputIterator,
             typename = typename std::iterator_traits<InputIterator>::iterator_category>
-  device_vector(InputIterator first, InputIterator last) : device_vector() { assign(first, last); }
+  device_vector(InputIterator first, InputIterator last, const Alloc& alloc = Alloc()) : device_vector(alloc) {
+    assign(first, last);
+  }
   ~device_vector() { release(); }
 
   device_vector& operator=(const device_vector& o) {
@@ -87,12 +102,13 @@ class device_vector {
   reference front() { return reference(data_); }
   reference back() { return reference(data_ + size_ - 1); }
 
+  allocator_type get_allocator() const { return alloc_; }
   void reserve(size_type n) {
     if (n <= capacity_) return;
     T* fresh = allocate(n);
     if (size_) copy_raw(fresh, data_, size_, THRUST_AMD_D2D);
     sync();
-    free_raw(data_);
+    free_raw(data_, capacity_);
     data_ = fresh;
     capacity_ = n;
   }
@@ -133,6 +149,7 @@ class device_vector {
     std::swap(data_, o.data_);
     std::swap(size_, o.size_);
     std::swap(capacity_, o.capacity_);
+    std::swap(alloc_, o.alloc_);
   }
 
   // Host copy of the contents.
@@ -141,18 +158,19 @@ class device_vector {
   }
 
  private:
-  template <typename U> friend class device_vector;
+  template <typename U, typename A2> friend class device_vector;
 
-  static T* allocate(size_type n) {
+  static T* to_raw(T* p) { return p; }
+  template <typename P>
+  static T* to_raw(const P& p) { return p.get(); }
+  T* allocate(size_type n) {
     if (n == 0) return nullptr;
     if (n > (~size_type(0)) / sizeof(T)) throw system::detail::bad_alloc("device_vector: size overflow");
-    void* p = nullptr;
-    const int rc = thrust_amd_malloc(&p, n * sizeof(T));
-    if (rc != 0) throw system::detail::bad_alloc(thrust_amd_error_string(rc));
-    return static_cast<T*>(p);
+    return to_raw(alloc_.allocate(n));
   }
-  static void free_raw(T* p) {
-    if (p) (void)thrust_amd_free(p);
+  void free_raw(T* p, size_type n) {
+    typedef decltype(std::declval<Alloc&>().allocate(size_type())) alloc_pointer;
+    if (p) alloc_.deallocate(alloc_pointer(p), n);
   }
   static void sync() {
     system::hip::detail::throw_on_error(thrust_amd_stream_synchronize(nullptr), "device_vector synchronize");
@@ -162,7 +180,7 @@ class device_vector {
                                         "device_vector copy");
   }
   void release() {
-    free_raw(data_);
+    free_raw(data_, capacity_);
     data_ = nullptr;
     size_ = capacity_ = 0;
   }
@@ -197,32 +215,35 @@ class device_vector {
 
   T* data_;
   size_type size_, capacity_;
+  Alloc alloc_;
 };
 
-template <typename T>
-inline void swap(device_vector<T>& a, device_vector<T>& b) { a.swap(b); }
+template <typename T, typename DA>
+inline void swap(device_vector<T, DA>& a, device_vector<T, DA>& b) { a.swap(b); }
 
 template <typename T, typename Alloc>
-host_vector<T, Alloc>::host_vector(const device_vector<T>& d) : base(d.size()) {
+template <typename DA>
+host_vector<T, Alloc>::host_vector(const device_vector<T, DA>& d) : base(d.size()) {
   d.copy_to_host(this->data());
 }
 template <typename T, typename Alloc>
-host_vector<T, Alloc>& host_vector<T, Alloc>::operator=(const device_vector<T>& d) {
+template <typename DA>
+host_vector<T, Alloc>& host_vector<T, Alloc>::operator=(const device_vector<T, DA>& d) {
   this->resize(d.size());
   d.copy_to_host(this->data());
   return *this;
 }
 
-template <typename T>
-inline bool operator==(const device_vector<T>& a, const device_vector<T>& b) {
+template <typename T, typename DA, typename DB>
+inline bool operator==(const device_vector<T, DA>& a, const device_vector<T, DB>& b) {
   return host_vector<T>(a) == host_vector<T>(b);
 }
-template <typename T, typename A>
-inline bool operator==(const device_vector<T>& a, const std::vector<T, A>& b) {
+template <typename T, typename DA, typename A>
+inline bool operator==(const device_vector<T, DA>& a, const std::vector<T, A>& b) {
   host_vector<T> h(a);
   return h.size() == b.size() && std::equal(h.begin(), h.end(), b.begin());
 }
-template <typename T, typename A>
-inline bool operator==(const std::vector<T, A>& a, const device_vector<T>& b) { return b == a; }
+template <typename T, typename DA, typename A>
+inline bool operator==(const std::vector<T, A>& a, const device_vector<T, DA>& b) { return b == a; }
 
 }  // namespace thrust

@@ -68,11 +68,44 @@ inline detail::temp_source get_temp_source(const allocator_policy<Alloc>& p) {
                              &detail::allocator_thunks<Alloc>::release};
 }
 
+// Policy carrying a memory resource for temporary storage: thrust::hip::par(&resource) with
+// resource a thrust::mr::memory_resource whose pointer is void* (device-accessible) or
+// device_ptr<void> (the reference accepts a resource pointer in the same place,
+// thrust/detail/allocator_aware_execution_policy.h:60-90).
+template <typename Resource>
+struct resource_policy : execution_policy<resource_policy<Resource> > {
+  Resource* resource;
+  void* stream;
+  explicit resource_policy(Resource* r, void* s = nullptr) : resource(r), stream(s) {}
+  resource_policy on(void* s) const { return resource_policy(resource, s); }
+};
+template <typename Resource>
+inline void* get_stream(const resource_policy<Resource>& p) { return p.stream; }
+namespace detail {
+template <typename Resource>
+struct resource_thunks {
+  static void* to_raw(void* p) { return p; }
+  template <typename P>
+  static void* to_raw(const P& p) { return p.get(); }
+  static void* acquire(void* ctx, std::size_t bytes) { return to_raw(static_cast<Resource*>(ctx)->allocate(bytes, 256)); }
+  static void release(void* ctx, void* p, std::size_t bytes) {
+    static_cast<Resource*>(ctx)->deallocate(typename Resource::pointer(p), bytes, 256);
+  }
+};
+}  // namespace detail
+template <typename Resource>
+inline detail::temp_source get_temp_source(const resource_policy<Resource>& p) {
+  return detail::temp_source{p.resource, &detail::resource_thunks<Resource>::acquire,
+                             &detail::resource_thunks<Resource>::release};
+}
+
 struct par_t : execution_policy<par_t> {
   // `stream` is a hipStream_t; it is taken as void* so that user code needs no HIP headers.
   stream_policy on(void* stream) const { return stream_policy(stream); }
   template <typename Alloc>
   allocator_policy<Alloc> operator()(Alloc& alloc) const { return allocator_policy<Alloc>(alloc); }
+  template <typename Resource>
+  resource_policy<Resource> operator()(Resource* resource) const { return resource_policy<Resource>(resource); }
   template <typename... Events>
   after_policy after(const Events&... events) const;  // defined in thrust/future.h
 };
@@ -99,6 +132,10 @@ struct device_t : thrust::device_execution_policy<device_t> {
   system::hip::stream_policy on(void* stream) const { return system::hip::stream_policy(stream); }
   template <typename Alloc>
   system::hip::allocator_policy<Alloc> operator()(Alloc& alloc) const { return system::hip::allocator_policy<Alloc>(alloc); }
+  template <typename Resource>
+  system::hip::resource_policy<Resource> operator()(Resource* resource) const {
+    return system::hip::resource_policy<Resource>(resource);
+  }
   template <typename... Events>
   system::hip::after_policy after(const Events&... events) const;  // defined in thrust/future.h
 };

@@ -6,7 +6,8 @@
 
 namespace thrust {
 
-template <typename T> class device_vector;
+template <typename T> class device_allocator;
+template <typename T, typename Alloc> class device_vector;
 
 template <typename T, typename Alloc = std::allocator<T> >
 class host_vector : public std::vector<T, Alloc> {
@@ -20,8 +21,10 @@ class host_vector : public std::vector<T, Alloc> {
   host_vector(host_vector&&) = default;
   host_vector& operator=(const host_vector&) = default;
   host_vector& operator=(host_vector&&) = default;
-  host_vector(const device_vector<T>& d);             // defined in device_vector.h
-  host_vector& operator=(const device_vector<T>& d);  // defined in device_vector.h
+  template <typename DA>
+  host_vector(const device_vector<T, DA>& d);             // defined in device_vector.h
+  template <typename DA>
+  host_vector& operator=(const device_vector<T, DA>& d);  // defined in device_vector.h
 };
 
 }  // namespace thrust

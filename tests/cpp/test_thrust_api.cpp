@@ -15,6 +15,7 @@
 #include <thrust/async/sort.h>
 #include <thrust/copy.h>
 #include <thrust/count.h>
+#include <thrust/device_allocator.h>
 #include <thrust/device_vector.h>
 #include <thrust/execution_policy.h>
 #include <thrust/fill.h>
@@ -23,6 +24,8 @@
 #include <thrust/host_vector.h>
 #include <thrust/inner_product.h>
 #include <thrust/merge.h>
+#include <thrust/mr/allocator.h>
+#include <thrust/mr/pool.h>
 #include <thrust/partition.h>
 #include <thrust/reduce.h>
 #include <thrust/remove.h>
@@ -60,8 +63,8 @@ static bool same(const A& a, const B& b) {
 
 template <typename T>
 static thrust::host_vector<T> hv(std::initializer_list<T> l) { return thrust::host_vector<T>(std::vector<T>(l)); }
-template <typename T>
-static thrust::host_vector<T> to_host(const thrust::device_vector<T>& d) { return thrust::host_vector<T>(d); }
+template <typename T, typename A>
+static thrust::host_vector<T> to_host(const thrust::device_vector<T, A>& d) { return thrust::host_vector<T>(d); }
 
 // deterministic inputs: an index hash, in the spirit of testing/unittest/random.h:12-21
 static uint64_t mix(uint64_t z) {
@@ -981,6 +984,80 @@ static void TestAsyncAlgorithms() {
   ASSERT_TRUE(thrust_amd_stream_destroy(user_stream) == 0);
 }
 
+// Memory resources, allocators over them and allocator-aware device_vector (the reference:
+// testing/mr_pool.cu, testing/allocator.cu, testing/caching_allocator.cu,
+// examples/mr_basic.cu).
+static void TestMemoryResources() {
+  g_test = "MemoryResources";
+  typedef thrust::mr::unsynchronized_pool_resource<thrust::device_memory_resource> Pool;
+  thrust::device_memory_resource upstream;
+  {
+    Pool pool(&upstream);
+    // the resource interface: blocks of a size class come back from the cache
+    thrust::device_ptr<void> a = pool.allocate(1000);
+    thrust::device_ptr<void> b = pool.allocate(1000);
+    ASSERT_TRUE(a.get() != nullptr && b.get() != nullptr && a.get() != b.get());
+    ASSERT_TRUE(pool.upstream_allocations() == 2);
+    pool.deallocate(a, 1000);
+    thrust::device_ptr<void> c = pool.allocate(900);  // same class (1024)
+    ASSERT_TRUE(c.get() == a.get() && pool.upstream_allocations() == 2);
+    pool.deallocate(b, 1000);
+    pool.deallocate(c, 900);
+    ASSERT_TRUE(pool.cached_bytes() == 2048);
+    pool.release();
+    ASSERT_TRUE(pool.cached_bytes() == 0);
+    ASSERT_TRUE(pool == pool && !(pool != pool));
+
+    // a vector over the pool: growing and shrinking reuses cached blocks
+    typedef thrust::mr::allocator<int, Pool> PoolAlloc;
+    PoolAlloc alloc(&pool);
+    const std::size_t before = pool.upstream_allocations();
+    {
+      thrust::device_vector<int, PoolAlloc> v(1000, 7, alloc);
+      ASSERT_TRUE(thrust::reduce(v.begin(), v.end()) == 7000);
+      thrust::host_vector<int> h = random_integers<int>(1000, 9, 0);
+      thrust::device_vector<int, PoolAlloc> w(alloc);
+      w = thrust::device_vector<int, PoolAlloc>(h.begin(), h.end(), alloc);
+      (void)w;
+    }
+    {
+      thrust::device_vector<int, PoolAlloc> v(1000, 1, alloc);  // the block the first vector returned
+      ASSERT_TRUE(pool.upstream_allocations() - before <= 2);
+      thrust::host_vector<int> h = random_integers<int>(1000, 9, 0), hs = h;
+      thrust::copy(h.begin(), h.end(), v.begin());
+      thrust::sort(v.begin(), v.end());
+      std::sort(hs.begin(), hs.end());
+      ASSERT_EQUAL_VEC(to_host(v), hs);
+      ASSERT_TRUE(v.get_allocator() == alloc);
+      // vectors with different allocators compare and convert
+      thrust::device_vector<int> plain(v);
+      ASSERT_TRUE(plain == v);
+    }
+    // temporary storage of the algorithms from the pool: thrust::device(&pool)
+    thrust::host_vector<int> h = random_integers<int>(1 << 16, 3, 0), hs = h;
+    std::sort(hs.begin(), hs.end());
+    thrust::device_vector<int> d = h;
+    const std::size_t before_sort = pool.upstream_allocations();
+    for (int round = 0; round < 3; ++round) {
+      d = h;
+      thrust::sort(thrust::device(&pool), d.begin(), d.end());
+      ASSERT_EQUAL_VEC(to_host(d), hs);
+    }
+    ASSERT_TRUE(pool.upstream_allocations() - before_sort == 1);  // one new block, reused twice
+    ASSERT_TRUE(thrust::reduce(thrust::hip::par(&pool).on(nullptr), d.begin(), d.end(), 0) ==
+                thrust::reduce(d.begin(), d.end(), 0));
+  }
+  // the default allocator: stateless, all instances equal, usable directly
+  thrust::device_allocator<int> da, db;
+  ASSERT_TRUE(da == db);
+  thrust::device_ptr<int> p = da.allocate(10);
+  thrust::fill(p, p + 10, 3);
+  ASSERT_TRUE(thrust::reduce(p, p + 10) == 30);
+  da.deallocate(p, 10);
+  thrust::device_vector<int> dv(5, 2);
+  ASSERT_TRUE(dv.get_allocator() == da);
+}
+
 int main() {
   TestReduceSimple();
   TestReduceWithOperatorTable();
@@ -1016,6 +1093,7 @@ int main() {
   TestTempArenaReuse();
   TestCustomTemporaryAllocation();
   TestAsyncAlgorithms();
+  TestMemoryResources();
   std::printf("%s: %d checks, %d failed\n", g_failed ? "FAILED" : "PASSED", g_checks, g_failed);
   return g_failed ? 1 : 0;
 }
