@@ -48,13 +48,18 @@ __global__ __launch_bounds__(256) void rbk_init_kernel(uint64_t* __restrict__ wo
 
 // K is the key's comparison class: an unsigned integer type of the key's size (integer
 // keys are equal iff their bits are) or float / double (operator==).
+//
+// Layout: a lane owns ITEMS = 16 consecutive elements (four 16-byte key vectors for 4-byte
+// keys), so the flags and the lane's fold are a serial pass over registers and the whole
+// tile needs ONE wave scan of pairs per wave.  (Lanes of a wave then read 16-byte pieces
+// 64 bytes apart; the four loads of a lane cover its cache lines completely.)
 template <typename K, typename V, typename Op>
 __global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
   constexpr int VEC = Vec16<K>::N;
   constexpr int CHUNKS = RBK_ITEMS / VEC >= 1 ? RBK_ITEMS / VEC : 1;
+  constexpr int ITEMS = CHUNKS * VEC;
   constexpr int WAVES = RBK_BLOCK / WAVE;
-  constexpr uint32_t WAVE_SPAN = WAVE * CHUNKS * VEC;
-  constexpr uint32_t TILE = WAVES * WAVE_SPAN;
+  constexpr uint32_t TILE = RBK_BLOCK * ITEMS;
   using WV = typename SegValue<V>::type;
   using Pair = SegPair<WV>;
   using VV = RbkValueVec<V, VEC>;
@@ -62,9 +67,18 @@ __global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
   const V vid = Op::template identity<V>();
   const Pair pid{0u, (WV)vid};
 
+  // Outputs of a tile with RBK_SPARSE .. RBK_STAGED runs are gathered in LDS and leave in
+  // coalesced stores.  A tile with more runs writes them directly (its run beginnings are
+  // dense, so neighbouring lanes write neighbouring addresses anyway), and so does a tile
+  // with very few (nothing to coalesce; its waves retire without another barrier).
+  constexpr uint32_t RBK_STAGED = 4096;
+  constexpr uint32_t RBK_SPARSE = 128;
   __shared__ uint32_t s_tile;
   __shared__ Pair s_wave_agg[WAVES];
   __shared__ Pair s_prefix;
+  __shared__ K s_keys_out[RBK_STAGED];
+  __shared__ V s_values_out[RBK_STAGED + 1];
+  __shared__ uint32_t s_first_is_head, s_last_is_tail;
 
   if (threadIdx.x == 0) s_tile = atomicAdd(a.ticket, 1u);
   __syncthreads();
@@ -73,72 +87,63 @@ __global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
   const uint32_t valid = (uint32_t)((a.n - tile_base < TILE) ? (a.n - tile_base) : TILE);
   const int wave = threadIdx.x / WAVE;
   const int lane = threadIdx.x % WAVE;
-  const uint32_t lane_off = wave * WAVE_SPAN + lane * VEC;
+  const uint32_t lane_off = threadIdx.x * ITEMS;
+  const uint64_t first = tile_base + lane_off;  // global index of the lane's first element
   const bool full = valid == TILE;
 
   // ---- load
-  Vec16<K> k[CHUNKS];
-  VV v[CHUNKS];
+  K k[ITEMS];
+  V v[ITEMS];
   if (full && a.aligned) {
+    Vec16<K> kv[CHUNKS];
+    VV vv[CHUNKS];
 #pragma unroll
     for (int j = 0; j < CHUNKS; ++j) {
-      const uint64_t off = tile_base + lane_off + j * (WAVE * VEC);
-      k[j] = *reinterpret_cast<const Vec16<K>*>(a.keys + off);
-      v[j] = *reinterpret_cast<const VV*>(a.values + off);
+      kv[j] = *reinterpret_cast<const Vec16<K>*>(a.keys + first + j * VEC);
+      vv[j] = *reinterpret_cast<const VV*>(a.values + first + j * VEC);
     }
-  } else {
 #pragma unroll
     for (int j = 0; j < CHUNKS; ++j) {
 #pragma unroll
       for (int i = 0; i < VEC; ++i) {
-        const uint32_t e = lane_off + j * (WAVE * VEC) + i;
-        k[j].v[i] = (e < valid) ? a.keys[tile_base + e] : K{};
-        v[j].v[i] = (e < valid) ? a.values[tile_base + e] : vid;
+        k[j * VEC + i] = kv[j].v[i];
+        v[j * VEC + i] = vv[j].v[i];
       }
+    }
+  } else {
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      const uint32_t e = lane_off + i;
+      k[i] = (e < valid) ? a.keys[tile_base + e] : K{};
+      v[i] = (e < valid) ? a.values[tile_base + e] : vid;
     }
   }
 
-  // ---- head / tail flags per chunk (bit i = element i), lane-local inclusive pairs
-  uint32_t head[CHUNKS], tail[CHUNKS];
-  Pair lane_excl[CHUNKS];
-  Pair carry = pid;
+  // ---- head / tail flags (bit i = element i) and the fold of the lane's elements
+  K prev = dpp_move<0x138 /* wave_shr:1 */>(k[ITEMS - 1], k[ITEMS - 1]);
+  K next = dpp_move<0x130 /* wave_shl:1 */>(k[0], k[0]);
+  if (lane == 0 && first > 0 && first < a.n) prev = a.keys[first - 1];
+  if (lane == WAVE - 1 && first + ITEMS < a.n) next = a.keys[first + ITEMS];
+  // differs[i]: element i differs from its predecessor; bit ITEMS: the lane's successor differs
+  uint32_t differs = 0;
 #pragma unroll
-  for (int j = 0; j < CHUNKS; ++j) {
-    const uint64_t first = tile_base + lane_off + j * (WAVE * VEC);
-    K prev = dpp_move<0x138 /* wave_shr:1 */>(k[j].v[VEC - 1], k[j].v[VEC - 1]);
-    K next = dpp_move<0x130 /* wave_shl:1 */>(k[j].v[0], k[j].v[0]);
-    bool first_of_all = false, last_of_all = false;
-    if (lane == 0) {
-      if (first == 0) first_of_all = true;
-      else if (first < a.n) prev = a.keys[first - 1];
-    }
-    if (lane == WAVE - 1) {
-      if (first + VEC < a.n) next = a.keys[first + VEC];
-    }
-    uint32_t h = 0, t = 0;
+  for (int i = 0; i < ITEMS; ++i) differs |= (uint32_t)(!(((i == 0) ? prev : k[i - 1]) == k[i])) << i;
+  differs |= (uint32_t)(!(k[ITEMS - 1] == next)) << ITEMS;
+  if (tile == 0 && threadIdx.x == 0) differs |= 1u;  // the very first element starts a run
+  const uint32_t live = (lane_off >= valid) ? 0u
+                        : ((valid - lane_off >= (uint32_t)ITEMS) ? ((1u << ITEMS) - 1u) : ((1u << (valid - lane_off)) - 1u));
+  // the very last element ends a run (it is in the last tile, at local index valid - 1)
+  const bool last_tile = tile_base + valid == a.n;
+  const uint32_t last_bit = (last_tile && valid - 1 >= lane_off && valid - 1 - lane_off < (uint32_t)ITEMS)
+                                ? (1u << (valid - 1 - lane_off)) : 0u;
+  const uint32_t head = differs & live;
+  const uint32_t tail = ((differs >> 1) | last_bit) & live;
+  Pair agg{head & 1u, (WV)v[0]};
 #pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      const uint64_t pos = first + i;
-      const K p = (i == 0) ? prev : k[j].v[i - 1];
-      const K nx = (i == VEC - 1) ? next : k[j].v[i + 1];
-      const bool in_range = pos < a.n;
-      const bool hd = in_range && ((i == 0 && first_of_all) || !(p == k[j].v[i]));
-      const bool tl = in_range && (pos + 1 == a.n || !(k[j].v[i] == nx));
-      h |= (uint32_t)hd << i;
-      t |= (uint32_t)tl << i;
-    }
-    (void)last_of_all;
-    head[j] = h;
-    tail[j] = t;
-    // fold of the lane's VEC elements
-    Pair agg{h & 1u, (WV)v[j].v[0]};
-#pragma unroll
-    for (int i = 1; i < VEC; ++i) agg = sop(agg, Pair{(h >> i) & 1u, (WV)v[j].v[i]});
-    const Pair incl = wave_inclusive_scan(agg, sop, pid);
-    lane_excl[j] = sop(carry, dpp_move<0x138>(pid, incl));
-    carry = sop(carry, readlane(incl, WAVE - 1));
-  }
-  if (lane == 0) s_wave_agg[wave] = carry;
+  for (int i = 1; i < ITEMS; ++i) agg = sop(agg, Pair{(head >> i) & 1u, (WV)v[i]});
+  const Pair incl = wave_inclusive_scan(agg, sop, pid);
+  const Pair lane_excl = dpp_move<0x138>(pid, incl);
+  if (lane == WAVE - 1) s_wave_agg[wave] = incl;
   __syncthreads();
   Pair wave_prefix = pid, tile_agg = pid;
 #pragma unroll
@@ -165,19 +170,38 @@ __global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
     }
   }
   __syncthreads();
-  const Pair before_wave = sop(s_prefix, wave_prefix);
 
   // ---- emit first keys at run beginnings, run totals at run ends
+  const uint32_t runs_before = s_prefix.heads;  // runs begun before this tile
+  const uint32_t tile_runs = tile_agg.heads;    // runs begun in this tile
+  Pair run = sop(sop(s_prefix, wave_prefix), lane_excl);
+  if (tile_runs > RBK_STAGED || tile_runs < RBK_SPARSE) {
 #pragma unroll
-  for (int j = 0; j < CHUNKS; ++j) {
-    Pair run = sop(before_wave, lane_excl[j]);
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      run = sop(run, Pair{(head[j] >> i) & 1u, (WV)v[j].v[i]});
-      if ((head[j] >> i) & 1u) a.keys_out[run.heads - 1] = k[j].v[i];
-      if ((tail[j] >> i) & 1u) a.values_out[run.heads - 1] = (V)run.value;
+    for (int i = 0; i < ITEMS; ++i) {
+      run = sop(run, Pair{(head >> i) & 1u, (WV)v[i]});
+      if ((head >> i) & 1u) a.keys_out[run.heads - 1] = k[i];
+      if ((tail >> i) & 1u) a.values_out[run.heads - 1] = (V)run.value;
     }
+    return;
   }
+  // Run r (global index) keeps its key in slot r - runs_before and its total in slot
+  // r - runs_before + 1: slot 0 of the totals belongs to a run that began in an earlier
+  // tile and ends here.
+  if (threadIdx.x == 0) s_first_is_head = head & 1u;
+  if (valid - 1 >= lane_off && valid - 1 - lane_off < (uint32_t)ITEMS) s_last_is_tail = (tail >> (valid - 1 - lane_off)) & 1u;
+#pragma unroll
+  for (int i = 0; i < ITEMS; ++i) {
+    run = sop(run, Pair{(head >> i) & 1u, (WV)v[i]});
+    if ((head >> i) & 1u) s_keys_out[run.heads - 1 - runs_before] = k[i];
+    if ((tail >> i) & 1u) s_values_out[run.heads - runs_before] = (V)run.value;
+  }
+  __syncthreads();
+  for (uint32_t j = threadIdx.x; j < tile_runs; j += RBK_BLOCK) a.keys_out[(uint64_t)runs_before + j] = s_keys_out[j];
+  // totals present: every run touched by the tile except a last one that goes on
+  const uint32_t lo = s_first_is_head ? 1u : 0u;
+  const uint32_t hi = s_last_is_tail ? tile_runs + 1u : tile_runs;  // exclusive
+  for (uint32_t j = lo + threadIdx.x; j < hi; j += RBK_BLOCK)
+    a.values_out[(uint64_t)runs_before + j - 1] = s_values_out[j];
 }
 
 template <typename K, typename V, typename Op>
