@@ -6,11 +6,14 @@
 
 namespace ta {
 
-// 16 elements per lane; the pair scan needs ~110 VGPRs, so a CU holds 16 waves.  For
+// 16 elements per lane; the pair scan needs ~105 VGPRs, so a CU holds 16 waves.  For
 // reduce_by_key one workgroup of 1024 threads measured best (large tiles keep the number of
-// tiles in flight, and the look-back, small: 0.73 against 0.77 ms with 512 threads at 2^28
+// tiles in flight, and the look-back, small: 0.69 against 0.72 ms with 512 threads at 2^28
 // pairs); scan_by_key, which also writes every element, prefers two workgroups of 512 that
-// overlap each other's load, scan and store phases (0.71 against 0.79 ms).
+// overlap each other's load, scan and store phases (0.71 against 0.79 ms).  reduce_by_key
+// gives each lane 16 consecutive elements (one pair scan per wave); scan_by_key keeps the
+// wave-striped vectors: with consecutive elements its 16-byte stores land 64 bytes apart
+// and the kernel measured 0.81 ms.
 constexpr int RBK_BLOCK = 1024;
 constexpr int SBK_BLOCK = 512;
 constexpr int RBK_ITEMS = 16;  // elements per lane
