@@ -90,18 +90,23 @@ pair<KOut, VOut> reduce_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, KOu
 }  // namespace cpp
 
 namespace hip {
+// The accumulator has the type of init; elements of another arithmetic type are converted
+// to it first, as plus<T> does in the reference (testing/reduce.cu:99-129).
 template <typename D, typename It, typename T, typename Op>
 T reduce(execution_policy<D>& exec, It first, It last, T init, Op) {
   typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
   static_assert(std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value,
                 "thrust::reduce on the device system needs device_ptr / device_vector iterators or raw device pointers");
-  static_assert(detail::is_abi_type<T>::value && std::is_same<V, T>::value,
-                "thrust::reduce on the device system: init must have the (arithmetic) element type");
+  static_assert(detail::is_abi_type<T>::value && detail::is_abi_type<V>::value,
+                "thrust::reduce on the device system: elements and init must have arithmetic types");
   static_assert(detail::binop_code<Op, T>::value >= 0,
-                "thrust::reduce on the device system supports thrust::plus, thrust::minimum and thrust::maximum");
+                "thrust::reduce on the device system supports thrust::plus, thrust::minimum and thrust::maximum "
+                "of the type of init");
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
-  const void* in = n ? (const void*)thrust::detail::raw(first) : nullptr;
+  detail::temp_storage converted(stream, detail::temp_source_of(exec));
+  const void* in = n ? (const void*)detail::input_as<T>(static_cast<const V*>(thrust::detail::raw(first)), n, stream, converted)
+                     : nullptr;
   detail::temp_storage temp(stream, detail::temp_source_of(exec));
   void* d_out = nullptr;
   // the result slot is the `extra` region, which run() only knows after the size query

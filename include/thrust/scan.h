@@ -152,32 +152,40 @@ Out exclusive_scan_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, Out resu
 
 namespace hip {
 namespace detail {
-template <typename In, typename Out, typename T, typename Op>
+// A is the accumulator's type: the input's element type for inclusive_scan, the type of
+// init for exclusive_scan; input and output may hold other arithmetic types, converted on
+// the way in and out as the reference does (testing/scan.cu:236-295).
+template <typename In, typename Out, typename A, typename Op>
 struct scan_checks {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  typedef typename iterator_value<Out>::type U;
   static_assert((std::is_pointer<In>::value || thrust::detail::is_device_iterator<In>::value) &&
                     (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value),
                 "scan on the device system needs device_ptr / device_vector iterators or raw device pointers");
-  static_assert(is_abi_type<V>::value && std::is_same<V, T>::value &&
-                    std::is_same<typename iterator_value<Out>::type, V>::value,
-                "scan on the device system: input, output and init must share one arithmetic type");
-  static_assert(binop_code<Op, V>::value >= 0,
-                "scan on the device system supports thrust::plus, thrust::minimum and thrust::maximum");
+  static_assert(is_abi_type<V>::value && is_abi_type<A>::value && is_abi_type<U>::value,
+                "scan on the device system: input, output and init must have arithmetic types");
+  static_assert(binop_code<Op, A>::value >= 0,
+                "scan on the device system supports thrust::plus, thrust::minimum and thrust::maximum "
+                "of the accumulator's type");
 };
 }  // namespace detail
 
 template <typename D, typename In, typename Out, typename Op>
 Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  typedef typename iterator_value<Out>::type U;
   (void)sizeof(detail::scan_checks<In, Out, V, Op>);
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
+  detail::temp_storage staged(stream, detail::temp_source_of(exec));
+  V* computed = detail::output_as<V>(static_cast<U*>(thrust::detail::raw(result)), n, staged);
   detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "inclusive_scan failed", [&](void* t, std::size_t* b) {
-    return thrust_amd_inclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
-                                     detail::dtype_of<V>::value, detail::binop_code<Op, V>::value, stream);
+    return thrust_amd_inclusive_scan(t, b, thrust::detail::raw(first), computed, n, detail::dtype_of<V>::value,
+                                     detail::binop_code<Op, V>::value, stream);
   });
+  detail::finish_output(computed, static_cast<U*>(thrust::detail::raw(result)), n, stream);
   detail::synchronize(stream, "inclusive_scan: synchronize");
   return result + n;
 }
@@ -185,15 +193,21 @@ Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op)
 template <typename D, typename In, typename Out, typename T, typename Op>
 Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T init, Op) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  typedef typename iterator_value<Out>::type U;
   (void)sizeof(detail::scan_checks<In, Out, T, Op>);
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
+  detail::temp_storage converted(stream, detail::temp_source_of(exec));
+  const T* in = detail::input_as<T>(static_cast<const V*>(thrust::detail::raw(first)), n, stream, converted);
+  detail::temp_storage staged(stream, detail::temp_source_of(exec));
+  T* computed = detail::output_as<T>(static_cast<U*>(thrust::detail::raw(result)), n, staged);
   detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "exclusive_scan failed", [&](void* t, std::size_t* b) {
-    return thrust_amd_exclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
-                                     detail::dtype_of<V>::value, detail::binop_code<Op, V>::value, &init, stream);
+    return thrust_amd_exclusive_scan(t, b, in, computed, n, detail::dtype_of<T>::value,
+                                     detail::binop_code<Op, T>::value, &init, stream);
   });
+  detail::finish_output(computed, static_cast<U*>(thrust::detail::raw(result)), n, stream);
   detail::synchronize(stream, "exclusive_scan: synchronize");
   return result + n;
 }

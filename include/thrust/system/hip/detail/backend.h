@@ -154,6 +154,52 @@ inline void* run(temp_storage& temp, std::size_t extra, const char* what, Call c
   return static_cast<char*>(temp.ptr()) + aligned;
 }
 
+// Mixed element types: the reference converts every element to the accumulator's type as
+// it is read and the result to the output's type as it is written.  Here the conversion is
+// a pass of its own into (out of) temporary storage; same types cost nothing.
+template <typename T, typename V>
+inline const T* input_as(const V* in, uint64_t, void*, temp_storage&, std::true_type) {
+  return in;
+}
+template <typename T, typename V>
+inline const T* input_as(const V* in, uint64_t n, void* stream, temp_storage& holder, std::false_type) {
+  static_assert(is_abi_type<T>::value && is_abi_type<V>::value, "mixed element types must both be arithmetic");
+  holder.ensure((std::size_t)n * sizeof(T));
+  throw_on_error(thrust_amd_convert(in, dtype_of<V>::value, holder.ptr(), dtype_of<T>::value, n, stream),
+                 "element type conversion failed");
+  return static_cast<const T*>(holder.ptr());
+}
+template <typename T, typename V>
+inline const T* input_as(const V* in, uint64_t n, void* stream, temp_storage& holder) {
+  return input_as<T>(in, n, stream, holder, std::is_same<T, V>());
+}
+// Where an algorithm that computes in T writes when the caller's output holds U.
+template <typename T, typename U>
+inline T* output_as(U* out, uint64_t, temp_storage&, std::true_type) {
+  return out;
+}
+template <typename T, typename U>
+inline T* output_as(U*, uint64_t n, temp_storage& holder, std::false_type) {
+  static_assert(is_abi_type<T>::value && is_abi_type<U>::value, "mixed element types must both be arithmetic");
+  holder.ensure((std::size_t)n * sizeof(T));
+  return static_cast<T*>(holder.ptr());
+}
+template <typename T, typename U>
+inline T* output_as(U* out, uint64_t n, temp_storage& holder) {
+  return output_as<T>(out, n, holder, std::is_same<T, U>());
+}
+template <typename T, typename U>
+inline void finish_output(const T*, U*, uint64_t, void*, std::true_type) {}
+template <typename T, typename U>
+inline void finish_output(const T* computed, U* out, uint64_t n, void* stream, std::false_type) {
+  throw_on_error(thrust_amd_convert(computed, dtype_of<T>::value, out, dtype_of<U>::value, n, stream),
+                 "element type conversion failed");
+}
+template <typename T, typename U>
+inline void finish_output(const T* computed, U* out, uint64_t n, void* stream) {
+  finish_output(computed, out, n, stream, std::is_same<T, U>());
+}
+
 inline void synchronize(void* stream, const char* what) {
   throw_on_error(thrust_amd_stream_synchronize(stream), what);
 }

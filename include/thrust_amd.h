@@ -128,6 +128,16 @@ int thrust_amd_memcpy(void* dst, const void* src, size_t bytes, int kind, void* 
  * cuda_cub::synchronize (thrust/system/cuda/detail/util.h:75-104). */
 int thrust_amd_stream_synchronize(void* stream);
 
+/* out[i] = (out_dtype)in[i] with the conversions of C++ (floating point to integer truncates
+ * toward zero).  The front end uses it where the reference's algorithms mix types: the
+ * accumulator of reduce and exclusive_scan has the type of init, that of inclusive_scan the
+ * input's type, and results are converted to the output's element type
+ * (thrust/system/detail/generic/reduce.inl:35-53, thrust/system/cuda/detail/scan.h:76-122;
+ * testing/reduce.cu:99-129, testing/scan.cu:236-295).  in and out must not overlap unless
+ * they are the same address and the types have the same size. */
+int thrust_amd_convert(const void* in, int in_dtype, void* out, int out_dtype, uint64_t n,
+                       void* stream);
+
 /* Streams and events for callers that overlap work (the asynchronous algorithms of the
  * front end).  A stream created here is independent of the null stream; an event is
  * recorded on one stream and another stream can be made to wait for it without blocking

@@ -205,6 +205,27 @@ class _Base:
                                             _p(out), *self._extra()), "inner_product")
         return out[0]
 
+    def convert(self, x, dtype):
+        x = _c(x)
+        out = np.empty(x.size, dtype)
+        self._ok(self._fn("convert")(_p(x), _code(x), _p(out), _code(out), ctypes.c_uint64(x.size)), "convert")
+        return out
+
+    # The reference's type rules for mixed element types (see oracle_convert).
+    def reduce_as(self, x, init, op=PLUS):
+        """reduce(first, last, init): the accumulator has init's type."""
+        init = np.asarray(init)
+        return self.reduce(self.convert(x, init.dtype), op, init[()])
+
+    def inclusive_scan_as(self, x, out_dtype, op=PLUS):
+        """inclusive_scan(first, last, result): accumulates in the input's type, converts on output."""
+        return self.convert(self.inclusive_scan(x, op), out_dtype)
+
+    def exclusive_scan_as(self, x, init, out_dtype, op=PLUS):
+        """exclusive_scan(first, last, result, init): accumulates in init's type, converts on output."""
+        init = np.asarray(init)
+        return self.convert(self.exclusive_scan(self.convert(x, init.dtype), init[()], op), out_dtype)
+
     def set_operation(self, op, a, b, descending=False):
         a, b = _c(a), _c(b)
         out = np.empty(a.size + b.size, a.dtype)
@@ -292,3 +313,30 @@ class Reference(_Base):
     def __init__(self, kind):
         super().__init__(REF_LIBS[kind])
         self.kind = kind
+
+    # The real mixed-type calls, int32 <-> float32 only: these run the reference's own type
+    # deduction, where the methods of the same names above restate it with conversions.
+    def reduce_as(self, x, init, op=PLUS):
+        x, init = _c(x), np.asarray(init)
+        if op != PLUS:
+            raise ValueError("the reference driver instantiates plus only for mixed types")
+        iv, out = np.array([init], init.dtype), np.empty(1, init.dtype)
+        self._ok(self._fn("reduce_mixed")(_p(x), _code(x), ctypes.c_uint64(x.size), _code(iv), _p(iv), _p(out)),
+                 "reduce_mixed")
+        return out[0]
+
+    def _scan_mixed(self, x, out_dtype, exclusive, init):
+        x = _c(x)
+        out = np.empty(x.size, out_dtype)
+        if {x.dtype, out.dtype} != {np.dtype(np.int32), np.dtype(np.float32)}:
+            raise ValueError("the reference driver instantiates int32 <-> float32 only")
+        iv = np.array([0 if init is None else init], np.int32 if init is None else np.asarray(init).dtype)
+        self._ok(self._fn("scan_mixed")(_p(x), _code(x), _p(out), ctypes.c_uint64(x.size), exclusive, _code(iv),
+                                        _p(iv)), "scan_mixed")
+        return out
+
+    def inclusive_scan_as(self, x, out_dtype, op=PLUS):
+        return self._scan_mixed(x, out_dtype, -1, None)
+
+    def exclusive_scan_as(self, x, init, out_dtype, op=PLUS):
+        return self._scan_mixed(x, out_dtype, 1, init)

@@ -320,6 +320,46 @@ REF_API int ref_inner_product(const void* a, const void* b, uint64_t n, int dtyp
   });
 }
 
+// Mixed element types through the real reference, for the pairs the tests use: x is int32
+// or float32, the other type is the other one of the two.
+REF_API int ref_convert(const void* in, int in_dtype, void* out, int out_dtype, uint64_t n) {
+  return with_dtype(in_dtype, [&](auto zi) {
+    using TI = decltype(zi);
+    return with_dtype(out_dtype, [&](auto zo) {
+      using TO = decltype(zo);
+      thrust::copy(thrust::device, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out));  // converting copy
+      return 0;
+    });
+  });
+}
+REF_API int ref_reduce_mixed(const void* in, int in_dtype, uint64_t n, int init_dtype, const void* init, void* out) {
+  if (in_dtype == THRUST_AMD_F32 && init_dtype == THRUST_AMD_I32)
+    *(int32_t*)out = thrust::reduce(thrust::device, dp<float>(in), dp<float>(in) + n, *(const int32_t*)init);
+  else if (in_dtype == THRUST_AMD_I32 && init_dtype == THRUST_AMD_F32)
+    *(float*)out = thrust::reduce(thrust::device, dp<int32_t>(in), dp<int32_t>(in) + n, *(const float*)init);
+  else
+    return -1;
+  return 0;
+}
+// inclusive_scan(in, out) and exclusive_scan(in, out, init) with out of the other type;
+// init has init_dtype (THRUST_AMD_I32 or THRUST_AMD_F32); exclusive < 0: inclusive scan
+REF_API int ref_scan_mixed(const void* in, int in_dtype, void* out, uint64_t n, int exclusive, int init_dtype,
+                           const void* init) {
+  auto run = [&](auto zi, auto zo) {
+    using TI = decltype(zi);
+    using TO = decltype(zo);
+    if (exclusive < 0) thrust::inclusive_scan(thrust::device, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out));
+    else if (init_dtype == THRUST_AMD_I32)
+      thrust::exclusive_scan(thrust::device, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out), *(const int32_t*)init);
+    else
+      thrust::exclusive_scan(thrust::device, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out), *(const float*)init);
+    return 0;
+  };
+  if (in_dtype == THRUST_AMD_F32) return run((float)0, (int32_t)0);
+  if (in_dtype == THRUST_AMD_I32) return run((int32_t)0, (float)0);
+  return -1;
+}
+
 namespace {
 // The real set operations; C is thrust::less<K> or thrust::greater<K>.
 template <typename K, typename C>

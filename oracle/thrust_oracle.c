@@ -445,6 +445,19 @@ ORACLE_API int oracle_count_if(const void* in, uint64_t n, int dtype, int cmp, c
   return 0;
 }
 
+/* Conversion between element types as C++'s static_cast does it (floating point to integer
+ * truncates toward zero), the conversion the reference's iterators and function objects
+ * apply where an algorithm mixes types: reduce's accumulator has the type of init and
+ * every element is converted to it before plus<T> adds (generic/reduce.inl:35-53 with
+ * functional.h:211-230), inclusive_scan accumulates in the input's type and converts on
+ * output, exclusive_scan accumulates in the type of init (sequential/scan.h:48-115). */
+ORACLE_API int oracle_convert(const void* in, int in_dtype, void* out, int out_dtype, uint64_t n) {
+#define BODY(S, T) return convert_from_##S((const T*)in, out, out_dtype, (size_t)n);
+  DISPATCH(in_dtype, BODY)
+#undef BODY
+  return -1;
+}
+
 /* The four set operations and their by-key forms; values are opaque items of value_bytes
  * that travel with the key the reference's tuple loop emits. */
 static int set_operation_impl(int op, const void* ka, uint64_t na, const void* kb, uint64_t nb,

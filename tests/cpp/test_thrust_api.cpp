@@ -65,6 +65,8 @@ template <typename T>
 static thrust::host_vector<T> hv(std::initializer_list<T> l) { return thrust::host_vector<T>(std::vector<T>(l)); }
 template <typename T, typename A>
 static thrust::host_vector<T> to_host(const thrust::device_vector<T, A>& d) { return thrust::host_vector<T>(d); }
+template <typename T>
+static thrust::host_vector<T> to_host(const thrust::host_vector<T>& h) { return h; }
 
 // deterministic inputs: an index hash, in the spirit of testing/unittest/random.h:12-21
 static uint64_t mix(uint64_t z) {
@@ -140,6 +142,60 @@ static void TestScanSimple() {  // testing/scan.cu:23-93
   input = in;
   thrust::exclusive_scan(input.begin(), input.end(), output.begin());
   ASSERT_EQUAL_VEC(to_host(output), hv<int>({0, 1, 4, 2, 6}));
+}
+
+// testing/reduce.cu:98-129 and testing/scan.cu:236-295: the accumulator is init's type for
+// reduce and exclusive_scan and the input's type for inclusive_scan; the plus<int>-on-float
+// case of the scan test is outside the device system's operator set and is left out.
+template <typename IntVector, typename FloatVector>
+static void MixedTypes() {
+  IntVector int_input(hv<int>({1, 2, 3, 4}));
+  FloatVector float_input(hv<float>({1.5f, 2.5f, 3.5f, 4.5f}));
+  ASSERT_TRUE(thrust::reduce(float_input.begin(), float_input.end(), (int)0) == 10);
+  ASSERT_TRUE(thrust::reduce(int_input.begin(), int_input.end(), (float)0.5) == 10.5f);
+
+  IntVector int_output(4);
+  FloatVector float_output(4);
+  thrust::inclusive_scan(float_input.begin(), float_input.end(), int_output.begin());
+  ASSERT_EQUAL_VEC(to_host(int_output), hv<int>({1, 4, 7, 12}));
+  thrust::exclusive_scan(float_input.begin(), float_input.end(), int_output.begin());
+  ASSERT_EQUAL_VEC(to_host(int_output), hv<int>({0, 1, 4, 7}));
+  thrust::exclusive_scan(float_input.begin(), float_input.end(), int_output.begin(), (float)5.5);
+  ASSERT_EQUAL_VEC(to_host(int_output), hv<int>({5, 7, 9, 13}));
+  thrust::inclusive_scan(int_input.begin(), int_input.end(), float_output.begin());
+  ASSERT_EQUAL_VEC(to_host(float_output), hv<float>({1.f, 3.f, 6.f, 10.f}));
+  thrust::exclusive_scan(int_input.begin(), int_input.end(), float_output.begin(), (float)5.5);
+  ASSERT_EQUAL_VEC(to_host(float_output), hv<float>({5.5f, 6.5f, 8.5f, 11.5f}));
+}
+
+static void TestMixedTypes() {
+  g_test = "MixedTypesHost";
+  MixedTypes<thrust::host_vector<int>, thrust::host_vector<float>>();
+  g_test = "MixedTypesDevice";
+  MixedTypes<thrust::device_vector<int>, thrust::device_vector<float>>();
+
+  // widening and narrowing at a size that spans several tiles, against the host system
+  g_test = "MixedTypesLarge";
+  const std::size_t n = 100003;
+  thrust::host_vector<short> h(n);
+  for (std::size_t i = 0; i < n; ++i) h[i] = (short)((i * 2654435761u >> 7) % 2001) - 1000;
+  thrust::device_vector<short> d(h);
+  ASSERT_TRUE(thrust::reduce(d.begin(), d.end(), (long long)5) == thrust::reduce(h.begin(), h.end(), (long long)5));
+  ASSERT_TRUE(thrust::reduce(d.begin(), d.end(), (long long)-7, thrust::maximum<long long>()) ==
+              thrust::reduce(h.begin(), h.end(), (long long)-7, thrust::maximum<long long>()));
+  thrust::host_vector<long long> h_wide(n);
+  thrust::device_vector<long long> d_wide(n);
+  thrust::exclusive_scan(h.begin(), h.end(), h_wide.begin(), (long long)1 << 40);
+  thrust::exclusive_scan(d.begin(), d.end(), d_wide.begin(), (long long)1 << 40);
+  ASSERT_EQUAL_VEC(to_host(d_wide), h_wide);
+  thrust::inclusive_scan(h.begin(), h.end(), h_wide.begin());  // short accumulator wraps, then widens
+  thrust::inclusive_scan(d.begin(), d.end(), d_wide.begin());
+  ASSERT_EQUAL_VEC(to_host(d_wide), h_wide);
+  thrust::host_vector<unsigned char> h_narrow(n);
+  thrust::device_vector<unsigned char> d_narrow(n);
+  thrust::exclusive_scan(h.begin(), h.end(), h_narrow.begin(), 3);  // int accumulator, bytes out
+  thrust::exclusive_scan(d.begin(), d.end(), d_narrow.begin(), 3);
+  ASSERT_EQUAL_VEC(to_host(d_narrow), h_narrow);
 }
 
 static void TestScanByKeySimple() {  // testing/scan_by_key.cu:9-60 and :121-180
@@ -1062,6 +1118,7 @@ int main() {
   TestReduceSimple();
   TestReduceWithOperatorTable();
   TestScanSimple();
+  TestMixedTypes();
   TestScanByKeySimple();
   TestCountSimple();
   TestInnerProductSimple();

@@ -104,6 +104,26 @@ def test_known_transform_reduce_and_scans(oracle):
         assert got.tolist() == c["out"]
 
 
+def test_known_mixed_types(oracle):
+    """testing/reduce.cu:98-129 and testing/scan.cu:236-297: which type accumulates."""
+    for c in KA["reduce_mixed"]:
+        init = np.dtype(c["init_dtype"]).type(c["init"])
+        got = oracle.reduce_as(np.array(c["in"], c["in_dtype"]), init)
+        assert got.dtype == init.dtype and got == c["out"], c["source"]
+    for c in KA["scan_mixed"]:
+        x = np.array(c["in"], c["in_dtype"])
+        if c["kind"] == "inclusive":
+            got = oracle.inclusive_scan_as(x, np.dtype(c["out_dtype"]))
+        else:
+            got = oracle.exclusive_scan_as(x, np.dtype(c["init_dtype"]).type(c["init"]), np.dtype(c["out_dtype"]))
+        assert got.dtype == np.dtype(c["out_dtype"]) and got.tolist() == c["out"], c["source"]
+    # conversions follow C's rules: truncation toward zero, wrap-around for narrower integers
+    assert oracle.convert(np.array([-1.9, -0.5, 0.5, 1.9, 126.99], np.float64), np.int8).tolist() == [-1, 0, 0, 1, 126]
+    assert oracle.convert(np.array([-1, 255, 256, 70000], np.int32), np.uint8).tolist() == [255, 255, 0, 112]
+    assert oracle.convert(np.array([-1, 3], np.int8), np.uint64).tolist() == [2 ** 64 - 1, 3]
+    assert oracle.convert(np.array([2 ** 24 + 1], np.int32), np.float32).tolist() == [float(2 ** 24)]
+
+
 def test_known_set_operations(oracle):
     codes = {"difference": cpu.SET_DIFFERENCE, "intersection": cpu.SET_INTERSECTION,
              "symmetric_difference": cpu.SET_SYMMETRIC_DIFFERENCE, "union": cpu.SET_UNION}
@@ -227,6 +247,23 @@ def test_oracle_matches_live_reference_on_ragged_sizes(oracle, oracle_seq):
                                     cpp.set_operation(op, sa[::-1].copy(), sb[::-1].copy(), True)), (dt, n, op)
                 x, y = oracle.set_operation_by_key(op, sa, sb, wa, wb), omp.set_operation_by_key(op, sa, sb, wa, wb)
                 assert _bytes_equal(x[0], y[0]) and np.array_equal(x[1], y[1]), (dt, n, op)
+        # mixed element types: the reference's own type deduction against the restated rule
+        fx = (datagen.u01(23, n) * 64 - 32).astype(np.float32)
+        ix = (datagen.splitmix64(29, n) % np.uint64(2001)).astype(np.int32) - np.int32(1000)
+        for ref in (omp, cpp):
+            assert oracle.reduce_as(fx, np.int32(7)) == ref.reduce_as(fx, np.int32(7)), n
+            assert _bytes_equal(oracle.exclusive_scan_as(ix, np.int32(3), np.float32), ref.exclusive_scan_as(ix, np.int32(3), np.float32))
+            assert _bytes_equal(oracle.inclusive_scan_as(ix, np.float32), ref.inclusive_scan_as(ix, np.float32))
+            for dt_in, dt_out in ((np.float32, np.int32), (np.int64, np.uint8), (np.uint16, np.float64), (np.float64, np.float32)):
+                src = (fx.astype(np.float64) * 1.37).astype(dt_in) if np.dtype(dt_in).kind == "f" else ix.astype(dt_in)
+                if np.dtype(dt_out).kind != "f" and np.dtype(dt_in).kind == "f":
+                    src = np.clip(src, -1e6, 1e6).astype(dt_in)
+                assert _bytes_equal(oracle.convert(src, dt_out), ref.convert(src, dt_out)), (dt_in, dt_out)
+        # float accumulators: one thread, so that the order of additions is the sequential one
+        assert oracle_seq.reduce_as(ix, np.float32(0.5)) == cpp.reduce_as(ix, np.float32(0.5)), n
+        assert _bytes_equal(oracle_seq.inclusive_scan_as(fx, np.int32), cpp.inclusive_scan_as(fx, np.int32))
+        assert _bytes_equal(oracle_seq.exclusive_scan_as(fx, np.float32(5.5), np.int32), cpp.exclusive_scan_as(fx, np.float32(5.5), np.int32))
+        assert _bytes_equal(oracle_seq.exclusive_scan_as(ix, np.float32(5.5), np.float32), cpp.exclusive_scan_as(ix, np.float32(5.5), np.float32))
         keys = np.sort((datagen.splitmix64(7, n) % np.uint64(50)).astype(np.int32))
         vals = datagen.u01(9, n)
         a, b = oracle.reduce_by_key(keys, vals), omp.reduce_by_key(keys, vals)

@@ -50,6 +50,7 @@ SIGNATURES = {
     "thrust_amd_temp_bytes_held": (_sz, []),
     "thrust_amd_profile_enable": (_int, [_int]),
     "thrust_amd_profile_collect": (_int, [_c.c_char_p, _sz, _szp]),
+    "thrust_amd_convert": (_int, [_vp, _int, _vp, _int, _u64, _vp]),
     "thrust_amd_stream_create": (_int, [ctypes.POINTER(_vp)]),
     "thrust_amd_stream_destroy": (_int, [_vp]),
     "thrust_amd_stream_query": (_int, [_vp, ctypes.POINTER(_int)]),
@@ -211,6 +212,12 @@ def reduce(x, op=PLUS, init=0, temp=None, out=None):
     iv = _scalar(x.dtype, init)
     _run("thrust_amd_reduce", temp, lambda fn, t, b: fn(
         t, b, x.ptr, x.n, x.dtype, op, iv.ctypes.data, out.ptr, stream_ptr()))
+    return out
+
+
+def convert(x, out_dtype, out=None):
+    out = out or DeviceArray(x.n, out_dtype)
+    check(load().thrust_amd_convert(x.ptr, x.dtype, out.ptr, out_dtype, x.n, stream_ptr()), "thrust_amd_convert")
     return out
 
 

@@ -161,6 +161,35 @@ TA_EXPORT int thrust_amd_fill(void* dst, uint64_t n, size_t elem_bytes, const vo
   });
 }
 
+namespace ta {
+template <typename In, typename Out>
+__global__ __launch_bounds__(256) void convert_kernel(const In* in, Out* out, uint64_t n) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = static_cast<Out>(in[i]);
+}
+}  // namespace ta
+
+TA_EXPORT int thrust_amd_convert(const void* in, int in_dtype, void* out, int out_dtype, uint64_t n,
+                                 void* stream) {
+  using namespace ta;
+  if (!valid_dtype(in_dtype) || !valid_dtype(out_dtype)) return (int)hipErrorInvalidValue;
+  if (n == 0) return 0;
+  if (!in || !out) return (int)hipErrorInvalidValue;
+  return with_dtype(in_dtype, [&](auto it) {
+    using In = typename decltype(it)::type;
+    return with_dtype(out_dtype, [&](auto ot) {
+      using Out = typename decltype(ot)::type;
+      uint64_t blocks = (n + 255) / 256;
+      const uint64_t cap = (uint64_t)NUM_CU * 32;
+      if (blocks > cap) blocks = cap;
+      TA_LAUNCH("convert", (hipStream_t)stream, (convert_kernel<In, Out>), dim3((uint32_t)blocks), dim3(256),
+                static_cast<const In*>(in), static_cast<Out*>(out), n);
+      TA_CHECK_LAUNCH();
+      return 0;
+    });
+  });
+}
+
 // ------------------------------------------------------------------ temp arena
 // Blocks are rounded up to size classes (powers of two from 4 KiB to 64 MiB, then
 // multiples of 64 MiB -- a 2^28-key radix sort needs ~1.2 GiB and must not round to
