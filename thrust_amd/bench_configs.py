@@ -108,6 +108,8 @@ def main():
                 lambda: capi.reduce_by_key(dk, dv, temp=t, keys_out=ko, values_out=vo), 8 * n + 8 * runs)
             run(f"C4 unique_by_key mean run {mean}",
                 lambda: capi.unique_by_key(dk, dv, keys_out=ko, values_out=vo, temp=t), 8 * n + 8 * runs)
+            run(f"C4 unique (keys only) mean run {mean}",
+                lambda: capi.unique(dk, out=ko, temp=t), 4 * n + 4 * runs)
             del keys, vals, dk, dv, ko, vo, t, u, lens
     if "c5" in which:
         x = torch.rand(n, device="cuda", generator=g)

@@ -8,9 +8,10 @@
 // and the exclusive prefix sum of the flags -- inside the lane, then across the wave with
 // DPP, across the waves through LDS, across tiles by decoupled look-back with a dynamic
 // tile ticket -- is the output position of each selected element; a rejected element goes
-// to (its index - selected before it) of the second output when there is one.  Elements
-// are written straight from registers: the selected elements of a wave's 1 KiB load are
-// contiguous in the output, so the partial-line stores of a wave meet in L2.
+// to (its index - selected before it) of the second output when there is one.  The selected
+// elements of a wave are contiguous in the output (and so are its rejected ones); each wave
+// compacts them in its own piece of LDS first, so that its store instructions cover
+// contiguous addresses.
 //
 // Outputs may alias inputs where the header says so: a tile learns its output offset
 // only after every earlier tile has published its count, and a tile publishes only after
@@ -29,8 +30,97 @@ namespace ta {
 
 enum SelectFlagMode { FLAG_PRED = 0, FLAG_HEAD = 1, FLAG_BYTE = 2 };
 
+// Two shapes.  Without a payload and with elements of up to four bytes, 16 elements per
+// lane keep the kernel within 64 registers, so two 1024-thread workgroups share a CU and
+// one loads while the other waits for its prefix: that beats a larger tile (measured:
+// copy_if of 2^28 float32 0.40 ms against 0.45 ms with 32 elements per lane).  Every other
+// combination needs more registers than that anyway and takes a larger tile (192 bytes of
+// input per lane, at most 32 elements: narrow elements are unpacked into a register each),
+// because every tile draws a ticket from one counter and waits for the prefix to travel
+// to it, and both costs are per tile (unique_by_key of int32 + float32: 0.63 -> 0.57 ms;
+// 512-thread workgroups for these shapes were slower, 0.63 ms).
 constexpr int SELECT_BLOCK = 1024;
-constexpr int SELECT_ITEMS = 16;  // elements per lane
+constexpr int SELECT_LEAN_ITEMS = 16;
+constexpr int SELECT_LANE_BYTES = 192;
+constexpr int SELECT_MIN_ITEMS = 8;   // sizes the descriptor array
+constexpr int SELECT_MAX_ITEMS = 32;
+
+template <typename T, typename U, bool HAS_PAYLOAD>
+struct SelectShape {
+  static constexpr int VEC = Vec16<T>::N;
+  static constexpr bool LEAN = !HAS_PAYLOAD && sizeof(T) <= 4;
+  static constexpr int BLOCK = SELECT_BLOCK;
+  // 8 = registers for two lean workgroups per CU (a few spilled registers in the head-flag
+  // form cost less than the second workgroup brings)
+  static constexpr int WAVES_PER_SIMD = LEAN ? 8 : 4;  // registers for two lean workgroups per CU
+  static constexpr int BY_BYTES = SELECT_LANE_BYTES / (int)(sizeof(T) + (HAS_PAYLOAD ? sizeof(U) : 0));
+  static constexpr int WANTED =
+      LEAN ? SELECT_LEAN_ITEMS
+           : (BY_BYTES < SELECT_MIN_ITEMS ? SELECT_MIN_ITEMS : (BY_BYTES > SELECT_MAX_ITEMS ? SELECT_MAX_ITEMS : BY_BYTES));
+  static constexpr int CHUNKS = WANTED / VEC >= 1 ? WANTED / VEC : 1;
+  static constexpr uint32_t TILE = (uint32_t)BLOCK * CHUNKS * VEC;
+  // LDS of one wave for the write-out: four 16-byte vectors per lane, or one chunk of the
+  // payload where that is more
+  static constexpr uint32_t PAYLOAD_CHUNK_BYTES = HAS_PAYLOAD ? (uint32_t)(WAVE * VEC * sizeof(U)) : 0u;
+  static constexpr uint32_t STAGE_BYTES = PAYLOAD_CHUNK_BYTES > 4096u ? PAYLOAD_CHUNK_BYTES : 4096u;
+};
+
+// Write-out of one stream of a wave through the wave's own LDS region.  The wave's
+// elements are handled in groups of G chunks: every lane drops its selected elements at
+// their rank inside the group and (when there is a second output) its rejected elements
+// behind them, in order; then consecutive lanes read consecutive slots, so that every
+// store instruction covers one contiguous piece of the output.  The region is private to
+// the wave and LDS executes a wave's instructions in order, so no barrier is needed
+// between the two steps, only a compiler fence.
+//   chunk_base[j]  selected elements of the wave before chunk j (wave-uniform)
+//   lane_excl[j]   selected elements of the wave before this lane's part of chunk j
+//   wave_valid     elements of the wave's span that exist (ragged last tile)
+//   out_true       where the wave's first selected element goes
+//   out_false      where the wave's first rejected element goes, or nullptr
+template <bool HAS_FALSE, int CHUNKS, int VEC, int G, typename S, typename Get>
+TA_DEVICE void select_emit(S* stage, const uint32_t (&fl)[CHUNKS], const uint32_t (&lane_excl)[CHUNKS],
+                           const uint32_t (&chunk_base)[CHUNKS + 1], int lane, uint32_t wave_valid,
+                           S* out_true, S* out_false, Get get) {
+  constexpr uint32_t CHUNK_ELEMS = WAVE * VEC;
+#pragma unroll
+  for (int g0 = 0; g0 < CHUNKS; g0 += G) {
+    const int ge = (CHUNKS - g0 < G) ? CHUNKS - g0 : G;
+    const uint32_t sel0 = chunk_base[g0];
+    const uint32_t sel_g = chunk_base[g0 + ge] - sel0;
+    const uint32_t e0 = (uint32_t)g0 * CHUNK_ELEMS;
+    const uint32_t left = wave_valid > e0 ? wave_valid - e0 : 0u;
+    const uint32_t e_cnt = left < (uint32_t)ge * CHUNK_ELEMS ? left : (uint32_t)ge * CHUNK_ELEMS;
+#pragma unroll
+    for (int jj = 0; jj < G; ++jj) {
+      const int j = g0 + jj;
+      if (j < CHUNKS) {
+        uint32_t r = lane_excl[j] - sel0;
+        // slot of a rejected element = sel_g + (its offset in the group) - (selected before it)
+        uint32_t rej = sel_g + (uint32_t)jj * CHUNK_ELEMS + (uint32_t)lane * VEC - r;
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          const bool sel = (fl[j] >> i) & 1u;
+          if constexpr (HAS_FALSE) {
+            const uint32_t e = (uint32_t)jj * CHUNK_ELEMS + (uint32_t)lane * VEC + i;
+            if (sel || e < e_cnt) stage[sel ? r : rej] = get(j, i);
+            rej += sel ? 0u : 1u;
+          } else {
+            if (sel) stage[r] = get(j, i);
+          }
+          r += sel ? 1u : 0u;
+        }
+      }
+    }
+    asm volatile("" ::: "memory");
+    const uint32_t limit = HAS_FALSE ? e_cnt : sel_g;
+    for (uint32_t slot = lane; slot < limit; slot += WAVE) {
+      const S v = stage[slot];
+      if (!HAS_FALSE || slot < sel_g) out_true[sel0 + slot] = v;
+      else out_false[(e0 - sel0) + (slot - sel_g)] = v;
+    }
+    asm volatile("" ::: "memory");
+  }
+}
 
 template <typename T, typename U>
 struct SelectArgs {
@@ -68,17 +158,20 @@ __global__ __launch_bounds__(256) void select_init_kernel(uint64_t* __restrict__
 }
 
 template <typename T, typename U, int MODE, bool HAS_PAYLOAD>
-__global__ __launch_bounds__(SELECT_BLOCK, 4) void select_kernel(SelectArgs<T, U> a) {
-  constexpr int VEC = Vec16<T>::N;
-  constexpr int CHUNKS = SELECT_ITEMS / VEC >= 1 ? SELECT_ITEMS / VEC : 1;
-  constexpr int WAVES = SELECT_BLOCK / WAVE;
+__global__ __launch_bounds__((SelectShape<T, U, HAS_PAYLOAD>::BLOCK), (SelectShape<T, U, HAS_PAYLOAD>::WAVES_PER_SIMD))
+void select_kernel(SelectArgs<T, U> a) {
+  using Shape = SelectShape<T, U, HAS_PAYLOAD>;
+  constexpr int VEC = Shape::VEC;
+  constexpr int CHUNKS = Shape::CHUNKS;
+  constexpr int WAVES = Shape::BLOCK / WAVE;
   constexpr uint32_t WAVE_SPAN = WAVE * CHUNKS * VEC;
-  constexpr uint32_t TILE = WAVES * WAVE_SPAN;
+  constexpr uint32_t TILE = Shape::TILE;
   using PV = PayloadVec<U, VEC>;
 
   __shared__ uint32_t s_tile;
   __shared__ uint32_t s_wave_cnt[WAVES];
   __shared__ uint64_t s_prefix;
+  __shared__ __attribute__((aligned(16))) unsigned char s_stage[(size_t)WAVES * Shape::STAGE_BYTES];
 
   if (threadIdx.x == 0) s_tile = atomicAdd(a.ticket, 1u);
   __syncthreads();
@@ -91,6 +184,13 @@ __global__ __launch_bounds__(SELECT_BLOCK, 4) void select_kernel(SelectArgs<T, U
   const bool full = valid == TILE;
 
   // ---- load
+  T wave_prev = T{};
+  if constexpr (MODE == FLAG_HEAD) {
+    // every lane reads the one element before the wave's span, unconditionally, so that
+    // this load is in flight together with the tile's
+    const uint64_t first = tile_base + (uint64_t)wave * WAVE_SPAN;
+    wave_prev = a.tested[(first > 0 && first < a.n) ? first - 1 : 0];
+  }
   Vec16<T> x[CHUNKS];
   PV y[HAS_PAYLOAD ? CHUNKS : 1];
   if (full && a.aligned) {
@@ -99,6 +199,18 @@ __global__ __launch_bounds__(SELECT_BLOCK, 4) void select_kernel(SelectArgs<T, U
       const uint64_t off = tile_base + lane_off + j * (WAVE * VEC);
       x[j] = *reinterpret_cast<const Vec16<T>*>(a.tested + off);
       if constexpr (HAS_PAYLOAD) y[j] = *reinterpret_cast<const PV*>(a.payload + off);
+    }
+  } else if (full) {
+    // pointers that do not allow whole vectors: element loads, still without predicates
+    // (a predicated load makes the compiler wait for it before issuing the next one)
+#pragma unroll
+    for (int j = 0; j < CHUNKS; ++j) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const uint64_t off = tile_base + lane_off + j * (WAVE * VEC) + i;
+        x[j].v[i] = a.tested[off];
+        if constexpr (HAS_PAYLOAD) y[j].v[i] = a.payload[off];
+      }
     }
   } else {
 #pragma unroll
@@ -117,14 +229,16 @@ __global__ __launch_bounds__(SELECT_BLOCK, 4) void select_kernel(SelectArgs<T, U
   if constexpr (MODE == FLAG_HEAD) {
 #pragma unroll
     for (int j = 0; j < CHUNKS; ++j) {
-      // predecessor of the lane's first element: last element of the previous lane, or,
-      // for lane 0, the element just before the wave's chunk in memory
+      // predecessor of the lane's first element: last element of the previous lane; for
+      // lane 0 the last element of the previous chunk (lane 63 holds it) or, for the first
+      // chunk, the element just before the wave's span, loaded with the tile
       T prev = dpp_move<0x138 /* wave_shr:1 */>(x[j].v[VEC - 1], x[j].v[VEC - 1]);
+      const T before = (j == 0) ? wave_prev : readlane(x[j > 0 ? j - 1 : 0].v[VEC - 1], WAVE - 1);
       const uint64_t first = tile_base + lane_off + j * (WAVE * VEC);
       bool head0 = false;
       if (lane == 0) {
         if (first == 0) head0 = true;
-        else if (first < a.n) prev = a.tested[first - 1];
+        else prev = before;
       }
       uint32_t f = 0;
 #pragma unroll
@@ -159,15 +273,16 @@ __global__ __launch_bounds__(SELECT_BLOCK, 4) void select_kernel(SelectArgs<T, U
 
   // ---- ranks: lane -> wave (DPP scans chained over the chunks) -> workgroup
   uint32_t lane_excl[CHUNKS];
-  uint32_t carry = 0;
+  uint32_t chunk_base[CHUNKS + 1];  // wave-uniform
+  chunk_base[0] = 0;
 #pragma unroll
   for (int j = 0; j < CHUNKS; ++j) {
     const uint32_t c = __builtin_popcount(fl[j]);
     const uint32_t incl = wave_inclusive_scan(c, OpPlus{});
-    lane_excl[j] = carry + dpp_move<0x138>(0u, incl);
-    carry += readlane(incl, WAVE - 1);
+    lane_excl[j] = chunk_base[j] + dpp_move<0x138>(0u, incl);
+    chunk_base[j + 1] = chunk_base[j] + readlane(incl, WAVE - 1);
   }
-  if (lane == 0) s_wave_cnt[wave] = carry;
+  if (lane == 0) s_wave_cnt[wave] = chunk_base[CHUNKS];
   // every load of this wave has returned before the tile's count can become visible:
   // in-place callers rely on it (see the file comment)
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -197,35 +312,30 @@ __global__ __launch_bounds__(SELECT_BLOCK, 4) void select_kernel(SelectArgs<T, U
     }
   }
   __syncthreads();
-  const uint64_t true_base = s_prefix + wave_prefix;  // + rank inside the wave
-  // a rejected element at tile offset e with r selected elements before it in the tile
+  // the wave's selected elements start at s_prefix + wave_prefix of the first output; a
+  // rejected element at tile offset e with r selected elements before it in the tile
   // lands at (tile_base - s_prefix) + e - r of the second output
-  const uint64_t false_base = tile_base - s_prefix;
-  const bool want_false = (a.tested_false != nullptr) || (HAS_PAYLOAD && a.payload_false != nullptr);
+  const uint64_t true_base = s_prefix + wave_prefix;
+  const uint32_t wave_e0 = (uint32_t)wave * WAVE_SPAN;
+  const uint64_t false_base = tile_base - s_prefix + wave_e0 - wave_prefix;
+  const uint32_t wave_valid = valid > wave_e0 ? (valid - wave_e0 < WAVE_SPAN ? valid - wave_e0 : WAVE_SPAN) : 0u;
 
-  // ---- scatter straight from registers
-#pragma unroll
-  for (int j = 0; j < CHUNKS; ++j) {
-    uint32_t r = lane_excl[j];
-#pragma unroll
-    for (int i = 0; i < VEC; ++i) {
-      const bool sel = (fl[j] >> i) & 1u;
-      if (sel) {
-        const uint64_t pos = true_base + r;
-        if (a.tested_true) a.tested_true[pos] = x[j].v[i];
-        if constexpr (HAS_PAYLOAD) a.payload_true[pos] = y[j].v[i];
-        ++r;
-      } else if (want_false) {
-        const uint32_t e = lane_off + j * (WAVE * VEC) + i;
-        if (e < valid) {
-          const uint64_t pos = false_base + e - (wave_prefix + r);
-          if (a.tested_false) a.tested_false[pos] = x[j].v[i];
-          if constexpr (HAS_PAYLOAD)
-            if (a.payload_false) a.payload_false[pos] = y[j].v[i];
-        }
-      }
-    }
-  }
+  // ---- write-out
+  auto emit = [&](auto* out_true, auto* out_false, auto get) {
+    using S = std::remove_pointer_t<decltype(out_true)>;
+    constexpr int G = (int)(Shape::STAGE_BYTES / (WAVE * VEC * sizeof(S)));
+    S* stage = reinterpret_cast<S*>(s_stage + (size_t)wave * Shape::STAGE_BYTES);
+    if (out_false)
+      select_emit<true, CHUNKS, VEC, G>(stage, fl, lane_excl, chunk_base, lane, wave_valid, out_true, out_false, get);
+    else
+      select_emit<false, CHUNKS, VEC, G>(stage, fl, lane_excl, chunk_base, lane, wave_valid, out_true, out_false, get);
+  };
+  if (a.tested_true)
+    emit(a.tested_true + true_base, a.tested_false ? a.tested_false + false_base : (T*)nullptr,
+         [&](int j, int i) { return x[j].v[i]; });
+  if constexpr (HAS_PAYLOAD)
+    emit(a.payload_true + true_base, a.payload_false ? a.payload_false + false_base : (U*)nullptr,
+         [&](int j, int i) { return y[j].v[i]; });
 }
 
 // Stencil forms: flags[i] = stencil[i] CMP threshold as one byte each.
@@ -240,6 +350,8 @@ __global__ __launch_bounds__(256) void select_flag_kernel(const T* __restrict__ 
 
 // Second step of the in-place partition: the rejected elements, parked in temp storage
 // in order, move behind the selected ones.
+// Plain element copies: 16-byte stores on the destination's grid with loads that are only
+// element-aligned were measured slower (0.48 against 0.45 ms for 0.95 * 2^28 float32).
 template <typename U>
 __global__ __launch_bounds__(256) void partition_tail_kernel(U* __restrict__ data,
                                                              const U* __restrict__ parked,
@@ -257,11 +369,12 @@ struct SelectTemp {
   uint64_t tiles;
 };
 
+// Sized for the smallest tile any payload type leads to, so that the temp size does not
+// depend on the payload; the launch uses the tile count of its own shape.
 template <typename T>
 static SelectTemp select_layout(uint64_t n, size_t extra_bytes) {
   constexpr int VEC = Vec16<T>::N;
-  constexpr int CHUNKS = SELECT_ITEMS / VEC >= 1 ? SELECT_ITEMS / VEC : 1;
-  constexpr uint64_t TILE = (uint64_t)SELECT_BLOCK * CHUNKS * VEC;
+  constexpr uint64_t TILE = (uint64_t)SELECT_BLOCK * (VEC > SELECT_MIN_ITEMS ? VEC : SELECT_MIN_ITEMS);
   SelectTemp t;
   t.tiles = (n + TILE - 1) / TILE;
   TempLayout lay;
@@ -274,20 +387,22 @@ static SelectTemp select_layout(uint64_t n, size_t extra_bytes) {
 
 template <typename T, typename U, int MODE, bool HAS_PAYLOAD>
 static int select_launch(char* temp, const SelectTemp& lay, SelectArgs<T, U> a, hipStream_t stream) {
-  if (lay.tiles > 0xffffffffull) return (int)hipErrorInvalidValue;
+  constexpr uint64_t TILE = SelectShape<T, U, HAS_PAYLOAD>::TILE;
+  const uint64_t tiles = (a.n + TILE - 1) / TILE;
+  if (tiles > 0xffffffffull || tiles > lay.tiles) return (int)hipErrorInvalidValue;
   a.ticket = reinterpret_cast<uint32_t*>(temp + lay.off_ticket);
   a.status = reinterpret_cast<uint64_t*>(temp + lay.off_status);
   constexpr size_t PAY_ALIGN = alignof(PayloadVec<U, Vec16<T>::N>);
   a.aligned = is_aligned16(a.tested) &&
               (!HAS_PAYLOAD || (reinterpret_cast<uintptr_t>(a.payload) % PAY_ALIGN) == 0);
-  const uint64_t words = lay.tiles * TileWords<uint64_t>::W;
+  const uint64_t words = tiles * TileWords<uint64_t>::W;
   const uint64_t init_threads = words ? words : 1;
   TA_LAUNCH("select_init", stream, select_init_kernel, dim3((uint32_t)((init_threads + 255) / 256)),
             dim3(256), a.status, words, a.ticket, a.d_num_true);
   TA_CHECK_LAUNCH();
   if (a.n == 0) return 0;
-  TA_LAUNCH("select", stream, (select_kernel<T, U, MODE, HAS_PAYLOAD>), dim3((uint32_t)lay.tiles),
-            dim3(SELECT_BLOCK), a);
+  TA_LAUNCH("select", stream, (select_kernel<T, U, MODE, HAS_PAYLOAD>), dim3((uint32_t)tiles),
+            dim3(SelectShape<T, U, HAS_PAYLOAD>::BLOCK), a);
   TA_CHECK_LAUNCH();
   return 0;
 }
