@@ -282,6 +282,21 @@ int thrust_amd_sort_pairs(void* temp, size_t* temp_bytes, void* keys, void* valu
                           int key_dtype, size_t value_bytes, int descending, int begin_bit,
                           int end_bit, void* stream);
 
+/* Stable comparison sort (merge sort) by operator< (descending != 0: operator>), the path
+ * thrust::sort takes when the comparator is not thrust::less / thrust::greater of an
+ * arithmetic key.  The order is the comparison's, not the bit pattern's: for floating-point
+ * keys -0.0 and +0.0 are equivalent and keep their input order (the radix entry points put
+ * -0.0 first); NaN keys are outside a strict weak order and not supported.  Same temp
+ * convention; n * (key + value) bytes of temp plus 8 bytes per 4096 elements.
+ * The kernels are the templates of include/thrust/system/hip/detail/merge_sort_kernels.h,
+ * which a translation unit compiled with hipcc instantiates for its own comparators.
+ * Replaces cuda_cub::__merge_sort::merge_sort (thrust/system/cuda/detail/sort.h:1278-1322;
+ * BlockSortAgent :235-633, PartitionAgent :638-694, MergeAgent :701-1138). */
+int thrust_amd_merge_sort_keys(void* temp, size_t* temp_bytes, void* keys, uint64_t n, int key_dtype,
+                               int descending, void* stream);
+int thrust_amd_merge_sort_pairs(void* temp, size_t* temp_bytes, void* keys, void* values, uint64_t n,
+                                int key_dtype, size_t value_bytes, int descending, void* stream);
+
 /* ---------------------------------------------------------- set operations */
 
 /* out = a OP b for two ranges sorted by operator< (descending != 0: by operator>), OP a

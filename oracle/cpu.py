@@ -25,6 +25,7 @@ NP_DTYPES = {I8: np.int8, U8: np.uint8, I16: np.int16, U16: np.uint16, I32: np.i
 DTYPE_OF_NP = {np.dtype(v): k for k, v in NP_DTYPES.items()}
 PLUS, MIN, MAX = range(3)
 LT, LE, GT, GE, EQ, NE, NONZERO = range(7)
+CMP_SORT_LESS, CMP_SORT_GREATER, CMP_SORT_LESS_DIV = 0, 1, 2
 IDENTITY, NEGATE, SQUARE = range(3)
 SET_DIFFERENCE, SET_INTERSECTION, SET_SYMMETRIC_DIFFERENCE, SET_UNION = range(4)
 
@@ -225,6 +226,15 @@ class _Base:
         """exclusive_scan(first, last, result, init): accumulates in init's type, converts on output."""
         init = np.asarray(init)
         return self.convert(self.exclusive_scan(self.convert(x, init.dtype), init[()], op), out_dtype)
+
+    def comparison_sort(self, keys, values=None, comparator=CMP_SORT_LESS, param=0):
+        """stable_sort(_by_key) with a user comparator: returns sorted copies."""
+        k = _c(keys).copy()
+        v = None if values is None else _c(values).copy()
+        self._ok(self._fn("comparison_sort")(_p(k), _p(v) if v is not None else None, ctypes.c_uint64(k.size),
+                                              _code(k), ctypes.c_uint64(0 if v is None else v.itemsize),
+                                              int(comparator), ctypes.c_long(int(param))), "comparison_sort")
+        return k if v is None else (k, v)
 
     def set_operation(self, op, a, b, descending=False):
         a, b = _c(a), _c(b)

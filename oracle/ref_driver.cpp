@@ -158,6 +158,45 @@ REF_API int ref_sort_pairs(void* keys, void* values, uint64_t n, int dtype, uint
   });
 }
 
+namespace {
+// User-defined comparators: not thrust::less / thrust::greater, so the reference takes its
+// comparison sort (sequential/sort.inl:103-197 via the OMP system's intervals).
+template <typename T> struct user_less {
+  __host__ __device__ bool operator()(const T& a, const T& b) const { return a < b; }
+};
+template <typename T> struct user_greater {
+  __host__ __device__ bool operator()(const T& a, const T& b) const { return b < a; }
+};
+template <typename T> struct user_less_div {  // testing/stable_sort.cu:43-47 with a parameter
+  int d;
+  __host__ __device__ bool operator()(const T& a, const T& b) const { return ((int)a) / d < ((int)b) / d; }
+};
+template <typename T, typename C>
+void comparison_sort(void* keys, void* values, uint64_t n, uint64_t value_bytes, C comp) {
+  if (!values) {
+    thrust::stable_sort(thrust::device, dp<T>(keys), dp<T>(keys) + n, comp);
+    return;
+  }
+  with_bytes(value_bytes, [&](auto vz) {
+    using V = decltype(vz);
+    thrust::stable_sort_by_key(thrust::device, dp<T>(keys), dp<T>(keys) + n, dp<V>(values), comp);
+    return 0;
+  });
+}
+}  // namespace
+
+REF_API int ref_comparison_sort(void* keys, void* values, uint64_t n, int dtype, uint64_t value_bytes,
+                                int comparator, long param) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    if (comparator == 0) comparison_sort<T>(keys, values, n, value_bytes, user_less<T>());
+    else if (comparator == 1) comparison_sort<T>(keys, values, n, value_bytes, user_greater<T>());
+    else if (comparator == 2 && param != 0) comparison_sort<T>(keys, values, n, value_bytes, user_less_div<T>{(int)param});
+    else return -1;
+    return 0;
+  });
+}
+
 REF_API int ref_merge(const void* a, uint64_t na, const void* b, uint64_t nb, void* out, int dtype,
                       int descending) {
   return with_dtype(dtype, [&](auto z) {

@@ -246,6 +246,33 @@ ORACLE_API int oracle_sort_pairs(void* keys, void* values, uint64_t n, int dtype
   return 0;
 }
 
+/* stable_sort(_by_key) with a comparator that is not less / greater of a primitive key: the
+ * OMP and CPP systems both end in the sequential merge sort for each interval
+ * (sequential/sort.inl:103-197 -> stable_merge_sort.inl); any stable sort gives the same
+ * result, so the one-interval form is restated.  comparator: 0 operator<, 1 operator>,
+ * 2 less_div(param).  values == NULL: keys only. */
+ORACLE_API int oracle_comparison_sort(void* keys, void* values, uint64_t n, int dtype, uint64_t value_bytes,
+                                      int comparator, long param) {
+  if (comparator < 0 || comparator > 2 || (comparator == 2 && param == 0)) return -1;
+  if (n == 0) return 0;
+  size_t* perm = NULL;
+  if (values) {
+    perm = (size_t*)malloc((size_t)n * sizeof(size_t));
+    for (size_t i = 0; i < n; i++) perm[i] = i;
+  }
+#define BODY(S, T) comparison_sort_##S((T*)keys, perm, (size_t)n, comparator, param);
+  DISPATCH(dtype, BODY)
+#undef BODY
+  if (values) {
+    void* tmp = malloc((size_t)n * value_bytes);
+    memcpy(tmp, values, (size_t)n * value_bytes);
+    gather_bytes(tmp, perm, (size_t)n, value_bytes, values);
+    free(tmp);
+    free(perm);
+  }
+  return 0;
+}
+
 /* sequential::merge(_by_key) -- the OMP system inherits it (omp/detail/merge.h:21-22). */
 ORACLE_API int oracle_merge_by_key(const void* ka, uint64_t na, const void* kb, uint64_t nb,
                                    const void* va, const void* vb, void* kout, void* vout,

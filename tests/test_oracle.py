@@ -124,6 +124,38 @@ def test_known_mixed_types(oracle):
     assert oracle.convert(np.array([2 ** 24 + 1], np.int32), np.float32).tolist() == [float(2 ** 24)]
 
 
+def test_known_comparison_sort(oracle):
+    """testing/stable_sort.cu:49-90, stable_sort_by_key.cu:50-95: less_div_10 keeps the input order of equivalents."""
+    kinds = {"less": cpu.CMP_SORT_LESS, "greater": cpu.CMP_SORT_GREATER, "less_div": cpu.CMP_SORT_LESS_DIV}
+    for c in KA["comparison_sort"]:
+        keys = np.array(c["keys"], I32)
+        if "values" in c:
+            k, v = oracle.comparison_sort(keys, np.array(c["values"], np.uint32), kinds[c["comparator"]], c["param"])
+            assert k.tolist() == c["keys_out"] and v.tolist() == c["values_out"], c["source"]
+        else:
+            assert oracle.comparison_sort(keys, None, kinds[c["comparator"]], c["param"]).tolist() == c["keys_out"], c["source"]
+
+
+def test_comparison_sort_against_numpy_stable_sort(oracle):
+    """Stability fixes the answer: numpy's stable argsort of the comparator's key gives the same permutation."""
+    for dtype in (np.int8, np.uint16, np.int32, np.uint64, np.float32, np.float64):
+        for n in (0, 1, 31, 32, 33, 64, 65, 1000, 50001):
+            x = ((datagen.splitmix64(71, n) % np.uint64(97)).astype(np.int64) - (0 if np.dtype(dtype).kind == "u" else 48)).astype(dtype)
+            v = np.arange(n, dtype=np.uint32)
+            k, w = oracle.comparison_sort(x, v, cpu.CMP_SORT_LESS)
+            order = np.argsort(x, kind="stable")
+            assert np.array_equal(w, order.astype(np.uint32)) and np.array_equal(k, x[order]), (dtype, n)
+            k, w = oracle.comparison_sort(x, v, cpu.CMP_SORT_GREATER)
+            order = np.argsort(-x.astype(np.float64), kind="stable")
+            assert np.array_equal(w, order.astype(np.uint32)) and np.array_equal(k, x[order]), (dtype, n)
+            k, w = oracle.comparison_sort(x, v, cpu.CMP_SORT_LESS_DIV, 10)
+            order = np.argsort(np.trunc(x.astype(np.float64) / 10), kind="stable")  # C division truncates
+            assert np.array_equal(w, order.astype(np.uint32)) and np.array_equal(k, x[order]), (dtype, n)
+    # -0.0 and +0.0 are equivalent under operator< and keep their input order
+    z = np.array([0.0, -0.0, 1.0, -0.0, 0.0, -1.0], np.float32)
+    assert oracle.comparison_sort(z).tobytes() == np.array([-1.0, 0.0, -0.0, -0.0, 0.0, 1.0], np.float32).tobytes()
+
+
 def test_known_set_operations(oracle):
     codes = {"difference": cpu.SET_DIFFERENCE, "intersection": cpu.SET_INTERSECTION,
              "symmetric_difference": cpu.SET_SYMMETRIC_DIFFERENCE, "union": cpu.SET_UNION}
@@ -247,6 +279,16 @@ def test_oracle_matches_live_reference_on_ragged_sizes(oracle, oracle_seq):
                                     cpp.set_operation(op, sa[::-1].copy(), sb[::-1].copy(), True)), (dt, n, op)
                 x, y = oracle.set_operation_by_key(op, sa, sb, wa, wb), omp.set_operation_by_key(op, sa, sb, wa, wb)
                 assert _bytes_equal(x[0], y[0]) and np.array_equal(x[1], y[1]), (dt, n, op)
+        # comparison sort: user-defined comparators take the reference's merge sort
+        cx = (datagen.splitmix64(31, n) % np.uint64(199)).astype(np.int32) - np.int32(99)
+        cf = np.where(datagen.u01(33, n) < 0.1, np.float32(-0.0), cx.astype(np.float32) / 4).astype(np.float32)
+        cv = np.arange(n, dtype=np.uint32)
+        for ref in (omp, cpp):
+            for comparator, param in ((cpu.CMP_SORT_LESS, 0), (cpu.CMP_SORT_GREATER, 0), (cpu.CMP_SORT_LESS_DIV, 10)):
+                for keys in (cx, cf, cx.astype(np.int8), cx.astype(np.int64)):
+                    x, y = oracle.comparison_sort(keys, cv, comparator, param), ref.comparison_sort(keys, cv, comparator, param)
+                    assert _bytes_equal(x[0], y[0]) and np.array_equal(x[1], y[1]), (n, comparator, keys.dtype)
+                assert _bytes_equal(oracle.comparison_sort(cf, None, comparator, param), ref.comparison_sort(cf, None, comparator, param))
         # mixed element types: the reference's own type deduction against the restated rule
         fx = (datagen.u01(23, n) * 64 - 32).astype(np.float32)
         ix = (datagen.splitmix64(29, n) % np.uint64(2001)).astype(np.int32) - np.int32(1000)

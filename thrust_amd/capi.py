@@ -73,6 +73,8 @@ SIGNATURES = {
                                                _int, _sz, _int, _vp]),
     "thrust_amd_sort_keys": (_int, [_vp, _szp, _vp, _u64, _int, _int, _int, _int, _vp]),
     "thrust_amd_sort_pairs": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _sz, _int, _int, _int, _vp]),
+    "thrust_amd_merge_sort_keys": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp]),
+    "thrust_amd_merge_sort_pairs": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _sz, _int, _vp]),
     "thrust_amd_copy_if": (_int, [_vp, _szp, _vp, _vp, _vp, _vp, _u64, _sz, _int, _int, _vp, _vp]),
     "thrust_amd_partition_copy": (_int, [_vp, _szp, _vp, _vp, _vp, _vp, _vp, _u64, _sz, _int, _int, _vp, _vp]),
     "thrust_amd_stable_partition": (_int, [_vp, _szp, _vp, _vp, _vp, _u64, _sz, _int, _int, _vp, _vp]),
@@ -302,6 +304,17 @@ def sort_pairs(keys, values, descending=False, begin_bit=0, end_bit=None, temp=N
     return _run("thrust_amd_sort_pairs", temp, lambda fn, t, b: fn(
         t, b, keys.ptr, values.ptr, keys.n, keys.dtype, values.itemsize, int(descending),
         begin_bit, end_bit, stream_ptr()))
+
+
+def merge_sort_keys(keys, descending=False, temp=None):
+    """Stable comparison sort in place (operator< / operator>)."""
+    return _run("thrust_amd_merge_sort_keys", temp, lambda fn, t, b: fn(
+        t, b, keys.ptr, keys.n, keys.dtype, int(descending), stream_ptr()))
+
+
+def merge_sort_pairs(keys, values, descending=False, temp=None):
+    return _run("thrust_amd_merge_sort_pairs", temp, lambda fn, t, b: fn(
+        t, b, keys.ptr, values.ptr, keys.n, keys.dtype, values.itemsize, int(descending), stream_ptr()))
 
 
 def _count(dev_u64):
