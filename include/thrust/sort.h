@@ -4,8 +4,11 @@
 // (thrust/system/detail/generic/sort.inl:57-64).  The device system takes the radix path
 // for arithmetic keys with exactly thrust::less or thrust::greater -- the reference's own
 // condition for its primitive sort (thrust/system/detail/sequential/sort.inl:139-148,
-// thrust/system/cuda/detail/sort.h:1518-1523); other comparators are not available on
-// the device system yet and fail to compile with a message.
+// thrust/system/cuda/detail/sort.h:1518-1523).  Every other comparator or key type takes
+// the stable merge sort, as in the reference (cuda/detail/sort.h:1278-1322).  Its kernels
+// are templates on the comparator, so that path exists in translation units compiled
+// with hipcc (the comparator must be callable on the device: __host__ __device__); a
+// translation unit compiled by a plain host compiler stops there with a message.
 #pragma once
 #include <algorithm>
 #include <numeric>
@@ -13,6 +16,9 @@
 
 #include <thrust/functional.h>
 #include <thrust/system/hip/detail/backend.h>
+#if defined(__HIPCC__)
+#include <thrust/system/hip/detail/merge_sort_kernels.h>
+#endif
 
 namespace thrust {
 
@@ -78,40 +84,85 @@ void stable_sort_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, Comp comp)
 }  // namespace cpp
 
 namespace hip {
+namespace detail {
+// true: arithmetic key ordered by thrust::less / thrust::greater -> radix sort through the C ABI
+template <typename K, typename Comp, bool = is_abi_type<K>::value>
+struct takes_radix_path : std::integral_constant<bool, (order_code<Comp, K>::value >= 0)> {};
+template <typename K, typename Comp>
+struct takes_radix_path<K, Comp, false> : std::false_type {};
+
+template <typename T>
+struct needs_hipcc : std::false_type {};
+
+template <typename K, typename Comp>
+void sort_keys(void* stream, temp_source source, K* keys, uint64_t n, Comp, std::true_type) {
+  temp_storage temp(stream, source);
+  run(temp, 0, "sort failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_sort_keys(t, b, keys, n, dtype_of<K>::value, order_code<Comp, K>::value, 0,
+                                (int)sizeof(K) * 8, stream);
+  });
+}
+template <typename K, typename V, typename Comp>
+void sort_pairs(void* stream, temp_source source, K* keys, V* values, uint64_t n, Comp, std::true_type) {
+  static_assert(is_abi_item<V>::value, "sort_by_key on the device system supports values of 1, 2, 4 or 8 bytes");
+  temp_storage temp(stream, source);
+  run(temp, 0, "sort_by_key failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_sort_pairs(t, b, keys, values, n, dtype_of<K>::value, sizeof(V), order_code<Comp, K>::value, 0,
+                                 (int)sizeof(K) * 8, stream);
+  });
+}
+#if defined(__HIPCC__)
+template <typename K, typename Comp>
+void sort_keys(void* stream, temp_source source, K* keys, uint64_t n, Comp comp, std::false_type) {
+  temp_storage temp(stream, source);
+  run(temp, 0, "sort (comparison path) failed", [&](void* t, std::size_t* b) {
+    return thrust::system::hip::merge_sort::sort<K, unsigned, false>(t, b, keys, (unsigned*)nullptr, n, comp,
+                                                                     (hipStream_t)stream);
+  });
+}
+template <typename K, typename V, typename Comp>
+void sort_pairs(void* stream, temp_source source, K* keys, V* values, uint64_t n, Comp comp, std::false_type) {
+  temp_storage temp(stream, source);
+  run(temp, 0, "sort_by_key (comparison path) failed", [&](void* t, std::size_t* b) {
+    return thrust::system::hip::merge_sort::sort<K, V, true>(t, b, keys, values, n, comp, (hipStream_t)stream);
+  });
+}
+#else
+template <typename K, typename Comp>
+void sort_keys(void*, temp_source, K*, uint64_t, Comp, std::false_type) {
+  static_assert(needs_hipcc<Comp>::value,
+                "sort on the device system: comparators other than thrust::less / thrust::greater of an arithmetic "
+                "key run as kernels instantiated for the comparator; compile this translation unit with hipcc");
+}
+template <typename K, typename V, typename Comp>
+void sort_pairs(void*, temp_source, K*, V*, uint64_t, Comp, std::false_type) {
+  static_assert(needs_hipcc<Comp>::value,
+                "sort_by_key on the device system: comparators other than thrust::less / thrust::greater of an "
+                "arithmetic key run as kernels instantiated for the comparator; compile this translation unit with hipcc");
+}
+#endif
+}  // namespace detail
+
 template <typename D, typename It, typename Comp>
-void stable_sort(execution_policy<D>& exec, It first, It last, Comp) {
+void stable_sort(execution_policy<D>& exec, It first, It last, Comp comp) {
   typedef typename iterator_value<It>::type K;
   static_assert(std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value,
                 "sort on the device system needs device_ptr / device_vector iterators or raw device pointers");
-  static_assert(detail::is_abi_type<K>::value && detail::order_code<Comp, K>::value >= 0,
-                "sort on the device system supports arithmetic keys ordered by thrust::less or thrust::greater");
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n < 2) return;
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
-  detail::run(temp, 0, "sort failed", [&](void* t, std::size_t* b) {
-    return thrust_amd_sort_keys(t, b, thrust::detail::raw(first), n, detail::dtype_of<K>::value,
-                                detail::order_code<Comp, K>::value, 0, (int)sizeof(K) * 8, stream);
-  });
+  detail::sort_keys(stream, detail::temp_source_of(exec), thrust::detail::raw(first), n, comp,
+                    detail::takes_radix_path<K, Comp>());
   detail::synchronize(stream, "sort: synchronize");
 }
 template <typename D, typename KIt, typename VIt, typename Comp>
-void stable_sort_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Comp) {
+void stable_sort_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Comp comp) {
   typedef typename iterator_value<KIt>::type K;
-  typedef typename iterator_value<VIt>::type V;
-  static_assert(detail::is_abi_type<K>::value && detail::order_code<Comp, K>::value >= 0,
-                "sort_by_key on the device system supports arithmetic keys ordered by thrust::less or thrust::greater");
-  static_assert(detail::is_abi_item<V>::value,
-                "sort_by_key on the device system supports values of 1, 2, 4 or 8 bytes");
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n < 2) return;
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
-  detail::run(temp, 0, "sort_by_key failed", [&](void* t, std::size_t* b) {
-    return thrust_amd_sort_pairs(t, b, thrust::detail::raw(kf), thrust::detail::raw(vf), n,
-                                 detail::dtype_of<K>::value, sizeof(V), detail::order_code<Comp, K>::value, 0,
-                                 (int)sizeof(K) * 8, stream);
-  });
+  detail::sort_pairs(stream, detail::temp_source_of(exec), thrust::detail::raw(kf), thrust::detail::raw(vf), n, comp,
+                     detail::takes_radix_path<K, Comp>());
   detail::synchronize(stream, "sort_by_key: synchronize");
 }
 }  // namespace hip

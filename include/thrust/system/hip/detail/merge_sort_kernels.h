@@ -71,17 +71,25 @@ __global__ __launch_bounds__(BLOCK) void block_sort_kernel(const K* keys_in, con
   const uint32_t run0 = tid * ITEMS;
 
   // ---- coalesced load, then every lane picks up its ITEMS consecutive elements
+  K k[ITEMS];
+  V v[HAS_VALUES ? ITEMS : 1];
 #pragma unroll
   for (int q = 0; q < ITEMS; ++q) {
     const uint32_t e = (uint32_t)q * BLOCK + tid;
     if (e < valid) {
-      s_keys[slot_of(e)] = keys_in[tile_base + e];
-      if constexpr (HAS_VALUES) s_vals[slot_of(e)] = vals_in[tile_base + e];
+      k[q] = keys_in[tile_base + e];
+      if constexpr (HAS_VALUES) v[q] = vals_in[tile_base + e];
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < ITEMS; ++q) {
+    const uint32_t e = (uint32_t)q * BLOCK + tid;
+    if (e < valid) {
+      s_keys[slot_of(e)] = k[q];
+      if constexpr (HAS_VALUES) s_vals[slot_of(e)] = v[q];
     }
   }
   __syncthreads();
-  K k[ITEMS];
-  V v[HAS_VALUES ? ITEMS : 1];
 #pragma unroll
   for (int i = 0; i < ITEMS; ++i) {
     const uint32_t e = run0 + i;
@@ -231,11 +239,19 @@ __global__ __launch_bounds__(BLOCK) void merge_pass_kernel(const K* keys_in, con
   const K* b = keys_in + p.b_begin + b0;
   const uint64_t out_base = p.a_begin + p.out0;
 
-  // ---- stage the keys: A's piece first, then B's
+  // ---- stage the keys: A's piece first, then B's (all loads issued before the first LDS write)
+  {
+    K in[ITEMS];
 #pragma unroll
-  for (int q = 0; q < ITEMS; ++q) {
-    const uint32_t e = (uint32_t)q * BLOCK + tid;
-    if (e < count) s_keys[e] = (e < ca) ? a[e] : b[e - ca];
+    for (int q = 0; q < ITEMS; ++q) {
+      const uint32_t e = (uint32_t)q * BLOCK + tid;
+      if (e < count) in[q] = (e < ca) ? a[e] : b[e - ca];
+    }
+#pragma unroll
+    for (int q = 0; q < ITEMS; ++q) {
+      const uint32_t e = (uint32_t)q * BLOCK + tid;
+      if (e < count) s_keys[e] = in[q];
+    }
   }
   __syncthreads();
 
@@ -276,10 +292,18 @@ __global__ __launch_bounds__(BLOCK) void merge_pass_kernel(const K* keys_in, con
     const V* va = vals_in + p.a_begin + a0;
     const V* vb = vals_in + p.b_begin + b0;
     __syncthreads();  // the key write-out has read the exchange buffer
+    {
+      V in[ITEMS];
 #pragma unroll
-    for (int q = 0; q < ITEMS; ++q) {
-      const uint32_t e = (uint32_t)q * BLOCK + tid;
-      if (e < count) s_vals[e] = (e < ca) ? va[e] : vb[e - ca];
+      for (int q = 0; q < ITEMS; ++q) {
+        const uint32_t e = (uint32_t)q * BLOCK + tid;
+        if (e < count) in[q] = (e < ca) ? va[e] : vb[e - ca];
+      }
+#pragma unroll
+      for (int q = 0; q < ITEMS; ++q) {
+        const uint32_t e = (uint32_t)q * BLOCK + tid;
+        if (e < count) s_vals[e] = in[q];
+      }
     }
     __syncthreads();
     V v[ITEMS];

@@ -1,0 +1,184 @@
+// Front-end test compiled with hipcc: thrust::sort / stable_sort / sort_by_key with user
+// comparators and a struct key take the comparison (merge sort) path, whose kernels are
+// instantiated in this translation unit.  Known answers are the reference's:
+// testing/stable_sort.cu:49-90 (less_div_10), :125-173 (comparator with an external table),
+// testing/stable_sort_by_key.cu:50-95; the rest is the reference's host-against-device
+// differential pattern (testing/stable_sort.cu:93-108) over its size list.
+#include <thrust/device_vector.h>
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/host_vector.h>
+#include <thrust/sort.h>
+
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdint>
+#include <cstdio>
+#include <vector>
+
+static int g_failed = 0, g_checks = 0;
+static const char* g_test = "";
+#define ASSERT_TRUE(c)                                                                    \
+  do {                                                                                    \
+    ++g_checks;                                                                           \
+    if (!(c)) { ++g_failed; std::printf("FAIL [%s] %s:%d: %s\n", g_test, __FILE__, __LINE__, #c); } \
+  } while (0)
+
+template <typename A, typename B>
+static bool same(const A& a, const B& b) {
+  if (a.size() != b.size()) return false;
+  for (size_t i = 0; i < a.size(); ++i)
+    if (!(a[i] == b[i])) return false;
+  return true;
+}
+template <typename T>
+static thrust::host_vector<T> hv(std::initializer_list<T> l) { return thrust::host_vector<T>(std::vector<T>(l)); }
+template <typename T>
+static thrust::host_vector<T> to_host(const thrust::device_vector<T>& d) { return thrust::host_vector<T>(d); }
+
+static uint64_t mix(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+
+template <typename T>
+struct less_div_10 {
+  __host__ __device__ bool operator()(const T& lhs, const T& rhs) const { return ((int)lhs) / 10 < ((int)rhs) / 10; }
+};
+template <typename T>
+struct comp_mod3 {
+  const T* table;
+  __host__ __device__ bool operator()(T a, T b) const { return table[(int)a] < table[(int)b]; }
+};
+template <typename T>
+struct my_greater {
+  __host__ __device__ bool operator()(const T& a, const T& b) const { return b < a; }
+};
+
+struct Record {  // a key that is not arithmetic
+  int group;
+  float weight;
+  __host__ __device__ bool operator==(const Record& o) const { return group == o.group && weight == o.weight; }
+};
+struct by_group_then_heavier {
+  __host__ __device__ bool operator()(const Record& a, const Record& b) const {
+    return a.group != b.group ? a.group < b.group : b.weight < a.weight;
+  }
+};
+struct by_group {
+  __host__ __device__ bool operator()(const Record& a, const Record& b) const { return a.group < b.group; }
+};
+
+static const size_t kSizes[] = {0, 1, 2, 3, 15, 16, 17, 31, 32, 33, 255, 256, 257, 1023, 1024, 1025, 4095, 4096, 4097,
+                                8191, 8192, 8193, 12293, 16384, 20485, 65533, 65536, 65539, 300007};
+
+static void TestKnownAnswers() {
+  g_test = "StableSortSimple";
+  thrust::device_vector<int> keys(hv<int>({25, 14, 35, 16, 26, 34, 36, 24, 15}));
+  thrust::stable_sort(keys.begin(), keys.end(), less_div_10<int>());
+  ASSERT_TRUE(same(to_host(keys), hv<int>({14, 16, 15, 25, 26, 24, 35, 34, 36})));
+
+  g_test = "StableSortByKeySimple";
+  thrust::device_vector<int> k2(hv<int>({25, 14, 35, 16, 26, 34, 36, 24, 15}));
+  thrust::device_vector<int> v2(hv<int>({0, 1, 2, 3, 4, 5, 6, 7, 8}));
+  thrust::stable_sort_by_key(k2.begin(), k2.end(), v2.begin(), less_div_10<int>());
+  ASSERT_TRUE(same(to_host(k2), hv<int>({14, 16, 15, 25, 26, 24, 35, 34, 36})));
+  ASSERT_TRUE(same(to_host(v2), hv<int>({1, 3, 8, 0, 4, 7, 2, 5, 6})));
+
+  g_test = "StableSortWithIndirection";
+  thrust::device_vector<int> data(hv<int>({1, 3, 5, 3, 0, 2, 1}));
+  thrust::device_vector<int> table(hv<int>({0, 1, 2, 0, 1, 2}));
+  thrust::stable_sort(data.begin(), data.end(), comp_mod3<int>{thrust::raw_pointer_cast(table.data())});
+  ASSERT_TRUE(same(to_host(data), hv<int>({3, 3, 0, 1, 1, 5, 2})));
+
+  g_test = "SortWithUserGreater";
+  thrust::device_vector<int> d(hv<int>({1, 3, 6, 5, 2, 0, 4}));
+  thrust::sort(thrust::device, d.begin(), d.end(), my_greater<int>());
+  ASSERT_TRUE(same(to_host(d), hv<int>({6, 5, 4, 3, 2, 1, 0})));
+}
+
+template <typename T>
+static void Differential(const char* name) {
+  g_test = name;
+  for (size_t n : kSizes) {
+    thrust::host_vector<T> h(n);
+    thrust::host_vector<unsigned> hvls(n);
+    for (size_t i = 0; i < n; ++i) {
+      h[i] = (T)(mix(17 * n + i) % 201);
+      hvls[i] = (unsigned)i;
+    }
+    thrust::device_vector<T> d(h);
+    thrust::stable_sort(h.begin(), h.end(), less_div_10<T>());
+    thrust::stable_sort(d.begin(), d.end(), less_div_10<T>());
+    ASSERT_TRUE(same(to_host(d), h));
+
+    for (size_t i = 0; i < n; ++i) h[i] = (T)(mix(29 * n + i) % 57);
+    d = h;
+    thrust::device_vector<unsigned> dv(hvls);
+    thrust::sort_by_key(h.begin(), h.end(), hvls.begin(), my_greater<T>());
+    thrust::sort_by_key(d.begin(), d.end(), dv.begin(), my_greater<T>());
+    ASSERT_TRUE(same(to_host(d), h));
+    ASSERT_TRUE(same(to_host(dv), hvls));
+  }
+}
+
+static void TestStructKeys() {
+  g_test = "StructKeys";
+  for (size_t n : kSizes) {
+    std::vector<Record> h(n);
+    for (size_t i = 0; i < n; ++i) h[i] = Record{(int)(mix(i + 3 * n) % 23), (float)(mix(i + 7 * n) % 1000) / 8.0f};
+    Record* dptr = nullptr;
+    unsigned long long* dval = nullptr;
+    if (n) {
+      dptr = thrust::raw_pointer_cast(thrust::device_malloc<Record>(n));
+      dval = thrust::raw_pointer_cast(thrust::device_malloc<unsigned long long>(n));
+    }
+    std::vector<unsigned long long> hval(n);
+    for (size_t i = 0; i < n; ++i) hval[i] = i;
+    if (n) {
+      (void)hipMemcpy(dptr, h.data(), n * sizeof(Record), hipMemcpyHostToDevice);
+      (void)hipMemcpy(dval, hval.data(), n * sizeof(unsigned long long), hipMemcpyHostToDevice);
+    }
+    // total order on the struct
+    thrust::sort(thrust::device, dptr, dptr + n, by_group_then_heavier());
+    std::vector<Record> want(h);
+    std::stable_sort(want.begin(), want.end(), by_group_then_heavier());
+    std::vector<Record> got(n);
+    if (n) (void)hipMemcpy(got.data(), dptr, n * sizeof(Record), hipMemcpyDeviceToHost);
+    ASSERT_TRUE(same(got, want));
+    // a partial order with 8-byte values: stability decides
+    if (n) (void)hipMemcpy(dptr, h.data(), n * sizeof(Record), hipMemcpyHostToDevice);
+    thrust::stable_sort_by_key(thrust::device, dptr, dptr + n, dval, by_group());
+    std::vector<size_t> order(n);
+    for (size_t i = 0; i < n; ++i) order[i] = i;
+    std::stable_sort(order.begin(), order.end(), [&](size_t a, size_t b) { return h[a].group < h[b].group; });
+    std::vector<unsigned long long> gotv(n);
+    if (n) {
+      (void)hipMemcpy(got.data(), dptr, n * sizeof(Record), hipMemcpyDeviceToHost);
+      (void)hipMemcpy(gotv.data(), dval, n * sizeof(unsigned long long), hipMemcpyDeviceToHost);
+    }
+    bool ok = true;
+    for (size_t i = 0; i < n; ++i) ok = ok && got[i] == h[order[i]] && gotv[i] == order[i];
+    ASSERT_TRUE(ok);
+    if (n) {
+      thrust::device_free(thrust::device_pointer_cast(dptr));
+      thrust::device_free(thrust::device_pointer_cast(dval));
+    }
+  }
+}
+
+int main() {
+  TestKnownAnswers();
+  Differential<signed char>("signed char");
+  Differential<short>("short");
+  Differential<int>("int");
+  Differential<long long>("long long");
+  Differential<float>("float");
+  TestStructKeys();
+  std::printf("%d checks, %d failed\n", g_checks, g_failed);
+  std::printf(g_failed ? "FAILED\n" : "PASSED\n");
+  return g_failed ? 1 : 0;
+}

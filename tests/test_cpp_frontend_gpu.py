@@ -1,7 +1,7 @@
 """Runs the C++ front-end test programs (the thrust:: API over the C ABI) on the GPU.
 
 The programs are built by tests/cpp/Makefile (driven by __graft_entry__.build) with the
-plain host compiler; they replay the reference's literal known-answer vectors and its
+plain host compiler (one of them, for user comparators, with hipcc); they replay the reference's literal known-answer vectors and its
 host-vs-device differential pattern through device_vector.
 """
 import os
@@ -32,3 +32,9 @@ def test_thrust_api_known_answers_and_differential():
 def test_c_abi_from_plain_c():
     out = _run("test_thrust_c11")
     assert "PASS" in out
+
+
+def test_user_comparators_and_struct_keys_compiled_with_hipcc():
+    # thrust::sort with user comparators: the merge sort kernels are instantiated in the test's own translation unit
+    out = _run("test_user_comparator")
+    assert "PASSED" in out

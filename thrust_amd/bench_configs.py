@@ -16,9 +16,12 @@ with the algorithmic bytes of the call and the resulting fraction of the 8 TB/s 
 
   C7  the four set operations on two sorted ranges of 2^27 uint32 with runs of about four
       and two equal keys (bytes: both inputs read, the result written)
+  C8  the stable comparison sort (merge sort) of 2^28 uint32 keys and of 2^27 uint64 keys
+      with uint32 values (bytes: one block sort and ceil(log2(n / 4096)) merge passes, each
+      reading and writing every element)
 
 Inputs are generated on the device from a seeded generator.  Usage:
-  python3 thrust_amd/bench_configs.py [c2] [c3] [c4] [c5] [c6] [c7]
+  python3 thrust_amd/bench_configs.py [c2] [c3] [c4] [c5] [c6] [c7] [c8]
 """
 import os
 import sys
@@ -37,7 +40,7 @@ def main():
     if not torch.cuda.is_available():
         raise SystemExit("bench_configs.py needs a GPU")
     capi.load()
-    which = [a.lower() for a in sys.argv[1:]] or ["c2", "c3", "c4", "c5", "c6", "c7"]
+    which = [a.lower() for a in sys.argv[1:]] or ["c2", "c3", "c4", "c5", "c6", "c7", "c8"]
     g = torch.Generator(device="cuda")
     g.manual_seed(1)
 
@@ -181,6 +184,26 @@ def main():
         run("C7 set_union_by_key 2 x 2^27 u32+u32",
             lambda: capi.set_operation_by_key(3, da, db, dva, dvb, keys_out=out, values_out=vo, temp=t2),
             4 * (2 * m + cnt) + 8 * cnt, extra=f"{cnt} out")
+        del ka, kb, da, db, out, t, va, dva, dvb, vo, t2
+    if "c8" in which:
+        def passes(count):
+            return 1 + int(np.ceil(np.log2(max(1.0, count / 4096))))
+        r = torch.randint(-(1 << 31), 1 << 31, (n,), dtype=torch.int32, device="cuda", generator=g)
+        src, work, t = dev(r, capi.U32), capi.DeviceArray(n, capi.U32), capi.Temp()
+        run("C8 comparison sort u32 2^28", lambda: capi.merge_sort_keys(work, temp=t), passes(n) * 8 * n,
+            setup=lambda: work.storage.copy_(src.storage), extra=f"{passes(n)} x 8 B/key")
+        del r, src, work, t
+        m = 1 << 27
+        r = torch.randint(-(1 << 62), 1 << 62, (m,), dtype=torch.int64, device="cuda", generator=g)
+        v = torch.arange(m, dtype=torch.int32, device="cuda")
+        sk, sv = dev(r, capi.U64), dev(v, capi.U32)
+        wk, wv, t = capi.DeviceArray(m, capi.U64), capi.DeviceArray(m, capi.U32), capi.Temp()
+
+        def setup():
+            wk.storage.copy_(sk.storage)
+            wv.storage.copy_(sv.storage)
+        run("C8 comparison sort_by_key u64+u32 2^27", lambda: capi.merge_sort_pairs(wk, wv, temp=t),
+            passes(m) * 24 * m, setup=setup, extra=f"{passes(m)} x 24 B/pair")
 
 
 if __name__ == "__main__":
