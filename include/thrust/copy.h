@@ -10,7 +10,9 @@
 #include <vector>
 
 #include <thrust/functional.h>
+#include <thrust/iterator/transform_iterator.h>
 #include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/device_input.h>
 
 namespace thrust {
 
@@ -87,12 +89,51 @@ Out copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred)
 }  // namespace cpp
 
 namespace hip {
+namespace detail {
 template <typename D, typename In, typename Out>
-Out copy(execution_policy<D>& exec, In first, In last, Out result) {
+Out copy(execution_policy<D>& exec, In first, In last, Out result, std::false_type) {
   // explicit device policy: raw pointers are device pointers
   const bool in_dev = thrust::detail::is_device_iterator<In>::value || std::is_pointer<In>::value;
   const bool out_dev = thrust::detail::is_device_iterator<Out>::value || std::is_pointer<Out>::value;
-  return thrust::detail::copy_dispatch(first, last, result, in_dev, out_dev, detail::stream_of(exec));
+  return thrust::detail::copy_dispatch(first, last, result, in_dev, out_dev, stream_of(exec));
+}
+// from a fancy iterator to device memory: the materialisation kernel writes straight into
+// the destination; to host memory: the iterator is walked on the host
+template <typename D, typename In, typename Out>
+Out copy_fancy(execution_policy<D>& exec, In first, In last, Out result, std::true_type) {
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  materialize(stream, first, thrust::detail::raw(result), n);
+  synchronize(stream, "copy: synchronize");
+  return result + n;
+}
+template <typename D, typename In, typename Out>
+Out copy_fancy(execution_policy<D>&, In first, In last, Out result, std::false_type) {
+  for (; first != last; ++first, ++result) *result = *first;
+  return result;
+}
+template <typename D, typename In, typename Out>
+Out copy(execution_policy<D>& exec, In first, In last, Out result, std::true_type) {
+  return copy_fancy(exec, first, last, result,
+                    std::integral_constant<bool, thrust::detail::is_device_iterator<Out>::value ||
+                                                     std::is_pointer<Out>::value>());
+}
+// a user predicate as one byte per element, for the stencil form of the selection kernels
+template <typename Pred>
+struct as_flag {
+  Pred pred;
+  template <typename V>
+  __host__ __device__ unsigned char operator()(const V& x) const { return pred(x) ? 1 : 0; }
+};
+template <typename Pred, typename T, bool = is_abi_type<T>::value>
+struct selects_in_kernel : std::integral_constant<bool, unary_pred<Pred, T>::supported> {};
+template <typename Pred, typename T>
+struct selects_in_kernel<Pred, T, false> : std::false_type {};
+}  // namespace detail
+
+template <typename D, typename In, typename Out>
+Out copy(execution_policy<D>& exec, In first, In last, Out result) {
+  return detail::copy(exec, first, last, result, thrust::detail::is_fancy_iterator<In>());
 }
 
 namespace detail {
@@ -134,20 +175,54 @@ inline uint64_t run_selection(void* stream, const temp_source& source, const Pre
 }
 }  // namespace detail
 
+namespace detail {
+// recognised predicate on the tested elements themselves: compared inside the selection kernel
+template <typename D, typename In, typename St, typename Out, typename Pred>
+Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, bool has_stencil, Out result, Pred pred,
+                 std::true_type) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  device_input<In> source(stream, temp_source_of(exec), first, n);
+  device_input<St> tested(stream, temp_source_of(exec), stencil, has_stencil ? n : 0);
+  const uint64_t cnt = run_selection<S>(stream, temp_source_of(exec), pred, "copy_if failed",
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_copy_if(t, b, source.ptr(), has_stencil ? (const void*)tested.ptr() : nullptr,
+                                  thrust::detail::raw(result), d_num, n, sizeof(T), dtype_of<S>::value, cmp, thr,
+                                  stream);
+      });
+  return result + cnt;
+}
+// any other predicate: one byte per element from a transform iterator, then the stencil form
+template <typename D, typename In, typename St, typename Out, typename Pred>
+Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, bool, Out result, Pred pred,
+                 std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  const as_flag<Pred> flag = {pred};
+  device_input<In> source(stream, temp_source_of(exec), first, n);
+  device_input<thrust::transform_iterator<as_flag<Pred>, St> > flags(
+      stream, temp_source_of(exec), thrust::make_transform_iterator(stencil, flag), n);
+  const uint64_t cnt = run_selection<unsigned char>(
+      stream, temp_source_of(exec), thrust::identity<unsigned char>(), "copy_if failed",
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_copy_if(t, b, source.ptr(), flags.ptr(), thrust::detail::raw(result), d_num, n, sizeof(T),
+                                  THRUST_AMD_U8, cmp, thr, stream);
+      });
+  return result + cnt;
+}
+}  // namespace detail
+
 template <typename D, typename In, typename Out, typename Pred>
 Out copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  static_assert(std::is_same<typename iterator_value<Out>::type, T>::value,
-                "thrust::copy_if on the device system: input and output element types must match");
-  void* stream = detail::stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return result;
-  const uint64_t cnt = detail::run_selection<T>(stream, detail::temp_source_of(exec), pred, "copy_if failed",
-      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_copy_if(t, b, thrust::detail::raw(first), nullptr, thrust::detail::raw(result), d_num, n,
-                                  sizeof(T), detail::dtype_of<T>::value, cmp, thr, stream);
-      });
-  return result + cnt;
+  static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
+                "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
+  return detail::copy_if_impl(exec, first, last, first, false, result, pred, detail::selects_in_kernel<Pred, T>());
 }
 template <typename D, typename In, typename St, typename Out, typename Pred>
 Out copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result, Pred pred) {
@@ -155,16 +230,7 @@ Out copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result
   typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
   static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
                 "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  void* stream = detail::stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return result;
-  const uint64_t cnt = detail::run_selection<S>(stream, detail::temp_source_of(exec), pred, "copy_if failed",
-      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_copy_if(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil),
-                                  thrust::detail::raw(result), d_num, n, sizeof(T), detail::dtype_of<S>::value, cmp,
-                                  thr, stream);
-      });
-  return result + cnt;
+  return detail::copy_if_impl(exec, first, last, stencil, true, result, pred, detail::selects_in_kernel<Pred, S>());
 }
 }  // namespace hip
 }  // namespace system
@@ -175,10 +241,19 @@ Out copy(const detail::execution_policy_base<D>& exec, In first, In last, Out re
   return copy(detail::derived_cast(detail::strip_const(exec)), first, last, result);
 }
 // Without a policy the two iterators may live in different systems.
+namespace detail {
+template <typename In, typename Out>
+Out copy_any(In first, In last, Out result, std::false_type) {
+  return copy_dispatch(first, last, result, is_device_iterator<In>::value, is_device_iterator<Out>::value, nullptr);
+}
+template <typename In, typename Out>
+Out copy_any(In first, In last, Out result, std::true_type) {  // fancy input: its own system decides
+  return thrust::copy(policy_for<In>(), first, last, result);
+}
+}  // namespace detail
 template <typename In, typename Out>
 Out copy(In first, In last, Out result) {
-  return thrust::detail::copy_dispatch(first, last, result, detail::is_device_iterator<In>::value,
-                                       detail::is_device_iterator<Out>::value, nullptr);
+  return detail::copy_any(first, last, result, detail::is_fancy_iterator<In>());
 }
 template <typename D, typename In, typename Size, typename Out>
 Out copy_n(const detail::execution_policy_base<D>& exec, In first, Size n, Out result) {

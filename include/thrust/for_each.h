@@ -1,0 +1,3 @@
+// thrust::for_each lives with the other element-wise algorithms.
+#pragma once
+#include <thrust/transform.h>

@@ -1,0 +1,3 @@
+// thrust::gather lives with the other element-wise algorithms.
+#pragma once
+#include <thrust/transform.h>

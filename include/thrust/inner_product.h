@@ -7,6 +7,7 @@
 #pragma once
 #include <thrust/functional.h>
 #include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/device_input.h>
 
 namespace thrust {
 
@@ -39,9 +40,9 @@ template <typename D, typename It1, typename It2, typename T, typename Op1, type
 T inner_product(execution_policy<D>& exec, It1 first1, It1 last1, It2 first2, T init, Op1, Op2) {
   typedef typename std::remove_const<typename iterator_value<It1>::type>::type V1;
   typedef typename std::remove_const<typename iterator_value<It2>::type>::type V2;
-  static_assert((std::is_pointer<It1>::value || thrust::detail::is_device_iterator<It1>::value) &&
-                    (std::is_pointer<It2>::value || thrust::detail::is_device_iterator<It2>::value),
-                "thrust::inner_product on the device system needs device_ptr / device_vector iterators or raw device pointers");
+  static_assert(detail::is_device_input<It1>::value && detail::is_device_input<It2>::value,
+                "thrust::inner_product on the device system needs device_ptr / device_vector iterators, raw device "
+                "pointers or fancy iterators over them");
   static_assert(detail::is_abi_type<T>::value && std::is_same<V1, T>::value && std::is_same<V2, T>::value,
                 "thrust::inner_product on the device system: both ranges and init must share one arithmetic type");
   static_assert(detail::binop_code<Op1, T>::value == THRUST_AMD_PLUS &&
@@ -50,11 +51,13 @@ T inner_product(execution_policy<D>& exec, It1 first1, It1 last1, It2 first2, T 
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last1 - first1);
   if (n == 0) return init;
+  detail::device_input<It1> source1(stream, detail::temp_source_of(exec), first1, n);
+  detail::device_input<It2> source2(stream, detail::temp_source_of(exec), first2, n);
   detail::temp_storage temp(stream, detail::temp_source_of(exec));
   void* d_out = nullptr;
   std::size_t need = 0;
   auto call = [&](void* t, std::size_t* b) {
-    return thrust_amd_inner_product(t, b, thrust::detail::raw(first1), thrust::detail::raw(first2), n,
+    return thrust_amd_inner_product(t, b, source1.ptr(), source2.ptr(), n,
                                     detail::dtype_of<T>::value, &init, d_out, stream);
   };
   detail::throw_on_error(call(nullptr, &need), "inner_product: temp size query");

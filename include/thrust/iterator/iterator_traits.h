@@ -24,6 +24,11 @@ namespace detail {
 template <typename It> struct is_device_iterator : std::false_type {};
 template <typename T> struct is_device_iterator<device_ptr<T> > : std::true_type {};
 
+// Iterators whose elements are computed (counting, constant, transform, permutation) derive from this.
+struct fancy_iterator_marker {};
+template <typename It>
+struct is_fancy_iterator : std::is_base_of<fancy_iterator_marker, It> {};
+
 // Raw address of the element an iterator points at.  Device iterators are device_ptr or,
 // under an explicit device policy, plain pointers; host iterators must be contiguous
 // (pointers, std::vector / host_vector iterators).
@@ -31,10 +36,16 @@ template <typename T> inline T* raw(const device_ptr<T>& p) { return p.get(); }
 template <typename T> inline T* raw(T* p) { return p; }
 template <typename It>
 inline auto raw(It it) -> typename std::enable_if<
-    !std::is_pointer<It>::value && !is_device_iterator<It>::value,
+    !std::is_pointer<It>::value && !is_device_iterator<It>::value && !is_fancy_iterator<It>::value,
     typename std::remove_reference<decltype(*it)>::type*>::type {
   // never dereferences: callers pass begin() of a non-empty contiguous range or use n == 0
   return std::addressof(*it);
+}
+// a fancy iterator has no address; code that reaches this at run time took a wrong turn
+template <typename It>
+inline auto raw(It) -> typename std::enable_if<is_fancy_iterator<It>::value,
+                                               typename std::iterator_traits<It>::value_type*>::type {
+  return nullptr;
 }
 
 template <typename It>

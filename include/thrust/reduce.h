@@ -8,6 +8,7 @@
 #include <thrust/functional.h>
 #include <thrust/pair.h>
 #include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/device_input.h>
 
 namespace thrust {
 
@@ -95,8 +96,9 @@ namespace hip {
 template <typename D, typename It, typename T, typename Op>
 T reduce(execution_policy<D>& exec, It first, It last, T init, Op) {
   typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
-  static_assert(std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value,
-                "thrust::reduce on the device system needs device_ptr / device_vector iterators or raw device pointers");
+  static_assert(detail::is_device_input<It>::value,
+                "thrust::reduce on the device system needs device_ptr / device_vector iterators, raw device pointers "
+                "or fancy iterators over them");
   static_assert(detail::is_abi_type<T>::value && detail::is_abi_type<V>::value,
                 "thrust::reduce on the device system: elements and init must have arithmetic types");
   static_assert(detail::binop_code<Op, T>::value >= 0,
@@ -104,9 +106,9 @@ T reduce(execution_policy<D>& exec, It first, It last, T init, Op) {
                 "of the type of init");
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
+  detail::device_input<It> source(stream, detail::temp_source_of(exec), first, n);
   detail::temp_storage converted(stream, detail::temp_source_of(exec));
-  const void* in = n ? (const void*)detail::input_as<T>(static_cast<const V*>(thrust::detail::raw(first)), n, stream, converted)
-                     : nullptr;
+  const void* in = n ? (const void*)detail::input_as<T>(source.ptr(), n, stream, converted) : nullptr;
   detail::temp_storage temp(stream, detail::temp_source_of(exec));
   void* d_out = nullptr;
   // the result slot is the `extra` region, which run() only knows after the size query
@@ -140,11 +142,13 @@ pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n == 0) return thrust::make_pair(ko, vo);
+  detail::device_input<KIt> keys_in(stream, detail::temp_source_of(exec), kf, n);
+  detail::device_input<VIt> values_in(stream, detail::temp_source_of(exec), vf, n);
   detail::temp_storage temp(stream, detail::temp_source_of(exec));
   uint64_t* d_runs = nullptr;
   std::size_t need = 0;
   auto call = [&](void* t, std::size_t* b) {
-    return thrust_amd_reduce_by_key(t, b, thrust::detail::raw(kf), thrust::detail::raw(vf),
+    return thrust_amd_reduce_by_key(t, b, keys_in.ptr(), values_in.ptr(),
                                     thrust::detail::raw(ko), thrust::detail::raw(vo), d_runs, n,
                                     detail::dtype_of<K>::value, detail::dtype_of<V>::value,
                                     detail::binop_code<Op, V>::value, stream);

@@ -12,6 +12,7 @@
 #pragma once
 #include <thrust/functional.h>
 #include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/device_input.h>
 
 namespace thrust {
 
@@ -159,9 +160,10 @@ template <typename In, typename Out, typename A, typename Op>
 struct scan_checks {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
   typedef typename iterator_value<Out>::type U;
-  static_assert((std::is_pointer<In>::value || thrust::detail::is_device_iterator<In>::value) &&
+  static_assert(is_device_input<In>::value &&
                     (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value),
-                "scan on the device system needs device_ptr / device_vector iterators or raw device pointers");
+                "scan on the device system needs device_ptr / device_vector iterators or raw device pointers "
+                "(fancy iterators as input only)");
   static_assert(is_abi_type<V>::value && is_abi_type<A>::value && is_abi_type<U>::value,
                 "scan on the device system: input, output and init must have arithmetic types");
   static_assert(binop_code<Op, A>::value >= 0,
@@ -178,11 +180,12 @@ Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op)
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
+  detail::device_input<In> source(stream, detail::temp_source_of(exec), first, n);
   detail::temp_storage staged(stream, detail::temp_source_of(exec));
   V* computed = detail::output_as<V>(static_cast<U*>(thrust::detail::raw(result)), n, staged);
   detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "inclusive_scan failed", [&](void* t, std::size_t* b) {
-    return thrust_amd_inclusive_scan(t, b, thrust::detail::raw(first), computed, n, detail::dtype_of<V>::value,
+    return thrust_amd_inclusive_scan(t, b, source.ptr(), computed, n, detail::dtype_of<V>::value,
                                      detail::binop_code<Op, V>::value, stream);
   });
   detail::finish_output(computed, static_cast<U*>(thrust::detail::raw(result)), n, stream);
@@ -198,8 +201,9 @@ Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T i
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
+  detail::device_input<In> source(stream, detail::temp_source_of(exec), first, n);
   detail::temp_storage converted(stream, detail::temp_source_of(exec));
-  const T* in = detail::input_as<T>(static_cast<const V*>(thrust::detail::raw(first)), n, stream, converted);
+  const T* in = detail::input_as<T>(source.ptr(), n, stream, converted);
   detail::temp_storage staged(stream, detail::temp_source_of(exec));
   T* computed = detail::output_as<T>(static_cast<U*>(thrust::detail::raw(result)), n, staged);
   detail::temp_storage temp(stream, detail::temp_source_of(exec));

@@ -1,0 +1,55 @@
+// Element-wise kernels that take iterators and functors by value: materialisation of a
+// fancy iterator, for_each, binary transform, scatter.  They are templates on types only
+// the user's translation unit knows, so they exist where that unit is compiled with hipcc
+// (the reference instantiates its kernels the same way: thrust/system/cuda/detail/core/
+// util.h:527-561 LoadIterator, parallel_for.h).  HBM traffic: what the iterators read and
+// one write per element.
+#pragma once
+#if !defined(__HIPCC__)
+#error "thrust/system/hip/detail/fancy_kernels.h is HIP code: compile this translation unit with hipcc"
+#endif
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace thrust {
+namespace system {
+namespace hip {
+namespace detail {
+
+constexpr int ELEMENTWISE_BLOCK = 256;
+inline unsigned elementwise_grid(uint64_t n) {
+  const uint64_t blocks = (n + ELEMENTWISE_BLOCK - 1) / ELEMENTWISE_BLOCK;
+  const uint64_t cap = 256 * 16;  // grid-stride beyond that
+  return (unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap));
+}
+
+template <typename View, typename T>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void materialize_kernel(View first, T* out, uint64_t n) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = (T)first[i];
+}
+
+template <typename T, typename F>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void for_each_kernel(T* first, uint64_t n, F f) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) f(first[i]);
+}
+
+template <typename ViewA, typename ViewB, typename T, typename F>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform2_kernel(ViewA a, ViewB b, T* out, uint64_t n, F f) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = (T)f(a[i], b[i]);
+}
+
+template <typename ViewIn, typename ViewMap, typename T>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void scatter_kernel(ViewIn in, ViewMap map, T* out, uint64_t n) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[map[i]] = (T)in[i];
+}
+
+inline int launch_status() { return (int)hipGetLastError(); }
+
+}  // namespace detail
+}  // namespace hip
+}  // namespace system
+}  // namespace thrust

@@ -1,0 +1,217 @@
+// thrust::transform (unary and binary), thrust::for_each, thrust::sequence, thrust::gather,
+// thrust::scatter: the element-wise callers on either side of the reduce / scan / sort path
+// (thrust/system/detail/generic/transform.inl, sequence.inl, gather.inl, scatter.inl;
+// thrust/system/cuda/detail/for_each.h).  On the device system they run as kernels that
+// take the functor and the iterators by value, so they need a translation unit compiled
+// with hipcc (functors __host__ __device__); the host system runs plain loops.
+#pragma once
+#include <algorithm>
+
+#include <thrust/copy.h>
+#include <thrust/iterator/counting_iterator.h>
+#include <thrust/iterator/permutation_iterator.h>
+#include <thrust/iterator/transform_iterator.h>
+#include <thrust/system/hip/detail/device_input.h>
+
+namespace thrust {
+namespace system {
+namespace cpp {
+template <typename D, typename In, typename Out, typename F>
+Out transform(execution_policy<D>&, In first, In last, Out result, F f) {
+  for (; first != last; ++first, ++result) *result = f(*first);
+  return result;
+}
+template <typename D, typename In1, typename In2, typename Out, typename F>
+Out transform(execution_policy<D>&, In1 first1, In1 last1, In2 first2, Out result, F f) {
+  for (; first1 != last1; ++first1, ++first2, ++result) *result = f(*first1, *first2);
+  return result;
+}
+template <typename D, typename It, typename F>
+It for_each(execution_policy<D>&, It first, It last, F f) {
+  for (; first != last; ++first) f(*first);
+  return first;
+}
+template <typename D, typename It, typename T>
+void sequence(execution_policy<D>&, It first, It last, T init, T step) {
+  typedef typename iterator_value<It>::type V;
+  for (std::size_t i = 0; first != last; ++first, ++i) *first = (V)(init + step * (T)i);
+}
+template <typename D, typename MapIt, typename In, typename Out>
+Out gather(execution_policy<D>&, MapIt map_first, MapIt map_last, In input, Out result) {
+  for (; map_first != map_last; ++map_first, ++result) *result = input[*map_first];
+  return result;
+}
+template <typename D, typename In, typename MapIt, typename Out>
+void scatter(execution_policy<D>&, In first, In last, MapIt map, Out output) {
+  for (; first != last; ++first, ++map) output[*map] = *first;
+}
+}  // namespace cpp
+
+namespace hip {
+namespace detail {
+template <typename T>
+struct sequence_value {  // element i of thrust::sequence(first, last, init, step)
+  T init, step;
+  __host__ __device__ T operator()(unsigned long long i) const { return (T)(init + step * (T)i); }
+};
+template <typename It>
+struct is_device_output
+    : std::integral_constant<bool, std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value> {};
+}  // namespace detail
+
+template <typename D, typename In, typename Out, typename F>
+Out transform(execution_policy<D>& exec, In first, In last, Out result, F f) {
+  return thrust::copy(exec, thrust::make_transform_iterator(first, f), thrust::make_transform_iterator(last, f), result);
+}
+template <typename D, typename In1, typename In2, typename Out, typename F>
+Out transform(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, Out result, F f) {
+  static_assert(detail::is_device_input<In1>::value && detail::is_device_input<In2>::value &&
+                    detail::is_device_output<Out>::value,
+                "thrust::transform on the device system reads device or fancy iterators and writes device memory");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last1 - first1);
+  if (n == 0) return result;
+#if defined(__HIPCC__)
+  typedef typename iterator_value<Out>::type U;
+  hipLaunchKernelGGL((detail::transform2_kernel<typename thrust::detail::device_view_of<In1>::type,
+                                                typename thrust::detail::device_view_of<In2>::type, U, F>),
+                     dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
+                     thrust::detail::device_view(first1), thrust::detail::device_view(first2),
+                     thrust::detail::raw(result), n, f);
+  detail::throw_on_error(detail::launch_status(), "transform: kernel launch");
+  detail::synchronize(stream, "transform: synchronize");
+#else
+  static_assert(detail::fancy_needs_hipcc<F>::value,
+                "thrust::transform on the device system runs the functor in a kernel; compile this translation unit with hipcc");
+#endif
+  return result + n;
+}
+template <typename D, typename It, typename F>
+It for_each(execution_policy<D>& exec, It first, It last, F f) {
+  static_assert(detail::is_device_output<It>::value,
+                "thrust::for_each on the device system needs device_ptr / device_vector iterators or raw device pointers");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return last;
+#if defined(__HIPCC__)
+  typedef typename std::remove_pointer<decltype(thrust::detail::raw(first))>::type T;
+  hipLaunchKernelGGL((detail::for_each_kernel<T, F>), dim3(detail::elementwise_grid(n)),
+                     dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream, thrust::detail::raw(first), n, f);
+  detail::throw_on_error(detail::launch_status(), "for_each: kernel launch");
+  detail::synchronize(stream, "for_each: synchronize");
+#else
+  static_assert(detail::fancy_needs_hipcc<F>::value,
+                "thrust::for_each on the device system runs the functor in a kernel; compile this translation unit with hipcc");
+#endif
+  return last;
+}
+template <typename D, typename It, typename T>
+void sequence(execution_policy<D>& exec, It first, It last, T init, T step) {
+  const detail::sequence_value<T> value = {init, step};
+  thrust::counting_iterator<unsigned long long> zero(0);
+  thrust::copy(exec, thrust::make_transform_iterator(zero, value),
+               thrust::make_transform_iterator(zero + (last - first), value), first);
+}
+template <typename D, typename MapIt, typename In, typename Out>
+Out gather(execution_policy<D>& exec, MapIt map_first, MapIt map_last, In input, Out result) {
+  return thrust::copy(exec, thrust::make_permutation_iterator(input, map_first),
+                      thrust::make_permutation_iterator(input, map_last), result);
+}
+template <typename D, typename In, typename MapIt, typename Out>
+void scatter(execution_policy<D>& exec, In first, In last, MapIt map, Out output) {
+  static_assert(detail::is_device_input<In>::value && detail::is_device_input<MapIt>::value &&
+                    detail::is_device_output<Out>::value,
+                "thrust::scatter on the device system reads device or fancy iterators and writes device memory");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return;
+#if defined(__HIPCC__)
+  typedef typename iterator_value<Out>::type U;
+  hipLaunchKernelGGL((detail::scatter_kernel<typename thrust::detail::device_view_of<In>::type,
+                                             typename thrust::detail::device_view_of<MapIt>::type, U>),
+                     dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
+                     thrust::detail::device_view(first), thrust::detail::device_view(map),
+                     thrust::detail::raw(output), n);
+  detail::throw_on_error(detail::launch_status(), "scatter: kernel launch");
+  detail::synchronize(stream, "scatter: synchronize");
+#else
+  static_assert(detail::fancy_needs_hipcc<In>::value,
+                "thrust::scatter on the device system runs as a kernel over the iterators; compile this translation unit with hipcc");
+#endif
+}
+}  // namespace hip
+}  // namespace system
+
+// ------------------------------------------------------------------ entry points
+template <typename D, typename In, typename Out, typename F>
+Out transform(const detail::execution_policy_base<D>& exec, In first, In last, Out result, F f) {
+  return transform(detail::derived_cast(detail::strip_const(exec)), first, last, result, f);
+}
+template <typename D, typename In1, typename In2, typename Out, typename F>
+Out transform(const detail::execution_policy_base<D>& exec, In1 first1, In1 last1, In2 first2, Out result, F f) {
+  return transform(detail::derived_cast(detail::strip_const(exec)), first1, last1, first2, result, f);
+}
+template <typename In, typename Out, typename F,
+          typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>
+Out transform(In first, In last, Out result, F f) {
+  return thrust::transform(detail::policy_for<Out>(), first, last, result, f);
+}
+template <typename In1, typename In2, typename Out, typename F,
+          typename = typename std::enable_if<!detail::is_execution_policy<In1>::value>::type>
+Out transform(In1 first1, In1 last1, In2 first2, Out result, F f) {
+  return thrust::transform(detail::policy_for<Out>(), first1, last1, first2, result, f);
+}
+
+template <typename D, typename It, typename F>
+It for_each(const detail::execution_policy_base<D>& exec, It first, It last, F f) {
+  return for_each(detail::derived_cast(detail::strip_const(exec)), first, last, f);
+}
+template <typename It, typename F>
+It for_each(It first, It last, F f) {
+  return thrust::for_each(detail::policy_for<It>(), first, last, f);
+}
+
+template <typename D, typename It, typename T>
+void sequence(const detail::execution_policy_base<D>& exec, It first, It last, T init, T step) {
+  sequence(detail::derived_cast(detail::strip_const(exec)), first, last, init, step);
+}
+template <typename D, typename It, typename T>
+void sequence(const detail::execution_policy_base<D>& exec, It first, It last, T init) {
+  thrust::sequence(exec, first, last, init, T(1));
+}
+template <typename D, typename It>
+void sequence(const detail::execution_policy_base<D>& exec, It first, It last) {
+  typedef typename iterator_value<It>::type T;
+  thrust::sequence(exec, first, last, T(0), T(1));
+}
+template <typename It>
+void sequence(It first, It last) {
+  thrust::sequence(detail::policy_for<It>(), first, last);
+}
+template <typename It, typename T, typename = typename std::enable_if<!detail::is_execution_policy<It>::value>::type>
+void sequence(It first, It last, T init) {
+  thrust::sequence(detail::policy_for<It>(), first, last, init);
+}
+template <typename It, typename T, typename = typename std::enable_if<!detail::is_execution_policy<It>::value>::type>
+void sequence(It first, It last, T init, T step) {
+  thrust::sequence(detail::policy_for<It>(), first, last, init, step);
+}
+
+template <typename D, typename MapIt, typename In, typename Out>
+Out gather(const detail::execution_policy_base<D>& exec, MapIt map_first, MapIt map_last, In input, Out result) {
+  return gather(detail::derived_cast(detail::strip_const(exec)), map_first, map_last, input, result);
+}
+template <typename MapIt, typename In, typename Out>
+Out gather(MapIt map_first, MapIt map_last, In input, Out result) {
+  return thrust::gather(detail::policy_for<Out>(), map_first, map_last, input, result);
+}
+template <typename D, typename In, typename MapIt, typename Out>
+void scatter(const detail::execution_policy_base<D>& exec, In first, In last, MapIt map, Out output) {
+  scatter(detail::derived_cast(detail::strip_const(exec)), first, last, map, output);
+}
+template <typename In, typename MapIt, typename Out>
+void scatter(In first, In last, MapIt map, Out output) {
+  thrust::scatter(detail::policy_for<Out>(), first, last, map, output);
+}
+
+}  // namespace thrust

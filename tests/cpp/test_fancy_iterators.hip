@@ -1,0 +1,253 @@
+// Front-end test compiled with hipcc: fancy iterators as inputs of the device system's
+// algorithms, user functors in transform / for_each / transform_reduce / count_if /
+// copy_if, and sequence / gather / scatter.  Literal vectors are the reference's
+// (testing/gather.cu:14-32, scatter.cu:10-32, sequence.cu:43-76, transform.cu:11-28 and
+// :261-280, counting_iterator.cu, constant_iterator.cu); everything else compares the
+// device system with the sequential host system on the same inputs.
+#include <thrust/copy.h>
+#include <thrust/count.h>
+#include <thrust/device_vector.h>
+#include <thrust/execution_policy.h>
+#include <thrust/for_each.h>
+#include <thrust/functional.h>
+#include <thrust/gather.h>
+#include <thrust/host_vector.h>
+#include <thrust/inner_product.h>
+#include <thrust/iterator/constant_iterator.h>
+#include <thrust/iterator/counting_iterator.h>
+#include <thrust/iterator/permutation_iterator.h>
+#include <thrust/iterator/transform_iterator.h>
+#include <thrust/reduce.h>
+#include <thrust/scan.h>
+#include <thrust/scatter.h>
+#include <thrust/sequence.h>
+#include <thrust/transform.h>
+#include <thrust/transform_reduce.h>
+
+#include <cstdint>
+#include <cstdio>
+#include <vector>
+
+static int g_failed = 0, g_checks = 0;
+static const char* g_test = "";
+#define ASSERT_TRUE(c)                                                                    \
+  do {                                                                                    \
+    ++g_checks;                                                                           \
+    if (!(c)) { ++g_failed; std::printf("FAIL [%s] %s:%d: %s\n", g_test, __FILE__, __LINE__, #c); } \
+  } while (0)
+
+template <typename A, typename B>
+static bool same(const A& a, const B& b) {
+  if (a.size() != b.size()) return false;
+  for (size_t i = 0; i < a.size(); ++i)
+    if (!(a[i] == b[i])) return false;
+  return true;
+}
+template <typename T>
+static thrust::host_vector<T> hv(std::initializer_list<T> l) { return thrust::host_vector<T>(std::vector<T>(l)); }
+template <typename T>
+static thrust::host_vector<T> to_host(const thrust::device_vector<T>& d) { return thrust::host_vector<T>(d); }
+
+static uint64_t mix(uint64_t z) {
+  z += 0x9E3779B97F4A7C15ull;
+  z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+  z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+  return z ^ (z >> 31);
+}
+template <typename T>
+static thrust::host_vector<T> random_values(size_t n, uint64_t seed, uint64_t modulus) {
+  thrust::host_vector<T> h(n);
+  for (size_t i = 0; i < n; ++i) h[i] = (T)(mix(seed * 1000003ull + i) % modulus);
+  return h;
+}
+
+static const size_t kSizes[] = {0, 1, 2, 63, 64, 65, 255, 256, 257, 1000, 4095, 4096, 4097, 65533, 65536, 65539,
+                                (1u << 20) + 3};
+
+struct times_three_plus_one {
+  __host__ __device__ int operator()(int x) const { return 3 * x + 1; }
+};
+struct saxpy {
+  float a;
+  __host__ __device__ float operator()(float x, float y) const { return a * x + y; }
+};
+struct is_even {
+  __host__ __device__ bool operator()(int x) const { return (x & 1) == 0; }
+};
+struct double_in_place {
+  __host__ __device__ void operator()(int& x) const { x = 2 * x + 1; }
+};
+struct widen_square {
+  __host__ __device__ long long operator()(int x) const { return (long long)x * x; }
+};
+
+static void TestKnownAnswers() {
+  g_test = "GatherSimple";
+  {
+    thrust::device_vector<int> map(hv<int>({6, 2, 1, 7, 2})), src(hv<int>({0, 1, 2, 3, 4, 5, 6, 7})), dst(5, 0);
+    auto end = thrust::gather(map.begin(), map.end(), src.begin(), dst.begin());
+    ASSERT_TRUE(end - dst.begin() == 5);
+    ASSERT_TRUE(same(to_host(dst), hv<int>({6, 2, 1, 7, 2})));
+  }
+  g_test = "ScatterSimple";
+  {
+    thrust::device_vector<int> map(hv<int>({6, 3, 1, 7, 2})), src(hv<int>({0, 1, 2, 3, 4})), dst(8, 0);
+    thrust::scatter(src.begin(), src.end(), map.begin(), dst.begin());
+    ASSERT_TRUE(same(to_host(dst), hv<int>({0, 2, 4, 1, 0, 0, 0, 3})));
+  }
+  g_test = "SequenceSimple";
+  {
+    thrust::device_vector<int> v(5);
+    thrust::sequence(v.begin(), v.end());
+    ASSERT_TRUE(same(to_host(v), hv<int>({0, 1, 2, 3, 4})));
+    thrust::sequence(v.begin(), v.end(), 10);
+    ASSERT_TRUE(same(to_host(v), hv<int>({10, 11, 12, 13, 14})));
+    thrust::sequence(v.begin(), v.end(), 10, 2);
+    ASSERT_TRUE(same(to_host(v), hv<int>({10, 12, 14, 16, 18})));
+  }
+  g_test = "TransformSimple";
+  {
+    thrust::device_vector<int> in(hv<int>({1, -2, 3})), in2(hv<int>({-4, 5, 6})), out(3);
+    auto it = thrust::transform(in.begin(), in.end(), out.begin(), thrust::negate<int>());
+    ASSERT_TRUE(it - out.begin() == 3);
+    ASSERT_TRUE(same(to_host(out), hv<int>({-1, 2, -3})));
+    it = thrust::transform(in.begin(), in.end(), in2.begin(), out.begin(), thrust::minus<int>());
+    ASSERT_TRUE(it - out.begin() == 3);
+    ASSERT_TRUE(same(to_host(out), hv<int>({5, -7, -3})));
+  }
+  g_test = "CountingAndConstant";
+  {
+    thrust::counting_iterator<int> first(0);
+    ASSERT_TRUE(*first == 0 && first[5] == 5 && (first + 3) - first == 3);
+    ASSERT_TRUE(thrust::reduce(first, first + 100) == 4950);
+    ASSERT_TRUE(thrust::reduce(thrust::device, first + 1, first + 4) == 6);  // testing/counting_iterator.cu sums 1 + 2 + 3
+    thrust::constant_iterator<int> seven(7);
+    ASSERT_TRUE(*seven == 7 && seven[12] == 7 && (seven + 9) - seven == 9);
+    ASSERT_TRUE(thrust::reduce(seven, seven + 1000) == 7000);
+    thrust::device_vector<int> out(4);
+    thrust::copy(first + 3, first + 7, out.begin());
+    ASSERT_TRUE(same(to_host(out), hv<int>({3, 4, 5, 6})));
+    thrust::exclusive_scan(seven, seven + 4, out.begin());
+    ASSERT_TRUE(same(to_host(out), hv<int>({0, 7, 14, 21})));
+  }
+}
+
+static void Differential() {
+  for (size_t n : kSizes) {
+    const thrust::host_vector<int> h = random_values<int>(n, 3, 2001);
+    const thrust::device_vector<int> d(h);
+
+    g_test = "transform_iterator inputs";
+    {
+      auto hf = thrust::make_transform_iterator(h.begin(), times_three_plus_one());
+      auto df = thrust::make_transform_iterator(d.begin(), times_three_plus_one());
+      ASSERT_TRUE(thrust::reduce(df, df + n, 5) == thrust::reduce(hf, hf + n, 5));
+      ASSERT_TRUE(thrust::reduce(df, df + n, -1000000, thrust::maximum<int>()) ==
+                  thrust::reduce(hf, hf + n, -1000000, thrust::maximum<int>()));
+      thrust::host_vector<int> hs(n);
+      thrust::device_vector<int> ds(n);
+      thrust::inclusive_scan(hf, hf + n, hs.begin());
+      thrust::inclusive_scan(df, df + n, ds.begin());
+      ASSERT_TRUE(same(to_host(ds), hs));
+      thrust::exclusive_scan(hf, hf + n, hs.begin(), 11);
+      thrust::exclusive_scan(df, df + n, ds.begin(), 11);
+      ASSERT_TRUE(same(to_host(ds), hs));
+    }
+    g_test = "user functors";
+    {
+      ASSERT_TRUE(thrust::transform_reduce(d.begin(), d.end(), widen_square(), (long long)3, thrust::plus<long long>()) ==
+                  thrust::transform_reduce(h.begin(), h.end(), widen_square(), (long long)3, thrust::plus<long long>()));
+      ASSERT_TRUE(thrust::count_if(d.begin(), d.end(), is_even()) == thrust::count_if(h.begin(), h.end(), is_even()));
+      thrust::host_vector<int> ho(n);
+      thrust::device_vector<int> dout(n);
+      auto he = thrust::copy_if(h.begin(), h.end(), ho.begin(), is_even());
+      auto de = thrust::copy_if(d.begin(), d.end(), dout.begin(), is_even());
+      ASSERT_TRUE(de - dout.begin() == he - ho.begin());
+      ho.resize(he - ho.begin());
+      dout.resize(de - dout.begin());
+      ASSERT_TRUE(same(to_host(dout), ho));
+      // stencil form: keep h[i] where the stencil is even
+      const thrust::host_vector<int> hst = random_values<int>(n, 9, 10);
+      const thrust::device_vector<int> dst(hst);
+      ho.resize(n);
+      dout.resize(n);
+      he = thrust::copy_if(h.begin(), h.end(), hst.begin(), ho.begin(), is_even());
+      de = thrust::copy_if(d.begin(), d.end(), dst.begin(), dout.begin(), is_even());
+      ASSERT_TRUE(de - dout.begin() == he - ho.begin());
+      ho.resize(he - ho.begin());
+      dout.resize(de - dout.begin());
+      ASSERT_TRUE(same(to_host(dout), ho));
+    }
+    g_test = "transform / for_each / sequence";
+    {
+      thrust::host_vector<float> hx(n), hy(n), hz(n);
+      for (size_t i = 0; i < n; ++i) { hx[i] = (float)(mix(i) % 1000) / 8.0f; hy[i] = (float)(mix(i + n) % 1000) / 4.0f; }
+      thrust::device_vector<float> dx(hx), dy(hy), dz(n);
+      thrust::transform(hx.begin(), hx.end(), hy.begin(), hz.begin(), saxpy{2.5f});
+      thrust::transform(dx.begin(), dx.end(), dy.begin(), dz.begin(), saxpy{2.5f});
+      ASSERT_TRUE(same(to_host(dz), hz));
+      thrust::host_vector<int> h2(h);
+      thrust::device_vector<int> d2(d);
+      thrust::for_each(h2.begin(), h2.end(), double_in_place());
+      thrust::for_each(d2.begin(), d2.end(), double_in_place());
+      ASSERT_TRUE(same(to_host(d2), h2));
+      thrust::transform(h.begin(), h.end(), h2.begin(), times_three_plus_one());
+      thrust::transform(d.begin(), d.end(), d2.begin(), times_three_plus_one());
+      ASSERT_TRUE(same(to_host(d2), h2));
+      thrust::host_vector<long long> hq(n);
+      thrust::device_vector<long long> dq(n);
+      thrust::sequence(hq.begin(), hq.end(), (long long)-5, (long long)3);
+      thrust::sequence(dq.begin(), dq.end(), (long long)-5, (long long)3);
+      ASSERT_TRUE(same(to_host(dq), hq));
+    }
+    g_test = "gather / scatter / permutation";
+    if (n) {
+      // a permutation of 0..n-1: i -> (a*i + b) mod n with gcd(a, n) = 1
+      size_t a = 7;
+      while (a > 1 && (n % a == 0 || std::__gcd(a, n) != 1)) ++a;
+      thrust::host_vector<unsigned> hmap(n);
+      for (size_t i = 0; i < n; ++i) hmap[i] = (unsigned)((a * i + 3) % n);
+      thrust::device_vector<unsigned> dmap(hmap);
+      thrust::host_vector<int> hg(n), hsc(n, -1);
+      thrust::device_vector<int> dg(n), dsc(n, -1);
+      thrust::gather(hmap.begin(), hmap.end(), h.begin(), hg.begin());
+      thrust::gather(dmap.begin(), dmap.end(), d.begin(), dg.begin());
+      ASSERT_TRUE(same(to_host(dg), hg));
+      thrust::scatter(h.begin(), h.end(), hmap.begin(), hsc.begin());
+      thrust::scatter(d.begin(), d.end(), dmap.begin(), dsc.begin());
+      ASSERT_TRUE(same(to_host(dsc), hsc));
+      auto hp = thrust::make_permutation_iterator(h.begin(), hmap.begin());
+      auto dp = thrust::make_permutation_iterator(d.begin(), dmap.begin());
+      ASSERT_TRUE(thrust::reduce(dp, dp + n / 2, 1) == thrust::reduce(hp, hp + n / 2, 1));
+    }
+    g_test = "reduce_by_key with a constant iterator";
+    {
+      thrust::host_vector<int> hk(n);
+      for (size_t i = 0; i < n; ++i) hk[i] = (int)(i / 3 + (mix(i / 3) % 2));
+      thrust::device_vector<int> dk(hk), dko(n), dvo(n);
+      thrust::host_vector<int> hko(n), hvo(n);
+      auto hr = thrust::reduce_by_key(hk.begin(), hk.end(), thrust::constant_iterator<int>(1), hko.begin(), hvo.begin());
+      auto dr = thrust::reduce_by_key(dk.begin(), dk.end(), thrust::constant_iterator<int>(1), dko.begin(), dvo.begin());
+      ASSERT_TRUE(dr.first - dko.begin() == hr.first - hko.begin());
+      const size_t runs = hr.first - hko.begin();
+      hko.resize(runs); hvo.resize(runs); dko.resize(runs); dvo.resize(runs);
+      ASSERT_TRUE(same(to_host(dko), hko));
+      ASSERT_TRUE(same(to_host(dvo), hvo));
+    }
+    g_test = "inner_product with a counting iterator";
+    {
+      thrust::counting_iterator<int> c(1);
+      long long want = 0;
+      for (size_t i = 0; i < n; ++i) want += (long long)h[i] * (long long)(1 + (int)i);
+      ASSERT_TRUE((long long)thrust::inner_product(d.begin(), d.end(), c, 0) == (long long)(int)want);
+    }
+  }
+}
+
+int main() {
+  TestKnownAnswers();
+  Differential();
+  std::printf("%d checks, %d failed\n", g_checks, g_failed);
+  std::printf(g_failed ? "FAILED\n" : "PASSED\n");
+  return g_failed ? 1 : 0;
+}

@@ -38,3 +38,9 @@ def test_user_comparators_and_struct_keys_compiled_with_hipcc():
     # thrust::sort with user comparators: the merge sort kernels are instantiated in the test's own translation unit
     out = _run("test_user_comparator")
     assert "PASSED" in out
+
+
+def test_fancy_iterators_and_user_functors_compiled_with_hipcc():
+    # counting / constant / transform / permutation iterators as inputs, transform, for_each, sequence, gather, scatter
+    out = _run("test_fancy_iterators")
+    assert "PASSED" in out

@@ -110,6 +110,14 @@ __global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
         v[j * VEC + i] = vv[j].v[i];
       }
     }
+  } else if (full) {
+    // pointers that do not allow whole vectors: element loads, still without predicates
+    // (a predicated load makes the compiler wait for it before issuing the next one)
+#pragma unroll
+    for (int i = 0; i < ITEMS; ++i) {
+      k[i] = a.keys[first + i];
+      v[i] = a.values[first + i];
+    }
   } else {
 #pragma unroll
     for (int i = 0; i < ITEMS; ++i) {

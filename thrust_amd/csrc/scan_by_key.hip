@@ -82,6 +82,18 @@ __global__ __launch_bounds__(SBK_BLOCK, 4) void sbk_kernel(SbkArgs<K, V> a) {
       k[j] = *reinterpret_cast<const Vec16<K>*>(a.keys + off);
       v[j] = *reinterpret_cast<const VV*>(a.values + off);
     }
+  } else if (full) {
+    // pointers that do not allow whole vectors: element loads, still without predicates
+    // (a predicated load makes the compiler wait for it before issuing the next one)
+#pragma unroll
+    for (int j = 0; j < CHUNKS; ++j) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) {
+        const uint64_t off = tile_base + lane_off + j * (WAVE * VEC) + i;
+        k[j].v[i] = a.keys[off];
+        v[j].v[i] = a.values[off];
+      }
+    }
   } else {
 #pragma unroll
     for (int j = 0; j < CHUNKS; ++j) {
