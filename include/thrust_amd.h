@@ -118,6 +118,14 @@ size_t thrust_amd_dtype_size(int dtype);
 int thrust_amd_malloc(void** ptr, size_t bytes);
 int thrust_amd_free(void* ptr);
 
+/* Universal memory: one pointer that host code and kernels both dereference.  Replaces the
+ * managed allocation behind thrust::universal_vector (thrust/system/cuda/memory_resource.h:
+ * 40-110, universal_memory_resource over cudaMallocManaged).  Here it is pinned host memory
+ * mapped into the device's address space: nothing migrates, device accesses cross the host
+ * link.  Any entry point takes such a pointer where it takes device memory. */
+int thrust_amd_malloc_universal(void** ptr, size_t bytes);
+int thrust_amd_free_universal(void* ptr);
+
 /* Copy between host and device or device and device, ordered on `stream`; the H2D/D2H
  * forms return after the copy has completed (pageable host memory), the D2D form is
  * asynchronous.  Replaces cuda_cub::trivial_copy_{to,from}_device / trivial_copy_device_to_device

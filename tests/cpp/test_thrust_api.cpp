@@ -35,6 +35,7 @@
 #include <thrust/transform_reduce.h>
 #include <thrust/transform_scan.h>
 #include <thrust/unique.h>
+#include <thrust/universal_vector.h>
 
 #include <cstdint>
 #include <cstdio>
@@ -1043,6 +1044,37 @@ static void TestAsyncAlgorithms() {
 // Memory resources, allocators over them and allocator-aware device_vector (the reference:
 // testing/mr_pool.cu, testing/allocator.cu, testing/caching_allocator.cu,
 // examples/mr_basic.cu).
+static void TestUniversalVector() {  // testing/universal_memory.cu:25-82: one pointer for host code and algorithms
+  g_test = "UniversalVector";
+  const size_t n = 100003;
+  thrust::universal_vector<unsigned int> u(n);
+  unsigned int* direct = thrust::raw_pointer_cast(u.data());
+  thrust::host_vector<unsigned int> h(n);
+  for (size_t i = 0; i < n; ++i) h[i] = direct[i] = (unsigned int)mix(i * 77 + 1);  // written by plain host stores
+  thrust::sort(u.begin(), u.end());                                                 // sorted by the device system
+  thrust::sort(h.begin(), h.end());
+  bool ok = true;
+  for (size_t i = 0; i < n; ++i) ok = ok && direct[i] == h[i];                      // read back by plain host loads
+  ASSERT_TRUE(ok);
+  ASSERT_TRUE(thrust::reduce(u.begin(), u.end(), 0u) == thrust::reduce(h.begin(), h.end(), 0u));
+  ASSERT_TRUE(u[5] == h[5]);
+  u[5] = 123u;
+  ASSERT_TRUE(direct[5] == 123u);
+  thrust::device_vector<unsigned int> d(u.begin(), u.end());  // universal -> device
+  h[5] = 123u;
+  ASSERT_EQUAL_VEC(to_host(d), h);
+  thrust::universal_vector<unsigned int> scanned(n);
+  thrust::inclusive_scan(d.begin(), d.end(), scanned.begin());  // device -> universal output
+  thrust::host_vector<unsigned int> hs(n);
+  thrust::inclusive_scan(h.begin(), h.end(), hs.begin());
+  ok = true;
+  const unsigned int* sdirect = thrust::raw_pointer_cast(scanned.data());
+  for (size_t i = 0; i < n; ++i) ok = ok && sdirect[i] == hs[i];
+  ASSERT_TRUE(ok);
+  thrust::universal_vector<int> empty;
+  ASSERT_TRUE(empty.size() == 0 && empty.begin() == empty.end());
+}
+
 static void TestMemoryResources() {
   g_test = "MemoryResources";
   typedef thrust::mr::unsynchronized_pool_resource<thrust::device_memory_resource> Pool;
@@ -1151,6 +1183,7 @@ int main() {
   TestCustomTemporaryAllocation();
   TestAsyncAlgorithms();
   TestMemoryResources();
+  TestUniversalVector();
   std::printf("%s: %d checks, %d failed\n", g_failed ? "FAILED" : "PASSED", g_checks, g_failed);
   return g_failed ? 1 : 0;
 }

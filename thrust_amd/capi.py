@@ -73,6 +73,8 @@ SIGNATURES = {
                                                _int, _sz, _int, _vp]),
     "thrust_amd_sort_keys": (_int, [_vp, _szp, _vp, _u64, _int, _int, _int, _int, _vp]),
     "thrust_amd_sort_pairs": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _sz, _int, _int, _int, _vp]),
+    "thrust_amd_malloc_universal": (_int, [_c.POINTER(_vp), _sz]),
+    "thrust_amd_free_universal": (_int, [_vp]),
     "thrust_amd_merge_sort_keys": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp]),
     "thrust_amd_merge_sort_pairs": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _sz, _int, _vp]),
     "thrust_amd_copy_if": (_int, [_vp, _szp, _vp, _vp, _vp, _vp, _u64, _sz, _int, _int, _vp, _vp]),

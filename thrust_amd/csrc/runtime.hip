@@ -46,19 +46,38 @@ TA_EXPORT int thrust_amd_free(void* ptr) {
   return (int)hipFree(ptr);
 }
 
+// Universal memory: pinned host memory that the device addresses directly.  Both sides can
+// dereference the same pointer and no page ever migrates or faults.
+TA_EXPORT int thrust_amd_malloc_universal(void** ptr, size_t bytes) {
+  if (!ptr) return (int)hipErrorInvalidValue;
+  *ptr = nullptr;
+  if (bytes == 0) return 0;
+  hipError_t e = hipHostMalloc(ptr, bytes, hipHostMallocDefault);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    *ptr = nullptr;
+  }
+  return (int)e;
+}
+
+TA_EXPORT int thrust_amd_free_universal(void* ptr) {
+  if (!ptr) return 0;
+  return (int)hipHostFree(ptr);
+}
+
 TA_EXPORT int thrust_amd_memcpy(void* dst, const void* src, size_t bytes, int kind, void* stream) {
   if (bytes == 0) return 0;
   if (!dst || !src) return (int)hipErrorInvalidValue;
   hipStream_t s = (hipStream_t)stream;
   switch (kind) {
+    // the runtime resolves the address spaces itself (hipMemcpyDefault), so that universal
+    // memory may stand on either side; `kind` keeps deciding whether the call blocks
     case THRUST_AMD_H2D:
-      TA_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, s));
-      return (int)hipStreamSynchronize(s);
     case THRUST_AMD_D2H:
-      TA_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, s));
+      TA_CHECK(hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, s));
       return (int)hipStreamSynchronize(s);
     case THRUST_AMD_D2D:
-      return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, s);
+      return (int)hipMemcpyAsync(dst, src, bytes, hipMemcpyDefault, s);
     default:
       return (int)hipErrorInvalidValue;
   }
