@@ -479,10 +479,17 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   }
   if constexpr (HAS_VALUES) {
     V v[ITEMS];
+    if (valid == (uint32_t)TILE) {
+      // whole tile: no predicates, so that all loads are in flight together (a predicated
+      // load makes the compiler wait for it before issuing the next one)
 #pragma unroll
-    for (int r = 0; r < ITEMS; ++r) {
-      const uint32_t pos = span + r * WAVE;
-      v[r] = (pos < valid) ? vals_in[tile_base + pos] : V{};
+      for (int r = 0; r < ITEMS; ++r) v[r] = vals_in[tile_base + span + r * WAVE];
+    } else {
+#pragma unroll
+      for (int r = 0; r < ITEMS; ++r) {
+        const uint32_t pos = span + r * WAVE;
+        v[r] = (pos < valid) ? vals_in[tile_base + pos] : V{};
+      }
     }
     __syncthreads();  // keys have been read out of the exchange buffer
 #pragma unroll
