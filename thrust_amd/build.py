@@ -21,8 +21,15 @@ FLAGS = [
 ]
 
 
+# Sources that take longest to compile (many template instances) go first, so that the
+# worker pool does not end on one of them.
+SLOWEST_FIRST = ["transform_scan.hip", "transform_scan_exclusive.hip", "merge_sort.hip", "scan.hip",
+                 "reduce_by_key.hip", "radix_sort.hip", "scan_by_key.hip", "transform_reduce.hip"]
+
+
 def sources():
-    return sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+    found = sorted(f for f in os.listdir(CSRC) if f.endswith(".hip"))
+    return [f for f in SLOWEST_FIRST if f in found] + [f for f in found if f not in SLOWEST_FIRST]
 
 
 def _compile(src):
