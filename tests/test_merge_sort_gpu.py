@@ -112,3 +112,43 @@ def test_merge_sort_temp_and_arguments(dev):
     assert lib.thrust_amd_merge_sort_keys(d.ptr, ctypes.byref(small), d.ptr, 1 << 20, i32, 0, dev.stream_ptr()) != 0
     assert lib.thrust_amd_merge_sort_keys(None, ctypes.byref(need), None, 10, 99, 0, dev.stream_ptr()) != 0
     assert lib.thrust_amd_merge_sort_pairs(None, ctypes.byref(need), None, None, 10, i32, 3, 0, dev.stream_ptr()) != 0
+
+
+def test_merge_sort_full_size_properties(dev):
+    """2^28 uint32 keys: sortedness, a 64-bit sum checksum and a histogram of the top byte; then
+    2^27 pairs with 256 distinct keys, where stability fixes the order of the values: inside a
+    run of equal keys the values (input positions) must increase.  All checked on the device."""
+    import torch
+    n = 1 << 28
+    g = torch.Generator(device="cuda")
+    g.manual_seed(11)
+    src = torch.randint(-(1 << 31), 1 << 31, (n,), dtype=torch.int32, device="cuda", generator=g)
+
+    def u32(t):
+        return t.to(torch.int64) & 0xFFFFFFFF
+
+    s_sum = int(u32(src).sum().item())
+    s_hist = torch.bincount((u32(src) >> 24).to(torch.int64), minlength=256)
+    d = dev.DeviceArray(n, dev.U32, src.view(torch.uint8).clone())
+    del src
+    dev.merge_sort_keys(d)
+    o = u32(d.storage.view(torch.int32))
+    assert bool((o[1:] >= o[:-1]).all().item())
+    assert int(o.sum().item()) == s_sum
+    assert torch.equal(torch.bincount((o >> 24).to(torch.int64), minlength=256), s_hist)
+    del o, d
+
+    m = 1 << 27
+    keys = torch.randint(0, 256, (m,), dtype=torch.int32, device="cuda", generator=g)
+    vals = torch.arange(m, dtype=torch.int32, device="cuda")
+    counts = torch.bincount(keys.to(torch.int64), minlength=256)
+    dk = dev.DeviceArray(m, dev.I32, keys.view(torch.uint8).clone())
+    dv = dev.DeviceArray(m, dev.U32, vals.view(torch.uint8).clone())
+    dev.merge_sort_pairs(dk, dv, descending=True)
+    ok = dk.storage.view(torch.int32)
+    ov = dv.storage.view(torch.int32)
+    assert bool((ok[1:] <= ok[:-1]).all().item())
+    assert torch.equal(torch.bincount(ok.to(torch.int64), minlength=256), counts)
+    assert bool((keys[ov.to(torch.int64)] == ok).all().item())          # every value still sits with its key
+    same = ok[1:] == ok[:-1]
+    assert bool((ov[1:][same] > ov[:-1][same]).all().item())            # equal keys keep their input order
