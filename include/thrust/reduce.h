@@ -9,6 +9,9 @@
 #include <thrust/pair.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#if defined(__HIPCC__)
+#include <thrust/system/hip/detail/generic_kernels.h>
+#endif
 
 namespace thrust {
 
@@ -93,37 +96,78 @@ pair<KOut, VOut> reduce_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, KOu
 namespace hip {
 // The accumulator has the type of init; elements of another arithmetic type are converted
 // to it first, as plus<T> does in the reference (testing/reduce.cu:99-129).
+namespace detail {
 template <typename D, typename It, typename T, typename Op>
-T reduce(execution_policy<D>& exec, It first, It last, T init, Op) {
+T reduce(execution_policy<D>& exec, It first, It last, T init, Op, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
-  static_assert(detail::is_device_input<It>::value,
-                "thrust::reduce on the device system needs device_ptr / device_vector iterators, raw device pointers "
-                "or fancy iterators over them");
-  static_assert(detail::is_abi_type<T>::value && detail::is_abi_type<V>::value,
-                "thrust::reduce on the device system: elements and init must have arithmetic types");
-  static_assert(detail::binop_code<Op, T>::value >= 0,
-                "thrust::reduce on the device system supports thrust::plus, thrust::minimum and thrust::maximum "
-                "of the type of init");
-  void* stream = detail::stream_of(exec);
+  void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
-  detail::device_input<It> source(stream, detail::temp_source_of(exec), first, n);
-  detail::temp_storage converted(stream, detail::temp_source_of(exec));
-  const void* in = n ? (const void*)detail::input_as<T>(source.ptr(), n, stream, converted) : nullptr;
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
+  device_input<It> source(stream, temp_source_of(exec), first, n);
+  temp_storage converted(stream, temp_source_of(exec));
+  const void* in = n ? (const void*)input_as<T>(source.ptr(), n, stream, converted) : nullptr;
+  temp_storage temp(stream, temp_source_of(exec));
   void* d_out = nullptr;
   // the result slot is the `extra` region, which run() only knows after the size query
   std::size_t need = 0;
-  detail::throw_on_error(thrust_amd_reduce(nullptr, &need, in, n, detail::dtype_of<T>::value,
-                                           detail::binop_code<Op, T>::value, &init, nullptr, stream),
+  throw_on_error(thrust_amd_reduce(nullptr, &need, in, n, dtype_of<T>::value,
+                                           binop_code<Op, T>::value, &init, nullptr, stream),
                          "reduce: temp size query");
   const std::size_t aligned = (need + 255) / 256 * 256;
   temp.ensure(aligned + 256);
   d_out = static_cast<char*>(temp.ptr()) + aligned;
   std::size_t bytes = aligned;
-  detail::throw_on_error(thrust_amd_reduce(temp.ptr(), &bytes, in, n, detail::dtype_of<T>::value,
-                                           detail::binop_code<Op, T>::value, &init, d_out, stream),
+  throw_on_error(thrust_amd_reduce(temp.ptr(), &bytes, in, n, dtype_of<T>::value,
+                                           binop_code<Op, T>::value, &init, d_out, stream),
                          "reduce failed");
-  return detail::read_scalar<T>(d_out, stream, "reduce: result copy");
+  return read_scalar<T>(d_out, stream, "reduce: result copy");
+}
+
+// A user's operator or element type: kernels instantiated for them (hipcc translation units).
+template <typename D, typename It, typename T, typename Op>
+T reduce(execution_policy<D>& exec, It first, It last, T init, Op op, std::false_type) {
+#if defined(__HIPCC__)
+  namespace gk = thrust::system::hip::generic;
+  typedef typename thrust::detail::device_view_of<It>::type View;
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return init;
+  uint64_t chunks = (n + gk::TILE - 1) / gk::TILE;
+  if (chunks > 1024) chunks = 1024;
+  const uint64_t chunk = (n + chunks - 1) / chunks;
+  chunks = (n + chunk - 1) / chunk;  // every chunk holds at least one element
+  const std::size_t partial_bytes = ((std::size_t)chunks * sizeof(T) + 255) / 256 * 256;
+  temp_storage temp(stream, temp_source_of(exec));
+  temp.ensure(partial_bytes + 256);
+  T* partials = static_cast<T*>(temp.ptr());
+  T* d_out = reinterpret_cast<T*>(static_cast<char*>(temp.ptr()) + partial_bytes);
+  hipLaunchKernelGGL((gk::reduce_chunks_kernel<View, T, Op>), dim3((unsigned)chunks), dim3(gk::BLOCK), 0,
+                     (hipStream_t)stream, thrust::detail::device_view(first), n, chunk, op, partials);
+  throw_on_error(launch_status(), "reduce: kernel launch");
+  hipLaunchKernelGGL((gk::reduce_final_kernel<T, Op>), dim3(1), dim3(gk::BLOCK), 0, (hipStream_t)stream,
+                     (const T*)partials, (uint32_t)chunks, init, op, d_out);
+  throw_on_error(launch_status(), "reduce: kernel launch");
+  return read_scalar<T>(d_out, stream, "reduce: result copy");
+#else
+  static_assert(fancy_needs_hipcc<Op>::value,
+                "thrust::reduce on the device system: operators other than thrust::plus / minimum / maximum of an "
+                "arithmetic type run in kernels instantiated for the operator; compile this translation unit with hipcc");
+  return init;
+#endif
+}
+
+template <typename T, typename V, typename Op, bool = is_abi_type<T>::value && is_abi_type<V>::value>
+struct reduces_in_library : std::integral_constant<bool, (binop_code<Op, T>::value >= 0)> {};
+template <typename T, typename V, typename Op>
+struct reduces_in_library<T, V, Op, false> : std::false_type {};
+}  // namespace detail
+
+template <typename D, typename It, typename T, typename Op>
+T reduce(execution_policy<D>& exec, It first, It last, T init, Op op) {
+  typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
+  static_assert(detail::is_device_input<It>::value,
+                "thrust::reduce on the device system needs device_ptr / device_vector iterators, raw device pointers "
+                "or fancy iterators over them");
+  return detail::reduce(exec, first, last, init, op, detail::reduces_in_library<T, V, Op>());
 }
 
 template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>

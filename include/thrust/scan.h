@@ -13,6 +13,9 @@
 #include <thrust/functional.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#if defined(__HIPCC__)
+#include <thrust/system/hip/detail/generic_kernels.h>
+#endif
 
 namespace thrust {
 
@@ -152,68 +155,120 @@ Out exclusive_scan_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, Out resu
 }  // namespace cpp
 
 namespace hip {
+// The accumulator's type is the input's element type for inclusive_scan and the type of init
+// for exclusive_scan; input and output may hold other arithmetic types, converted on the way
+// in and out as the reference does (testing/scan.cu:236-295).
 namespace detail {
-// A is the accumulator's type: the input's element type for inclusive_scan, the type of
-// init for exclusive_scan; input and output may hold other arithmetic types, converted on
-// the way in and out as the reference does (testing/scan.cu:236-295).
-template <typename In, typename Out, typename A, typename Op>
-struct scan_checks {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
-  typedef typename iterator_value<Out>::type U;
-  static_assert(is_device_input<In>::value &&
-                    (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value),
-                "scan on the device system needs device_ptr / device_vector iterators or raw device pointers "
-                "(fancy iterators as input only)");
-  static_assert(is_abi_type<V>::value && is_abi_type<A>::value && is_abi_type<U>::value,
-                "scan on the device system: input, output and init must have arithmetic types");
-  static_assert(binop_code<Op, A>::value >= 0,
-                "scan on the device system supports thrust::plus, thrust::minimum and thrust::maximum "
-                "of the accumulator's type");
-};
-}  // namespace detail
-
 template <typename D, typename In, typename Out, typename Op>
-Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op) {
+Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
   typedef typename iterator_value<Out>::type U;
-  (void)sizeof(detail::scan_checks<In, Out, V, Op>);
-  void* stream = detail::stream_of(exec);
+  void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  detail::device_input<In> source(stream, detail::temp_source_of(exec), first, n);
-  detail::temp_storage staged(stream, detail::temp_source_of(exec));
-  V* computed = detail::output_as<V>(static_cast<U*>(thrust::detail::raw(result)), n, staged);
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
-  detail::run(temp, 0, "inclusive_scan failed", [&](void* t, std::size_t* b) {
-    return thrust_amd_inclusive_scan(t, b, source.ptr(), computed, n, detail::dtype_of<V>::value,
-                                     detail::binop_code<Op, V>::value, stream);
+  device_input<In> source(stream, temp_source_of(exec), first, n);
+  temp_storage staged(stream, temp_source_of(exec));
+  V* computed = output_as<V>(static_cast<U*>(thrust::detail::raw(result)), n, staged);
+  temp_storage temp(stream, temp_source_of(exec));
+  run(temp, 0, "inclusive_scan failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_inclusive_scan(t, b, source.ptr(), computed, n, dtype_of<V>::value,
+                                     binop_code<Op, V>::value, stream);
   });
-  detail::finish_output(computed, static_cast<U*>(thrust::detail::raw(result)), n, stream);
-  detail::synchronize(stream, "inclusive_scan: synchronize");
+  finish_output(computed, static_cast<U*>(thrust::detail::raw(result)), n, stream);
+  synchronize(stream, "inclusive_scan: synchronize");
   return result + n;
 }
 
 template <typename D, typename In, typename Out, typename T, typename Op>
-Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T init, Op) {
+Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T init, Op, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
   typedef typename iterator_value<Out>::type U;
-  (void)sizeof(detail::scan_checks<In, Out, T, Op>);
-  void* stream = detail::stream_of(exec);
+  void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  detail::device_input<In> source(stream, detail::temp_source_of(exec), first, n);
-  detail::temp_storage converted(stream, detail::temp_source_of(exec));
-  const T* in = detail::input_as<T>(source.ptr(), n, stream, converted);
-  detail::temp_storage staged(stream, detail::temp_source_of(exec));
-  T* computed = detail::output_as<T>(static_cast<U*>(thrust::detail::raw(result)), n, staged);
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
-  detail::run(temp, 0, "exclusive_scan failed", [&](void* t, std::size_t* b) {
-    return thrust_amd_exclusive_scan(t, b, in, computed, n, detail::dtype_of<T>::value,
-                                     detail::binop_code<Op, T>::value, &init, stream);
+  device_input<In> source(stream, temp_source_of(exec), first, n);
+  temp_storage converted(stream, temp_source_of(exec));
+  const T* in = input_as<T>(source.ptr(), n, stream, converted);
+  temp_storage staged(stream, temp_source_of(exec));
+  T* computed = output_as<T>(static_cast<U*>(thrust::detail::raw(result)), n, staged);
+  temp_storage temp(stream, temp_source_of(exec));
+  run(temp, 0, "exclusive_scan failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_exclusive_scan(t, b, in, computed, n, dtype_of<T>::value,
+                                     binop_code<Op, T>::value, &init, stream);
   });
-  detail::finish_output(computed, static_cast<U*>(thrust::detail::raw(result)), n, stream);
-  detail::synchronize(stream, "exclusive_scan: synchronize");
+  finish_output(computed, static_cast<U*>(thrust::detail::raw(result)), n, stream);
+  synchronize(stream, "exclusive_scan: synchronize");
   return result + n;
+}
+
+// A user's operator or element type: three kernels instantiated for them (hipcc translation
+// units).  A is the accumulator's type, as in the library path.
+template <bool EXCLUSIVE, typename A, typename D, typename In, typename Out, typename Op>
+Out scan_generic(execution_policy<D>& exec, In first, In last, Out result, A init, Op op) {
+  static_assert(is_device_input<In>::value &&
+                    (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value),
+                "scan on the device system needs device_ptr / device_vector iterators or raw device pointers "
+                "(fancy iterators as input only)");
+#if defined(__HIPCC__)
+  namespace gk = thrust::system::hip::generic;
+  typedef typename thrust::detail::device_view_of<In>::type View;
+  typedef typename iterator_value<Out>::type U;
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  const uint64_t tiles = (n + gk::TILE - 1) / gk::TILE;
+  if (tiles > 0xffffffffull) throw_on_error(1, "scan: range too long");
+  temp_storage temp(stream, temp_source_of(exec));
+  temp.ensure((std::size_t)tiles * sizeof(A));
+  A* tile_total = static_cast<A*>(temp.ptr());
+  hipLaunchKernelGGL((gk::scan_tile_totals_kernel<View, A, Op>), dim3((unsigned)tiles), dim3(gk::BLOCK), 0,
+                     (hipStream_t)stream, thrust::detail::device_view(first), n, op, tile_total);
+  throw_on_error(launch_status(), "scan: kernel launch");
+  hipLaunchKernelGGL((gk::scan_tile_prefix_kernel<A, Op>), dim3(1), dim3(gk::BLOCK), 0, (hipStream_t)stream,
+                     tile_total, (uint32_t)tiles, op);
+  throw_on_error(launch_status(), "scan: kernel launch");
+  hipLaunchKernelGGL((gk::scan_tiles_kernel<EXCLUSIVE, View, A, U, Op>), dim3((unsigned)tiles), dim3(gk::BLOCK), 0,
+                     (hipStream_t)stream, thrust::detail::device_view(first), thrust::detail::raw(result), n, op, init,
+                     (const A*)tile_total);
+  throw_on_error(launch_status(), "scan: kernel launch");
+  synchronize(stream, "scan: synchronize");
+  return result + n;
+#else
+  static_assert(fancy_needs_hipcc<Op>::value,
+                "scan on the device system: operators other than thrust::plus / minimum / maximum of an arithmetic "
+                "type run in kernels instantiated for the operator; compile this translation unit with hipcc");
+  return result;
+#endif
+}
+template <typename D, typename In, typename Out, typename Op>
+Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op op, std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  return scan_generic<false, V>(exec, first, last, result, V(), op);
+}
+template <typename D, typename In, typename Out, typename T, typename Op>
+Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T init, Op op, std::false_type) {
+  return scan_generic<true, T>(exec, first, last, result, init, op);
+}
+
+// library path: arithmetic input, output and accumulator with plus / minimum / maximum of the accumulator's type
+template <typename V, typename U, typename A, typename Op,
+          bool = is_abi_type<V>::value && is_abi_type<U>::value && is_abi_type<A>::value>
+struct scans_in_library : std::integral_constant<bool, (binop_code<Op, A>::value >= 0)> {};
+template <typename V, typename U, typename A, typename Op>
+struct scans_in_library<V, U, A, Op, false> : std::false_type {};
+}  // namespace detail
+
+template <typename D, typename In, typename Out, typename Op>
+Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op op) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  typedef typename iterator_value<Out>::type U;
+  return detail::inclusive_scan(exec, first, last, result, op, detail::scans_in_library<V, U, V, Op>());
+}
+template <typename D, typename In, typename Out, typename T, typename Op>
+Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T init, Op op) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  typedef typename iterator_value<Out>::type U;
+  return detail::exclusive_scan(exec, first, last, result, init, op, detail::scans_in_library<V, U, T, Op>());
 }
 
 namespace detail {

@@ -24,6 +24,8 @@
 #include <thrust/transform.h>
 #include <thrust/transform_reduce.h>
 
+#include <hip/hip_runtime.h>
+
 #include <cstdint>
 #include <cstdio>
 #include <vector>
@@ -80,6 +82,92 @@ struct double_in_place {
 struct widen_square {
   __host__ __device__ long long operator()(int x) const { return (long long)x * x; }
 };
+
+// user operators for reduce and the scans
+struct Affine {  // x -> a * x + b over unsigned wrap-around; composition is associative, not commutative
+  unsigned a, b;
+  __host__ __device__ bool operator==(const Affine& o) const { return a == o.a && b == o.b; }
+};
+struct compose {  // apply the left function first, then the right one
+  __host__ __device__ Affine operator()(const Affine& f, const Affine& g) const { return Affine{f.a * g.a, f.b * g.a + g.b}; }
+};
+struct MinMax {
+  int lo, hi;
+  __host__ __device__ bool operator==(const MinMax& o) const { return lo == o.lo && hi == o.hi; }
+};
+struct to_minmax {
+  __host__ __device__ MinMax operator()(int x) const { return MinMax{x, x}; }
+};
+struct merge_minmax {  // associative and commutative
+  __host__ __device__ MinMax operator()(const MinMax& a, const MinMax& b) const {
+    return MinMax{a.lo < b.lo ? a.lo : b.lo, a.hi > b.hi ? a.hi : b.hi};
+  }
+};
+struct bit_xor_op {
+  __host__ __device__ unsigned operator()(unsigned a, unsigned b) const { return a ^ b; }
+};
+
+static void TestUserOperators() {
+  for (size_t n : kSizes) {
+    g_test = "reduce with user operators";
+    {
+      const thrust::host_vector<int> h = random_values<int>(n, 21, 100001);
+      const thrust::device_vector<int> d(h);
+      const MinMax init = {1 << 30, -(1 << 30)};
+      // the minimum / maximum example of the reference (examples/minmax.cu): one pass, a struct as the sum
+      const MinMax want = thrust::transform_reduce(h.begin(), h.end(), to_minmax(), init, merge_minmax());
+      const MinMax got = thrust::transform_reduce(d.begin(), d.end(), to_minmax(), init, merge_minmax());
+      ASSERT_TRUE(got == want);
+      const thrust::host_vector<unsigned> hu = random_values<unsigned>(n, 22, 1u << 31);
+      const thrust::device_vector<unsigned> du(hu);
+      ASSERT_TRUE(thrust::reduce(du.begin(), du.end(), 5u, bit_xor_op()) == thrust::reduce(hu.begin(), hu.end(), 5u, bit_xor_op()));
+      ASSERT_TRUE(thrust::reduce(du.begin(), du.end(), 1u, thrust::multiplies<unsigned>()) ==
+                  thrust::reduce(hu.begin(), hu.end(), 1u, thrust::multiplies<unsigned>()));
+    }
+    g_test = "scans with user operators";
+    {
+      thrust::host_vector<Affine> h(n);
+      for (size_t i = 0; i < n; ++i) h[i] = Affine{(unsigned)(mix(i) | 1u), (unsigned)mix(i + 99)};
+      Affine* dptr = nullptr;
+      Affine* dout = nullptr;
+      if (n) {
+        dptr = thrust::raw_pointer_cast(thrust::device_malloc<Affine>(n));
+        dout = thrust::raw_pointer_cast(thrust::device_malloc<Affine>(n));
+        (void)hipMemcpy(dptr, h.data(), n * sizeof(Affine), hipMemcpyHostToDevice);
+      }
+      thrust::host_vector<Affine> want(n), got(n);
+      thrust::inclusive_scan(h.begin(), h.end(), want.begin(), compose());
+      thrust::inclusive_scan(thrust::device, dptr, dptr + n, dout, compose());
+      if (n) (void)hipMemcpy(got.data(), dout, n * sizeof(Affine), hipMemcpyDeviceToHost);
+      ASSERT_TRUE(same(got, want));
+      const Affine init = {3u, 7u};
+      thrust::exclusive_scan(h.begin(), h.end(), want.begin(), init, compose());
+      thrust::exclusive_scan(thrust::device, dptr, dptr + n, dout, init, compose());
+      if (n) (void)hipMemcpy(got.data(), dout, n * sizeof(Affine), hipMemcpyDeviceToHost);
+      ASSERT_TRUE(same(got, want));
+      // in place
+      thrust::inclusive_scan(h.begin(), h.end(), want.begin(), compose());
+      thrust::inclusive_scan(thrust::device, dptr, dptr + n, dptr, compose());
+      if (n) (void)hipMemcpy(got.data(), dptr, n * sizeof(Affine), hipMemcpyDeviceToHost);
+      ASSERT_TRUE(same(got, want));
+      if (n) {
+        thrust::device_free(thrust::device_pointer_cast(dptr));
+        thrust::device_free(thrust::device_pointer_cast(dout));
+      }
+      // an operator of thrust/functional.h outside the library's set, on arithmetic elements
+      const thrust::host_vector<unsigned> hu = random_values<unsigned>(n, 23, 1u << 31);
+      const thrust::device_vector<unsigned> du(hu);
+      thrust::host_vector<unsigned> hs(n);
+      thrust::device_vector<unsigned> ds(n);
+      thrust::inclusive_scan(hu.begin(), hu.end(), hs.begin(), thrust::multiplies<unsigned>());
+      thrust::inclusive_scan(du.begin(), du.end(), ds.begin(), thrust::multiplies<unsigned>());
+      ASSERT_TRUE(same(to_host(ds), hs));
+      thrust::exclusive_scan(hu.begin(), hu.end(), hs.begin(), 9u, bit_xor_op());
+      thrust::exclusive_scan(du.begin(), du.end(), ds.begin(), 9u, bit_xor_op());
+      ASSERT_TRUE(same(to_host(ds), hs));
+    }
+  }
+}
 
 static void TestKnownAnswers() {
   g_test = "GatherSimple";
@@ -247,6 +335,7 @@ static void Differential() {
 int main() {
   TestKnownAnswers();
   Differential();
+  TestUserOperators();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
   std::printf(g_failed ? "FAILED\n" : "PASSED\n");
   return g_failed ? 1 : 0;
