@@ -176,43 +176,58 @@ inline uint64_t run_selection(void* stream, const temp_source& source, const Pre
 }  // namespace detail
 
 namespace detail {
-// recognised predicate on the tested elements themselves: compared inside the selection kernel
+// What a selection kernel tests.  A recognised predicate on arithmetic elements is evaluated
+// inside the kernel on the elements themselves (or on the stencil); any other predicate is
+// evaluated first, by a kernel instantiated for it, into one byte per element, and the
+// selection kernel takes those bytes as its stencil.
+template <typename St, typename Pred,
+          bool InKernel = selects_in_kernel<Pred, typename std::remove_const<typename iterator_value<St>::type>::type>::value>
+class tested_stream {
+ public:
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type tested_type;
+  typedef Pred predicate_type;
+  tested_stream(void* stream, const temp_source& source, St tested, uint64_t n, Pred pred, bool has_stencil)
+      : input_(stream, source, tested, has_stencil ? n : 0), pred_(pred), has_stencil_(has_stencil) {}
+  const void* stencil() const { return has_stencil_ ? (const void*)input_.ptr() : nullptr; }
+  int dtype() const { return dtype_of<tested_type>::value; }
+  const Pred& predicate() const { return pred_; }
+
+ private:
+  device_input<St> input_;
+  Pred pred_;
+  bool has_stencil_;
+};
+template <typename St, typename Pred>
+class tested_stream<St, Pred, false> {
+ public:
+  typedef unsigned char tested_type;
+  typedef thrust::identity<unsigned char> predicate_type;
+  tested_stream(void* stream, const temp_source& source, St tested, uint64_t n, Pred pred, bool)
+      : flags_(stream, source, thrust::make_transform_iterator(tested, as_flag<Pred>{pred}), n) {}
+  const void* stencil() const { return flags_.ptr(); }
+  int dtype() const { return THRUST_AMD_U8; }
+  predicate_type predicate() const { return predicate_type(); }
+
+ private:
+  device_input<thrust::transform_iterator<as_flag<Pred>, St> > flags_;
+};
+
 template <typename D, typename In, typename St, typename Out, typename Pred>
 Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, bool has_stencil, Out result, Pred pred,
-                 std::true_type) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
-  void* stream = stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return result;
-  device_input<In> source(stream, temp_source_of(exec), first, n);
-  device_input<St> tested(stream, temp_source_of(exec), stencil, has_stencil ? n : 0);
-  const uint64_t cnt = run_selection<S>(stream, temp_source_of(exec), pred, "copy_if failed",
-      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_copy_if(t, b, source.ptr(), has_stencil ? (const void*)tested.ptr() : nullptr,
-                                  thrust::detail::raw(result), d_num, n, sizeof(T), dtype_of<S>::value, cmp, thr,
-                                  stream);
-      });
-  return result + cnt;
-}
-// any other predicate: one byte per element from a transform iterator, then the stencil form
-template <typename D, typename In, typename St, typename Out, typename Pred>
-Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, bool, Out result, Pred pred,
-                 std::false_type) {
+                 bool negate) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  const as_flag<Pred> flag = {pred};
   device_input<In> source(stream, temp_source_of(exec), first, n);
-  device_input<thrust::transform_iterator<as_flag<Pred>, St> > flags(
-      stream, temp_source_of(exec), thrust::make_transform_iterator(stencil, flag), n);
-  const uint64_t cnt = run_selection<unsigned char>(
-      stream, temp_source_of(exec), thrust::identity<unsigned char>(), "copy_if failed",
+  tested_stream<St, Pred> tested(stream, temp_source_of(exec), stencil, n, pred, has_stencil);
+  const uint64_t cnt = run_selection<typename tested_stream<St, Pred>::tested_type>(
+      stream, temp_source_of(exec), tested.predicate(), "copy_if failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_copy_if(t, b, source.ptr(), flags.ptr(), thrust::detail::raw(result), d_num, n, sizeof(T),
-                                  THRUST_AMD_U8, cmp, thr, stream);
-      });
+        return thrust_amd_copy_if(t, b, source.ptr(), tested.stencil(), thrust::detail::raw(result), d_num, n,
+                                  sizeof(T), tested.dtype(), cmp, thr, stream);
+      },
+      negate);
   return result + cnt;
 }
 }  // namespace detail
@@ -222,7 +237,7 @@ Out copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred)
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
   static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
                 "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  return detail::copy_if_impl(exec, first, last, first, false, result, pred, detail::selects_in_kernel<Pred, T>());
+  return detail::copy_if_impl(exec, first, last, first, false, result, pred, false);
 }
 template <typename D, typename In, typename St, typename Out, typename Pred>
 Out copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result, Pred pred) {
@@ -230,7 +245,7 @@ Out copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result
   typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
   static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
                 "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  return detail::copy_if_impl(exec, first, last, stencil, true, result, pred, detail::selects_in_kernel<Pred, S>());
+  return detail::copy_if_impl(exec, first, last, stencil, true, result, pred, false);
 }
 }  // namespace hip
 }  // namespace system

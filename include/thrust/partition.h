@@ -48,74 +48,65 @@ pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In l
 }  // namespace cpp
 
 namespace hip {
-template <typename D, typename It, typename Pred>
-It stable_partition(execution_policy<D>& exec, It first, It last, Pred pred) {
+namespace detail {
+template <typename D, typename It, typename St, typename Pred>
+It stable_partition_impl(execution_policy<D>& exec, It first, It last, St stencil, bool has_stencil, Pred pred) {
   typedef typename iterator_value<It>::type T;
-  void* stream = detail::stream_of(exec);
+  static_assert(is_abi_item<T>::value, "stable_partition on the device system: items of 1, 2, 4 or 8 bytes");
+  void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return first;
-  const uint64_t cnt = detail::run_selection<T>(stream, detail::temp_source_of(exec), pred, "stable_partition failed",
+  tested_stream<St, Pred> tested(stream, temp_source_of(exec), stencil, n, pred, has_stencil);
+  const uint64_t cnt = run_selection<typename tested_stream<St, Pred>::tested_type>(
+      stream, temp_source_of(exec), tested.predicate(), "stable_partition failed",
       [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_stable_partition(t, b, thrust::detail::raw(first), nullptr, d_num, n, sizeof(T),
-                                           detail::dtype_of<T>::value, cmp, thr, stream);
+        return thrust_amd_stable_partition(t, b, thrust::detail::raw(first), tested.stencil(), d_num, n, sizeof(T),
+                                           tested.dtype(), cmp, thr, stream);
       });
-  detail::synchronize(stream, "stable_partition: synchronize");
+  synchronize(stream, "stable_partition: synchronize");
   return first + cnt;
+}
+template <typename D, typename In, typename St, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy_impl(execution_policy<D>& exec, In first, In last, St stencil, bool has_stencil,
+                                            Out1 out_true, Out2 out_false, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  static_assert(is_abi_item<T>::value && std::is_same<typename iterator_value<Out1>::type, T>::value &&
+                    std::is_same<typename iterator_value<Out2>::type, T>::value,
+                "partition_copy on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return thrust::make_pair(out_true, out_false);
+  device_input<In> source(stream, temp_source_of(exec), first, n);
+  tested_stream<St, Pred> tested(stream, temp_source_of(exec), stencil, n, pred, has_stencil);
+  const uint64_t cnt = run_selection<typename tested_stream<St, Pred>::tested_type>(
+      stream, temp_source_of(exec), tested.predicate(), "partition_copy failed",
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_partition_copy(t, b, source.ptr(), tested.stencil(), thrust::detail::raw(out_true),
+                                         thrust::detail::raw(out_false), d_num, n, sizeof(T), tested.dtype(), cmp, thr,
+                                         stream);
+      });
+  synchronize(stream, "partition_copy: synchronize");
+  return thrust::make_pair(out_true + cnt, out_false + (n - cnt));
+}
+}  // namespace detail
+
+template <typename D, typename It, typename Pred>
+It stable_partition(execution_policy<D>& exec, It first, It last, Pred pred) {
+  return detail::stable_partition_impl(exec, first, last, first, false, pred);
 }
 template <typename D, typename It, typename St, typename Pred>
 It stable_partition(execution_policy<D>& exec, It first, It last, St stencil, Pred pred) {
-  typedef typename iterator_value<It>::type T;
-  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
-  static_assert(detail::is_abi_item<T>::value, "stable_partition on the device system: items of 1, 2, 4 or 8 bytes");
-  void* stream = detail::stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return first;
-  const uint64_t cnt = detail::run_selection<S>(stream, detail::temp_source_of(exec), pred, "stable_partition failed",
-      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_stable_partition(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil), d_num, n,
-                                           sizeof(T), detail::dtype_of<S>::value, cmp, thr, stream);
-      });
-  detail::synchronize(stream, "stable_partition: synchronize");
-  return first + cnt;
+  return detail::stable_partition_impl(exec, first, last, stencil, true, pred);
 }
 template <typename D, typename In, typename Out1, typename Out2, typename Pred>
 pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In last, Out1 out_true, Out2 out_false,
                                        Pred pred) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  static_assert(std::is_same<typename iterator_value<Out1>::type, T>::value &&
-                    std::is_same<typename iterator_value<Out2>::type, T>::value,
-                "partition_copy on the device system: input and output element types must match");
-  void* stream = detail::stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return thrust::make_pair(out_true, out_false);
-  const uint64_t cnt = detail::run_selection<T>(stream, detail::temp_source_of(exec), pred, "partition_copy failed",
-      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_partition_copy(t, b, thrust::detail::raw(first), nullptr, thrust::detail::raw(out_true),
-                                         thrust::detail::raw(out_false), d_num, n, sizeof(T),
-                                         detail::dtype_of<T>::value, cmp, thr, stream);
-      });
-  detail::synchronize(stream, "partition_copy: synchronize");
-  return thrust::make_pair(out_true + cnt, out_false + (n - cnt));
+  return detail::stable_partition_copy_impl(exec, first, last, first, false, out_true, out_false, pred);
 }
 template <typename D, typename In, typename St, typename Out1, typename Out2, typename Pred>
 pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In last, St stencil, Out1 out_true,
                                        Out2 out_false, Pred pred) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
-  static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out1>::type, T>::value &&
-                    std::is_same<typename iterator_value<Out2>::type, T>::value,
-                "partition_copy on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  void* stream = detail::stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return thrust::make_pair(out_true, out_false);
-  const uint64_t cnt = detail::run_selection<S>(stream, detail::temp_source_of(exec), pred, "partition_copy failed",
-      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_partition_copy(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil),
-                                         thrust::detail::raw(out_true), thrust::detail::raw(out_false), d_num, n,
-                                         sizeof(T), detail::dtype_of<S>::value, cmp, thr, stream);
-      });
-  detail::synchronize(stream, "partition_copy: synchronize");
-  return thrust::make_pair(out_true + cnt, out_false + (n - cnt));
+  return detail::stable_partition_copy_impl(exec, first, last, stencil, true, out_true, out_false, pred);
 }
 }  // namespace hip
 }  // namespace system

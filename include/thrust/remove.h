@@ -67,34 +67,16 @@ namespace hip {
 template <typename D, typename In, typename Out, typename Pred>
 Out remove_copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  static_assert(std::is_same<typename iterator_value<Out>::type, T>::value,
-                "thrust::remove_copy_if on the device system: input and output element types must match");
-  void* stream = detail::stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return result;
-  const uint64_t cnt = detail::run_selection<T>(stream, detail::temp_source_of(exec), pred, "remove_copy_if failed",
-      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_copy_if(t, b, thrust::detail::raw(first), nullptr, thrust::detail::raw(result), d_num, n,
-                                  sizeof(T), detail::dtype_of<T>::value, cmp, thr, stream);
-      }, true);
-  return result + cnt;
+  static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
+                "thrust::remove_copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
+  return detail::copy_if_impl(exec, first, last, first, false, result, pred, true);
 }
 template <typename D, typename In, typename St, typename Out, typename Pred>
 Out remove_copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result, Pred pred) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
   static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
                 "thrust::remove_copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  void* stream = detail::stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return result;
-  const uint64_t cnt = detail::run_selection<S>(stream, detail::temp_source_of(exec), pred, "remove_copy_if failed",
-      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
-        return thrust_amd_copy_if(t, b, thrust::detail::raw(first), thrust::detail::raw(stencil),
-                                  thrust::detail::raw(result), d_num, n, sizeof(T), detail::dtype_of<S>::value, cmp,
-                                  thr, stream);
-      }, true);
-  return result + cnt;
+  return detail::copy_if_impl(exec, first, last, stencil, true, result, pred, true);
 }
 // in place: the compaction kernel writes a tile only after every earlier tile has been read
 template <typename D, typename It, typename Pred>

@@ -17,6 +17,8 @@
 #include <thrust/iterator/counting_iterator.h>
 #include <thrust/iterator/permutation_iterator.h>
 #include <thrust/iterator/transform_iterator.h>
+#include <thrust/partition.h>
+#include <thrust/remove.h>
 #include <thrust/reduce.h>
 #include <thrust/scan.h>
 #include <thrust/scatter.h>
@@ -265,6 +267,32 @@ static void Differential() {
       ho.resize(he - ho.begin());
       dout.resize(de - dout.begin());
       ASSERT_TRUE(same(to_host(dout), ho));
+    }
+    g_test = "partition / remove_if with a user predicate";
+    {
+      thrust::host_vector<int> hp(h);
+      thrust::device_vector<int> dp(d);
+      auto hmid = thrust::stable_partition(hp.begin(), hp.end(), is_even());
+      auto dmid = thrust::stable_partition(dp.begin(), dp.end(), is_even());
+      ASSERT_TRUE(dmid - dp.begin() == hmid - hp.begin());
+      ASSERT_TRUE(same(to_host(dp), hp));
+      thrust::host_vector<int> ht(n), hf(n);
+      thrust::device_vector<int> dt(n), df(n);
+      auto hr = thrust::partition_copy(h.begin(), h.end(), ht.begin(), hf.begin(), is_even());
+      auto dr = thrust::partition_copy(d.begin(), d.end(), dt.begin(), df.begin(), is_even());
+      ASSERT_TRUE(dr.first - dt.begin() == hr.first - ht.begin() && dr.second - df.begin() == hr.second - hf.begin());
+      ht.resize(hr.first - ht.begin()); hf.resize(hr.second - hf.begin());
+      dt.resize(dr.first - dt.begin()); df.resize(dr.second - df.begin());
+      ASSERT_TRUE(same(to_host(dt), ht));
+      ASSERT_TRUE(same(to_host(df), hf));
+      hp = h;
+      dp = d;
+      auto hend = thrust::remove_if(hp.begin(), hp.end(), is_even());
+      auto dend = thrust::remove_if(dp.begin(), dp.end(), is_even());
+      ASSERT_TRUE(dend - dp.begin() == hend - hp.begin());
+      hp.resize(hend - hp.begin());
+      dp.resize(dend - dp.begin());
+      ASSERT_TRUE(same(to_host(dp), hp));
     }
     g_test = "transform / for_each / sequence";
     {
