@@ -11,6 +11,7 @@
 #include <thrust/system/hip/detail/device_input.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/generic_kernels.h>
+#include <thrust/system/hip/detail/generic_by_key.h>
 #endif
 
 namespace thrust {
@@ -170,41 +171,65 @@ T reduce(execution_policy<D>& exec, It first, It last, T init, Op op) {
   return detail::reduce(exec, first, last, init, op, detail::reduces_in_library<T, V, Op>());
 }
 
+namespace detail {
+// library path: arithmetic keys and values, equal_to, plus / minimum / maximum, same types in and out
+template <typename K, typename V, typename KO, typename VO, typename Pred, typename Op,
+          bool = is_abi_type<K>::value && is_abi_type<V>::value && std::is_same<KO, K>::value && std::is_same<VO, V>::value>
+struct reduces_by_key_in_library
+    : std::integral_constant<bool, is_equal_to<Pred, K>::value && (binop_code<Op, V>::value >= 0)> {};
+template <typename K, typename V, typename KO, typename VO, typename Pred, typename Op>
+struct reduces_by_key_in_library<K, V, KO, VO, Pred, Op, false> : std::false_type {};
+
 template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
-pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred, Op) {
+pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred pred, Op op,
+                               std::false_type) {
+#if defined(__HIPCC__)
+  return reduce_by_key_generic(exec, kf, kl, vf, ko, vo, pred, op);
+#else
+  static_assert(fancy_needs_hipcc<Op>::value,
+                "thrust::reduce_by_key on the device system: key predicates other than thrust::equal_to, operators other "
+                "than thrust::plus / minimum / maximum and non-arithmetic elements run in kernels instantiated for "
+                "them; compile this translation unit with hipcc");
+  return thrust::make_pair(ko, vo);
+#endif
+}
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred, Op,
+                               std::true_type) {
   typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
   typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
-  static_assert(detail::is_abi_type<K>::value && detail::is_abi_type<V>::value,
-                "thrust::reduce_by_key on the device system needs arithmetic keys and values");
-  static_assert(std::is_same<typename iterator_value<KOut>::type, K>::value &&
-                    std::is_same<typename iterator_value<VOut>::type, V>::value,
-                "thrust::reduce_by_key on the device system: output element types must equal the input types");
-  static_assert(detail::is_equal_to<Pred, K>::value,
-                "thrust::reduce_by_key on the device system supports thrust::equal_to as key predicate");
-  static_assert(detail::binop_code<Op, V>::value >= 0,
-                "thrust::reduce_by_key on the device system supports thrust::plus, minimum and maximum");
-  void* stream = detail::stream_of(exec);
+  void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n == 0) return thrust::make_pair(ko, vo);
-  detail::device_input<KIt> keys_in(stream, detail::temp_source_of(exec), kf, n);
-  detail::device_input<VIt> values_in(stream, detail::temp_source_of(exec), vf, n);
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
+  device_input<KIt> keys_in(stream, temp_source_of(exec), kf, n);
+  device_input<VIt> values_in(stream, temp_source_of(exec), vf, n);
+  temp_storage temp(stream, temp_source_of(exec));
   uint64_t* d_runs = nullptr;
   std::size_t need = 0;
   auto call = [&](void* t, std::size_t* b) {
     return thrust_amd_reduce_by_key(t, b, keys_in.ptr(), values_in.ptr(),
                                     thrust::detail::raw(ko), thrust::detail::raw(vo), d_runs, n,
-                                    detail::dtype_of<K>::value, detail::dtype_of<V>::value,
-                                    detail::binop_code<Op, V>::value, stream);
+                                    dtype_of<K>::value, dtype_of<V>::value,
+                                    binop_code<Op, V>::value, stream);
   };
-  detail::throw_on_error(call(nullptr, &need), "reduce_by_key: temp size query");
+  throw_on_error(call(nullptr, &need), "reduce_by_key: temp size query");
   const std::size_t aligned = (need + 255) / 256 * 256;
   temp.ensure(aligned + 256);
   d_runs = reinterpret_cast<uint64_t*>(static_cast<char*>(temp.ptr()) + aligned);
   std::size_t bytes = aligned;
-  detail::throw_on_error(call(temp.ptr(), &bytes), "reduce_by_key failed");
-  const uint64_t runs = detail::read_scalar<uint64_t>(d_runs, stream, "reduce_by_key: count copy");
+  throw_on_error(call(temp.ptr(), &bytes), "reduce_by_key failed");
+  const uint64_t runs = read_scalar<uint64_t>(d_runs, stream, "reduce_by_key: count copy");
   return thrust::make_pair(ko + runs, vo + runs);
+}
+}  // namespace detail
+
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred pred, Op op) {
+  typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
+  return detail::reduce_by_key(exec, kf, kl, vf, ko, vo, pred, op,
+                               detail::reduces_by_key_in_library<K, V, typename iterator_value<KOut>::type,
+                                                                 typename iterator_value<VOut>::type, Pred, Op>());
 }
 }  // namespace hip
 }  // namespace system

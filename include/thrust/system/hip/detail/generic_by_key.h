@@ -1,0 +1,174 @@
+// unique, unique_by_key and reduce_by_key for a user's key predicate, operator or element
+// structs (hipcc translation units).  They are put together from pieces that exist already:
+//
+//   run flags   one kernel, instantiated for the predicate: head[i] = i == 0 || !pred(k[i-1], k[i])
+//               and tail[i] = i == n-1 || !pred(k[i], k[i+1]), one byte each
+//               (thrust/detail/range/head_flags.h:130-160, tail_flags.h in the reference)
+//   selection   the library's compaction kernel with those bytes as its stencil: the keys at the
+//               heads, the values at the heads (unique_by_key) or at the tails (reduce_by_key)
+//   sums        reduce_by_key scans (head, value) pairs with the segmented form of the operator
+//               through the generic in-order scan, exactly the reference's formulation
+//               (thrust/system/detail/generic/reduce_by_key.inl:50-136); the value at a run's
+//               tail is the run's sum
+//
+// Keys and values are moved by the selection kernel as items of 1, 2, 4 or 8 bytes.
+#pragma once
+#if !defined(__HIPCC__)
+#error "thrust/system/hip/detail/generic_by_key.h is HIP code: compile this translation unit with hipcc"
+#endif
+#include <thrust/copy.h>
+#include <thrust/iterator/transform_iterator.h>
+#include <thrust/pair.h>
+#include <thrust/scan.h>
+#include <thrust/system/hip/detail/device_input.h>
+
+namespace thrust {
+namespace system {
+namespace hip {
+namespace detail {
+
+template <typename ViewK, typename Pred>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void run_flags_kernel(ViewK keys, uint64_t n, Pred pred,
+                                                                      unsigned char* head, unsigned char* tail) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    head[i] = (i == 0 || !pred(keys[i - 1], keys[i])) ? 1 : 0;
+    if (tail) tail[i] = (i == n - 1 || !pred(keys[i], keys[i + 1])) ? 1 : 0;
+  }
+}
+
+template <typename V>
+struct seg_pair {
+  V value;
+  unsigned char head;
+};
+template <typename V, typename Op>
+struct seg_op {  // the operator of a segmented scan: a head on the right starts over
+  Op op;
+  __host__ __device__ seg_pair<V> operator()(const seg_pair<V>& a, const seg_pair<V>& b) const {
+    seg_pair<V> r;
+    r.head = (unsigned char)(a.head | b.head);
+    r.value = b.head ? b.value : (V)op(a.value, b.value);
+    return r;
+  }
+};
+template <typename V>
+struct pair_value {
+  __host__ __device__ V operator()(const seg_pair<V>& p) const { return p.value; }
+};
+template <typename ViewV, typename V>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void seg_pairs_kernel(ViewV values, const unsigned char* head,
+                                                                      uint64_t n, seg_pair<V>* pairs) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    seg_pair<V> p;
+    p.value = (V)values[i];
+    p.head = head[i];
+    pairs[i] = p;
+  }
+}
+
+// items[i] with flags[i] != 0, compacted in order into out; returns how many.
+inline uint64_t select_by_flags(void* stream, const temp_source& source, const void* items, const unsigned char* flags,
+                                void* out, uint64_t n, std::size_t item_bytes, const char* what) {
+  return run_selection<unsigned char>(
+      stream, source, thrust::identity<unsigned char>(), what,
+      [&](void* t, std::size_t* b, uint64_t* d_num, int cmp, const void* thr) {
+        return thrust_amd_copy_if(t, b, items, flags, out, d_num, n, item_bytes, THRUST_AMD_U8, cmp, thr, stream);
+      });
+}
+
+template <typename D, typename KIn, typename Pred>
+inline void launch_run_flags(execution_policy<D>& exec, KIn kf, uint64_t n, Pred pred, unsigned char* head,
+                             unsigned char* tail) {
+  typedef typename thrust::detail::device_view_of<KIn>::type View;
+  hipLaunchKernelGGL((run_flags_kernel<View, Pred>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
+                     (hipStream_t)stream_of(exec), thrust::detail::device_view(kf), n, pred, head, tail);
+  throw_on_error(launch_status(), "run flags: kernel launch");
+}
+
+template <typename D, typename In, typename Out, typename Pred>
+Out unique_copy_generic(execution_policy<D>& exec, In first, In last, Out result, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  static_assert(is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
+                "unique on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  device_input<In> source(stream, temp_source_of(exec), first, n);
+  temp_storage flags(stream, temp_source_of(exec));
+  flags.ensure((std::size_t)n);
+  unsigned char* head = static_cast<unsigned char*>(flags.ptr());
+  launch_run_flags(exec, source.ptr(), n, pred, head, nullptr);
+  const uint64_t cnt = select_by_flags(stream, temp_source_of(exec), source.ptr(), head, thrust::detail::raw(result), n,
+                                       sizeof(T), "unique failed");
+  return result + cnt;
+}
+
+template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred>
+pair<KOut, VOut> unique_by_key_copy_generic(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo,
+                                            Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<KIn>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<VIn>::type>::type V;
+  static_assert(is_abi_item<K>::value && std::is_same<typename iterator_value<KOut>::type, K>::value &&
+                    is_abi_item<V>::value && std::is_same<typename iterator_value<VOut>::type, V>::value,
+                "unique_by_key on the device system: keys and values of 1, 2, 4 or 8 bytes, same types in and out");
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(kl - kf);
+  if (n == 0) return thrust::make_pair(ko, vo);
+  device_input<KIn> keys(stream, temp_source_of(exec), kf, n);
+  device_input<VIn> values(stream, temp_source_of(exec), vf, n);
+  temp_storage flags(stream, temp_source_of(exec));
+  flags.ensure((std::size_t)n);
+  unsigned char* head = static_cast<unsigned char*>(flags.ptr());
+  launch_run_flags(exec, keys.ptr(), n, pred, head, nullptr);
+  // the flags are made, so the two compactions may overwrite their inputs (in-place forms)
+  const uint64_t cnt = select_by_flags(stream, temp_source_of(exec), values.ptr(), head, thrust::detail::raw(vo), n,
+                                       sizeof(V), "unique_by_key failed");
+  (void)select_by_flags(stream, temp_source_of(exec), keys.ptr(), head, thrust::detail::raw(ko), n, sizeof(K),
+                        "unique_by_key failed");
+  return thrust::make_pair(ko + cnt, vo + cnt);
+}
+
+template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key_generic(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo, Pred pred,
+                                       Op op) {
+  typedef typename std::remove_const<typename iterator_value<KIn>::type>::type K;
+  typedef typename iterator_value<VOut>::type V;  // sums have the output's value type
+  static_assert(is_abi_item<K>::value && std::is_same<typename iterator_value<KOut>::type, K>::value &&
+                    is_abi_item<V>::value,
+                "reduce_by_key on the device system: keys and sums of 1, 2, 4 or 8 bytes, same key type in and out");
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(kl - kf);
+  if (n == 0) return thrust::make_pair(ko, vo);
+  device_input<KIn> keys(stream, temp_source_of(exec), kf, n);
+  temp_storage flags(stream, temp_source_of(exec));
+  flags.ensure((std::size_t)n * 2);
+  unsigned char* head = static_cast<unsigned char*>(flags.ptr());
+  unsigned char* tail = head + n;
+  launch_run_flags(exec, keys.ptr(), n, pred, head, tail);
+
+  typedef seg_pair<V> P;
+  temp_storage pair_store(stream, temp_source_of(exec));
+  pair_store.ensure((std::size_t)n * sizeof(P));
+  P* pairs = static_cast<P*>(pair_store.ptr());
+  typedef typename thrust::detail::device_view_of<VIn>::type ViewV;
+  hipLaunchKernelGGL((seg_pairs_kernel<ViewV, V>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
+                     (hipStream_t)stream, thrust::detail::device_view(vf), (const unsigned char*)head, n, pairs);
+  throw_on_error(launch_status(), "reduce_by_key: kernel launch");
+  const seg_op<V, Op> sop = {op};
+  scan_generic<false, P>(exec, pairs, pairs + n, pairs, P(), sop);  // in place, in input order
+
+  device_input<thrust::transform_iterator<pair_value<V>, const P*> > sums(
+      stream, temp_source_of(exec), thrust::make_transform_iterator((const P*)pairs, pair_value<V>()), n);
+  const uint64_t runs = select_by_flags(stream, temp_source_of(exec), sums.ptr(), tail, thrust::detail::raw(vo), n,
+                                        sizeof(V), "reduce_by_key failed");
+  (void)select_by_flags(stream, temp_source_of(exec), keys.ptr(), head, thrust::detail::raw(ko), n, sizeof(K),
+                        "reduce_by_key failed");
+  return thrust::make_pair(ko + runs, vo + runs);
+}
+
+}  // namespace detail
+}  // namespace hip
+}  // namespace system
+}  // namespace thrust

@@ -8,6 +8,10 @@
 #include <thrust/functional.h>
 #include <thrust/pair.h>
 #include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/device_input.h>
+#if defined(__HIPCC__)
+#include <thrust/system/hip/detail/generic_by_key.h>
+#endif
 
 namespace thrust {
 
@@ -83,57 +87,97 @@ pair<KOut, VOut> unique_by_key_copy(execution_policy<D>&, KIn kf, KIn kl, VIn vf
 }  // namespace cpp
 
 namespace hip {
+namespace detail {
+template <typename K, typename KO, typename Pred, bool = is_abi_type<K>::value && std::is_same<KO, K>::value>
+struct uniques_in_library : std::integral_constant<bool, is_equal_to<Pred, K>::value> {};
+template <typename K, typename KO, typename Pred>
+struct uniques_in_library<K, KO, Pred, false> : std::false_type {};
+
+// a user's predicate or element struct: head flags from a kernel instantiated for it
 template <typename D, typename In, typename Out, typename Pred>
-Out unique_copy(execution_policy<D>& exec, In first, In last, Out result, Pred) {
+Out unique_copy(execution_policy<D>& exec, In first, In last, Out result, Pred pred, std::false_type) {
+#if defined(__HIPCC__)
+  return unique_copy_generic(exec, first, last, result, pred);
+#else
+  static_assert(fancy_needs_hipcc<Pred>::value,
+                "unique on the device system: predicates other than thrust::equal_to of an arithmetic type run in "
+                "kernels instantiated for them; compile this translation unit with hipcc");
+  return result;
+#endif
+}
+template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred>
+pair<KOut, VOut> unique_by_key_copy(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo, Pred pred,
+                                    std::false_type) {
+#if defined(__HIPCC__)
+  return unique_by_key_copy_generic(exec, kf, kl, vf, ko, vo, pred);
+#else
+  static_assert(fancy_needs_hipcc<Pred>::value,
+                "unique_by_key on the device system: predicates other than thrust::equal_to of an arithmetic type run "
+                "in kernels instantiated for them; compile this translation unit with hipcc");
+  return thrust::make_pair(ko, vo);
+#endif
+}
+
+template <typename D, typename In, typename Out, typename Pred>
+Out unique_copy(execution_policy<D>& exec, In first, In last, Out result, Pred, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  static_assert(detail::is_abi_type<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
-                "unique on the device system needs one arithmetic element type for input and output");
-  static_assert(detail::is_equal_to<Pred, T>::value, "unique on the device system supports thrust::equal_to");
-  void* stream = detail::stream_of(exec);
+  void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
+  temp_storage temp(stream, temp_source_of(exec));
   uint64_t* d_num = nullptr;
   auto call = [&](void* t, std::size_t* b) {
     return thrust_amd_unique(t, b, thrust::detail::raw(first), thrust::detail::raw(result), d_num, n,
-                             detail::dtype_of<T>::value, stream);
+                             dtype_of<T>::value, stream);
   };
   std::size_t need = 0;
-  detail::throw_on_error(call(nullptr, &need), "unique: temp size query");
+  throw_on_error(call(nullptr, &need), "unique: temp size query");
   const std::size_t aligned = (need + 255) / 256 * 256;
   temp.ensure(aligned + 256);
   d_num = reinterpret_cast<uint64_t*>(static_cast<char*>(temp.ptr()) + aligned);
   std::size_t bytes = aligned;
-  detail::throw_on_error(call(temp.ptr(), &bytes), "unique failed");
-  return result + detail::read_scalar<uint64_t>(d_num, stream, "unique: count copy");
+  throw_on_error(call(temp.ptr(), &bytes), "unique failed");
+  return result + read_scalar<uint64_t>(d_num, stream, "unique: count copy");
 }
 template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred>
-pair<KOut, VOut> unique_by_key_copy(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo, Pred) {
+pair<KOut, VOut> unique_by_key_copy(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo, Pred,
+                                    std::true_type) {
   typedef typename std::remove_const<typename iterator_value<KIn>::type>::type K;
   typedef typename std::remove_const<typename iterator_value<VIn>::type>::type V;
-  static_assert(detail::is_abi_type<K>::value && std::is_same<typename iterator_value<KOut>::type, K>::value,
-                "unique_by_key on the device system needs one arithmetic key type for input and output");
-  static_assert(detail::is_abi_item<V>::value && std::is_same<typename iterator_value<VOut>::type, V>::value,
+  static_assert(is_abi_item<V>::value && std::is_same<typename iterator_value<VOut>::type, V>::value,
                 "unique_by_key on the device system supports values of 1, 2, 4 or 8 bytes, same type in and out");
-  static_assert(detail::is_equal_to<Pred, K>::value, "unique_by_key on the device system supports thrust::equal_to");
-  void* stream = detail::stream_of(exec);
+  void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n == 0) return thrust::make_pair(ko, vo);
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
+  temp_storage temp(stream, temp_source_of(exec));
   uint64_t* d_num = nullptr;
   auto call = [&](void* t, std::size_t* b) {
     return thrust_amd_unique_by_key(t, b, thrust::detail::raw(kf), thrust::detail::raw(vf), thrust::detail::raw(ko),
-                                    thrust::detail::raw(vo), d_num, n, detail::dtype_of<K>::value, sizeof(V), stream);
+                                    thrust::detail::raw(vo), d_num, n, dtype_of<K>::value, sizeof(V), stream);
   };
   std::size_t need = 0;
-  detail::throw_on_error(call(nullptr, &need), "unique_by_key: temp size query");
+  throw_on_error(call(nullptr, &need), "unique_by_key: temp size query");
   const std::size_t aligned = (need + 255) / 256 * 256;
   temp.ensure(aligned + 256);
   d_num = reinterpret_cast<uint64_t*>(static_cast<char*>(temp.ptr()) + aligned);
   std::size_t bytes = aligned;
-  detail::throw_on_error(call(temp.ptr(), &bytes), "unique_by_key failed");
-  const uint64_t cnt = detail::read_scalar<uint64_t>(d_num, stream, "unique_by_key: count copy");
+  throw_on_error(call(temp.ptr(), &bytes), "unique_by_key failed");
+  const uint64_t cnt = read_scalar<uint64_t>(d_num, stream, "unique_by_key: count copy");
   return thrust::make_pair(ko + cnt, vo + cnt);
+}
+}  // namespace detail
+
+template <typename D, typename In, typename Out, typename Pred>
+Out unique_copy(execution_policy<D>& exec, In first, In last, Out result, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  return detail::unique_copy(exec, first, last, result, pred,
+                             detail::uniques_in_library<T, typename iterator_value<Out>::type, Pred>());
+}
+template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred>
+pair<KOut, VOut> unique_by_key_copy(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<KIn>::type>::type K;
+  return detail::unique_by_key_copy(exec, kf, kl, vf, ko, vo, pred,
+                                    detail::uniques_in_library<K, typename iterator_value<KOut>::type, Pred>());
 }
 }  // namespace hip
 }  // namespace system

@@ -25,6 +25,7 @@
 #include <thrust/sequence.h>
 #include <thrust/transform.h>
 #include <thrust/transform_reduce.h>
+#include <thrust/unique.h>
 
 #include <hip/hip_runtime.h>
 
@@ -168,6 +169,82 @@ static void TestUserOperators() {
       thrust::exclusive_scan(du.begin(), du.end(), ds.begin(), 9u, bit_xor_op());
       ASSERT_TRUE(same(to_host(ds), hs));
     }
+  }
+}
+
+struct same_tens {  // the key predicate of testing/reduce_by_key.cu:60-112 and unique.cu:125-142
+  __host__ __device__ bool operator()(int a, int b) const { return a / 10 == b / 10; }
+};
+
+static void TestUserPredicatesByKey() {
+  g_test = "by-key known answers with a user predicate";
+  {
+    // testing/unique.cu:105-142: [11,11,12,20,29,21,21,31,31,37] with "same tens" -> [11,20,31]
+    thrust::device_vector<int> d(hv<int>({11, 11, 12, 20, 29, 21, 21, 31, 31, 37}));
+    auto end = thrust::unique(d.begin(), d.end(), same_tens());
+    ASSERT_TRUE(end - d.begin() == 3);
+    d.resize(3);
+    ASSERT_TRUE(same(to_host(d), hv<int>({11, 20, 31})));
+    // testing/reduce_by_key.cu:60-112: keys [11,11,21,20,21,21,21,37,37], values 0..8, "same tens" -> [11,21,37] / [1,20,15]
+    thrust::device_vector<int> k(hv<int>({11, 11, 21, 20, 21, 21, 21, 37, 37})), v(hv<int>({0, 1, 2, 3, 4, 5, 6, 7, 8}));
+    thrust::device_vector<int> ko(9), vo(9);
+    auto r = thrust::reduce_by_key(k.begin(), k.end(), v.begin(), ko.begin(), vo.begin(), same_tens());
+    ASSERT_TRUE(r.first - ko.begin() == 3 && r.second - vo.begin() == 3);
+    ko.resize(3); vo.resize(3);
+    ASSERT_TRUE(same(to_host(ko), hv<int>({11, 21, 37})));
+    ASSERT_TRUE(same(to_host(vo), hv<int>({1, 20, 15})));
+    // testing/unique_by_key.cu:160-253 with the same predicate -> keys [11,21,37], values [0,2,7]
+    thrust::device_vector<int> k2(k), v2(v);
+    auto u = thrust::unique_by_key(k2.begin(), k2.end(), v2.begin(), same_tens());
+    ASSERT_TRUE(u.first - k2.begin() == 3);
+    k2.resize(3); v2.resize(3);
+    ASSERT_TRUE(same(to_host(k2), hv<int>({11, 21, 37})));
+    ASSERT_TRUE(same(to_host(v2), hv<int>({0, 2, 7})));
+  }
+  for (size_t n : kSizes) {
+    g_test = "by-key differentials with user predicate and operator";
+    thrust::host_vector<int> hk(n);
+    for (size_t i = 0; i < n; ++i) hk[i] = (int)(i / 2 + mix(i / 5) % 7);
+    const thrust::host_vector<unsigned> hvv = random_values<unsigned>(n, 31, 1u << 20);
+    const thrust::device_vector<int> dk(hk);
+    const thrust::device_vector<unsigned> dv(hvv);
+    thrust::host_vector<int> hko(n);
+    thrust::host_vector<unsigned> hvo(n);
+    thrust::device_vector<int> dko(n);
+    thrust::device_vector<unsigned> dvo(n);
+    auto hr = thrust::reduce_by_key(hk.begin(), hk.end(), hvv.begin(), hko.begin(), hvo.begin(), same_tens(), bit_xor_op());
+    auto dr = thrust::reduce_by_key(dk.begin(), dk.end(), dv.begin(), dko.begin(), dvo.begin(), same_tens(), bit_xor_op());
+    ASSERT_TRUE(dr.first - dko.begin() == hr.first - hko.begin());
+    size_t runs = hr.first - hko.begin();
+    hko.resize(runs); hvo.resize(runs); dko.resize(runs); dvo.resize(runs);
+    ASSERT_TRUE(same(to_host(dko), hko));
+    ASSERT_TRUE(same(to_host(dvo), hvo));
+    // equal_to with an operator outside the library's set
+    hko.resize(n); hvo.resize(n); dko.resize(n); dvo.resize(n);
+    hr = thrust::reduce_by_key(hk.begin(), hk.end(), hvv.begin(), hko.begin(), hvo.begin(), thrust::equal_to<int>(),
+                               thrust::multiplies<unsigned>());
+    dr = thrust::reduce_by_key(dk.begin(), dk.end(), dv.begin(), dko.begin(), dvo.begin(), thrust::equal_to<int>(),
+                               thrust::multiplies<unsigned>());
+    runs = hr.first - hko.begin();
+    ASSERT_TRUE((size_t)(dr.first - dko.begin()) == runs);
+    hko.resize(runs); hvo.resize(runs); dko.resize(runs); dvo.resize(runs);
+    ASSERT_TRUE(same(to_host(dko), hko));
+    ASSERT_TRUE(same(to_host(dvo), hvo));
+    // unique_copy and unique_by_key_copy
+    hko.resize(n); dko.resize(n); hvo.resize(n); dvo.resize(n);
+    auto he = thrust::unique_copy(hk.begin(), hk.end(), hko.begin(), same_tens());
+    auto de = thrust::unique_copy(dk.begin(), dk.end(), dko.begin(), same_tens());
+    ASSERT_TRUE(de - dko.begin() == he - hko.begin());
+    hko.resize(he - hko.begin()); dko.resize(de - dko.begin());
+    ASSERT_TRUE(same(to_host(dko), hko));
+    hko.resize(n); dko.resize(n);
+    auto hu = thrust::unique_by_key_copy(hk.begin(), hk.end(), hvv.begin(), hko.begin(), hvo.begin(), same_tens());
+    auto du = thrust::unique_by_key_copy(dk.begin(), dk.end(), dv.begin(), dko.begin(), dvo.begin(), same_tens());
+    runs = hu.first - hko.begin();
+    ASSERT_TRUE((size_t)(du.first - dko.begin()) == runs);
+    hko.resize(runs); hvo.resize(runs); dko.resize(runs); dvo.resize(runs);
+    ASSERT_TRUE(same(to_host(dko), hko));
+    ASSERT_TRUE(same(to_host(dvo), hvo));
   }
 }
 
@@ -364,6 +441,7 @@ int main() {
   TestKnownAnswers();
   Differential();
   TestUserOperators();
+  TestUserPredicatesByKey();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
   std::printf(g_failed ? "FAILED\n" : "PASSED\n");
   return g_failed ? 1 : 0;
