@@ -7,6 +7,10 @@
 #include <thrust/functional.h>
 #include <thrust/pair.h>
 #include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/device_input.h>
+#if defined(__HIPCC__)
+#include <thrust/system/hip/detail/merge_sort_kernels.h>
+#endif
 
 namespace thrust {
 
@@ -61,55 +65,134 @@ pair<KOut, VOut> merge_by_key(execution_policy<D>&, K1 kf1, K1 kl1, K2 kf2, K2 k
 }  // namespace cpp
 
 namespace hip {
+namespace detail {
 template <typename D, typename In1, typename In2, typename Out, typename Comp>
-Out merge(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp) {
+Out merge(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<In1>::type>::type K;
-  static_assert(detail::is_abi_type<K>::value &&
+  static_assert(is_abi_type<K>::value &&
                     std::is_same<typename std::remove_const<typename iterator_value<In2>::type>::type, K>::value &&
                     std::is_same<typename iterator_value<Out>::type, K>::value,
                 "merge on the device system needs one arithmetic key type for both inputs and the output");
-  static_assert(detail::order_code<Comp, K>::value >= 0,
+  static_assert(order_code<Comp, K>::value >= 0,
                 "merge on the device system supports thrust::less and thrust::greater");
-  void* stream = detail::stream_of(exec);
+  void* stream = stream_of(exec);
   const uint64_t na = (uint64_t)(last1 - first1), nb = (uint64_t)(last2 - first2);
   if (na + nb == 0) return result;
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
-  detail::run(temp, 0, "merge failed", [&](void* t, std::size_t* b) {
+  temp_storage temp(stream, temp_source_of(exec));
+  run(temp, 0, "merge failed", [&](void* t, std::size_t* b) {
     return thrust_amd_merge(t, b, na ? thrust::detail::raw(first1) : nullptr, na,
                             nb ? thrust::detail::raw(first2) : nullptr, nb, thrust::detail::raw(result),
-                            detail::dtype_of<K>::value, detail::order_code<Comp, K>::value, stream);
+                            dtype_of<K>::value, order_code<Comp, K>::value, stream);
   });
-  detail::synchronize(stream, "merge: synchronize");
+  synchronize(stream, "merge: synchronize");
   return result + (na + nb);
 }
 template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
 pair<KOut, VOut> merge_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko,
-                              VOut vo, Comp) {
+                              VOut vo, Comp, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
   typedef typename std::remove_const<typename iterator_value<V1>::type>::type V;
-  static_assert(detail::is_abi_type<K>::value &&
+  static_assert(is_abi_type<K>::value &&
                     std::is_same<typename std::remove_const<typename iterator_value<K2>::type>::type, K>::value &&
                     std::is_same<typename iterator_value<KOut>::type, K>::value,
                 "merge_by_key on the device system needs one arithmetic key type for both inputs and the output");
-  static_assert(detail::is_abi_item<V>::value &&
+  static_assert(is_abi_item<V>::value &&
                     std::is_same<typename std::remove_const<typename iterator_value<V2>::type>::type, V>::value &&
                     std::is_same<typename iterator_value<VOut>::type, V>::value,
                 "merge_by_key on the device system supports values of 1, 2, 4 or 8 bytes, one type throughout");
-  static_assert(detail::order_code<Comp, K>::value >= 0,
+  static_assert(order_code<Comp, K>::value >= 0,
                 "merge_by_key on the device system supports thrust::less and thrust::greater");
-  void* stream = detail::stream_of(exec);
+  void* stream = stream_of(exec);
   const uint64_t na = (uint64_t)(kl1 - kf1), nb = (uint64_t)(kl2 - kf2);
   if (na + nb == 0) return thrust::make_pair(ko, vo);
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
-  detail::run(temp, 0, "merge_by_key failed", [&](void* t, std::size_t* b) {
+  temp_storage temp(stream, temp_source_of(exec));
+  run(temp, 0, "merge_by_key failed", [&](void* t, std::size_t* b) {
     return thrust_amd_merge_by_key(t, b, na ? thrust::detail::raw(kf1) : nullptr, na,
                                    nb ? thrust::detail::raw(kf2) : nullptr, nb,
                                    na ? thrust::detail::raw(vf1) : nullptr, nb ? thrust::detail::raw(vf2) : nullptr,
-                                   thrust::detail::raw(ko), thrust::detail::raw(vo), detail::dtype_of<K>::value,
-                                   sizeof(V), detail::order_code<Comp, K>::value, stream);
+                                   thrust::detail::raw(ko), thrust::detail::raw(vo), dtype_of<K>::value,
+                                   sizeof(V), order_code<Comp, K>::value, stream);
   });
-  detail::synchronize(stream, "merge_by_key: synchronize");
+  synchronize(stream, "merge_by_key: synchronize");
   return thrust::make_pair(ko + (na + nb), vo + (na + nb));
+}
+
+// A user's comparator or key type: both ranges are written one behind the other into temporary
+// storage (which also reads fancy iterators) and merged by the merge sort's kernels.
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
+void merge_generic(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko, VOut vo,
+                   Comp comp, bool has_values) {
+#if defined(__HIPCC__)
+  namespace ms = thrust::system::hip::merge_sort;
+  typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
+  typedef typename iterator_value<VOut>::type V;
+  static_assert(std::is_same<typename iterator_value<KOut>::type, K>::value,
+                "merge on the device system: the output holds the first range's key type");
+  void* stream = stream_of(exec);
+  const uint64_t na = (uint64_t)(kl1 - kf1), nb = (uint64_t)(kl2 - kf2), n = na + nb;
+  if (n == 0) return;
+  const uint64_t tiles = (n + ms::TILE - 1) / ms::TILE;
+  const std::size_t key_bytes = ((std::size_t)n * sizeof(K) + 255) / 256 * 256;
+  const std::size_t val_bytes = has_values ? ((std::size_t)n * sizeof(V) + 255) / 256 * 256 : 0;
+  temp_storage temp(stream, temp_source_of(exec));
+  temp.ensure(key_bytes + val_bytes + (std::size_t)(tiles + 1) * sizeof(uint64_t));
+  K* both = static_cast<K*>(temp.ptr());
+  V* both_values = reinterpret_cast<V*>(static_cast<char*>(temp.ptr()) + key_bytes);
+  uint64_t* split = reinterpret_cast<uint64_t*>(static_cast<char*>(temp.ptr()) + key_bytes + val_bytes);
+  materialize(stream, kf1, both, na);
+  materialize(stream, kf2, both + na, nb);
+  int rc;
+  if (has_values) {
+    materialize(stream, vf1, both_values, na);
+    materialize(stream, vf2, both_values + na, nb);
+    rc = ms::merge_two<K, V, true>(both, both_values, na, n, thrust::detail::raw(ko), thrust::detail::raw(vo), split,
+                                   comp, (hipStream_t)stream);
+  } else {
+    rc = ms::merge_two<K, V, false>(both, (const V*)nullptr, na, n, thrust::detail::raw(ko), (V*)nullptr, split, comp,
+                                    (hipStream_t)stream);
+  }
+  throw_on_error(rc, "merge failed");
+  synchronize(stream, "merge: synchronize");
+#else
+  static_assert(fancy_needs_hipcc<Comp>::value,
+                "merge on the device system: comparators other than thrust::less / thrust::greater of an arithmetic key "
+                "run in kernels instantiated for the comparator; compile this translation unit with hipcc");
+#endif
+}
+template <typename D, typename In1, typename In2, typename Out, typename Comp>
+Out merge(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp, std::false_type) {
+  merge_generic(exec, first1, last1, first2, last2, first1, first2, result, result, comp, false);
+  return result + ((last1 - first1) + (last2 - first2));
+}
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
+pair<KOut, VOut> merge_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko,
+                              VOut vo, Comp comp, std::false_type) {
+  merge_generic(exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp, true);
+  const std::ptrdiff_t n = (kl1 - kf1) + (kl2 - kf2);
+  return thrust::make_pair(ko + n, vo + n);
+}
+
+template <typename K, typename K2, typename KO, typename Comp,
+          bool = is_abi_type<K>::value && std::is_same<K2, K>::value && std::is_same<KO, K>::value>
+struct merges_in_library : std::integral_constant<bool, (order_code<Comp, K>::value >= 0)> {};
+template <typename K, typename K2, typename KO, typename Comp>
+struct merges_in_library<K, K2, KO, Comp, false> : std::false_type {};
+}  // namespace detail
+
+template <typename D, typename In1, typename In2, typename Out, typename Comp>
+Out merge(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+  typedef typename std::remove_const<typename iterator_value<In1>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<In2>::type>::type K2;
+  return detail::merge(exec, first1, last1, first2, last2, result, comp,
+                       detail::merges_in_library<K, K2, typename iterator_value<Out>::type, Comp>());
+}
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
+pair<KOut, VOut> merge_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko,
+                              VOut vo, Comp comp) {
+  typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<K2>::type>::type Kb;
+  return detail::merge_by_key(exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp,
+                              detail::merges_in_library<K, Kb, typename iterator_value<KOut>::type, Comp>());
 }
 }  // namespace hip
 }  // namespace system

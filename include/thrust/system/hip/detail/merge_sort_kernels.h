@@ -193,9 +193,19 @@ struct PairOfRuns {
   uint64_t a_begin, na, b_begin, nb;  // A = [a_begin, a_begin + na), B follows it
   uint64_t out0;                      // offset of the tile's first output inside the pair
 };
+template <bool LONE>
 __device__ __forceinline__ PairOfRuns pair_of(uint64_t tile, uint64_t run, uint64_t n) {
   PairOfRuns p;
   const uint64_t d0 = tile * TILE;
+  if (LONE) {
+    // one pair of runs of any two lengths: A = [0, run), B = [run, n) -- thrust::merge of two ranges
+    p.a_begin = 0;
+    p.na = run;
+    p.b_begin = run;
+    p.nb = n - run;
+    p.out0 = d0;
+    return p;
+  }
   p.a_begin = d0 / (2 * run) * (2 * run);
   p.na = (n - p.a_begin < run) ? (n - p.a_begin) : run;
   p.b_begin = p.a_begin + p.na;
@@ -205,19 +215,19 @@ __device__ __forceinline__ PairOfRuns pair_of(uint64_t tile, uint64_t run, uint6
 }
 
 // split[t] = how many of the outputs of tile t's pair that precede tile t come from run A.
-template <typename K, typename Comp>
+template <typename K, typename Comp, bool LONE = false>
 __global__ __launch_bounds__(256) void merge_partition_kernel(const K* keys, uint64_t n, uint64_t run,
                                                               uint64_t tiles, Comp comp, uint64_t* split) {
   const uint64_t t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
   if (t >= tiles) return;
-  const PairOfRuns p = pair_of(t, run, n);
+  const PairOfRuns p = pair_of<LONE>(t, run, n);
   const K* a = keys + p.a_begin;
   const K* b = keys + p.b_begin;
   split[t] = merge_path<uint64_t>([&](uint64_t x) { return a[x]; }, p.na, [&](uint64_t x) { return b[x]; }, p.nb,
                                   p.out0, comp);
 }
 
-template <typename K, typename V, bool HAS_VALUES, typename Comp>
+template <typename K, typename V, bool HAS_VALUES, typename Comp, bool LONE = false>
 __global__ __launch_bounds__(BLOCK) void merge_pass_kernel(const K* keys_in, const V* vals_in, K* keys_out,
                                                            V* vals_out, uint64_t n, uint64_t run, uint64_t tiles,
                                                            const uint64_t* split, Comp comp) {
@@ -227,7 +237,7 @@ __global__ __launch_bounds__(BLOCK) void merge_pass_kernel(const K* keys_in, con
   V* s_vals = reinterpret_cast<V*>(s_raw);
   const uint32_t tid = threadIdx.x;
   const uint64_t tile = blockIdx.x;
-  const PairOfRuns p = pair_of(tile, run, n);
+  const PairOfRuns p = pair_of<LONE>(tile, run, n);
   const uint64_t pair_len = p.na + p.nb;
   const uint64_t out1 = (p.out0 + TILE < pair_len) ? p.out0 + TILE : pair_len;
   const uint64_t a0 = split[tile];
@@ -382,6 +392,24 @@ int sort(void* temp, size_t* temp_bytes, K* keys, V* vals, uint64_t n, Comp comp
     run *= 2;
   }
   return 0;
+}
+
+// Merges the sorted ranges both[0, na) and both[na, n) into out (and their values with them);
+// ties take the first range first.  split: (tiles + 1) 64-bit words of scratch.
+template <typename K, typename V, bool HAS_VALUES, typename Comp>
+int merge_two(const K* both, const V* both_values, uint64_t na, uint64_t n, K* out, V* out_values, uint64_t* split,
+              Comp comp, hipStream_t stream) {
+  if (n == 0) return 0;
+  const uint64_t tiles = (n + TILE - 1) / TILE;
+  if (tiles > 0x7fffffffull) return (int)hipErrorInvalidValue;
+  THRUST_AMD_MERGE_SORT_LAUNCH("merge_sort_partition", stream, (merge_partition_kernel<K, Comp, true>),
+                               dim3((uint32_t)((tiles + 255) / 256)), dim3(256), both, n, na, tiles, comp, split);
+  hipError_t err = hipGetLastError();
+  if (err != hipSuccess) return (int)err;
+  THRUST_AMD_MERGE_SORT_LAUNCH("merge_sort_pass", stream, (merge_pass_kernel<K, V, HAS_VALUES, Comp, true>),
+                               dim3((uint32_t)tiles), dim3(BLOCK), both, both_values, out, out_values, n, na, tiles,
+                               (const uint64_t*)split, comp);
+  return (int)hipGetLastError();
 }
 
 }  // namespace merge_sort

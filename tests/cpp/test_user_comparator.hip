@@ -8,6 +8,7 @@
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
 #include <thrust/host_vector.h>
+#include <thrust/merge.h>
 #include <thrust/sort.h>
 
 #include <hip/hip_runtime.h>
@@ -170,6 +171,57 @@ static void TestStructKeys() {
   }
 }
 
+template <typename T>
+struct my_less {
+  __host__ __device__ bool operator()(const T& a, const T& b) const { return a < b; }
+};
+
+static void TestMergeWithUserComparators() {
+  g_test = "MergeSimple";  // testing/merge.cu:11-38 and merge_by_key.cu:10-45 through a user-defined less
+  {
+    thrust::device_vector<int> a(hv<int>({0, 2, 4})), b(hv<int>({0, 3, 3, 4})), out(7);
+    auto end = thrust::merge(a.begin(), a.end(), b.begin(), b.end(), out.begin(), my_less<int>());
+    ASSERT_TRUE(end - out.begin() == 7);
+    ASSERT_TRUE(same(to_host(out), hv<int>({0, 0, 2, 3, 3, 4, 4})));
+    thrust::device_vector<int> va(hv<int>({13, 7, 42})), vb(hv<int>({42, 42, 7, 13})), ko(7), vo(7);
+    auto ends = thrust::merge_by_key(a.begin(), a.end(), b.begin(), b.end(), va.begin(), vb.begin(), ko.begin(),
+                                     vo.begin(), my_less<int>());
+    ASSERT_TRUE(ends.first - ko.begin() == 7 && ends.second - vo.begin() == 7);
+    ASSERT_TRUE(same(to_host(ko), hv<int>({0, 0, 2, 3, 3, 4, 4})));
+    ASSERT_TRUE(same(to_host(vo), hv<int>({13, 42, 7, 42, 7, 42, 13})));  // ties: the first range first
+  }
+  g_test = "MergeDifferential";
+  for (size_t n : kSizes) {
+    const size_t na = n, nb = n / 3 + (n % 5);
+    thrust::host_vector<int> ha(na), hb(nb);
+    for (size_t i = 0; i < na; ++i) ha[i] = (int)(mix(i + 11 * n) % 997);
+    for (size_t i = 0; i < nb; ++i) hb[i] = (int)(mix(i + 13 * n) % 997);
+    // equivalence classes of ten under less_div_10; inside a class the input order must survive
+    std::stable_sort(ha.begin(), ha.end(), less_div_10<int>());
+    std::stable_sort(hb.begin(), hb.end(), less_div_10<int>());
+    thrust::device_vector<int> da(ha), db(hb), dout(na + nb);
+    thrust::host_vector<int> hout(na + nb);
+    thrust::merge(ha.begin(), ha.end(), hb.begin(), hb.end(), hout.begin(), less_div_10<int>());
+    thrust::merge(da.begin(), da.end(), db.begin(), db.end(), dout.begin(), less_div_10<int>());
+    ASSERT_TRUE(same(to_host(dout), hout));
+    // descending with values
+    std::stable_sort(ha.begin(), ha.end(), my_greater<int>());
+    std::stable_sort(hb.begin(), hb.end(), my_greater<int>());
+    da = ha;
+    db = hb;
+    thrust::host_vector<unsigned> hva(na), hvb(nb), hvo(na + nb);
+    for (size_t i = 0; i < na; ++i) hva[i] = (unsigned)i;
+    for (size_t i = 0; i < nb; ++i) hvb[i] = (unsigned)(1000000 + i);
+    thrust::device_vector<unsigned> dva(hva), dvb(hvb), dvo(na + nb);
+    thrust::merge_by_key(ha.begin(), ha.end(), hb.begin(), hb.end(), hva.begin(), hvb.begin(), hout.begin(), hvo.begin(),
+                         my_greater<int>());
+    thrust::merge_by_key(da.begin(), da.end(), db.begin(), db.end(), dva.begin(), dvb.begin(), dout.begin(), dvo.begin(),
+                         my_greater<int>());
+    ASSERT_TRUE(same(to_host(dout), hout));
+    ASSERT_TRUE(same(to_host(dvo), hvo));
+  }
+}
+
 int main() {
   TestKnownAnswers();
   Differential<signed char>("signed char");
@@ -178,6 +230,7 @@ int main() {
   Differential<long long>("long long");
   Differential<float>("float");
   TestStructKeys();
+  TestMergeWithUserComparators();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
   std::printf(g_failed ? "FAILED\n" : "PASSED\n");
   return g_failed ? 1 : 0;
