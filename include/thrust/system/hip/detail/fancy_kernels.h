@@ -19,7 +19,8 @@ namespace detail {
 constexpr int ELEMENTWISE_BLOCK = 256;
 inline unsigned elementwise_grid(uint64_t n) {
   const uint64_t blocks = (n + ELEMENTWISE_BLOCK - 1) / ELEMENTWISE_BLOCK;
-  const uint64_t cap = 256 * 16;  // grid-stride beyond that
+  const uint64_t cap = (uint64_t)1 << 20;  // one element per lane up to 2^28 (many short workgroups keep more
+                                           // memory requests in flight than a few that loop); grid-stride beyond
   return (unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap));
 }
 

@@ -199,7 +199,7 @@ TA_EXPORT int thrust_amd_convert(const void* in, int in_dtype, void* out, int ou
     return with_dtype(out_dtype, [&](auto ot) {
       using Out = typename decltype(ot)::type;
       uint64_t blocks = (n + 255) / 256;
-      const uint64_t cap = (uint64_t)NUM_CU * 32;
+      const uint64_t cap = (uint64_t)1 << 20;  // one element per lane up to 2^28; short workgroups keep more requests in flight
       if (blocks > cap) blocks = cap;
       TA_LAUNCH("convert", (hipStream_t)stream, (convert_kernel<In, Out>), dim3((uint32_t)blocks), dim3(256),
                 static_cast<const In*>(in), static_cast<Out*>(out), n);
