@@ -34,9 +34,17 @@ inline void copy_raw(const T* src, bool src_device, T* dst, bool dst_device, std
   }
 }
 
+// Fancy iterators have no address: element by element through the iterators themselves
+// (host code; device_ptr ends go through their host-side proxies).
 template <typename In, typename Out>
-inline Out copy_dispatch(In first, In last, Out result, bool in_device, bool out_device, void* stream,
-                         bool blocking = true) {
+inline typename std::enable_if<is_fancy_iterator<In>::value || is_fancy_iterator<Out>::value, Out>::type copy_dispatch(
+    In first, In last, Out result, bool, bool, void*, bool = true) {
+  for (; first != last; ++first, ++result) *result = *first;
+  return result;
+}
+template <typename In, typename Out>
+inline typename std::enable_if<!is_fancy_iterator<In>::value && !is_fancy_iterator<Out>::value, Out>::type copy_dispatch(
+    In first, In last, Out result, bool in_device, bool out_device, void* stream, bool blocking = true) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
   typedef typename iterator_value<Out>::type U;
   const std::size_t n = (std::size_t)std::distance(first, last);
@@ -103,7 +111,7 @@ template <typename D, typename In, typename Out>
 Out copy_fancy(execution_policy<D>& exec, In first, In last, Out result, std::true_type) {
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
-  materialize(stream, first, thrust::detail::raw(result), n);
+  materialize(stream, first, result, n);
   synchronize(stream, "copy: synchronize");
   return result + n;
 }
@@ -114,9 +122,9 @@ Out copy_fancy(execution_policy<D>&, In first, In last, Out result, std::false_t
 }
 template <typename D, typename In, typename Out>
 Out copy(execution_policy<D>& exec, In first, In last, Out result, std::true_type) {
+  // both ends on the device side: one kernel; otherwise the iterators are walked on the host
   return copy_fancy(exec, first, last, result,
-                    std::integral_constant<bool, thrust::detail::is_device_iterator<Out>::value ||
-                                                     std::is_pointer<Out>::value>());
+                    std::integral_constant<bool, is_device_input<In>::value && is_device_output<Out>::value>());
 }
 // a user predicate as one byte per element, for the stencil form of the selection kernels
 template <typename Pred>
@@ -133,7 +141,9 @@ struct selects_in_kernel<Pred, T, false> : std::false_type {};
 
 template <typename D, typename In, typename Out>
 Out copy(execution_policy<D>& exec, In first, In last, Out result) {
-  return detail::copy(exec, first, last, result, thrust::detail::is_fancy_iterator<In>());
+  return detail::copy(exec, first, last, result,
+                      std::integral_constant<bool, thrust::detail::is_fancy_iterator<In>::value ||
+                                                       thrust::detail::is_fancy_iterator<Out>::value>());
 }
 
 namespace detail {
@@ -262,13 +272,15 @@ Out copy_any(In first, In last, Out result, std::false_type) {
   return copy_dispatch(first, last, result, is_device_iterator<In>::value, is_device_iterator<Out>::value, nullptr);
 }
 template <typename In, typename Out>
-Out copy_any(In first, In last, Out result, std::true_type) {  // fancy input: its own system decides
-  return thrust::copy(policy_for<In>(), first, last, result);
+Out copy_any(In first, In last, Out result, std::true_type) {  // a fancy end: the output's system decides
+  return thrust::copy(policy_for<Out>(), first, last, result);
 }
 }  // namespace detail
 template <typename In, typename Out>
 Out copy(In first, In last, Out result) {
-  return detail::copy_any(first, last, result, detail::is_fancy_iterator<In>());
+  return detail::copy_any(first, last, result,
+                          std::integral_constant<bool, detail::is_fancy_iterator<In>::value ||
+                                                           detail::is_fancy_iterator<Out>::value>());
 }
 template <typename D, typename In, typename Size, typename Out>
 Out copy_n(const detail::execution_policy_base<D>& exec, In first, Size n, Out result) {

@@ -41,13 +41,6 @@ inline auto raw(It it) -> typename std::enable_if<
   // never dereferences: callers pass begin() of a non-empty contiguous range or use n == 0
   return std::addressof(*it);
 }
-// a fancy iterator has no address; code that reaches this at run time took a wrong turn
-template <typename It>
-inline auto raw(It) -> typename std::enable_if<is_fancy_iterator<It>::value,
-                                               typename std::iterator_traits<It>::value_type*>::type {
-  return nullptr;
-}
-
 template <typename It>
 struct is_contiguous_host_iterator
     : std::integral_constant<bool,

@@ -12,10 +12,12 @@
 #pragma once
 #include <algorithm>
 #include <numeric>
+#include <tuple>
 #include <vector>
 
 #include <thrust/functional.h>
 #include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/device_input.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/merge_sort_kernels.h>
 #endif
@@ -94,6 +96,21 @@ struct takes_radix_path<K, Comp, false> : std::false_type {};
 template <typename T>
 struct needs_hipcc : std::false_type {};
 
+// Values travel as opaque items of 1, 2, 4 or 8 bytes: arithmetic types, small structs, and tuples
+// of such (a tuple of values is moved bit by bit although its assignment operator is user-written).
+template <typename V>
+struct is_plain_tuple : std::false_type {};
+template <typename... Ts>
+struct is_plain_tuple<thrust::tuple<Ts...> >
+    : std::integral_constant<bool, std::is_trivially_copyable<std::tuple<Ts...> >::value> {};
+template <typename V>
+struct is_sort_payload
+    : std::integral_constant<bool, (is_abi_item<V>::value || is_plain_tuple<V>::value) &&
+                                       (sizeof(V) == 1 || sizeof(V) == 2 || sizeof(V) == 4 || sizeof(V) == 8)> {};
+template <typename K, typename V, typename Comp>
+struct pairs_take_radix_path
+    : std::integral_constant<bool, takes_radix_path<K, Comp>::value && is_sort_payload<V>::value> {};
+
 template <typename K, typename Comp>
 void sort_keys(void* stream, temp_source source, K* keys, uint64_t n, Comp, std::true_type) {
   temp_storage temp(stream, source);
@@ -104,7 +121,6 @@ void sort_keys(void* stream, temp_source source, K* keys, uint64_t n, Comp, std:
 }
 template <typename K, typename V, typename Comp>
 void sort_pairs(void* stream, temp_source source, K* keys, V* values, uint64_t n, Comp, std::true_type) {
-  static_assert(is_abi_item<V>::value, "sort_by_key on the device system supports values of 1, 2, 4 or 8 bytes");
   temp_storage temp(stream, source);
   run(temp, 0, "sort_by_key failed", [&](void* t, std::size_t* b) {
     return thrust_amd_sort_pairs(t, b, keys, values, n, dtype_of<K>::value, sizeof(V), order_code<Comp, K>::value, 0,
@@ -143,26 +159,74 @@ void sort_pairs(void*, temp_source, K*, V*, uint64_t, Comp, std::false_type) {
 #endif
 }  // namespace detail
 
+namespace detail {
+// The array a sort works on.  Device pointers are sorted where they lie; a zip_iterator
+// (structure of arrays) is gathered into an array of tuples first and written back through
+// the zip afterwards.
+template <typename It, bool Fancy = thrust::detail::is_fancy_iterator<It>::value>
+class sortable_range {
+ public:
+  typedef typename iterator_value<It>::type value_type;
+  sortable_range(void*, const temp_source&, It first, uint64_t) : ptr_(thrust::detail::raw(first)) {}
+  value_type* ptr() const { return ptr_; }
+  void write_back() {}
+
+ private:
+  value_type* ptr_;
+};
+template <typename It>
+class sortable_range<It, true> {
+ public:
+  typedef typename iterator_value<It>::type value_type;
+  sortable_range(void* stream, const temp_source& source, It first, uint64_t n)
+      : holder_(stream, source), stream_(stream), first_(first), n_(n), ptr_(nullptr) {
+    static_assert(is_device_output<It>::value,
+                  "sort on the device system: a fancy iterator to sort through must be a zip of device iterators");
+    holder_.ensure((std::size_t)n * sizeof(value_type));
+    ptr_ = static_cast<value_type*>(holder_.ptr());
+    materialize(stream, first, ptr_, n);
+  }
+  value_type* ptr() const { return ptr_; }
+  void write_back() { materialize(stream_, (const value_type*)ptr_, first_, n_); }
+
+ private:
+  temp_storage holder_;
+  void* stream_;
+  It first_;
+  uint64_t n_;
+  value_type* ptr_;
+};
+}  // namespace detail
+
 template <typename D, typename It, typename Comp>
 void stable_sort(execution_policy<D>& exec, It first, It last, Comp comp) {
   typedef typename iterator_value<It>::type K;
-  static_assert(std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value,
-                "sort on the device system needs device_ptr / device_vector iterators or raw device pointers");
+  static_assert(detail::is_device_output<It>::value,
+                "sort on the device system needs device_ptr / device_vector iterators, raw device pointers or a zip of them");
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n < 2) return;
-  detail::sort_keys(stream, detail::temp_source_of(exec), thrust::detail::raw(first), n, comp,
-                    detail::takes_radix_path<K, Comp>());
+  detail::sortable_range<It> keys(stream, detail::temp_source_of(exec), first, n);
+  detail::sort_keys(stream, detail::temp_source_of(exec), keys.ptr(), n, comp, detail::takes_radix_path<K, Comp>());
+  keys.write_back();
   detail::synchronize(stream, "sort: synchronize");
 }
 template <typename D, typename KIt, typename VIt, typename Comp>
 void stable_sort_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Comp comp) {
   typedef typename iterator_value<KIt>::type K;
+  static_assert(detail::is_device_output<KIt>::value && detail::is_device_output<VIt>::value,
+                "sort_by_key on the device system needs device_ptr / device_vector iterators, raw device pointers or "
+                "zips of them");
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n < 2) return;
-  detail::sort_pairs(stream, detail::temp_source_of(exec), thrust::detail::raw(kf), thrust::detail::raw(vf), n, comp,
-                     detail::takes_radix_path<K, Comp>());
+  detail::sortable_range<KIt> keys(stream, detail::temp_source_of(exec), kf, n);
+  detail::sortable_range<VIt> values(stream, detail::temp_source_of(exec), vf, n);
+  typedef typename iterator_value<VIt>::type V;
+  detail::sort_pairs(stream, detail::temp_source_of(exec), keys.ptr(), values.ptr(), n, comp,
+                     detail::pairs_take_radix_path<K, V, Comp>());
+  keys.write_back();
+  values.write_back();
   detail::synchronize(stream, "sort_by_key: synchronize");
 }
 }  // namespace hip

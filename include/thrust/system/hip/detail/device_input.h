@@ -8,6 +8,7 @@
 // translation unit compiled with hipcc.
 #pragma once
 #include <thrust/iterator/detail/fancy_iterator_base.h>
+#include <thrust/iterator/zip_iterator.h>
 #include <thrust/system/hip/detail/backend.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/fancy_kernels.h>
@@ -23,17 +24,30 @@ struct is_device_input
     : std::integral_constant<bool, std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value ||
                                        thrust::detail::is_fancy_iterator<It>::value> {};
 
+// Where kernels that take iterators by value may write: device memory, or a zip of such.
+template <typename It>
+struct is_device_output
+    : std::integral_constant<bool, std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value> {};
+
+template <>
+struct is_device_output<thrust::zip_iterator<thrust::tuple<> > > : std::true_type {};
+template <typename H, typename... T>
+struct is_device_output<thrust::zip_iterator<thrust::tuple<H, T...> > >
+    : std::integral_constant<bool, is_device_output<H>::value &&
+                                       is_device_output<thrust::zip_iterator<thrust::tuple<T...> > >::value> {};
+
 template <typename It>
 struct fancy_needs_hipcc : std::false_type {};
 
-// Writes first[0, n) into out (device memory) on the stream.
-template <typename It, typename T>
-inline void materialize(void* stream, It first, T* out, uint64_t n) {
+// Writes first[0, n) to out[0, n) (a device pointer, device_ptr or a zip of them) on the stream.
+template <typename It, typename Out>
+inline void materialize(void* stream, It first, Out out, uint64_t n) {
 #if defined(__HIPCC__)
   if (n == 0) return;
   typedef typename thrust::detail::device_view_of<It>::type View;
-  hipLaunchKernelGGL((materialize_kernel<View, T>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
-                     (hipStream_t)stream, thrust::detail::device_view(first), out, n);
+  typedef typename thrust::detail::device_view_of<Out>::type OutView;
+  hipLaunchKernelGGL((materialize_kernel<View, OutView>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
+                     (hipStream_t)stream, thrust::detail::device_view(first), thrust::detail::device_view(out), n);
   throw_on_error(launch_status(), "fancy iterator: materialisation kernel");
 #else
   static_assert(fancy_needs_hipcc<It>::value,

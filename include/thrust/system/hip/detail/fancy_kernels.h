@@ -24,28 +24,29 @@ inline unsigned elementwise_grid(uint64_t n) {
   return (unsigned)(blocks < 1 ? 1 : (blocks < cap ? blocks : cap));
 }
 
-template <typename View, typename T>
-__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void materialize_kernel(View first, T* out, uint64_t n) {
+// out may be a pointer or a zip of pointers: out[i] is then a tuple of references, written through
+template <typename View, typename OutView>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void materialize_kernel(View first, OutView out, uint64_t n) {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = (T)first[i];
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = first[i];
 }
 
-template <typename T, typename F>
-__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void for_each_kernel(T* first, uint64_t n, F f) {
+template <typename View, typename F>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void for_each_kernel(View first, uint64_t n, F f) {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) f(first[i]);
 }
 
-template <typename ViewA, typename ViewB, typename T, typename F>
-__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform2_kernel(ViewA a, ViewB b, T* out, uint64_t n, F f) {
+template <typename ViewA, typename ViewB, typename OutView, typename F>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform2_kernel(ViewA a, ViewB b, OutView out, uint64_t n, F f) {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = (T)f(a[i], b[i]);
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = f(a[i], b[i]);
 }
 
-template <typename ViewIn, typename ViewMap, typename T>
-__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void scatter_kernel(ViewIn in, ViewMap map, T* out, uint64_t n) {
+template <typename ViewIn, typename ViewMap, typename OutView>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void scatter_kernel(ViewIn in, ViewMap map, OutView out, uint64_t n) {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[map[i]] = (T)in[i];
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[map[i]] = in[i];
 }
 
 inline int launch_status() { return (int)hipGetLastError(); }

@@ -58,7 +58,9 @@ __device__ __forceinline__ T block_fold(T value, bool has, Op& op, T* s_val, uns
 template <typename View, typename T, typename Op>
 __global__ __launch_bounds__(BLOCK) void reduce_chunks_kernel(View first, uint64_t n, uint64_t chunk, Op op,
                                                               T* partials) {
-  __shared__ T s_val[BLOCK];
+  // raw bytes: T may have a constructor, which shared arrays cannot run
+  __shared__ __attribute__((aligned(16))) unsigned char s_val_raw[BLOCK * sizeof(T)];
+  T* s_val = reinterpret_cast<T*>(s_val_raw);
   __shared__ unsigned char s_has[BLOCK];
   const uint64_t begin = (uint64_t)blockIdx.x * chunk;
   const uint64_t end = (begin + chunk < n) ? begin + chunk : n;
@@ -78,7 +80,9 @@ __global__ __launch_bounds__(BLOCK) void reduce_chunks_kernel(View first, uint64
 template <typename T, typename Op>
 __global__ __launch_bounds__(BLOCK) void reduce_final_kernel(const T* partials, uint32_t count, T init, Op op,
                                                              T* result) {
-  __shared__ T s_val[BLOCK];
+  // raw bytes: T may have a constructor, which shared arrays cannot run
+  __shared__ __attribute__((aligned(16))) unsigned char s_val_raw[BLOCK * sizeof(T)];
+  T* s_val = reinterpret_cast<T*>(s_val_raw);
   __shared__ unsigned char s_has[BLOCK];
   T acc = T();
   bool has = false;
@@ -116,7 +120,9 @@ __device__ __forceinline__ T block_inclusive(T value, bool has, Op& op, T* s_val
 // Step 1 of the scan: tile_total[t] = fold of tile t in input order (every tile holds an element).
 template <typename View, typename T, typename Op>
 __global__ __launch_bounds__(BLOCK) void scan_tile_totals_kernel(View first, uint64_t n, Op op, T* tile_total) {
-  __shared__ T s_val[BLOCK];
+  // raw bytes: T may have a constructor, which shared arrays cannot run
+  __shared__ __attribute__((aligned(16))) unsigned char s_val_raw[BLOCK * sizeof(T)];
+  T* s_val = reinterpret_cast<T*>(s_val_raw);
   __shared__ unsigned char s_has[BLOCK];
   const uint64_t base = (uint64_t)blockIdx.x * TILE + (uint64_t)threadIdx.x * ITEMS;
   T acc = T();
@@ -138,7 +144,9 @@ __global__ __launch_bounds__(BLOCK) void scan_tile_totals_kernel(View first, uin
 // every lane owns a contiguous piece of the array.
 template <typename T, typename Op>
 __global__ __launch_bounds__(BLOCK) void scan_tile_prefix_kernel(T* tile_total, uint32_t tiles, Op op) {
-  __shared__ T s_val[BLOCK];
+  // raw bytes: T may have a constructor, which shared arrays cannot run
+  __shared__ __attribute__((aligned(16))) unsigned char s_val_raw[BLOCK * sizeof(T)];
+  T* s_val = reinterpret_cast<T*>(s_val_raw);
   __shared__ unsigned char s_has[BLOCK];
   const uint32_t per = (tiles + BLOCK - 1) / BLOCK;
   const uint32_t begin = threadIdx.x * per;
@@ -176,7 +184,9 @@ __global__ __launch_bounds__(BLOCK) void scan_tile_prefix_kernel(T* tile_total, 
 template <bool EXCLUSIVE, typename View, typename T, typename U, typename Op>
 __global__ __launch_bounds__(BLOCK) void scan_tiles_kernel(View first, U* out, uint64_t n, Op op, T init,
                                                            const T* tile_prefix) {
-  __shared__ T s_val[BLOCK];
+  // raw bytes: T may have a constructor, which shared arrays cannot run
+  __shared__ __attribute__((aligned(16))) unsigned char s_val_raw[BLOCK * sizeof(T)];
+  T* s_val = reinterpret_cast<T*>(s_val_raw);
   __shared__ unsigned char s_has[BLOCK];
   const uint64_t base = (uint64_t)blockIdx.x * TILE + (uint64_t)threadIdx.x * ITEMS;
   T x[ITEMS];

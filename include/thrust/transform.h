@@ -54,9 +54,6 @@ struct sequence_value {  // element i of thrust::sequence(first, last, init, ste
   T init, step;
   __host__ __device__ T operator()(unsigned long long i) const { return (T)(init + step * (T)i); }
 };
-template <typename It>
-struct is_device_output
-    : std::integral_constant<bool, std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value> {};
 }  // namespace detail
 
 template <typename D, typename In, typename Out, typename F>
@@ -72,12 +69,12 @@ Out transform(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, Out 
   const uint64_t n = (uint64_t)(last1 - first1);
   if (n == 0) return result;
 #if defined(__HIPCC__)
-  typedef typename iterator_value<Out>::type U;
   hipLaunchKernelGGL((detail::transform2_kernel<typename thrust::detail::device_view_of<In1>::type,
-                                                typename thrust::detail::device_view_of<In2>::type, U, F>),
+                                                typename thrust::detail::device_view_of<In2>::type,
+                                                typename thrust::detail::device_view_of<Out>::type, F>),
                      dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
                      thrust::detail::device_view(first1), thrust::detail::device_view(first2),
-                     thrust::detail::raw(result), n, f);
+                     thrust::detail::device_view(result), n, f);
   detail::throw_on_error(detail::launch_status(), "transform: kernel launch");
   detail::synchronize(stream, "transform: synchronize");
 #else
@@ -89,14 +86,15 @@ Out transform(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, Out 
 template <typename D, typename It, typename F>
 It for_each(execution_policy<D>& exec, It first, It last, F f) {
   static_assert(detail::is_device_output<It>::value,
-                "thrust::for_each on the device system needs device_ptr / device_vector iterators or raw device pointers");
+                "thrust::for_each on the device system needs device_ptr / device_vector iterators, raw device pointers "
+                "or a zip of them");
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return last;
 #if defined(__HIPCC__)
-  typedef typename std::remove_pointer<decltype(thrust::detail::raw(first))>::type T;
-  hipLaunchKernelGGL((detail::for_each_kernel<T, F>), dim3(detail::elementwise_grid(n)),
-                     dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream, thrust::detail::raw(first), n, f);
+  hipLaunchKernelGGL((detail::for_each_kernel<typename thrust::detail::device_view_of<It>::type, F>),
+                     dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
+                     thrust::detail::device_view(first), n, f);
   detail::throw_on_error(detail::launch_status(), "for_each: kernel launch");
   detail::synchronize(stream, "for_each: synchronize");
 #else
@@ -126,12 +124,12 @@ void scatter(execution_policy<D>& exec, In first, In last, MapIt map, Out output
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return;
 #if defined(__HIPCC__)
-  typedef typename iterator_value<Out>::type U;
   hipLaunchKernelGGL((detail::scatter_kernel<typename thrust::detail::device_view_of<In>::type,
-                                             typename thrust::detail::device_view_of<MapIt>::type, U>),
+                                             typename thrust::detail::device_view_of<MapIt>::type,
+                                             typename thrust::detail::device_view_of<Out>::type>),
                      dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
                      thrust::detail::device_view(first), thrust::detail::device_view(map),
-                     thrust::detail::raw(output), n);
+                     thrust::detail::device_view(output), n);
   detail::throw_on_error(detail::launch_status(), "scatter: kernel launch");
   detail::synchronize(stream, "scatter: synchronize");
 #else

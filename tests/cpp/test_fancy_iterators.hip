@@ -17,6 +17,9 @@
 #include <thrust/iterator/counting_iterator.h>
 #include <thrust/iterator/permutation_iterator.h>
 #include <thrust/iterator/transform_iterator.h>
+#include <thrust/iterator/zip_iterator.h>
+#include <thrust/sort.h>
+#include <thrust/tuple.h>
 #include <thrust/partition.h>
 #include <thrust/remove.h>
 #include <thrust/reduce.h>
@@ -30,7 +33,9 @@
 #include <hip/hip_runtime.h>
 
 #include <cstdint>
+#include <algorithm>
 #include <cstdio>
+#include <utility>
 #include <vector>
 
 static int g_failed = 0, g_checks = 0;
@@ -248,6 +253,88 @@ static void TestUserPredicatesByKey() {
   }
 }
 
+struct add_first_two_into_third {  // the functor of examples/arbitrary_transformation.cu
+  template <typename Tuple>
+  __host__ __device__ void operator()(Tuple t) const { thrust::get<2>(t) = thrust::get<0>(t) + thrust::get<1>(t); }
+};
+struct swap_pair {
+  __host__ __device__ thrust::tuple<float, int> operator()(const thrust::tuple<int, float>& t) const {
+    return thrust::make_tuple(thrust::get<1>(t) * 2.0f, thrust::get<0>(t) + 1);
+  }
+};
+struct tuple_sum {
+  __host__ __device__ thrust::tuple<int, int> operator()(const thrust::tuple<int, int>& a, const thrust::tuple<int, int>& b) const {
+    return thrust::make_tuple(thrust::get<0>(a) + thrust::get<0>(b), thrust::get<1>(a) + thrust::get<1>(b));
+  }
+};
+
+static void TestZipIterator() {
+  g_test = "ZipSimple";
+  {
+    // testing/zip_iterator.cu: dereference, arithmetic, assignment through the tuple of references
+    thrust::device_vector<int> a(hv<int>({1, 2, 3, 4})), b(hv<int>({10, 20, 30, 40})), c(4, 0);
+    auto z = thrust::make_zip_iterator(thrust::make_tuple(a.begin(), b.begin(), c.begin()));
+    ASSERT_TRUE((z + 4) - z == 4);
+    thrust::tuple<int, int, int> second = z[1];
+    ASSERT_TRUE(thrust::get<0>(second) == 2 && thrust::get<1>(second) == 20 && thrust::get<2>(second) == 0);
+    thrust::for_each(z, z + 4, add_first_two_into_third());
+    ASSERT_TRUE(same(to_host(c), hv<int>({11, 22, 33, 44})));
+    // sort_by_key with two value arrays zipped
+    thrust::device_vector<int> keys(hv<int>({3, 1, 2, 1}));
+    thrust::sort_by_key(keys.begin(), keys.end(), thrust::make_zip_iterator(thrust::make_tuple(a.begin(), b.begin())));
+    ASSERT_TRUE(same(to_host(keys), hv<int>({1, 1, 2, 3})));
+    ASSERT_TRUE(same(to_host(a), hv<int>({2, 4, 3, 1})));
+    ASSERT_TRUE(same(to_host(b), hv<int>({20, 40, 30, 10})));
+    // sorting a structure of arrays lexicographically
+    thrust::device_vector<int> major(hv<int>({2, 1, 2, 1, 0})), minor(hv<int>({5, 9, 1, 3, 7}));
+    auto zz = thrust::make_zip_iterator(thrust::make_tuple(major.begin(), minor.begin()));
+    thrust::sort(zz, zz + 5);
+    ASSERT_TRUE(same(to_host(major), hv<int>({0, 1, 1, 2, 2})));
+    ASSERT_TRUE(same(to_host(minor), hv<int>({7, 3, 9, 1, 5})));
+  }
+  for (size_t n : kSizes) {
+    g_test = "ZipDifferential";
+    const thrust::host_vector<int> hi = random_values<int>(n, 41, 1000);
+    thrust::host_vector<float> hf(n);
+    for (size_t i = 0; i < n; ++i) hf[i] = (float)(mix(i + 5) % 4096) / 16.0f;
+    const thrust::device_vector<int> di(hi);
+    const thrust::device_vector<float> df(hf);
+    // transform from a zip to a zip
+    thrust::host_vector<float> hof(n);
+    thrust::host_vector<int> hoi(n);
+    thrust::device_vector<float> dof(n);
+    thrust::device_vector<int> doi(n);
+    thrust::transform(thrust::make_zip_iterator(thrust::make_tuple(hi.begin(), hf.begin())),
+                      thrust::make_zip_iterator(thrust::make_tuple(hi.end(), hf.end())),
+                      thrust::make_zip_iterator(thrust::make_tuple(hof.begin(), hoi.begin())), swap_pair());
+    thrust::transform(thrust::make_zip_iterator(thrust::make_tuple(di.begin(), df.begin())),
+                      thrust::make_zip_iterator(thrust::make_tuple(di.end(), df.end())),
+                      thrust::make_zip_iterator(thrust::make_tuple(dof.begin(), doi.begin())), swap_pair());
+    ASSERT_TRUE(same(to_host(dof), hof));
+    ASSERT_TRUE(same(to_host(doi), hoi));
+    // reduce of zipped ranges with a user operator: two sums in one pass
+    const thrust::tuple<int, int> zero = thrust::make_tuple(0, 0);
+    auto hz = thrust::make_zip_iterator(thrust::make_tuple(hi.begin(), hoi.begin()));
+    auto dz = thrust::make_zip_iterator(thrust::make_tuple(di.begin(), doi.begin()));
+    ASSERT_TRUE(thrust::reduce(dz, dz + n, zero, tuple_sum()) == thrust::reduce(hz, hz + n, zero, tuple_sum()));
+    // stable sort of a structure of arrays by a user comparator on the tuple, against the host system
+    thrust::host_vector<int> hk(hi), hv2(n);
+    for (size_t i = 0; i < n; ++i) hv2[i] = (int)i;
+    thrust::device_vector<int> dk(hk), dv2(hv2);
+    auto hzz = thrust::make_zip_iterator(thrust::make_tuple(hk.begin(), hv2.begin()));
+    auto dzz = thrust::make_zip_iterator(thrust::make_tuple(dk.begin(), dv2.begin()));
+    thrust::sort(dzz, dzz + n);
+    std::vector<std::pair<int, int> > ref(n);
+    for (size_t i = 0; i < n; ++i) ref[i] = std::make_pair(hi[i], (int)i);
+    std::sort(ref.begin(), ref.end());
+    bool ok = true;
+    const thrust::host_vector<int> gk = to_host(dk), gv = to_host(dv2);
+    for (size_t i = 0; i < n; ++i) ok = ok && gk[i] == ref[i].first && gv[i] == ref[i].second;
+    ASSERT_TRUE(ok);
+    (void)hzz;
+  }
+}
+
 static void TestKnownAnswers() {
   g_test = "GatherSimple";
   {
@@ -442,6 +529,7 @@ int main() {
   Differential();
   TestUserOperators();
   TestUserPredicatesByKey();
+  TestZipIterator();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
   std::printf(g_failed ? "FAILED\n" : "PASSED\n");
   return g_failed ? 1 : 0;
