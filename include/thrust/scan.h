@@ -290,8 +290,23 @@ struct scan_by_key_checks {
 };
 }  // namespace detail
 
+namespace detail {
+// library path: arithmetic keys and values of one type, equal_to, plus / minimum / maximum
+template <typename K, typename V, typename U, typename T, typename Pred, typename Op,
+          bool = is_abi_type<K>::value && is_abi_type<V>::value && std::is_same<V, T>::value && std::is_same<U, V>::value>
+struct scans_by_key_in_library
+    : std::integral_constant<bool, is_equal_to<Pred, K>::value && (binop_code<Op, V>::value >= 0)> {};
+template <typename K, typename V, typename U, typename T, typename Pred, typename Op>
+struct scans_by_key_in_library<K, V, U, T, Pred, Op, false> : std::false_type {};
+
+// a user's key predicate, operator or element types (defined with the other by-key pieces,
+// in translation units compiled with hipcc)
+template <bool EXCLUSIVE, typename D, typename KIt, typename VIt, typename Out, typename A, typename Pred, typename Op>
+Out scan_by_key_generic(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, A init, Pred pred, Op op);
+}  // namespace detail
+
 template <typename D, typename KIt, typename VIt, typename Out, typename Pred, typename Op>
-Out inclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred, Op) {
+Out inclusive_scan_by_key_library(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred, Op) {
   typedef detail::scan_by_key_checks<KIt, VIt, Out, typename std::remove_const<typename iterator_value<VIt>::type>::type, Pred, Op> C;
   typedef typename C::K K;
   typedef typename C::V V;
@@ -309,7 +324,7 @@ Out inclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out
 }
 
 template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
-Out exclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init, Pred, Op) {
+Out exclusive_scan_by_key_library(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init, Pred, Op) {
   typedef detail::scan_by_key_checks<KIt, VIt, Out, T, Pred, Op> C;
   typedef typename C::K K;
   typedef typename C::V V;
@@ -335,6 +350,64 @@ Out exclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out
   });
   detail::synchronize(stream, "exclusive_scan_by_key: synchronize");
   return result + n;
+}
+
+namespace detail {
+template <typename D, typename KIt, typename VIt, typename Out, typename Pred, typename Op>
+Out inclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred pred, Op op, std::true_type) {
+  return inclusive_scan_by_key_library(exec, kf, kl, vf, result, pred, op);
+}
+template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
+Out exclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init, Pred pred, Op op,
+                          std::true_type) {
+  return exclusive_scan_by_key_library(exec, kf, kl, vf, result, init, pred, op);
+}
+#if defined(__HIPCC__)
+template <typename D, typename KIt, typename VIt, typename Out, typename Pred, typename Op>
+Out inclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred pred, Op op, std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
+  return scan_by_key_generic<false>(exec, kf, kl, vf, result, V(), pred, op);
+}
+template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
+Out exclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init, Pred pred, Op op,
+                          std::false_type) {
+  return scan_by_key_generic<true>(exec, kf, kl, vf, result, init, pred, op);
+}
+#else
+template <typename D, typename KIt, typename VIt, typename Out, typename Pred, typename Op>
+Out inclusive_scan_by_key(execution_policy<D>&, KIt, KIt, VIt, Out result, Pred, Op, std::false_type) {
+  static_assert(fancy_needs_hipcc<Op>::value,
+                "scan_by_key on the device system: key predicates other than thrust::equal_to, operators other than "
+                "thrust::plus / minimum / maximum and non-arithmetic elements run in kernels instantiated for them; "
+                "compile this translation unit with hipcc");
+  return result;
+}
+template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
+Out exclusive_scan_by_key(execution_policy<D>&, KIt, KIt, VIt, Out result, T, Pred, Op, std::false_type) {
+  static_assert(fancy_needs_hipcc<Op>::value,
+                "scan_by_key on the device system: key predicates other than thrust::equal_to, operators other than "
+                "thrust::plus / minimum / maximum and non-arithmetic elements run in kernels instantiated for them; "
+                "compile this translation unit with hipcc");
+  return result;
+}
+#endif
+}  // namespace detail
+
+template <typename D, typename KIt, typename VIt, typename Out, typename Pred, typename Op>
+Out inclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred pred, Op op) {
+  typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
+  return detail::inclusive_scan_by_key(
+      exec, kf, kl, vf, result, pred, op,
+      detail::scans_by_key_in_library<K, V, typename iterator_value<Out>::type, V, Pred, Op>());
+}
+template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
+Out exclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init, Pred pred, Op op) {
+  typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
+  return detail::exclusive_scan_by_key(
+      exec, kf, kl, vf, result, init, pred, op,
+      detail::scans_by_key_in_library<K, V, typename iterator_value<Out>::type, T, Pred, Op>());
 }
 }  // namespace hip
 }  // namespace system
@@ -453,3 +526,7 @@ Out exclusive_scan_by_key(KIt kf, KIt kl, VIt vf, Out result, T init, Pred pred,
 }
 
 }  // namespace thrust
+
+#if defined(__HIPCC__)
+#include <thrust/system/hip/detail/generic_by_key.h>
+#endif

@@ -168,6 +168,55 @@ pair<KOut, VOut> reduce_by_key_generic(execution_policy<D>& exec, KIn kf, KIn kl
   return thrust::make_pair(ko + runs, vo + runs);
 }
 
+// inclusive / exclusive scan_by_key: the generic in-order scan over (head, value) pairs with the
+// segmented operator.  The exclusive form scans the values shifted right by one with init at
+// the heads, which is how the reference states it
+// (thrust/system/detail/generic/scan_by_key.inl:50-140).  A is the accumulator's type.
+template <typename ViewV, typename A>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void shifted_seg_pairs_kernel(ViewV values, const unsigned char* head,
+                                                                              uint64_t n, A init, seg_pair<A>* pairs) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) {
+    seg_pair<A> p;
+    p.head = head[i];
+    if (p.head) p.value = init;
+    else p.value = (A)values[i - 1];
+    pairs[i] = p;
+  }
+}
+
+template <bool EXCLUSIVE, typename D, typename KIt, typename VIt, typename Out, typename A, typename Pred, typename Op>
+Out scan_by_key_generic(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, A init, Pred pred, Op op) {
+  static_assert(is_device_input<KIt>::value && is_device_input<VIt>::value && is_device_output<Out>::value,
+                "scan_by_key on the device system reads device or fancy iterators and writes device memory");
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(kl - kf);
+  if (n == 0) return result;
+  temp_storage flags(stream, temp_source_of(exec));
+  flags.ensure((std::size_t)n);
+  unsigned char* head = static_cast<unsigned char*>(flags.ptr());
+  launch_run_flags(exec, kf, n, pred, head, nullptr);
+  typedef seg_pair<A> P;
+  temp_storage pair_store(stream, temp_source_of(exec));
+  pair_store.ensure((std::size_t)n * sizeof(P));
+  P* pairs = static_cast<P*>(pair_store.ptr());
+  typedef typename thrust::detail::device_view_of<VIt>::type ViewV;
+  if (EXCLUSIVE)
+    hipLaunchKernelGGL((shifted_seg_pairs_kernel<ViewV, A>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
+                       (hipStream_t)stream, thrust::detail::device_view(vf), (const unsigned char*)head, n, init, pairs);
+  else
+    hipLaunchKernelGGL((seg_pairs_kernel<ViewV, A>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
+                       (hipStream_t)stream, thrust::detail::device_view(vf), (const unsigned char*)head, n, pairs);
+  throw_on_error(launch_status(), "scan_by_key: kernel launch");
+  const seg_op<A, Op> sop = {op};
+  scan_generic<false, P>(exec, pairs, pairs + n, pairs, P(), sop);
+  // the values of the scanned pairs are the result (the pairs were built from a copy of the
+  // input, so the output may be the input)
+  materialize(stream, thrust::make_transform_iterator((const P*)pairs, pair_value<A>()), result, n);
+  synchronize(stream, "scan_by_key: synchronize");
+  return result + n;
+}
+
 }  // namespace detail
 }  // namespace hip
 }  // namespace system

@@ -235,6 +235,22 @@ static void TestUserPredicatesByKey() {
     hko.resize(runs); hvo.resize(runs); dko.resize(runs); dvo.resize(runs);
     ASSERT_TRUE(same(to_host(dko), hko));
     ASSERT_TRUE(same(to_host(dvo), hvo));
+    // scan_by_key with a user key predicate and operator (inclusive, exclusive with init, in place)
+    {
+      thrust::host_vector<unsigned> hs(n);
+      thrust::device_vector<unsigned> ds(n);
+      thrust::inclusive_scan_by_key(hk.begin(), hk.end(), hvv.begin(), hs.begin(), same_tens(), bit_xor_op());
+      thrust::inclusive_scan_by_key(dk.begin(), dk.end(), dv.begin(), ds.begin(), same_tens(), bit_xor_op());
+      ASSERT_TRUE(same(to_host(ds), hs));
+      thrust::exclusive_scan_by_key(hk.begin(), hk.end(), hvv.begin(), hs.begin(), 7u, same_tens(), thrust::multiplies<unsigned>());
+      thrust::exclusive_scan_by_key(dk.begin(), dk.end(), dv.begin(), ds.begin(), 7u, same_tens(), thrust::multiplies<unsigned>());
+      ASSERT_TRUE(same(to_host(ds), hs));
+      thrust::host_vector<unsigned> hin(hvv);
+      thrust::device_vector<unsigned> din(dv);
+      thrust::exclusive_scan_by_key(hk.begin(), hk.end(), hin.begin(), hin.begin(), 3u, thrust::equal_to<int>(), bit_xor_op());
+      thrust::exclusive_scan_by_key(dk.begin(), dk.end(), din.begin(), din.begin(), 3u, thrust::equal_to<int>(), bit_xor_op());
+      ASSERT_TRUE(same(to_host(din), hin));
+    }
     // unique_copy and unique_by_key_copy
     hko.resize(n); dko.resize(n); hvo.resize(n); dvo.resize(n);
     auto he = thrust::unique_copy(hk.begin(), hk.end(), hko.begin(), same_tens());
