@@ -93,6 +93,30 @@ __global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out,
     }
   }
 
+  // ---- the tile's aggregate first, and published at once: a later tile's look-back can pass
+  // this tile as soon as the sum is known, it does not have to wait for the scan below
+  // (plus, minimum and maximum commute, so the lanes may fold their own elements first)
+  {
+    T lane_total = id;
+#pragma unroll
+    for (int j = 0; j < SCAN_CHUNKS; ++j) {
+#pragma unroll
+      for (int i = 0; i < VEC; ++i) lane_total = op(lane_total, x[j].v[i]);
+    }
+    const T wave_total = wave_reduce(lane_total, op);
+    if (lane == 0) s_wave_agg[wave] = wave_total;
+  }
+  __syncthreads();
+  T wave_prefix = id;
+  T block_agg = id;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    if (w == wave) wave_prefix = block_agg;
+    block_agg = op(block_agg, s_wave_agg[w]);
+  }
+  uint64_t* my_slot = status + (size_t)tile * W;
+  if (threadIdx.x == 0) tile_publish<T>(my_slot, tile == 0 ? TS_INCLUSIVE : TS_PARTIAL, block_agg);
+
   // ---- wave-local scan in place: every element becomes the fold of the wave's span up to
   // it (inclusive), or up to but excluding it (exclusive); CHUNKS DPP wave scans chained by
   // the wave total.  Nothing but x[] and the carry stays live.
@@ -117,25 +141,11 @@ __global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out,
       }
     }
   }
-  if (lane == 0) s_wave_agg[wave] = carry;
-  __syncthreads();
-
-  T wave_prefix = id;
-  T block_agg = id;
-#pragma unroll
-  for (int w = 0; w < WAVES; ++w) {
-    if (w == wave) wave_prefix = block_agg;
-    block_agg = op(block_agg, s_wave_agg[w]);
-  }
 
   // ---- cross-tile prefix
-  uint64_t* my_slot = status + (size_t)tile * W;
   if (wave == 0) {
     T tile_excl = id;
-    if (tile == 0) {
-      if (lane == 0) tile_publish<T>(my_slot, TS_INCLUSIVE, block_agg);
-    } else {
-      if (lane == 0) tile_publish<T>(my_slot, TS_PARTIAL, block_agg);
+    if (tile != 0) {
       tile_excl = tile_lookback<T>(status, tile, op, id);
       if (lane == 0) tile_publish<T>(my_slot, TS_INCLUSIVE, op(tile_excl, block_agg));
     }
