@@ -9,8 +9,10 @@ import numpy as np
 from thrust_amd import datagen
 
 LT = 0
-SMALL = {"c1": 1 << 14, "c2": 1 << 14, "c3": 1 << 13, "c4": 1 << 15, "c5": 1 << 14, "c6": 1 << 15, "c7": 1 << 14}
-LARGE = {"c1": 1 << 22, "c2": 1 << 22, "c3": 1 << 21, "c4": 1 << 22, "c5": 1 << 22, "c6": 1 << 22, "c7": 1 << 22}
+SMALL = {"c1": 1 << 14, "c2": 1 << 14, "c3": 1 << 13, "c4": 1 << 15, "c5": 1 << 14, "c6": 1 << 15, "c7": 1 << 14,
+         "c8": 1 << 14}
+LARGE = {"c1": 1 << 22, "c2": 1 << 22, "c3": 1 << 21, "c4": 1 << 22, "c5": 1 << 22, "c6": 1 << 22, "c7": 1 << 22,
+         "c8": 1 << 21}
 
 
 def c1(impl, n):
@@ -122,7 +124,30 @@ def c7(impl, n):
     return out
 
 
-CASES = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5, "c6": c6, "c7": c7}
+def c8(impl, n):
+    """The comparison sort (stable_sort with user-defined comparators: the reference's merge sort) and the
+    reference's rules for mixed element types (conversions, accumulator of init's / the input's type)."""
+    out = {}
+    k = (datagen.c2_uint32(n) % np.uint32(1000)).astype(np.int32) - np.int32(500)
+    f = datagen.c2_float32(n)  # with +0.0 / -0.0, equivalent under operator<: their input order must survive
+    v = np.arange(n, dtype=np.uint32)
+    out["c8.comparison_sort_i32"] = impl.comparison_sort(k)
+    ko, vo = impl.comparison_sort(k, v, 1)
+    out["c8.comparison_sort_by_key_i32_greater.values"] = vo
+    ko, vo = impl.comparison_sort(f, v, 0)
+    out["c8.comparison_sort_by_key_f32.key_bits"] = ko.view(np.uint32)
+    out["c8.comparison_sort_by_key_f32.values"] = vo
+    x = datagen.c1_int32(n)
+    fx = x.astype(np.float32) / np.float32(4) - np.float32(100)
+    out["c8.convert_f32_to_i32"] = impl.convert(fx, np.int32)
+    out["c8.convert_i32_to_f32"] = impl.convert(x * np.int32(16777), np.float32)
+    out["c8.reduce_f32_into_i32"] = np.array([impl.reduce_as(fx, np.int32(3))], np.int32)
+    out["c8.inclusive_scan_i32_to_f32"] = impl.inclusive_scan_as(x, np.float32)
+    out["c8.exclusive_scan_i32_init5_to_f32"] = impl.exclusive_scan_as(x, np.int32(5), np.float32)
+    return out
+
+
+CASES = {"c1": c1, "c2": c2, "c3": c3, "c4": c4, "c5": c5, "c6": c6, "c7": c7, "c8": c8}
 
 
 def digest(a):

@@ -82,6 +82,32 @@ class DeviceImpl:
         ko, vo, cnt = self.dev.set_operation_by_key(op, self._d(ka), self._d(kb), self._d(va), self._d(vb), descending)
         return ko.numpy()[:cnt], vo.numpy()[:cnt]
 
+    def comparison_sort(self, keys, values=None, comparator=0, param=0):
+        dk = self._d(keys)
+        if values is None:
+            self.dev.merge_sort_keys(dk, descending=bool(comparator))
+            return dk.numpy()
+        dv = self._d(values)
+        self.dev.merge_sort_pairs(dk, dv, descending=bool(comparator))
+        return dk.numpy(), dv.numpy()
+
+    def convert(self, x, dtype):
+        return self.dev.convert(self._d(x), self.dev.DTYPE_OF_NP[np.dtype(dtype)]).numpy()
+
+    # mixed element types, composed the way the C++ front end composes them
+    def reduce_as(self, x, init, op=0):
+        init = np.asarray(init)
+        acc = self.dev.convert(self._d(x), self.dev.DTYPE_OF_NP[init.dtype])
+        return self.dev.reduce(acc, op, init[()]).numpy()[0]
+
+    def inclusive_scan_as(self, x, out_dtype, op=0):
+        return self.dev.convert(self.dev.inclusive_scan(self._d(x), op=op), self.dev.DTYPE_OF_NP[np.dtype(out_dtype)]).numpy()
+
+    def exclusive_scan_as(self, x, init, out_dtype, op=0):
+        init = np.asarray(init)
+        acc = self.dev.convert(self._d(x), self.dev.DTYPE_OF_NP[init.dtype])
+        return self.dev.convert(self.dev.exclusive_scan(acc, init[()], op=op), self.dev.DTYPE_OF_NP[np.dtype(out_dtype)]).numpy()
+
     def transform_reduce(self, x, unary, op=0, init=0):
         return self.dev.transform_reduce(self._d(x), unary, op=op, init=init).numpy()[0]
 
