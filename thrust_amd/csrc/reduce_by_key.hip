@@ -49,14 +49,14 @@ __global__ __launch_bounds__(256) void rbk_init_kernel(uint64_t* __restrict__ wo
 // K is the key's comparison class: an unsigned integer type of the key's size (integer
 // keys are equal iff their bits are) or float / double (operator==).
 //
-// Layout: a lane owns ITEMS = 16 consecutive elements (four 16-byte key vectors for 4-byte
-// keys), so the flags and the lane's fold are a serial pass over registers and the whole
+// Layout: a lane owns ITEMS = 16 or 20 consecutive elements (four or five 16-byte key vectors
+// for 4-byte keys), so the flags and the lane's fold are a serial pass over registers and the whole
 // tile needs ONE wave scan of pairs per wave.  (Lanes of a wave then read 16-byte pieces
 // 64 bytes apart; the four loads of a lane cover its cache lines completely.)
 template <typename K, typename V, typename Op>
 __global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
   constexpr int VEC = Vec16<K>::N;
-  constexpr int CHUNKS = RBK_ITEMS / VEC >= 1 ? RBK_ITEMS / VEC : 1;
+  constexpr int CHUNKS = RbkItems<K, V>::value / VEC >= 1 ? RbkItems<K, V>::value / VEC : 1;
   constexpr int ITEMS = CHUNKS * VEC;
   constexpr int WAVES = RBK_BLOCK / WAVE;
   constexpr uint32_t TILE = RBK_BLOCK * ITEMS;
@@ -217,7 +217,7 @@ static int rbk_run(void* temp, size_t* temp_bytes, const void* keys_in, const vo
                    void* keys_out, void* values_out, uint64_t* d_num_runs, uint64_t n,
                    hipStream_t stream) {
   constexpr int VEC = Vec16<K>::N;
-  constexpr int CHUNKS = RBK_ITEMS / VEC >= 1 ? RBK_ITEMS / VEC : 1;
+  constexpr int CHUNKS = RbkItems<K, V>::value / VEC >= 1 ? RbkItems<K, V>::value / VEC : 1;
   constexpr uint64_t TILE = (uint64_t)RBK_BLOCK * CHUNKS * VEC;
   using Pair = SegPair<typename SegValue<V>::type>;
   constexpr int W = TileWords<Pair>::W;
