@@ -8,13 +8,18 @@
 // first range's first min(m,n) copies for intersection, its last m-n for difference, and
 // for union all of the first range followed by the second range's last n-m.  The _by_key
 // forms carry one value with every kept key, taken from the range the key came from
-// (thrust/system/detail/generic/set_operations.inl:44-330).  The device system supports
-// arithmetic keys ordered by thrust::less or thrust::greater; results must not overlap
-// the inputs.
+// (thrust/system/detail/generic/set_operations.inl:44-330).  On the device system,
+// arithmetic keys ordered by thrust::less or thrust::greater run in the library's kernels;
+// other comparators and key structs run in kernels instantiated for them, in translation
+// units compiled with hipcc.  Results must not overlap the inputs.
 #pragma once
 #include <thrust/functional.h>
 #include <thrust/pair.h>
 #include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/device_input.h>
+#if defined(__HIPCC__)
+#include <thrust/system/hip/detail/generic_set_operations.h>
+#endif
 
 namespace thrust {
 namespace system {
@@ -66,20 +71,40 @@ inline pair<KOut, VOut> set_operation_by_key(K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 
 
 namespace hip {
 namespace detail {
+// The library's kernels take one arithmetic key type throughout, ordered by operator< or operator>.
+template <typename K, typename In2, typename Out, typename Comp,
+          bool = is_abi_type<K>::value &&
+                 std::is_same<typename std::remove_const<typename iterator_value<In2>::type>::type, K>::value &&
+                 std::is_same<typename iterator_value<Out>::type, K>::value>
+struct set_operation_in_library : std::integral_constant<bool, (order_code<Comp, K>::value >= 0)> {};
 template <typename K, typename In2, typename Out, typename Comp>
-struct set_key_checks {
-  static_assert(is_abi_type<K>::value &&
-                    std::is_same<typename std::remove_const<typename iterator_value<In2>::type>::type, K>::value &&
-                    std::is_same<typename iterator_value<Out>::type, K>::value,
-                "set operations on the device system need one arithmetic key type for both inputs and the output");
-  static_assert(order_code<Comp, K>::value >= 0,
-                "set operations on the device system support thrust::less and thrust::greater");
-};
+struct set_operation_in_library<K, In2, Out, Comp, false> : std::false_type {};
+
+// Everything else: kernels instantiated for the comparator.
+template <int OP, typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut,
+          typename Comp>
+inline uint64_t set_operation_other(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko,
+                                    VOut vo, Comp comp, bool has_values) {
+#if defined(__HIPCC__)
+  return set_operation_generic<OP>(exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp, has_values);
+#else
+  static_assert(fancy_needs_hipcc<Comp>::value,
+                "set operations on the device system: comparators other than thrust::less / thrust::greater of an "
+                "arithmetic key run in kernels instantiated for the comparator; compile this translation unit with hipcc");
+  return 0;
+#endif
+}
 
 template <int OP, typename D, typename In1, typename In2, typename Out, typename Comp>
-inline Out set_operation(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp) {
+inline Out set_operation(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp,
+                         std::false_type) {
+  return result + set_operation_other<OP>(exec, first1, last1, first2, last2, first1, first2, result, result, comp, false);
+}
+
+template <int OP, typename D, typename In1, typename In2, typename Out, typename Comp>
+inline Out set_operation(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp,
+                         std::true_type) {
   typedef typename std::remove_const<typename iterator_value<In1>::type>::type K;
-  (void)sizeof(set_key_checks<K, In2, Out, Comp>);
   void* stream = stream_of(exec);
   const uint64_t na = (uint64_t)(last1 - first1), nb = (uint64_t)(last2 - first2);
   if (na + nb == 0) return result;
@@ -100,13 +125,27 @@ inline Out set_operation(execution_policy<D>& exec, In1 first1, In1 last1, In2 f
   return result + read_scalar<uint64_t>(d_num, stream, "set operation: result size");
 }
 
+template <int OP, typename D, typename In1, typename In2, typename Out, typename Comp>
+inline Out set_operation(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+  typedef typename std::remove_const<typename iterator_value<In1>::type>::type K;
+  return set_operation<OP>(exec, first1, last1, first2, last2, result, comp,
+                           set_operation_in_library<K, In2, Out, Comp>());
+}
+
 template <int OP, typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut,
           typename Comp>
 inline pair<KOut, VOut> set_operation_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2,
-                                             KOut ko, VOut vo, Comp) {
+                                             KOut ko, VOut vo, Comp comp, std::false_type) {
+  const uint64_t cnt = set_operation_other<OP>(exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp, true);
+  return thrust::make_pair(ko + cnt, vo + cnt);
+}
+
+template <int OP, typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut,
+          typename Comp>
+inline pair<KOut, VOut> set_operation_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2,
+                                             KOut ko, VOut vo, Comp, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
   typedef typename std::remove_const<typename iterator_value<V1>::type>::type V;
-  (void)sizeof(set_key_checks<K, K2, KOut, Comp>);
   static_assert(is_abi_item<V>::value &&
                     std::is_same<typename std::remove_const<typename iterator_value<V2>::type>::type, V>::value &&
                     std::is_same<typename iterator_value<VOut>::type, V>::value,
@@ -133,6 +172,15 @@ inline pair<KOut, VOut> set_operation_by_key(execution_policy<D>& exec, K1 kf1, 
   throw_on_error(call(temp.ptr(), &bytes), "set operation by key failed");
   const uint64_t cnt = read_scalar<uint64_t>(d_num, stream, "set operation by key: result size");
   return thrust::make_pair(ko + cnt, vo + cnt);
+}
+
+template <int OP, typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut,
+          typename Comp>
+inline pair<KOut, VOut> set_operation_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2,
+                                             KOut ko, VOut vo, Comp comp) {
+  typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
+  return set_operation_by_key<OP>(exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp,
+                                  set_operation_in_library<K, K2, KOut, Comp>());
 }
 }  // namespace detail
 }  // namespace hip

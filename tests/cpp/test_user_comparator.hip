@@ -3,12 +3,16 @@
 // instantiated in this translation unit.  Known answers are the reference's:
 // testing/stable_sort.cu:49-90 (less_div_10), :125-173 (comparator with an external table),
 // testing/stable_sort_by_key.cu:50-95; the rest is the reference's host-against-device
-// differential pattern (testing/stable_sort.cu:93-108) over its size list.
+// differential pattern (testing/stable_sort.cu:93-108) over its size list.  merge and the
+// set operations with user comparators follow: testing/merge.cu:11-38, set_difference.cu:70-90,
+// set_intersection.cu:71-91, set_symmetric_difference.cu:70-90, set_union.cu:71-116,
+// set_union_by_key.cu:89-120, set_intersection_by_key.cu:83-112.
 #include <thrust/device_vector.h>
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
 #include <thrust/host_vector.h>
 #include <thrust/merge.h>
+#include <thrust/set_operations.h>
 #include <thrust/sort.h>
 
 #include <hip/hip_runtime.h>
@@ -222,6 +226,146 @@ static void TestMergeWithUserComparators() {
   }
 }
 
+static void TestSetOperationsWithUserComparators() {
+  g_test = "SetOperationsSimple";
+  {
+    thrust::device_vector<int> a(hv<int>({0, 2, 4, 5})), b(hv<int>({0, 3, 3, 4, 6})), out(9);
+    auto end = thrust::set_difference(a.begin(), a.end(), b.begin(), b.end(), out.begin(), my_less<int>());
+    ASSERT_TRUE(end - out.begin() == 2);
+    out.resize(2);
+    ASSERT_TRUE(same(to_host(out), hv<int>({2, 5})));
+  }
+  {
+    thrust::device_vector<int> a(hv<int>({0, 2, 4})), b(hv<int>({0, 3, 3, 4})), out(7);
+    auto end = thrust::set_intersection(a.begin(), a.end(), b.begin(), b.end(), out.begin(), my_less<int>());
+    ASSERT_TRUE(end - out.begin() == 2);
+    out.resize(2);
+    ASSERT_TRUE(same(to_host(out), hv<int>({0, 4})));
+    out.resize(7);
+    end = thrust::set_union(a.begin(), a.end(), b.begin(), b.end(), out.begin(), my_less<int>());
+    ASSERT_TRUE(end - out.begin() == 5);
+    out.resize(5);
+    ASSERT_TRUE(same(to_host(out), hv<int>({0, 2, 3, 3, 4})));
+    // by key: a tie takes the first range's value; the second range's surplus keeps its own
+    thrust::device_vector<int> va(hv<int>({0, 0, 0})), vb(hv<int>({1, 1, 1, 1})), ko(7), vo(7);
+    auto ends = thrust::set_union_by_key(a.begin(), a.end(), b.begin(), b.end(), va.begin(), vb.begin(), ko.begin(),
+                                         vo.begin(), my_less<int>());
+    ASSERT_TRUE(ends.first - ko.begin() == 5 && ends.second - vo.begin() == 5);
+    ko.resize(5);
+    vo.resize(5);
+    ASSERT_TRUE(same(to_host(ko), hv<int>({0, 2, 3, 3, 4})));
+    ASSERT_TRUE(same(to_host(vo), hv<int>({0, 0, 1, 1, 0})));
+    ko.resize(7);
+    vo.resize(7);
+    ends = thrust::set_intersection_by_key(a.begin(), a.end(), b.begin(), b.end(), va.begin(), ko.begin(), vo.begin(),
+                                           my_less<int>());
+    ASSERT_TRUE(ends.first - ko.begin() == 2 && ends.second - vo.begin() == 2);
+    ko.resize(2);
+    vo.resize(2);
+    ASSERT_TRUE(same(to_host(ko), hv<int>({0, 4})));
+    ASSERT_TRUE(same(to_host(vo), hv<int>({0, 0})));
+  }
+  {
+    thrust::device_vector<int> a(hv<int>({0, 2, 2})), b(hv<int>({0, 2, 2, 2, 3})), out(8);
+    auto end = thrust::set_union(a.begin(), a.end(), b.begin(), b.end(), out.begin(), my_less<int>());
+    ASSERT_TRUE(end - out.begin() == 5);
+    out.resize(5);
+    ASSERT_TRUE(same(to_host(out), hv<int>({0, 2, 2, 2, 3})));
+  }
+  {
+    thrust::device_vector<int> a(hv<int>({0, 2, 4, 6})), b(hv<int>({0, 3, 3, 4, 7})), out(9);
+    auto end = thrust::set_symmetric_difference(a.begin(), a.end(), b.begin(), b.end(), out.begin(), my_less<int>());
+    ASSERT_TRUE(end - out.begin() == 5);
+    out.resize(5);
+    ASSERT_TRUE(same(to_host(out), hv<int>({2, 3, 3, 6, 7})));
+  }
+  g_test = "SetOperationsDifferential";
+  for (size_t n : kSizes) {
+    const size_t na = n, nb = n / 2 + (n % 7);
+    // equivalence classes of ten under less_div_10, a few dozen elements in each for the
+    // larger sizes: which copies survive shows in the low digit
+    const uint64_t range = n < 64 ? 40 : (n < 5000 ? 400 : 3000);
+    thrust::host_vector<int> ha(na), hb(nb);
+    for (size_t i = 0; i < na; ++i) ha[i] = (int)(mix(i + 17 * n) % range);
+    for (size_t i = 0; i < nb; ++i) hb[i] = (int)(mix(i + 19 * n) % range);
+    std::stable_sort(ha.begin(), ha.end(), less_div_10<int>());
+    std::stable_sort(hb.begin(), hb.end(), less_div_10<int>());
+    thrust::host_vector<unsigned> hva(na), hvb(nb);
+    for (size_t i = 0; i < na; ++i) hva[i] = (unsigned)i;
+    for (size_t i = 0; i < nb; ++i) hvb[i] = (unsigned)(1000000 + i);
+    thrust::device_vector<int> da(ha), db(hb);
+    thrust::device_vector<unsigned> dva(hva), dvb(hvb);
+    thrust::host_vector<int> hout(na + nb);
+    thrust::device_vector<int> dout(na + nb);
+    thrust::host_vector<unsigned> hvo(na + nb);
+    thrust::device_vector<unsigned> dvo(na + nb);
+    const less_div_10<int> comp;
+    size_t hc, dc;
+#define CHECK_KEYS(NAME)                                                                                   \
+    hc = thrust::NAME(ha.begin(), ha.end(), hb.begin(), hb.end(), hout.begin(), comp) - hout.begin();      \
+    dc = thrust::NAME(da.begin(), da.end(), db.begin(), db.end(), dout.begin(), comp) - dout.begin();      \
+    ASSERT_TRUE(hc == dc);                                                                                 \
+    {                                                                                                      \
+      thrust::host_vector<int> got(dout);                                                                  \
+      ASSERT_TRUE(std::equal(hout.begin(), hout.begin() + hc, got.begin()));                               \
+    }
+    CHECK_KEYS(set_difference)
+    CHECK_KEYS(set_intersection)
+    CHECK_KEYS(set_symmetric_difference)
+    CHECK_KEYS(set_union)
+#undef CHECK_KEYS
+#define CHECK_BY_KEY(NAME)                                                                                 \
+    hc = thrust::NAME(ha.begin(), ha.end(), hb.begin(), hb.end(), hva.begin(), hvb.begin(), hout.begin(),  \
+                      hvo.begin(), comp).first - hout.begin();                                             \
+    dc = thrust::NAME(da.begin(), da.end(), db.begin(), db.end(), dva.begin(), dvb.begin(), dout.begin(),  \
+                      dvo.begin(), comp).first - dout.begin();                                             \
+    ASSERT_TRUE(hc == dc);                                                                                 \
+    {                                                                                                      \
+      thrust::host_vector<int> got(dout);                                                                  \
+      thrust::host_vector<unsigned> got_values(dvo);                                                       \
+      ASSERT_TRUE(std::equal(hout.begin(), hout.begin() + hc, got.begin()));                               \
+      ASSERT_TRUE(std::equal(hvo.begin(), hvo.begin() + hc, got_values.begin()));                          \
+    }
+    CHECK_BY_KEY(set_difference_by_key)
+    CHECK_BY_KEY(set_symmetric_difference_by_key)
+    CHECK_BY_KEY(set_union_by_key)
+#undef CHECK_BY_KEY
+    hc = thrust::set_intersection_by_key(ha.begin(), ha.end(), hb.begin(), hb.end(), hva.begin(), hout.begin(),
+                                         hvo.begin(), comp).first - hout.begin();
+    dc = thrust::set_intersection_by_key(da.begin(), da.end(), db.begin(), db.end(), dva.begin(), dout.begin(),
+                                         dvo.begin(), comp).first - dout.begin();
+    ASSERT_TRUE(hc == dc);
+    {
+      thrust::host_vector<int> got(dout);
+      thrust::host_vector<unsigned> got_values(dvo);
+      ASSERT_TRUE(std::equal(hout.begin(), hout.begin() + hc, got.begin()));
+      ASSERT_TRUE(std::equal(hvo.begin(), hvo.begin() + hc, got_values.begin()));
+    }
+  }
+  g_test = "SetOperationsStructKeys";
+  {
+    // records ordered by group only: the weight tells which copies were kept
+    const size_t na = 5000, nb = 3000;
+    thrust::host_vector<Record> ha(na), hb(nb);
+    for (size_t i = 0; i < na; ++i) ha[i] = Record{(int)(mix(i + 5) % 700), (float)i};
+    for (size_t i = 0; i < nb; ++i) hb[i] = Record{(int)(mix(i + 7) % 700), -(float)i};
+    std::stable_sort(ha.begin(), ha.end(), by_group());
+    std::stable_sort(hb.begin(), hb.end(), by_group());
+    thrust::device_vector<Record> da(ha), db(hb), dout(na + nb);
+    thrust::host_vector<Record> hout(na + nb);
+    size_t hc = thrust::set_union(ha.begin(), ha.end(), hb.begin(), hb.end(), hout.begin(), by_group()) - hout.begin();
+    size_t dc = thrust::set_union(da.begin(), da.end(), db.begin(), db.end(), dout.begin(), by_group()) - dout.begin();
+    ASSERT_TRUE(hc == dc);
+    thrust::host_vector<Record> got(dout);
+    ASSERT_TRUE(std::equal(hout.begin(), hout.begin() + hc, got.begin()));
+    hc = thrust::set_difference(ha.begin(), ha.end(), hb.begin(), hb.end(), hout.begin(), by_group()) - hout.begin();
+    dc = thrust::set_difference(da.begin(), da.end(), db.begin(), db.end(), dout.begin(), by_group()) - dout.begin();
+    ASSERT_TRUE(hc == dc);
+    got = dout;
+    ASSERT_TRUE(std::equal(hout.begin(), hout.begin() + hc, got.begin()));
+  }
+}
+
 int main() {
   TestKnownAnswers();
   Differential<signed char>("signed char");
@@ -231,6 +375,7 @@ int main() {
   Differential<float>("float");
   TestStructKeys();
   TestMergeWithUserComparators();
+  TestSetOperationsWithUserComparators();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
   std::printf(g_failed ? "FAILED\n" : "PASSED\n");
   return g_failed ? 1 : 0;
