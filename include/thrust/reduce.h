@@ -150,8 +150,8 @@ T reduce(execution_policy<D>& exec, It first, It last, T init, Op op, std::false
   return read_scalar<T>(d_out, stream, "reduce: result copy");
 #else
   static_assert(fancy_needs_hipcc<Op>::value,
-                "thrust::reduce on the device system: operators other than thrust::plus / minimum / maximum of an "
-                "arithmetic type run in kernels instantiated for the operator; compile this translation unit with hipcc");
+                "thrust::reduce on the device system: fancy iterators, and operators other than thrust::plus / minimum / "
+                "maximum of an arithmetic type, run in kernels instantiated for them; compile this translation unit with hipcc");
   return init;
 #endif
 }
@@ -168,7 +168,10 @@ T reduce(execution_policy<D>& exec, It first, It last, T init, Op op) {
   static_assert(detail::is_device_input<It>::value,
                 "thrust::reduce on the device system needs device_ptr / device_vector iterators, raw device pointers "
                 "or fancy iterators over them");
-  return detail::reduce(exec, first, last, init, op, detail::reduces_in_library<T, V, Op>());
+  // a fancy iterator is read where it is (the kernels instantiated for it), not written out first
+  return detail::reduce(exec, first, last, init, op,
+                        std::integral_constant<bool, detail::reduces_in_library<T, V, Op>::value &&
+                                                         !thrust::detail::is_fancy_iterator<It>::value>());
 }
 
 namespace detail {

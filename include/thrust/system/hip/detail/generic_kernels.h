@@ -65,11 +65,12 @@ __global__ __launch_bounds__(BLOCK) void reduce_chunks_kernel(View first, uint64
   const uint64_t begin = (uint64_t)blockIdx.x * chunk;
   const uint64_t end = (begin + chunk < n) ? begin + chunk : n;
   T acc = T();
-  bool has = false;
-  for (uint64_t i = begin + threadIdx.x; i < end; i += BLOCK) {
-    const T x = (T)first[i];
-    if (has) acc = op(acc, x);
-    else { acc = x; has = true; }
+  const bool has = begin + threadIdx.x < end;
+  if (has) {
+    // the lane's first element starts the fold, the rest follow in index order
+    acc = (T)first[begin + threadIdx.x];
+#pragma unroll 4
+    for (uint64_t i = begin + threadIdx.x + BLOCK; i < end; i += BLOCK) acc = op(acc, (T)first[i]);
   }
   bool any;
   const T total = block_fold(acc, has, op, s_val, s_has, any);

@@ -351,6 +351,23 @@ static void TestZipIterator() {
   }
 }
 
+// testing/reduce.cu:213-231: ranges of 2^30 .. 2^33 elements that exist only as an iterator
+static void TestReduceWithBigIndexes() {
+  g_test = "ReduceWithBigIndexes";
+  for (int magnitude = 30; magnitude <= 33; ++magnitude) {
+    thrust::constant_iterator<long long> begin(1);
+    thrust::constant_iterator<long long> end = begin + (1ll << magnitude);
+    ASSERT_TRUE(end - begin == (1ll << magnitude));
+    const long long result = thrust::reduce(thrust::device, begin, end);
+    ASSERT_TRUE(result == (1ll << magnitude));
+  }
+  // the same range counted: sum of 0 .. n-1
+  const long long n = (1ll << 31) + 12345;
+  thrust::counting_iterator<long long> first(0);
+  const long long sum = thrust::reduce(thrust::device, first, first + n, 0ll);
+  ASSERT_TRUE(sum == (long long)((unsigned long long)n * (unsigned long long)(n - 1) / 2));
+}
+
 static void TestKnownAnswers() {
   g_test = "GatherSimple";
   {
@@ -542,6 +559,7 @@ static void Differential() {
 
 int main() {
   TestKnownAnswers();
+  TestReduceWithBigIndexes();
   Differential();
   TestUserOperators();
   TestUserPredicatesByKey();
