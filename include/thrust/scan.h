@@ -216,17 +216,48 @@ Out scan_generic(execution_policy<D>& exec, In first, In last, Out result, A ini
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
-  const uint64_t tiles = (n + gk::TILE - 1) / gk::TILE;
+  constexpr uint64_t TILE = gk::scan_shape<A>::TILE;
+  const uint64_t tiles = (n + TILE - 1) / TILE;
   if (tiles > 0xffffffffull) throw_on_error(1, "scan: range too long");
+  // The tile totals are scanned in place: by one workgroup when there are few, otherwise by the
+  // same three steps one level up (their tile totals, scanned, then every tile of totals on top
+  // of what precedes it).  level[k] holds the totals of level k - 1's tiles; level[0] those of the input.
+  constexpr uint64_t ONE_WORKGROUP = 4 * gk::BLOCK;
+  constexpr int MAX_LEVELS = 8;
+  uint64_t count[MAX_LEVELS];
+  std::size_t offset[MAX_LEVELS];
+  int levels = 0;
+  std::size_t bytes = 0;
+  for (uint64_t c = tiles;; c = (c + TILE - 1) / TILE) {
+    count[levels] = c;
+    offset[levels] = bytes;
+    bytes += ((std::size_t)c * sizeof(A) + 255) / 256 * 256;
+    ++levels;
+    if (c <= ONE_WORKGROUP || levels == MAX_LEVELS) break;
+  }
   temp_storage temp(stream, temp_source_of(exec));
-  temp.ensure((std::size_t)tiles * sizeof(A));
-  A* tile_total = static_cast<A*>(temp.ptr());
+  temp.ensure(bytes);
+  A* level[MAX_LEVELS];
+  for (int k = 0; k < levels; ++k) level[k] = reinterpret_cast<A*>(static_cast<char*>(temp.ptr()) + offset[k]);
+  A* tile_total = level[0];
   hipLaunchKernelGGL((gk::scan_tile_totals_kernel<View, A, Op>), dim3((unsigned)tiles), dim3(gk::BLOCK), 0,
                      (hipStream_t)stream, thrust::detail::device_view(first), n, op, tile_total);
   throw_on_error(launch_status(), "scan: kernel launch");
+  for (int k = 1; k < levels; ++k) {
+    hipLaunchKernelGGL((gk::scan_tile_totals_kernel<const A*, A, Op>), dim3((unsigned)count[k]), dim3(gk::BLOCK), 0,
+                       (hipStream_t)stream, (const A*)level[k - 1], count[k - 1], op, level[k]);
+    throw_on_error(launch_status(), "scan: kernel launch");
+  }
   hipLaunchKernelGGL((gk::scan_tile_prefix_kernel<A, Op>), dim3(1), dim3(gk::BLOCK), 0, (hipStream_t)stream,
-                     tile_total, (uint32_t)tiles, op);
+                     level[levels - 1], (uint32_t)count[levels - 1], op);
   throw_on_error(launch_status(), "scan: kernel launch");
+  for (int k = levels - 1; k >= 1; --k) {
+    // in place: a workgroup reads its tile into registers before it writes
+    hipLaunchKernelGGL((gk::scan_tiles_kernel<false, const A*, A, A, Op>), dim3((unsigned)count[k]), dim3(gk::BLOCK), 0,
+                       (hipStream_t)stream, (const A*)level[k - 1], level[k - 1], count[k - 1], op, init,
+                       (const A*)level[k]);
+    throw_on_error(launch_status(), "scan: kernel launch");
+  }
   hipLaunchKernelGGL((gk::scan_tiles_kernel<EXCLUSIVE, View, A, U, Op>), dim3((unsigned)tiles), dim3(gk::BLOCK), 0,
                      (hipStream_t)stream, thrust::detail::device_view(first), thrust::detail::raw(result), n, op, init,
                      (const A*)tile_total);

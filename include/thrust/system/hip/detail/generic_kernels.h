@@ -7,13 +7,15 @@
 //           a tree over the lanes through LDS), a last workgroup folds the chunk results
 //           into init.  The operator must be associative and commutative, as the
 //           reference requires of reduce.
-//   scan    three steps: the fold of every 2048-element tile; an in-order scan of the tile
-//           results by one workgroup; every tile scanned again with what precedes it.
+//   scan    three steps: the fold of every tile (256 lanes, about 64 bytes each); an in-order scan of the tile
+//           results (by one workgroup when they are few, else by the same three steps one
+//           level up); every tile scanned again with what precedes it.
 //           Only associativity is used: operands always meet in input order.
 //
 // There is no identity for an arbitrary operator, so partial results carry a "holds a
 // value" flag where a lane or tile may be empty.  HBM traffic: reduce reads the range
-// once; the scans read it twice and write it once.
+// once; the scans read it twice and write it once, with consecutive lanes on consecutive
+// elements (the lanes' own order is made in LDS).
 #pragma once
 #if !defined(__HIPCC__)
 #error "thrust/system/hip/detail/generic_kernels.h is HIP code: compile this translation unit with hipcc"
@@ -96,49 +98,118 @@ __global__ __launch_bounds__(BLOCK) void reduce_final_kernel(const T* partials, 
   if (threadIdx.x == 0) *result = any ? op(init, total) : init;
 }
 
-// Inclusive scan of the lanes' values in lane order (Hillis-Steele through LDS).  Lanes
-// without a value take part as "nothing": incl_has tells whether anything precedes or sits
-// in the lane.  Returns the inclusive value.
+// The scans' tile: every lane owns ITEMS consecutive elements, about 64 bytes of them.  A tile
+// is loaded and stored with consecutive lanes on consecutive elements and turned into the
+// lanes' order through LDS; one spare slot after every ITEMS keeps the lanes, which walk
+// their own elements, on different banks.
+template <typename T>
+struct scan_shape {
+  static constexpr int WANTED = 64 / (int)sizeof(T);
+  static constexpr int ITEMS = WANTED < 1 ? 1 : (WANTED > 16 ? 16 : WANTED);
+  static constexpr int TILE = BLOCK * ITEMS;
+  static constexpr int SLOTS = TILE + BLOCK;
+  __host__ __device__ static constexpr unsigned slot(unsigned e) { return e + e / ITEMS; }
+};
+constexpr int WAVE_LANES = 64;
+constexpr int WAVES = BLOCK / WAVE_LANES;
+
+// LDS executes the instructions of one wave in order, so lanes of a wave exchange values
+// through it without a barrier; the compiler only has to keep the accesses where they are.
+__device__ __forceinline__ void wave_fence() { asm volatile("" ::: "memory"); }
+
+// Inclusive scan of the lanes' values in lane order: Hillis-Steele inside every wave through
+// the wave's own part of s_val / s_has, then the totals of the waves before.  Lanes without a
+// value take part as "nothing": incl_has tells whether anything precedes or sits in the lane.
+// One barrier inside; s_wave / s_wave_has hold WAVES entries.  Returns the inclusive value.
 template <typename T, typename Op>
-__device__ __forceinline__ T block_inclusive(T value, bool has, Op& op, T* s_val, unsigned char* s_has, bool& incl_has) {
-  const unsigned tid = threadIdx.x;
+__device__ __forceinline__ T block_inclusive(T value, bool has, Op& op, T* s_val, unsigned char* s_has, T* s_wave,
+                                             unsigned char* s_wave_has, bool& incl_has) {
+  const unsigned tid = threadIdx.x, lane = tid % WAVE_LANES, wave = tid / WAVE_LANES;
   T v = value;
   bool h = has;
-  for (unsigned step = 1; step < BLOCK; step <<= 1) {
+  for (unsigned step = 1; step < WAVE_LANES; step <<= 1) {
     s_val[tid] = v;
     s_has[tid] = h ? 1 : 0;
-    __syncthreads();
-    if (tid >= step && s_has[tid - step]) {
-      v = h ? op(s_val[tid - step], v) : s_val[tid - step];
+    wave_fence();
+    if (lane >= step && s_has[tid - step]) {
+      const T left = s_val[tid - step];
+      v = h ? op(left, v) : left;
       h = true;
     }
-    __syncthreads();
+    wave_fence();
+  }
+  if (lane == WAVE_LANES - 1) {
+    s_wave[wave] = v;
+    s_wave_has[wave] = h ? 1 : 0;
+  }
+  __syncthreads();
+  T before = T();
+  bool has_before = false;
+  for (unsigned w = 0; w < wave; ++w) {
+    if (s_wave_has[w]) {
+      before = has_before ? op(before, s_wave[w]) : s_wave[w];
+      has_before = true;
+    }
+  }
+  if (has_before) {
+    v = h ? op(before, v) : before;
+    h = true;
   }
   incl_has = h;
   return v;
 }
 
+// The tile's elements into s_tile, consecutive lanes on consecutive elements.
+template <typename T, typename View>
+__device__ __forceinline__ void load_tile(View first, uint64_t tile_base, unsigned valid, T* s_tile) {
+  typedef scan_shape<T> S;
+  T in[S::ITEMS];
+#pragma unroll
+  for (int q = 0; q < S::ITEMS; ++q) {
+    const unsigned e = (unsigned)q * BLOCK + threadIdx.x;
+    if (e < valid) in[q] = (T)first[tile_base + e];
+  }
+#pragma unroll
+  for (int q = 0; q < S::ITEMS; ++q) {
+    const unsigned e = (unsigned)q * BLOCK + threadIdx.x;
+    if (e < valid) s_tile[S::slot(e)] = in[q];
+  }
+}
+
+#define THRUST_AMD_SCAN_SHARED(T)                                                                      \
+  typedef scan_shape<T> S;                                                                             \
+  /* raw bytes: T may have a constructor, which shared arrays cannot run */                           \
+  __shared__ __attribute__((aligned(16))) unsigned char s_tile_raw[(size_t)S::SLOTS * sizeof(T)];      \
+  __shared__ __attribute__((aligned(16))) unsigned char s_val_raw[BLOCK * sizeof(T)];                  \
+  __shared__ __attribute__((aligned(16))) unsigned char s_wave_raw[WAVES * sizeof(T)];                 \
+  __shared__ unsigned char s_has[BLOCK];                                                               \
+  __shared__ unsigned char s_wave_has[WAVES];                                                          \
+  T* s_tile = reinterpret_cast<T*>(s_tile_raw);                                                        \
+  T* s_val = reinterpret_cast<T*>(s_val_raw);                                                          \
+  T* s_wave = reinterpret_cast<T*>(s_wave_raw);
+
 // Step 1 of the scan: tile_total[t] = fold of tile t in input order (every tile holds an element).
 template <typename View, typename T, typename Op>
 __global__ __launch_bounds__(BLOCK) void scan_tile_totals_kernel(View first, uint64_t n, Op op, T* tile_total) {
-  // raw bytes: T may have a constructor, which shared arrays cannot run
-  __shared__ __attribute__((aligned(16))) unsigned char s_val_raw[BLOCK * sizeof(T)];
-  T* s_val = reinterpret_cast<T*>(s_val_raw);
-  __shared__ unsigned char s_has[BLOCK];
-  const uint64_t base = (uint64_t)blockIdx.x * TILE + (uint64_t)threadIdx.x * ITEMS;
+  THRUST_AMD_SCAN_SHARED(T)
+  const uint64_t tile_base = (uint64_t)blockIdx.x * S::TILE;
+  const unsigned valid = (unsigned)((n - tile_base < (uint64_t)S::TILE) ? (n - tile_base) : (uint64_t)S::TILE);
+  load_tile<T>(first, tile_base, valid, s_tile);
+  __syncthreads();
   T acc = T();
   bool has = false;
 #pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
-    if (base + i < n) {
-      const T x = (T)first[base + i];
+  for (int i = 0; i < S::ITEMS; ++i) {
+    const unsigned e = threadIdx.x * S::ITEMS + i;
+    if (e < valid) {
+      const T x = s_tile[S::slot(e)];
       if (has) acc = op(acc, x);
       else { acc = x; has = true; }
     }
   }
-  bool any;
-  const T total = block_fold(acc, has, op, s_val, s_has, any);
-  if (threadIdx.x == 0) tile_total[blockIdx.x] = total;
+  bool incl_has;
+  const T incl = block_inclusive(acc, has, op, s_val, s_has, s_wave, s_wave_has, incl_has);
+  if (threadIdx.x == BLOCK - 1) tile_total[blockIdx.x] = incl;  // the last lane's value covers the tile
 }
 
 // Step 2: tile_total[t] becomes the fold of tiles 0 .. t (inclusive), in place, by one workgroup:
@@ -147,8 +218,11 @@ template <typename T, typename Op>
 __global__ __launch_bounds__(BLOCK) void scan_tile_prefix_kernel(T* tile_total, uint32_t tiles, Op op) {
   // raw bytes: T may have a constructor, which shared arrays cannot run
   __shared__ __attribute__((aligned(16))) unsigned char s_val_raw[BLOCK * sizeof(T)];
+  __shared__ __attribute__((aligned(16))) unsigned char s_wave_raw[WAVES * sizeof(T)];
   T* s_val = reinterpret_cast<T*>(s_val_raw);
+  T* s_wave = reinterpret_cast<T*>(s_wave_raw);
   __shared__ unsigned char s_has[BLOCK];
+  __shared__ unsigned char s_wave_has[WAVES];
   const uint32_t per = (tiles + BLOCK - 1) / BLOCK;
   const uint32_t begin = threadIdx.x * per;
   const uint32_t end = (begin + per < tiles) ? begin + per : tiles;
@@ -159,7 +233,7 @@ __global__ __launch_bounds__(BLOCK) void scan_tile_prefix_kernel(T* tile_total, 
     else { acc = tile_total[i]; has = true; }
   }
   bool incl_has;
-  const T incl = block_inclusive(acc, has, op, s_val, s_has, incl_has);
+  const T incl = block_inclusive(acc, has, op, s_val, s_has, s_wave, s_wave_has, incl_has);
   // what precedes this lane's piece: the previous lane's inclusive value
   s_val[threadIdx.x] = incl;
   s_has[threadIdx.x] = incl_has ? 1 : 0;
@@ -182,28 +256,30 @@ __global__ __launch_bounds__(BLOCK) void scan_tile_prefix_kernel(T* tile_total, 
 // Step 3: the tile scanned in input order on top of what precedes it.
 //   inclusive:  out[i] = x0 + ... + xi                    (init is not used)
 //   exclusive:  out[i] = init + x0 + ... + x(i-1)
+// out may be the input itself: a tile is read completely before any of it is written.
 template <bool EXCLUSIVE, typename View, typename T, typename U, typename Op>
 __global__ __launch_bounds__(BLOCK) void scan_tiles_kernel(View first, U* out, uint64_t n, Op op, T init,
                                                            const T* tile_prefix) {
-  // raw bytes: T may have a constructor, which shared arrays cannot run
-  __shared__ __attribute__((aligned(16))) unsigned char s_val_raw[BLOCK * sizeof(T)];
-  T* s_val = reinterpret_cast<T*>(s_val_raw);
-  __shared__ unsigned char s_has[BLOCK];
-  const uint64_t base = (uint64_t)blockIdx.x * TILE + (uint64_t)threadIdx.x * ITEMS;
-  T x[ITEMS];
+  THRUST_AMD_SCAN_SHARED(T)
+  const uint64_t tile_base = (uint64_t)blockIdx.x * S::TILE;
+  const unsigned valid = (unsigned)((n - tile_base < (uint64_t)S::TILE) ? (n - tile_base) : (uint64_t)S::TILE);
+  load_tile<T>(first, tile_base, valid, s_tile);
+  __syncthreads();
+  const unsigned mine = threadIdx.x * S::ITEMS;
+  T x[S::ITEMS];
   T acc = T();
   bool has = false;
 #pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
-    if (base + i < n) {
-      x[i] = (T)first[base + i];
+  for (int i = 0; i < S::ITEMS; ++i) {
+    if (mine + i < valid) {
+      x[i] = s_tile[S::slot(mine + i)];
       if (has) acc = op(acc, x[i]);
       else { acc = x[i]; has = true; }
     }
   }
   bool incl_has;
-  const T incl = block_inclusive(acc, has, op, s_val, s_has, incl_has);
-  s_val[threadIdx.x] = incl;
+  const T incl = block_inclusive(acc, has, op, s_val, s_has, s_wave, s_wave_has, incl_has);
+  s_val[threadIdx.x] = incl;  // every wave's scan is behind the barrier inside block_inclusive
   s_has[threadIdx.x] = incl_has ? 1 : 0;
   __syncthreads();
   // carry = everything before this lane's first element: init (exclusive form), the tiles
@@ -224,20 +300,28 @@ __global__ __launch_bounds__(BLOCK) void scan_tiles_kernel(View first, U* out, u
     carry = has_carry ? op(carry, before) : before;
     has_carry = true;
   }
+  // results go back to the lane's own slots, then out with consecutive lanes on consecutive elements
 #pragma unroll
-  for (int i = 0; i < ITEMS; ++i) {
-    if (base + i < n) {
+  for (int i = 0; i < S::ITEMS; ++i) {
+    if (mine + i < valid) {
       if (EXCLUSIVE) {
-        out[base + i] = (U)carry;  // has_carry is always true here
+        s_tile[S::slot(mine + i)] = carry;  // has_carry is always true here
         carry = op(carry, x[i]);
       } else {
         carry = has_carry ? op(carry, x[i]) : x[i];
         has_carry = true;
-        out[base + i] = (U)carry;
+        s_tile[S::slot(mine + i)] = carry;
       }
     }
   }
+  __syncthreads();
+#pragma unroll
+  for (int q = 0; q < S::ITEMS; ++q) {
+    const unsigned e = (unsigned)q * BLOCK + threadIdx.x;
+    if (e < valid) out[tile_base + e] = (U)s_tile[S::slot(e)];
+  }
 }
+#undef THRUST_AMD_SCAN_SHARED
 
 }  // namespace generic
 }  // namespace hip
