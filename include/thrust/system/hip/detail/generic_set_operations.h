@@ -14,7 +14,8 @@
 //   B_r  sits at (own index) + (elements of A not after x); it has a partner when the
 //        element r + 1 places before A's first "after x" is equivalent to x
 // One kernel, instantiated for the comparator, writes keys (and values) to their merged
-// positions with a keep byte each; the library's compaction kernel, with those bytes as
+// positions with a keep byte each (a workgroup takes a chunk of one range, whose ends bound
+// the chunk's searches in the other range); the library's compaction kernel, with those bytes as
 // its stencil, writes the result.  Keys and values are moved as items of 1, 2, 4 or 8 bytes.
 #pragma once
 #if !defined(__HIPCC__)
@@ -63,38 +64,49 @@ __device__ __forceinline__ uint64_t set_rank_in_run(const K* p, uint64_t i, cons
 }
 
 // a = both, b = both + na.  merged[p], merged_values[p], keep[p] for the merged position p of
-// every element of the two ranges.
+// every element of the two ranges.  A workgroup takes SET_CHUNK consecutive elements of one
+// range; the places of the chunk's first and last element in the other range bound every
+// search of the chunk there, so only two searches per workgroup run over the whole range.
+constexpr int SET_CHUNK = ELEMENTWISE_BLOCK * 8;
 template <typename K, typename V, bool HAS_VALUES, typename Comp>
 __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void set_place_kernel(const K* both, const V* both_values, uint64_t na,
-                                                                      uint64_t nb, int op, Comp comp, K* merged,
-                                                                      V* merged_values, unsigned char* keep) {
+                                                                      uint64_t nb, uint64_t chunks_a, int op, Comp comp,
+                                                                      K* merged, V* merged_values, unsigned char* keep) {
+  __shared__ uint64_t s_bound[2];
   const K* a = both;
   const K* b = both + na;
-  const uint64_t n = na + nb;
-  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   const bool a_alone = op != THRUST_AMD_SET_INTERSECTION;                                  // A without partner
   const bool a_paired = op == THRUST_AMD_SET_INTERSECTION || op == THRUST_AMD_SET_UNION;  // A with partner
   const bool b_alone = op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE || op == THRUST_AMD_SET_UNION;
-  for (uint64_t e = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; e < n; e += stride) {
-    const K x = both[e];
+  const bool from_a = blockIdx.x < chunks_a;
+  const K* own = from_a ? a : b;
+  const K* other = from_a ? b : a;
+  const uint64_t n_own = from_a ? na : nb, n_other = from_a ? nb : na;
+  const uint64_t begin = (from_a ? (uint64_t)blockIdx.x : (uint64_t)blockIdx.x - chunks_a) * SET_CHUNK;
+  const uint64_t end = begin + SET_CHUNK < n_own ? begin + SET_CHUNK : n_own;
+  // elements of the other range before the chunk's first key / not after its last key
+  if (threadIdx.x == 0) s_bound[0] = set_lower_bound(other, (uint64_t)0, n_other, own[begin], comp);
+  if (threadIdx.x == 64) s_bound[1] = set_upper_bound(other, (uint64_t)0, n_other, own[end - 1], comp);
+  __syncthreads();
+  const uint64_t lo = s_bound[0], hi = s_bound[1];
+  for (uint64_t i = begin + threadIdx.x; i < end; i += ELEMENTWISE_BLOCK) {
+    const K x = own[i];
+    const uint64_t r = set_rank_in_run(own, i, x, comp);
     uint64_t at;
     bool kept;
-    if (e < na) {
-      const uint64_t before = set_lower_bound(b, (uint64_t)0, nb, x, comp);
-      const uint64_t r = set_rank_in_run(a, e, x, comp);
+    if (from_a) {
+      const uint64_t before = set_lower_bound(b, lo, hi, x, comp);
       const bool partner = before + r < nb && !comp(x, b[before + r]);
-      at = e + before;
+      at = i + before;
       kept = partner ? a_paired : a_alone;
     } else {
-      const uint64_t j = e - na;
-      const uint64_t upto = set_upper_bound(a, (uint64_t)0, na, x, comp);
-      const uint64_t r = set_rank_in_run(b, j, x, comp);
+      const uint64_t upto = set_upper_bound(a, lo, hi, x, comp);
       const bool partner = r < upto && !comp(a[upto - 1 - r], x);
-      at = j + upto;
+      at = i + upto;
       kept = b_alone && !partner;
     }
     merged[at] = x;
-    if (HAS_VALUES) merged_values[at] = both_values[e];
+    if (HAS_VALUES) merged_values[at] = both_values[(from_a ? 0 : na) + i];
     keep[at] = kept ? 1 : 0;
   }
 }
@@ -126,16 +138,18 @@ uint64_t set_operation_generic(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2
   unsigned char* keep = reinterpret_cast<unsigned char*>(base + 2 * (key_bytes + val_bytes));
   materialize(stream, kf1, both, na);
   materialize(stream, kf2, both + na, nb);
+  const uint64_t chunks_a = (na + SET_CHUNK - 1) / SET_CHUNK, chunks_b = (nb + SET_CHUNK - 1) / SET_CHUNK;
+  if (chunks_a + chunks_b > 0x7fffffffull) throw_on_error(1, "set operation: ranges too long");
   if (has_values) {
     materialize(stream, vf1, both_values, na);
     if (keeps_second) materialize(stream, vf2, both_values + na, nb);
-    hipLaunchKernelGGL((set_place_kernel<K, V, true, Comp>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
-                       (hipStream_t)stream, (const K*)both, (const V*)both_values, na, nb, (int)OP, comp, merged,
-                       merged_values, keep);
+    hipLaunchKernelGGL((set_place_kernel<K, V, true, Comp>), dim3((unsigned)(chunks_a + chunks_b)),
+                       dim3(ELEMENTWISE_BLOCK), 0, (hipStream_t)stream, (const K*)both, (const V*)both_values, na, nb,
+                       chunks_a, (int)OP, comp, merged, merged_values, keep);
   } else {
-    hipLaunchKernelGGL((set_place_kernel<K, V, false, Comp>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
-                       (hipStream_t)stream, (const K*)both, (const V*)nullptr, na, nb, (int)OP, comp, merged,
-                       (V*)nullptr, keep);
+    hipLaunchKernelGGL((set_place_kernel<K, V, false, Comp>), dim3((unsigned)(chunks_a + chunks_b)),
+                       dim3(ELEMENTWISE_BLOCK), 0, (hipStream_t)stream, (const K*)both, (const V*)nullptr, na, nb,
+                       chunks_a, (int)OP, comp, merged, (V*)nullptr, keep);
   }
   throw_on_error(launch_status(), "set operation: kernel launch");
   const uint64_t cnt = select_by_flags(stream, temp_source_of(exec), merged, keep, thrust::detail::raw(ko), n, sizeof(K),
