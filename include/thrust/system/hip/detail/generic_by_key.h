@@ -8,7 +8,8 @@
 //               heads, the values at the heads (unique_by_key) or at the tails (reduce_by_key)
 //   sums        reduce_by_key scans (head, value) pairs with the segmented form of the operator
 //               through the generic in-order scan, exactly the reference's formulation
-//               (thrust/system/detail/generic/reduce_by_key.inl:50-136); the value at a run's
+//               (thrust/system/detail/generic/reduce_by_key.inl:50-136); the pairs are made as
+//               the scan reads them and only the values are written; the value at a run's
 //               tail is the run's sum
 //
 // Keys and values are moved by the selection kernel as items of 1, 2, 4 or 8 bytes.
@@ -17,6 +18,7 @@
 #error "thrust/system/hip/detail/generic_by_key.h is HIP code: compile this translation unit with hipcc"
 #endif
 #include <thrust/copy.h>
+#include <thrust/iterator/counting_iterator.h>
 #include <thrust/iterator/transform_iterator.h>
 #include <thrust/pair.h>
 #include <thrust/scan.h>
@@ -41,6 +43,20 @@ template <typename V>
 struct seg_pair {
   V value;
   unsigned char head;
+  // a scan over pairs may write the values alone
+  __host__ __device__ explicit operator V() const { return value; }
+};
+// element i of the (head, value) pairs of a segmented scan, made as it is read
+template <typename ViewV, typename V>
+struct seg_pair_at {
+  ViewV values;
+  const unsigned char* head;
+  __host__ __device__ seg_pair<V> operator()(uint64_t i) const {
+    seg_pair<V> p;
+    p.value = (V)values[i];
+    p.head = head[i];
+    return p;
+  }
 };
 template <typename V, typename Op>
 struct seg_op {  // the operator of a segmented scan: a head on the right starts over
@@ -148,20 +164,18 @@ pair<KOut, VOut> reduce_by_key_generic(execution_policy<D>& exec, KIn kf, KIn kl
   unsigned char* tail = head + n;
   launch_run_flags(exec, keys.ptr(), n, pred, head, tail);
 
+  // the running sums of the runs: the generic in-order scan reads (head, value) pairs made on
+  // the fly and writes the values alone
   typedef seg_pair<V> P;
-  temp_storage pair_store(stream, temp_source_of(exec));
-  pair_store.ensure((std::size_t)n * sizeof(P));
-  P* pairs = static_cast<P*>(pair_store.ptr());
   typedef typename thrust::detail::device_view_of<VIn>::type ViewV;
-  hipLaunchKernelGGL((seg_pairs_kernel<ViewV, V>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
-                     (hipStream_t)stream, thrust::detail::device_view(vf), (const unsigned char*)head, n, pairs);
-  throw_on_error(launch_status(), "reduce_by_key: kernel launch");
+  temp_storage sum_store(stream, temp_source_of(exec));
+  sum_store.ensure((std::size_t)n * sizeof(V));
+  V* sums = static_cast<V*>(sum_store.ptr());
+  const seg_pair_at<ViewV, V> pair_at = {thrust::detail::device_view(vf), head};
   const seg_op<V, Op> sop = {op};
-  scan_generic<false, P>(exec, pairs, pairs + n, pairs, P(), sop);  // in place, in input order
-
-  device_input<thrust::transform_iterator<pair_value<V>, const P*> > sums(
-      stream, temp_source_of(exec), thrust::make_transform_iterator((const P*)pairs, pair_value<V>()), n);
-  const uint64_t runs = select_by_flags(stream, temp_source_of(exec), sums.ptr(), tail, thrust::detail::raw(vo), n,
+  scan_generic<false, P>(exec, thrust::make_transform_iterator(thrust::counting_iterator<uint64_t>(0), pair_at),
+                         thrust::make_transform_iterator(thrust::counting_iterator<uint64_t>(n), pair_at), sums, P(), sop);
+  const uint64_t runs = select_by_flags(stream, temp_source_of(exec), sums, tail, thrust::detail::raw(vo), n,
                                         sizeof(V), "reduce_by_key failed");
   (void)select_by_flags(stream, temp_source_of(exec), keys.ptr(), head, thrust::detail::raw(ko), n, sizeof(K),
                         "reduce_by_key failed");
