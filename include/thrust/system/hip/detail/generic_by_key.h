@@ -211,10 +211,26 @@ Out scan_by_key_generic(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out r
   unsigned char* head = static_cast<unsigned char*>(flags.ptr());
   launch_run_flags(exec, kf, n, pred, head, nullptr);
   typedef seg_pair<A> P;
+  typedef typename thrust::detail::device_view_of<VIt>::type ViewV;
+  const seg_op<A, Op> sop = {op};
+  constexpr bool writes_values = !EXCLUSIVE &&
+                                 (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value) &&
+                                 std::is_same<typename iterator_value<Out>::type, A>::value;
+  if constexpr (writes_values) {
+    // inclusive: the pairs are made as the scan reads them and the values alone are written.
+    // The output may be the input: a tile is read completely before any of it is written,
+    // and no tile reads another tile's elements.
+    const seg_pair_at<ViewV, A> pair_at = {thrust::detail::device_view(vf), head};
+    scan_generic<false, P>(exec, thrust::make_transform_iterator(thrust::counting_iterator<uint64_t>(0), pair_at),
+                           thrust::make_transform_iterator(thrust::counting_iterator<uint64_t>(n), pair_at),
+                           thrust::detail::raw(result), P(), sop);
+    return result + n;
+  }
+  // exclusive: element i takes the value of element i - 1, which may lie in another tile, so
+  // the pairs are written out first
   temp_storage pair_store(stream, temp_source_of(exec));
   pair_store.ensure((std::size_t)n * sizeof(P));
   P* pairs = static_cast<P*>(pair_store.ptr());
-  typedef typename thrust::detail::device_view_of<VIt>::type ViewV;
   if (EXCLUSIVE)
     hipLaunchKernelGGL((shifted_seg_pairs_kernel<ViewV, A>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
                        (hipStream_t)stream, thrust::detail::device_view(vf), (const unsigned char*)head, n, init, pairs);
@@ -222,7 +238,6 @@ Out scan_by_key_generic(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out r
     hipLaunchKernelGGL((seg_pairs_kernel<ViewV, A>), dim3(elementwise_grid(n)), dim3(ELEMENTWISE_BLOCK), 0,
                        (hipStream_t)stream, thrust::detail::device_view(vf), (const unsigned char*)head, n, pairs);
   throw_on_error(launch_status(), "scan_by_key: kernel launch");
-  const seg_op<A, Op> sop = {op};
   scan_generic<false, P>(exec, pairs, pairs + n, pairs, P(), sop);
   // the values of the scanned pairs are the result (the pairs were built from a copy of the
   // input, so the output may be the input)

@@ -250,6 +250,11 @@ static void TestUserPredicatesByKey() {
       thrust::exclusive_scan_by_key(hk.begin(), hk.end(), hin.begin(), hin.begin(), 3u, thrust::equal_to<int>(), bit_xor_op());
       thrust::exclusive_scan_by_key(dk.begin(), dk.end(), din.begin(), din.begin(), 3u, thrust::equal_to<int>(), bit_xor_op());
       ASSERT_TRUE(same(to_host(din), hin));
+      hin = hvv;
+      din = dv;
+      thrust::inclusive_scan_by_key(hk.begin(), hk.end(), hin.begin(), hin.begin(), same_tens(), bit_xor_op());
+      thrust::inclusive_scan_by_key(dk.begin(), dk.end(), din.begin(), din.begin(), same_tens(), bit_xor_op());
+      ASSERT_TRUE(same(to_host(din), hin));
     }
     // unique_copy and unique_by_key_copy
     hko.resize(n); dko.resize(n); hvo.resize(n); dvo.resize(n);
