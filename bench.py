@@ -135,8 +135,30 @@ def cpu_baseline():
     x = datagen.c1_int32(1 << 26)
     t0 = time.perf_counter(); impl.reduce(x); t_red = time.perf_counter() - t0
     t0 = time.perf_counter(); impl.inclusive_scan(x); t_scan = time.perf_counter() - t0
+    # the other rows of the path on 2^24-element samples of their configurations (GB/s of the
+    # same algorithmic bytes the GPU figures use; one call each after building the inputs)
+    m = 1 << 24
+
+    def gbs(nbytes, fn):
+        t0 = time.perf_counter()
+        fn()
+        return round(nbytes / (time.perf_counter() - t0) / 1e9, 3)
+    ck, cv = datagen.c4_segments(m, 8)
+    runs = int(ck[-1]) + 1
+    f = datagen.c5_float32(m)
+    (ka, va), (kb, vb) = datagen.c5_merge_inputs(m // 2)
+    rows = {
+        "reduce_by_key_GBps": gbs(8.0 * m + 8.0 * runs, lambda: impl.reduce_by_key(ck, cv)),
+        "unique_by_key_GBps": gbs(8.0 * m + 8.0 * runs, lambda: impl.unique_by_key(ck, cv)),
+        "copy_if_half_GBps": gbs(6.0 * m, lambda: impl.copy_if(f, ocpu.LT, 0.5)),
+        "stable_partition_half_GBps": gbs(8.0 * m, lambda: impl.stable_partition(f.copy(), ocpu.LT, 0.5)),
+        "merge_by_key_GBps": gbs(16.0 * m, lambda: impl.merge_by_key(ka, kb, va, vb)),
+        "inclusive_scan_by_key_GBps": gbs(12.0 * m, lambda: impl.inclusive_scan_by_key(ck, cv)),
+        "set_union_GBps": gbs(8.0 * m, lambda: impl.set_operation(3, ka, kb)),
+    }
     return {
         "value": n / best / 1e9, "unit": "Gkeys/s", "cores": cores, "kind": kind,
+        "rows_2p24": rows,
         "sample": "thrust::sort of 2^26 uint32 (same generator as the GPU run's key space), best of 2, "
                   "timing includes one copy of the input made by the binding",
         "reduce_GBps": 4.0 * x.size / t_red / 1e9, "inclusive_scan_GBps": 8.0 * x.size / t_scan / 1e9,
