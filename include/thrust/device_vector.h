@@ -10,6 +10,8 @@
 // allocator whose allocate(n) yields a device_ptr<T> or a raw device pointer will do, e.g.
 // thrust::mr::allocator<T, Pool> over a pool resource (thrust/mr/pool.h).
 #pragma once
+#include <cstring>
+#include <new>
 #include <cstddef>
 #include <iterator>
 #include <type_traits>
@@ -116,8 +118,21 @@ class device_vector {
   void resize(size_type n, const T& value) {
     if (n > capacity_) reserve(n);
     if (n > size_) {
-      system::hip::detail::throw_on_error(
-          thrust_amd_fill(data_ + size_, n - size_, sizeof(T), &value, nullptr), "device_vector fill");
+      if (sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8) {
+        system::hip::detail::throw_on_error(
+            thrust_amd_fill(data_ + size_, n - size_, sizeof(T), &value, nullptr), "device_vector fill");
+      } else {
+        // the fill kernel moves items of 1, 2, 4 or 8 bytes; wider elements are laid out on
+        // the host, a piece at a time, and copied
+        const size_type piece = (size_type)((std::size_t)(1 << 20) / sizeof(T) + 1);
+        const size_type count = (n - size_) < piece ? (n - size_) : piece;
+        T* staged = static_cast<T*>(::operator new((std::size_t)count * sizeof(T)));
+        for (size_type i = 0; i < count; ++i) std::memcpy(static_cast<void*>(staged + i), &value, sizeof(T));
+        for (size_type done = size_; done < n; done += count)
+          copy_raw(data_ + done, staged, (n - done) < count ? (n - done) : count, THRUST_AMD_H2D);
+        sync();
+        ::operator delete(staged);
+      }
       sync();
     }
     size_ = n;

@@ -107,7 +107,8 @@ struct scan_shape {
   static constexpr int WANTED = 64 / (int)sizeof(T);
   static constexpr int ITEMS = WANTED < 1 ? 1 : (WANTED > 16 ? 16 : WANTED);
   static constexpr int TILE = BLOCK * ITEMS;
-  static constexpr int SLOTS = TILE + BLOCK;
+  // with one element per lane the two orders are the same and nothing is staged
+  static constexpr int SLOTS = ITEMS == 1 ? 1 : TILE + BLOCK;
   __host__ __device__ static constexpr unsigned slot(unsigned e) { return e + e / ITEMS; }
 };
 constexpr int WAVE_LANES = 64;
@@ -163,6 +164,7 @@ __device__ __forceinline__ T block_inclusive(T value, bool has, Op& op, T* s_val
 template <typename T, typename View>
 __device__ __forceinline__ void load_tile(View first, uint64_t tile_base, unsigned valid, T* s_tile) {
   typedef scan_shape<T> S;
+  if (S::ITEMS == 1) return;  // every lane reads its one element itself
   T in[S::ITEMS];
 #pragma unroll
   for (int q = 0; q < S::ITEMS; ++q) {
@@ -202,7 +204,7 @@ __global__ __launch_bounds__(BLOCK) void scan_tile_totals_kernel(View first, uin
   for (int i = 0; i < S::ITEMS; ++i) {
     const unsigned e = threadIdx.x * S::ITEMS + i;
     if (e < valid) {
-      const T x = s_tile[S::slot(e)];
+      const T x = S::ITEMS == 1 ? (T)first[tile_base + e] : s_tile[S::slot(e)];
       if (has) acc = op(acc, x);
       else { acc = x; has = true; }
     }
@@ -272,7 +274,7 @@ __global__ __launch_bounds__(BLOCK) void scan_tiles_kernel(View first, U* out, u
 #pragma unroll
   for (int i = 0; i < S::ITEMS; ++i) {
     if (mine + i < valid) {
-      x[i] = s_tile[S::slot(mine + i)];
+      x[i] = S::ITEMS == 1 ? (T)first[tile_base + mine] : s_tile[S::slot(mine + i)];
       if (has) acc = op(acc, x[i]);
       else { acc = x[i]; has = true; }
     }
@@ -305,15 +307,18 @@ __global__ __launch_bounds__(BLOCK) void scan_tiles_kernel(View first, U* out, u
   for (int i = 0; i < S::ITEMS; ++i) {
     if (mine + i < valid) {
       if (EXCLUSIVE) {
-        s_tile[S::slot(mine + i)] = carry;  // has_carry is always true here
+        if (S::ITEMS == 1) out[tile_base + mine] = (U)carry;
+        else s_tile[S::slot(mine + i)] = carry;  // has_carry is always true here
         carry = op(carry, x[i]);
       } else {
         carry = has_carry ? op(carry, x[i]) : x[i];
         has_carry = true;
-        s_tile[S::slot(mine + i)] = carry;
+        if (S::ITEMS == 1) out[tile_base + mine] = (U)carry;
+        else s_tile[S::slot(mine + i)] = carry;
       }
     }
   }
+  if (S::ITEMS == 1) return;
   __syncthreads();
 #pragma unroll
   for (int q = 0; q < S::ITEMS; ++q) {

@@ -91,6 +91,22 @@ struct widen_square {
   __host__ __device__ long long operator()(int x) const { return (long long)x * x; }
 };
 
+// an element wider than a lane's share of a tile: one element per lane in the scans
+struct Wide {
+  double v[12];
+  __host__ __device__ bool operator==(const Wide& o) const {
+    for (int i = 0; i < 12; ++i)
+      if (v[i] != o.v[i]) return false;
+    return true;
+  }
+};
+struct add_wide {
+  __host__ __device__ Wide operator()(const Wide& a, const Wide& b) const {
+    Wide r;
+    for (int i = 0; i < 12; ++i) r.v[i] = a.v[i] + b.v[i];
+    return r;
+  }
+};
 // user operators for reduce and the scans
 struct Affine {  // x -> a * x + b over unsigned wrap-around; composition is associative, not commutative
   unsigned a, b;
@@ -180,6 +196,25 @@ static void TestUserOperators() {
 struct same_tens {  // the key predicate of testing/reduce_by_key.cu:60-112 and unique.cu:125-142
   __host__ __device__ bool operator()(int a, int b) const { return a / 10 == b / 10; }
 };
+
+static void TestWideElements() {
+  g_test = "WideElements";
+  for (size_t n : {(size_t)1, (size_t)255, (size_t)256, (size_t)257, (size_t)5000}) {
+    thrust::host_vector<Wide> h(n);
+    for (size_t i = 0; i < n; ++i)
+      for (int k = 0; k < 12; ++k) h[i].v[k] = (double)((mix(i * 12 + k) % 1000));  // sums of integers: exact
+    thrust::device_vector<Wide> d(h), dout(n);
+    thrust::host_vector<Wide> hout(n);
+    thrust::inclusive_scan(h.begin(), h.end(), hout.begin(), add_wide());
+    thrust::inclusive_scan(d.begin(), d.end(), dout.begin(), add_wide());
+    ASSERT_TRUE(same(to_host(dout), hout));
+    Wide zero;
+    for (int k = 0; k < 12; ++k) zero.v[k] = 1.0;
+    thrust::exclusive_scan(h.begin(), h.end(), hout.begin(), zero, add_wide());
+    thrust::exclusive_scan(d.begin(), d.end(), d.begin(), zero, add_wide());  // in place
+    ASSERT_TRUE(same(to_host(d), hout));
+  }
+}
 
 static void TestUserPredicatesByKey() {
   g_test = "by-key known answers with a user predicate";
@@ -567,6 +602,7 @@ int main() {
   TestReduceWithBigIndexes();
   Differential();
   TestUserOperators();
+  TestWideElements();
   TestUserPredicatesByKey();
   TestZipIterator();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
