@@ -150,18 +150,9 @@ namespace detail {
 // Shared by copy_if and the partition family: runs `entry` (one of the three selection
 // entry points bound by the caller) and returns the number of selected elements.
 // `negate` selects the elements the predicate rejects (remove_if is copy_if of not1(pred),
-// thrust/system/cuda/detail/remove.h:40-66): every comparison code has its complement.
-inline int negated_cmp(int cmp) {
-  switch (cmp) {
-    case THRUST_AMD_LT: return THRUST_AMD_GE;
-    case THRUST_AMD_LE: return THRUST_AMD_GT;
-    case THRUST_AMD_GT: return THRUST_AMD_LE;
-    case THRUST_AMD_GE: return THRUST_AMD_LT;
-    case THRUST_AMD_EQ: return THRUST_AMD_NE;
-    case THRUST_AMD_NE: return THRUST_AMD_EQ;
-    default: return THRUST_AMD_EQ;  // "is non-zero" -> equal to the zero threshold it carries
-  }
-}
+// thrust/system/cuda/detail/remove.h:40-66).  The kernel evaluates the predicate and inverts
+// the result; swapping in the complementary comparison would drop NaNs, which fail both.
+inline int negated_cmp(int cmp) { return cmp ^ THRUST_AMD_CMP_NOT; }
 template <typename Tested, typename Pred, typename Call>
 inline uint64_t run_selection(void* stream, const temp_source& source, const Pred& pred, const char* what, Call call,
                               bool negate = false) {

@@ -89,16 +89,24 @@ struct square<void> {
 
 namespace detail {
 // `x CMP value` as a unary predicate; CMP is a thrust_amd_cmp code (0 LT .. 5 NE).
+#if defined(__GNUC__)
+#pragma GCC diagnostic push
+#pragma GCC diagnostic ignored "-Wsign-compare"  // the expression is the caller's, conversions included
+#endif
 template <int CMP, typename T>
 struct compare_with {
   T value;
-  constexpr bool operator()(const T& x) const {
+  // evaluated on the argument as it is, under the usual arithmetic conversions, as the
+  // reference's placeholder expression `_1 < t` does
+  template <typename A>
+  constexpr bool operator()(const A& x) const {
     return CMP == 0 ? x < value : CMP == 1 ? x <= value : CMP == 2 ? x > value
          : CMP == 3 ? x >= value : CMP == 4 ? x == value : x != value;
   }
-  template <typename A>
-  constexpr bool operator()(const A& x) const { return (*this)(static_cast<T>(x)); }
 };
+#if defined(__GNUC__)
+#pragma GCC diagnostic pop
+#endif
 struct placeholder1 {};
 }  // namespace detail
 

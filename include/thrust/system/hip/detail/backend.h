@@ -8,6 +8,8 @@
 //   - run(): the two-phase size-query / run protocol plus error conversion.
 #pragma once
 #include <cstdint>
+#include <cmath>
+#include <limits>
 #include <type_traits>
 
 #include <thrust/detail/execution_policy.h>
@@ -76,13 +78,86 @@ struct unary_pred {
   static int cmp(const Pred&) { return -1; }
   static T threshold(const Pred&) { return T(); }
 };
+// `x CMP t` with a threshold of type U on elements of type T.  C++ evaluates it after the usual
+// arithmetic conversions; the kernel compares two values of type T.  The two agree in three
+// situations, told apart by the types:
+//   SAME        converting t to T is the very conversion C++ applies (or loses nothing)
+//   MATH_INT    C++ compares the mathematical values of two integers: a threshold inside T's
+//               range is cast, one outside it makes the predicate constant
+//   MATH_FLOAT  integer elements against a floating threshold that every element converts to
+//               exactly: `x < 2.5` is `x < 3`, `x == 2.5` is never true
+// Every other combination (float elements against a double threshold, signed elements
+// converted to unsigned, ...) is not evaluated in the kernel; the caller's predicate is then
+// applied as it stands by a kernel instantiated for it.
 template <int CMP, typename U, typename T>
 struct unary_pred<thrust::detail::compare_with<CMP, U>, T> {
-  // the comparison happens in the tested type, as `x < t` would after the usual
-  // conversion of t when U converts to T without loss for the values in use
-  static const bool supported = std::is_convertible<U, T>::value;
-  static int cmp(const thrust::detail::compare_with<CMP, U>&) { return CMP; }
-  static T threshold(const thrust::detail::compare_with<CMP, U>& p) { return static_cast<T>(p.value); }
+  enum kind_t { NONE, SAME, MATH_INT, MATH_UINT, MATH_FLOAT };
+  template <typename A, typename B, bool = std::is_arithmetic<A>::value && std::is_arithmetic<B>::value>
+  struct classify { static const int value = NONE; };
+  template <typename A, typename B>
+  struct classify<A, B, true> {
+    typedef typename std::common_type<decltype(+A()), decltype(+B())>::type C;  // after promotion
+    static const bool a_f = std::is_floating_point<A>::value, b_f = std::is_floating_point<B>::value;
+    static const int value =
+        a_f ? ((!b_f || sizeof(B) <= sizeof(A)) ? SAME : NONE)
+        : b_f ? (((std::is_same<B, double>::value && sizeof(A) <= 4) || (std::is_same<B, float>::value && sizeof(A) <= 2))
+                     ? MATH_FLOAT : NONE)
+        : std::is_signed<C>::value ? MATH_INT
+        : std::is_unsigned<A>::value ? MATH_UINT
+                                     : NONE;
+  };
+  static const int kind = classify<T, U>::value;
+  static const bool supported = kind != NONE;
+
+  struct resolved { int cmp; T thr; };
+  static resolved constant(bool always) {
+    // always true: x >= lowest; always false: x < lowest
+    return resolved{always ? THRUST_AMD_GE : THRUST_AMD_LT, std::numeric_limits<T>::lowest()};
+  }
+  // x CMP w for x over T's whole range, w a wide integer of type Wide
+  template <typename Wide>
+  static resolved against_integer(int cmp, Wide w) {
+    const Wide lo = (Wide)std::numeric_limits<T>::lowest(), hi = (Wide)std::numeric_limits<T>::max();
+    if (w >= lo && w <= hi) return resolved{cmp, (T)w};
+    const bool above = w > hi;  // every element is below (above) the threshold
+    switch (cmp) {
+      case THRUST_AMD_LT: case THRUST_AMD_LE: return constant(above);
+      case THRUST_AMD_GT: case THRUST_AMD_GE: return constant(!above);
+      case THRUST_AMD_EQ: return constant(false);
+      default: return constant(true);
+    }
+  }
+  static resolved resolve(const thrust::detail::compare_with<CMP, U>& p, std::integral_constant<int, SAME>) {
+    return resolved{CMP, static_cast<T>(p.value)};
+  }
+  static resolved resolve(const thrust::detail::compare_with<CMP, U>& p, std::integral_constant<int, MATH_INT>) {
+    return against_integer<long long>(CMP, (long long)p.value);
+  }
+  static resolved resolve(const thrust::detail::compare_with<CMP, U>& p, std::integral_constant<int, MATH_UINT>) {
+    typedef typename classify<T, U>::C C;  // the threshold wraps to C, as in C++; elements keep their value
+    return against_integer<unsigned long long>(CMP, (unsigned long long)(C)p.value);
+  }
+  static resolved resolve(const thrust::detail::compare_with<CMP, U>& p, std::integral_constant<int, MATH_FLOAT>) {
+    const double v = (double)p.value;
+    if (v != v) return constant(CMP == THRUST_AMD_NE);  // NaN
+    const double fl = std::floor(v), ce = std::ceil(v);
+    const bool whole = fl == v;
+    int cmp = CMP;
+    double w = v;
+    switch (CMP) {
+      case THRUST_AMD_LT: case THRUST_AMD_GE: w = ce; break;
+      case THRUST_AMD_LE: case THRUST_AMD_GT: w = fl; break;
+      default: if (!whole) return constant(CMP == THRUST_AMD_NE); break;
+    }
+    // T has at most 32 bits here: anything beyond +-2^62 is outside its range on that side
+    const long long wide = w >= 4.0e18 ? (1LL << 62) : (w <= -4.0e18 ? -(1LL << 62) : (long long)w);
+    return against_integer<long long>(cmp, wide);
+  }
+  static resolved resolve(const thrust::detail::compare_with<CMP, U>&, std::integral_constant<int, NONE>) {
+    return resolved{-1, T()};
+  }
+  static int cmp(const thrust::detail::compare_with<CMP, U>& p) { return resolve(p, std::integral_constant<int, kind>()).cmp; }
+  static T threshold(const thrust::detail::compare_with<CMP, U>& p) { return resolve(p, std::integral_constant<int, kind>()).thr; }
 };
 template <typename I, typename T>
 struct unary_pred<thrust::identity<I>, T> {

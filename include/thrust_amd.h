@@ -61,7 +61,11 @@ typedef enum thrust_amd_binop {
 } thrust_amd_binop;
 
 /* Unary predicates `x CMP threshold` (threshold has the dtype of the tested array).
- * NONZERO is the reference's default "stencil element converted to bool". */
+ * NONZERO is the reference's default "stencil element converted to bool".  Any code may be
+ * or-ed with THRUST_AMD_CMP_NOT: the predicate is then !(x CMP threshold), the logical
+ * negation that remove_if applies (thrust/system/cuda/detail/remove.h:40-66 wraps the
+ * predicate in not1).  That is not the complementary comparison for floating point: a NaN
+ * fails `x < t` and `x >= t` alike, and passes !(x < t). */
 typedef enum thrust_amd_cmp {
   THRUST_AMD_LT = 0,
   THRUST_AMD_LE = 1,
@@ -70,7 +74,8 @@ typedef enum thrust_amd_cmp {
   THRUST_AMD_EQ = 4,
   THRUST_AMD_NE = 5,
   THRUST_AMD_NONZERO = 6,
-  THRUST_AMD_CMP_COUNT = 7
+  THRUST_AMD_CMP_COUNT = 7,
+  THRUST_AMD_CMP_NOT = 0x100
 } thrust_amd_cmp;
 
 /* Unary transforms applied to every input element by the transform_* entry points: the
@@ -169,10 +174,12 @@ int thrust_amd_fill(void* dst, uint64_t n, size_t elem_bytes, const void* value,
 /* Temporary-storage arena: a size-bucketed cache of device blocks, so that the blocking
  * thrust:: front end performs no hipMalloc in steady state.  `acquire` returns a block
  * of at least `bytes`, 256-byte aligned; `release` returns it to the cache once the
- * work enqueued so far on `stream` may be assumed ordered before its next use (blocks
- * are reused in stream order on the stream they were released on; a block released on
- * one stream is handed to another stream only after that stream was synchronised).
- * `trim` frees every cached block.  Replaces temporary_array<uint8_t,Derived> over
+ * work enqueued so far on `stream` may be assumed ordered before its next use: `release`
+ * records an event on `stream`, and the next `acquire` of that block makes its own stream
+ * wait for the event on the device (the host does not block).  The arena keeps the event,
+ * never the stream, so a stream may be destroyed while blocks released on it are cached.
+ * Blocks are cached per device (the device current at `acquire`); the cache itself is one
+ * per process and thread-safe.  `trim` frees every cached block.  Replaces temporary_array<uint8_t,Derived> over
  * get_temporary_buffer (thrust/detail/temporary_array.inl:62-140,
  * thrust/system/detail/generic/temporary_buffer.inl:33-47). */
 int thrust_amd_temp_acquire(void** ptr, size_t bytes, void* stream);

@@ -41,6 +41,7 @@
 #include <cstdio>
 #include <cstring>
 #include <functional>
+#include <limits>
 #include <string>
 #include <vector>
 
@@ -333,6 +334,126 @@ static void TestRemoveSimple() {  // testing/remove.cu:28-47,100-122,184-203,256
   thrust::host_vector<int> hst = hv<int>({0, 1, 0, 0, 1});
   h.resize(thrust::remove_if(h.begin(), h.end(), hst.begin(), thrust::identity<int>()) - h.begin());
   ASSERT_EQUAL_VEC(h, kept);
+}
+
+// Placeholder thresholds of another type than the elements: the device must select what C++
+// selects under the usual arithmetic conversions (the host system evaluates the expression
+// as written).  Covers a fractional threshold on integers, thresholds outside the element
+// type's range, a negative threshold on unsigned elements and an integer threshold on floats.
+template <typename T, typename Pred>
+static void check_mixed_predicate(const thrust::host_vector<T>& h, Pred pred) {
+  thrust::device_vector<T> d = h;
+  thrust::host_vector<T> want(h.size());
+  want.resize(thrust::copy_if(h.begin(), h.end(), want.begin(), pred) - want.begin());
+  thrust::device_vector<T> got(h.size());
+  got.resize(thrust::copy_if(d.begin(), d.end(), got.begin(), pred) - got.begin());
+  ASSERT_EQUAL_VEC(to_host(got), want);
+  ASSERT_TRUE((size_t)thrust::count_if(d.begin(), d.end(), pred) == want.size());
+  thrust::host_vector<T> hr = h;
+  hr.resize(thrust::remove_if(hr.begin(), hr.end(), pred) - hr.begin());
+  thrust::device_vector<T> dr = h;
+  dr.resize(thrust::remove_if(dr.begin(), dr.end(), pred) - dr.begin());
+  ASSERT_EQUAL_VEC(to_host(dr), hr);
+}
+static void TestMixedTypePlaceholders() {
+  g_test = "MixedTypePlaceholders";
+  using namespace thrust::placeholders;
+  const size_t n = 4099;
+  {
+    thrust::host_vector<int> h(n);
+    for (size_t i = 0; i < n; ++i) h[i] = (int)(mix(i) % 11) - 5;
+    check_mixed_predicate(h, _1 < 2.5);
+    check_mixed_predicate(h, _1 <= 2.5);
+    check_mixed_predicate(h, _1 > -2.5);
+    check_mixed_predicate(h, _1 >= -0.5);
+    check_mixed_predicate(h, _1 == 2.5);
+    check_mixed_predicate(h, _1 != 2.5);
+    check_mixed_predicate(h, _1 == 2.0);
+    check_mixed_predicate(h, _1 < 1e30);
+    check_mixed_predicate(h, _1 > 1e30);
+    check_mixed_predicate(h, _1 < 3ll);
+    check_mixed_predicate(h, _1 < (1ll << 40));
+    check_mixed_predicate(h, _1 >= -(1ll << 40));
+    check_mixed_predicate(h, _1 != (1ll << 40));
+  }
+  {
+    thrust::host_vector<int8_t> h(n);
+    for (size_t i = 0; i < n; ++i) h[i] = (int8_t)(mix(i) & 0xff);
+    check_mixed_predicate(h, _1 > 300);   // wraps to 44 if the threshold is cast to int8
+    check_mixed_predicate(h, _1 < 300);
+    check_mixed_predicate(h, _1 == 300);
+    check_mixed_predicate(h, _1 >= -200);
+    check_mixed_predicate(h, _1 < 17);
+    check_mixed_predicate(h, _1 < 16.5);
+  }
+  {
+    thrust::host_vector<uint16_t> h(n);
+    for (size_t i = 0; i < n; ++i) h[i] = (uint16_t)(mix(i) & 0xffff);
+    check_mixed_predicate(h, _1 > -1);     // compared as int: always true
+    check_mixed_predicate(h, _1 < 70000);
+    check_mixed_predicate(h, _1 >= 32768);
+  }
+  {
+    thrust::host_vector<uint32_t> h(n);
+    for (size_t i = 0; i < n; ++i) h[i] = (uint32_t)mix(i);
+    check_mixed_predicate(h, _1 < -2);     // compared as unsigned: below 4294967294
+    check_mixed_predicate(h, _1 > 1000);
+    check_mixed_predicate(h, _1 < (1ll << 31));
+  }
+  {
+    thrust::host_vector<float> h(n);
+    for (size_t i = 0; i < n; ++i) h[i] = (float)((double)(mix(i) % 2001) / 250.0 - 4.0);
+    check_mixed_predicate(h, _1 < 2);      // 2.5f < 2 is false: compared as float, not as int
+    check_mixed_predicate(h, _1 == 2);
+    check_mixed_predicate(h, _1 >= -1);
+  }
+  {
+    thrust::host_vector<double> h(n);
+    for (size_t i = 0; i < n; ++i) h[i] = (double)(mix(i) % 2001) / 250.0 - 4.0;
+    check_mixed_predicate(h, _1 < 0.3f);
+    check_mixed_predicate(h, _1 > 1);
+  }
+}
+
+// remove_if keeps what the predicate rejects.  A NaN fails `x < t` and is kept; it also fails
+// `x >= t`, so the complementary comparison would drop it.
+static void TestRemoveIfKeepsNaN() {
+  g_test = "RemoveIfKeepsNaN";
+  using namespace thrust::placeholders;
+  const size_t n = 5000;
+  const float nan = std::numeric_limits<float>::quiet_NaN();
+  thrust::host_vector<float> h(n);
+  size_t nans = 0;
+  for (size_t i = 0; i < n; ++i) {
+    h[i] = (mix(i) % 7 == 0) ? nan : (float)(mix(i) % 1000) / 1000.0f;
+    nans += h[i] != h[i];
+  }
+  auto bits = [](const thrust::host_vector<float>& v) {
+    thrust::host_vector<uint32_t> b(v.size());
+    for (size_t i = 0; i < v.size(); ++i) std::memcpy(&b[i], &v[i], 4);
+    return b;
+  };
+  thrust::host_vector<float> hr = h;
+  hr.resize(thrust::remove_if(hr.begin(), hr.end(), _1 < 0.5f) - hr.begin());
+  thrust::device_vector<float> dr = h;
+  dr.resize(thrust::remove_if(dr.begin(), dr.end(), _1 < 0.5f) - dr.begin());
+  ASSERT_EQUAL_VEC(bits(to_host(dr)), bits(hr));
+  size_t kept_nans = 0;
+  thrust::host_vector<float> back = dr;
+  for (size_t i = 0; i < back.size(); ++i) kept_nans += back[i] != back[i];
+  ASSERT_TRUE(kept_nans == nans && nans > 0);
+  thrust::device_vector<float> d = h, out(n);
+  out.resize(thrust::remove_copy_if(d.begin(), d.end(), out.begin(), _1 >= 0.5f) - out.begin());
+  thrust::host_vector<float> hout(n);
+  hout.resize(thrust::remove_copy_if(h.begin(), h.end(), hout.begin(), _1 >= 0.5f) - hout.begin());
+  ASSERT_EQUAL_VEC(bits(to_host(out)), bits(hout));
+  // partition: the NaNs fail the predicate and go behind the split point, in order
+  thrust::host_vector<float> hp = h;
+  thrust::device_vector<float> dp = h;
+  const size_t hs = thrust::stable_partition(hp.begin(), hp.end(), _1 < 0.5f) - hp.begin();
+  const size_t ds = thrust::stable_partition(dp.begin(), dp.end(), _1 < 0.5f) - dp.begin();
+  ASSERT_TRUE(hs == ds);
+  ASSERT_EQUAL_VEC(bits(to_host(dp)), bits(hp));
 }
 
 static void TestSetOperationsSimple() {
@@ -1075,6 +1196,51 @@ static void TestUniversalVector() {  // testing/universal_memory.cu:25-82: one p
   ASSERT_TRUE(empty.size() == 0 && empty.begin() == empty.end());
 }
 
+// A block released on a stream that is destroyed afterwards must stay usable: the arena keeps
+// an event per block, never the stream.  async::reduce runs on a stream of its own and gives
+// its temporary storage back on that stream; dropping the future destroys the stream; the
+// synchronous reduce of the same size on the null stream then picks that very block up.
+static void TestTempArenaOutlivesStream() {
+  g_test = "TempArenaOutlivesStream";
+  ASSERT_TRUE(thrust_amd_temp_trim() == 0);  // nothing cached: the next block is the only one
+  const size_t n = (1 << 20) + 3;
+  thrust::host_vector<int> h = random_integers<int>(n, 11, 0);
+  thrust::device_vector<int> d = h;
+  long long total = 0;
+  for (size_t i = 0; i < n; ++i) total += h[i];
+  {
+    auto f = thrust::async::reduce(d.begin(), d.end());
+    ASSERT_TRUE(f.get() == (int)total);
+  }  // the future, and with it its stream, is gone here
+  const size_t held = thrust_amd_temp_bytes_held();
+  ASSERT_TRUE(held > 0);
+  int got = 0;
+  bool threw = false;
+  try {
+    got = thrust::reduce(d.begin(), d.end());
+  } catch (...) {
+    threw = true;
+  }
+  ASSERT_TRUE(!threw);
+  ASSERT_TRUE(got == (int)total);
+  ASSERT_TRUE(thrust_amd_temp_bytes_held() == held);  // the cached block was reused, not lost
+  // the same through the C ABI with a user's stream: release, destroy, acquire elsewhere
+  void* s = nullptr;
+  ASSERT_TRUE(thrust_amd_stream_create(&s) == 0);
+  void* blk = nullptr;
+  ASSERT_TRUE(thrust_amd_temp_acquire(&blk, 1 << 16, s) == 0 && blk != nullptr);
+  ASSERT_TRUE(thrust_amd_temp_release(blk, s) == 0);
+  ASSERT_TRUE(thrust_amd_stream_synchronize(s) == 0);
+  ASSERT_TRUE(thrust_amd_stream_destroy(s) == 0);
+  void* again = nullptr;
+  ASSERT_TRUE(thrust_amd_temp_acquire(&again, 1 << 16, nullptr) == 0);
+  ASSERT_TRUE(again == blk);
+  ASSERT_TRUE(thrust_amd_temp_release(again, nullptr) == 0);
+  ASSERT_TRUE(thrust_amd_temp_release(again, nullptr) != 0);  // not handed out any more
+  ASSERT_TRUE(thrust_amd_temp_trim() == 0);
+  ASSERT_TRUE(thrust_amd_temp_bytes_held() == 0);
+}
+
 static void TestMemoryResources() {
   g_test = "MemoryResources";
   typedef thrust::mr::unsynchronized_pool_resource<thrust::device_memory_resource> Pool;
@@ -1179,9 +1345,12 @@ int main() {
   TestPoliciesAndRawPointers();
   TestDeviceVector();
   TestOutOfMemoryThrows();
+  TestMixedTypePlaceholders();
+  TestRemoveIfKeepsNaN();
   TestTempArenaReuse();
   TestCustomTemporaryAllocation();
   TestAsyncAlgorithms();
+  TestTempArenaOutlivesStream();
   TestMemoryResources();
   TestUniversalVector();
   std::printf("%s: %d checks, %d failed\n", g_failed ? "FAILED" : "PASSED", g_checks, g_failed);

@@ -276,15 +276,18 @@ TA_DEVICE int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_a
 // Comparison against a threshold chosen at run time (thrust_amd_cmp codes).
 template <typename T>
 TA_DEVICE bool apply_cmp(int cmp, T x, T t) {
-  switch (cmp) {
-    case THRUST_AMD_LT: return x < t;
-    case THRUST_AMD_LE: return x <= t;
-    case THRUST_AMD_GT: return x > t;
-    case THRUST_AMD_GE: return x >= t;
-    case THRUST_AMD_EQ: return x == t;
-    case THRUST_AMD_NE: return x != t;
-    default: return x != (T)0;
+  const bool negate = (cmp & THRUST_AMD_CMP_NOT) != 0;  // uniform: the logical negation of the code
+  bool r;
+  switch (cmp & ~THRUST_AMD_CMP_NOT) {
+    case THRUST_AMD_LT: r = x < t; break;
+    case THRUST_AMD_LE: r = x <= t; break;
+    case THRUST_AMD_GT: r = x > t; break;
+    case THRUST_AMD_GE: r = x >= t; break;
+    case THRUST_AMD_EQ: r = x == t; break;
+    case THRUST_AMD_NE: r = x != t; break;
+    default: r = x != (T)0; break;
   }
+  return r != negate;
 }
 
 // ------------------------------------------------------------------ search

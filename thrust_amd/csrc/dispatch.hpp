@@ -7,6 +7,8 @@ namespace ta {
 inline bool valid_dtype(int d) { return d >= 0 && d < THRUST_AMD_DTYPE_COUNT; }
 inline bool valid_binop(int o) { return o >= 0 && o < THRUST_AMD_BINOP_COUNT; }
 inline bool valid_cmp(int c) { return c >= 0 && c < THRUST_AMD_CMP_COUNT; }
+// ... or its logical negation (the selection entry points accept THRUST_AMD_CMP_NOT)
+inline bool valid_cmp_or_not(int c) { return c >= 0 && (c & ~THRUST_AMD_CMP_NOT) < THRUST_AMD_CMP_COUNT; }
 inline bool valid_unary(int u) { return u >= 0 && u < THRUST_AMD_UNARY_COUNT; }
 inline bool valid_item_bytes(size_t b) { return b == 1 || b == 2 || b == 4 || b == 8; }
 

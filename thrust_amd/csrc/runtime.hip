@@ -212,21 +212,26 @@ TA_EXPORT int thrust_amd_convert(const void* in, int in_dtype, void* out, int ou
 // ------------------------------------------------------------------ temp arena
 // Blocks are rounded up to size classes (powers of two from 4 KiB to 64 MiB, then
 // multiples of 64 MiB -- a 2^28-key radix sort needs ~1.2 GiB and must not round to
-// 2 GiB).  A released block remembers the stream it was released on.  It is handed out
-// again without further ado on the same stream (stream order makes the reuse safe);
-// for a different stream the releasing stream is synchronised first.
+// 2 GiB) and cached per device.  Every block owns one event.  Releasing a block records
+// that event on the releasing stream; handing the block out again makes the acquiring
+// stream wait for the event on the device (no host blocking).  The arena never keeps a
+// stream handle to call into later: the stream a block was released on may be destroyed at
+// any time, the event stays valid.  The handle is kept only as a tag, compared and never
+// used, to prefer a block last used on the same stream.
 namespace ta {
 
 struct ArenaBlock {
   void* ptr;
   size_t bytes;
-  hipStream_t released_on;
+  int device;
+  hipEvent_t released;        // recorded at the last release; null before the first one
+  const void* released_tag;   // value of the releasing stream handle (identity only)
 };
 
 struct Arena {
   std::mutex mu;
-  std::multimap<size_t, ArenaBlock> free_blocks;  // by size class
-  std::map<void*, size_t> live;                   // handed out -> size class
+  std::multimap<std::pair<int, size_t>, ArenaBlock> free_blocks;  // by (device, size class)
+  std::map<void*, ArenaBlock> live;                                // handed out
   size_t held = 0;
 };
 
@@ -246,6 +251,35 @@ static size_t size_class(size_t bytes) {
   return align_up(bytes, hi);
 }
 
+static int trim_device(int device, bool all_devices) {
+  Arena& a = arena();
+  std::vector<ArenaBlock> victims;
+  {
+    std::lock_guard<std::mutex> g(a.mu);
+    for (auto it = a.free_blocks.begin(); it != a.free_blocks.end();) {
+      if (all_devices || it->second.device == device) {
+        victims.push_back(it->second);
+        a.held -= it->second.bytes;
+        it = a.free_blocks.erase(it);
+      } else {
+        ++it;
+      }
+    }
+  }
+  int rc = 0;
+  for (auto& b : victims) {
+    hipError_t e = hipSuccess;
+    if (b.released) {
+      e = hipEventSynchronize(b.released);  // the last user of the block has finished
+      (void)hipEventDestroy(b.released);
+    }
+    const hipError_t f = hipFree(b.ptr);
+    if (e == hipSuccess) e = f;
+    if (e != hipSuccess && rc == 0) rc = (int)e;
+  }
+  return rc;
+}
+
 }  // namespace ta
 
 TA_EXPORT int thrust_amd_temp_acquire(void** ptr, size_t bytes, void* stream) {
@@ -253,27 +287,38 @@ TA_EXPORT int thrust_amd_temp_acquire(void** ptr, size_t bytes, void* stream) {
   if (!ptr) return (int)hipErrorInvalidValue;
   *ptr = nullptr;
   if (bytes == 0) return 0;
+  int device = 0;
+  TA_CHECK(hipGetDevice(&device));
   const size_t cls = size_class(bytes);
   Arena& a = arena();
-  ArenaBlock blk{nullptr, 0, nullptr};
+  ArenaBlock blk{nullptr, 0, device, nullptr, nullptr};
   {
     std::lock_guard<std::mutex> g(a.mu);
-    auto range = a.free_blocks.equal_range(cls);
+    auto range = a.free_blocks.equal_range(std::make_pair(device, cls));
     auto pick = range.second;
     for (auto it = range.first; it != range.second; ++it) {
-      if (it->second.released_on == (hipStream_t)stream) { pick = it; break; }
+      if (it->second.released_tag == (const void*)stream) { pick = it; break; }
       if (pick == range.second) pick = it;
     }
     if (pick != range.second) {
       blk = pick->second;
       a.free_blocks.erase(pick);
-      a.live[blk.ptr] = cls;
     }
   }
   if (blk.ptr) {
-    if (blk.released_on != (hipStream_t)stream) {
-      hipError_t e = hipStreamSynchronize(blk.released_on);
-      if (e != hipSuccess) return (int)e;
+    if (blk.released) {
+      // Work enqueued on `stream` from here on starts after the block's last use.  On the
+      // releasing stream itself this adds nothing that stream order did not already give.
+      const hipError_t e = hipStreamWaitEvent((hipStream_t)stream, blk.released, 0);
+      if (e != hipSuccess) {
+        std::lock_guard<std::mutex> g(a.mu);  // the block stays cached, not lost
+        a.free_blocks.emplace(std::make_pair(device, cls), blk);
+        return (int)e;
+      }
+    }
+    {
+      std::lock_guard<std::mutex> g(a.mu);
+      a.live[blk.ptr] = blk;
     }
     *ptr = blk.ptr;
     return 0;
@@ -281,9 +326,9 @@ TA_EXPORT int thrust_amd_temp_acquire(void** ptr, size_t bytes, void* stream) {
   void* p = nullptr;
   hipError_t e = hipMalloc(&p, cls);
   if (e != hipSuccess) {
-    // Out of memory: give the cached blocks back to the driver and try once more.
+    // Out of memory: give this device's cached blocks back to the driver and try once more.
     (void)hipGetLastError();
-    thrust_amd_temp_trim();
+    (void)trim_device(device, false);
     e = hipMalloc(&p, cls);
     if (e != hipSuccess) {
       (void)hipGetLastError();
@@ -292,7 +337,7 @@ TA_EXPORT int thrust_amd_temp_acquire(void** ptr, size_t bytes, void* stream) {
   }
   {
     std::lock_guard<std::mutex> g(a.mu);
-    a.live[p] = cls;
+    a.live[p] = ArenaBlock{p, cls, device, nullptr, nullptr};
     a.held += cls;
   }
   *ptr = p;
@@ -303,32 +348,34 @@ TA_EXPORT int thrust_amd_temp_release(void* ptr, void* stream) {
   using namespace ta;
   if (!ptr) return 0;
   Arena& a = arena();
-  std::lock_guard<std::mutex> g(a.mu);
-  auto it = a.live.find(ptr);
-  if (it == a.live.end()) return (int)hipErrorInvalidValue;
-  const size_t cls = it->second;
-  a.live.erase(it);
-  a.free_blocks.emplace(cls, ArenaBlock{ptr, cls, (hipStream_t)stream});
-  return 0;
-}
-
-TA_EXPORT int thrust_amd_temp_trim(void) {
-  using namespace ta;
-  Arena& a = arena();
-  std::vector<ArenaBlock> victims;
+  ArenaBlock blk;
   {
     std::lock_guard<std::mutex> g(a.mu);
-    for (auto& kv : a.free_blocks) victims.push_back(kv.second);
-    a.free_blocks.clear();
-    for (auto& b : victims) a.held -= b.bytes;
+    auto it = a.live.find(ptr);
+    if (it == a.live.end()) return (int)hipErrorInvalidValue;
+    blk = it->second;
+    a.live.erase(it);
   }
-  int rc = 0;
-  for (auto& b : victims) {
-    hipError_t e = hipFree(b.ptr);  // hipFree waits for outstanding work on the block
-    if (e != hipSuccess && rc == 0) rc = (int)e;
+  // Mark the end of the block's use on the releasing stream.  If that cannot be done the
+  // stream is drained instead, and the block goes back without an event to wait for.
+  hipError_t e = hipSuccess;
+  if (!blk.released) e = hipEventCreateWithFlags(&blk.released, hipEventDisableTiming);
+  if (e == hipSuccess) e = hipEventRecord(blk.released, (hipStream_t)stream);
+  if (e != hipSuccess) {
+    (void)hipGetLastError();
+    if (blk.released) (void)hipEventDestroy(blk.released);
+    blk.released = nullptr;
+    e = hipStreamSynchronize((hipStream_t)stream);
   }
-  return rc;
+  blk.released_tag = (const void*)stream;
+  {
+    std::lock_guard<std::mutex> g(a.mu);
+    a.free_blocks.emplace(std::make_pair(blk.device, blk.bytes), blk);
+  }
+  return (int)e;
 }
+
+TA_EXPORT int thrust_amd_temp_trim(void) { return ta::trim_device(0, true); }
 
 TA_EXPORT size_t thrust_amd_temp_bytes_held(void) {
   using namespace ta;

@@ -503,11 +503,11 @@ static int select_by_predicate(void* temp, size_t* temp_bytes, const void* in, c
                                void* out_true, void* out_false, uint64_t* d_num, uint64_t n,
                                size_t item_bytes, int stencil_dtype, int cmp, const void* threshold,
                                bool in_place, hipStream_t stream) {
-  if (!temp_bytes || !valid_item_bytes(item_bytes) || !valid_dtype(stencil_dtype) || !valid_cmp(cmp))
+  if (!temp_bytes || !valid_item_bytes(item_bytes) || !valid_dtype(stencil_dtype) || !valid_cmp_or_not(cmp))
     return (int)hipErrorInvalidValue;
   const size_t tested_bytes = thrust_amd_dtype_size(stencil_dtype);
   if (!stencil && tested_bytes != item_bytes) return (int)hipErrorInvalidValue;
-  if (cmp != THRUST_AMD_NONZERO && !threshold && temp) return (int)hipErrorInvalidValue;
+  if ((cmp & ~THRUST_AMD_CMP_NOT) != THRUST_AMD_NONZERO && !threshold && temp) return (int)hipErrorInvalidValue;
   const size_t park_bytes = in_place ? (size_t)n * item_bytes : 0;
 
   if (!stencil) {
