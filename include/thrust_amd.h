@@ -240,6 +240,18 @@ int thrust_amd_transform_reduce(void* temp, size_t* temp_bytes, const void* in, 
 int thrust_amd_inclusive_scan(void* temp, size_t* temp_bytes, const void* in, void* out,
                               uint64_t n, int dtype, int op, void* stream);
 
+/* thrust_amd_inclusive_scan for callers that cannot allocate (code under HIP graph capture,
+ * tight serving loops, harnesses that forbid hipMalloc): same result, no temporary storage
+ * argument.  It has no counterpart in the reference.  The tile descriptors live in a fixed
+ * 1 MiB array inside the library's device image (one copy per GPU, held until the process
+ * ends), cleared by a small kernel at every call; the call performs no hipMalloc / hipFree.
+ * n is limited by that array: up to 131040 tiles (about 6.4e9 elements of 4 bytes or less,
+ * 1.6e9 of 8 bytes); a larger n returns hipErrorInvalidValue and launches nothing.  Every
+ * call on a GPU shares that GPU's array: calls that may overlap in time on one GPU (two
+ * streams, two host threads) race and must be serialised by the caller. */
+int thrust_amd_inclusive_scan_static(const void* in, void* out, uint64_t n, int dtype, int op,
+                                     void* stream);
+
 /* out[0] = init, out[i] = init OP in[0] OP ... OP in[i-1]; out == in allowed.
  * `init` is a host pointer to one dtype element.
  * Replaces cuda_cub::exclusive_scan_n (thrust/system/cuda/detail/scan.h:132-200). */

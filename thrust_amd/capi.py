@@ -63,6 +63,7 @@ SIGNATURES = {
     "thrust_amd_count_if": (_int, [_vp, _szp, _vp, _u64, _int, _int, _vp, _vp, _vp]),
     "thrust_amd_inner_product": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _vp, _vp, _vp]),
     "thrust_amd_inclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _vp]),
+    "thrust_amd_inclusive_scan_static": (_int, [_vp, _vp, _u64, _int, _int, _vp]),
     "thrust_amd_exclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _vp, _vp]),
     "thrust_amd_transform_inclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _int, _vp]),
     "thrust_amd_transform_exclusive_scan": (_int, [_vp, _szp, _vp, _vp, _u64, _int, _int, _int, _vp, _vp]),
@@ -253,6 +254,14 @@ def inclusive_scan(x, out=None, op=PLUS, temp=None):
     out = out or DeviceArray(x.n, x.dtype)
     _run("thrust_amd_inclusive_scan", temp, lambda fn, t, b: fn(
         t, b, x.ptr, out.ptr, x.n, x.dtype, op, stream_ptr()))
+    return out
+
+
+def inclusive_scan_static(x, out=None, op=PLUS):
+    """The allocation-free entry point: no temp argument at all."""
+    out = out or DeviceArray(x.n, x.dtype)
+    check(load().thrust_amd_inclusive_scan_static(x.ptr, out.ptr, x.n, x.dtype, op, stream_ptr()),
+          "thrust_amd_inclusive_scan_static")
     return out
 
 
