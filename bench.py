@@ -9,7 +9,8 @@ JSON line follows the driver's contract.  `roofline` describes the dominant kern
 onesweep digit-binning pass: n keys read + n keys written), timed with events on the launch
 stream; `cpu_baseline` is the reference's own OpenMP device system (oracle/_ref, built from
 the reference sources) when that library travelled with the tree, else the C restatement,
-timed on a bounded sample on this machine's host cores.
+timed on this machine's host cores on the very keys and values the GPU legs used.  `configs`
+holds one verified row per other benchmark configuration (thrust_amd/bench_configs.py).
 """
 import argparse
 import json
@@ -33,11 +34,10 @@ PASS_TRAFFIC_BYTES = 2.318e9  # profiles/sort_u32_2p28_hbm_traffic.txt
 
 
 def device_random_u32(torch, n, seed):
-    """uint32 keys, uniform over the full range, generated on the device (seeded)."""
-    g = torch.Generator(device="cuda")
-    g.manual_seed(seed)
-    x = torch.randint(-(1 << 31), 1 << 31, (n,), dtype=torch.int32, device="cuda", generator=g)
-    return x.view(torch.uint8)
+    """uint32 keys, uniform over the full range: the seeded counter-based stream of
+    thrust_amd.datagen.c2_uint32, produced on the device (same bytes)."""
+    from thrust_amd import datagen_device
+    return datagen_device.c2_uint32(torch, n, seed).view(torch.uint8)
 
 
 def time_region(torch, fn, steps, warmup):
@@ -51,7 +51,7 @@ def time_region(torch, fn, steps, warmup):
     return (time.perf_counter() - t0) * 1e3 / steps
 
 
-def bench_sort(torch, capi, steps, warmup):
+def bench_sort(torch, capi, steps, warmup, want_host_copy):
     n = N_SORT
     src = device_random_u32(torch, n, 1)
     temp = capi.Temp()
@@ -70,6 +70,7 @@ def bench_sort(torch, capi, steps, warmup):
     if not ok:
         raise SystemExit("bench: sorted output failed the order/checksum check")
     del bufs, warm
+    host_keys = src.cpu().numpy().view(np.uint32) if want_host_copy else None
 
     # per-kernel durations of the same call, events on the launch stream
     capi.profile_enable(True)
@@ -83,14 +84,13 @@ def bench_sort(torch, capi, steps, warmup):
     launches, total_ms = prof["onesweep_pass"]
     pass_ms = total_ms / launches
     kernels_ms = {k: v[1] / reps for k, v in prof.items()}
-    return ms, pass_ms, kernels_ms
+    return ms, pass_ms, kernels_ms, host_keys
 
 
-def bench_c1(torch, capi, steps, warmup):
+def bench_c1(torch, capi, steps, warmup, want_host_copy):
     n = N_C1
-    g = torch.Generator(device="cuda")
-    g.manual_seed(42)
-    x = torch.randint(0, 1001, (n,), dtype=torch.int32, device="cuda", generator=g)
+    from thrust_amd import datagen_device
+    x = datagen_device.c1_int32(torch, n)  # the stream of thrust_amd.datagen.c1_int32 (seed 42)
     d = capi.DeviceArray(n, capi.I32, x.view(torch.uint8))
     out1 = capi.DeviceArray(1, capi.I32)
     outn = capi.DeviceArray(n, capi.I32)
@@ -106,43 +106,50 @@ def bench_c1(torch, capi, steps, warmup):
         raise SystemExit("bench: inclusive_scan total differs from the int64 sum modulo 2^32")
     ms_reduce = time_region(torch, lambda i, w: capi.reduce(d, temp=t_r, out=out1), steps, warmup)
     ms_scan = time_region(torch, lambda i, w: capi.inclusive_scan(d, out=outn, temp=t_s), steps, warmup)
-    return ms_reduce, ms_scan
+    return ms_reduce, ms_scan, (x.cpu().numpy() if want_host_copy else None)
 
 
-def cpu_baseline():
-    """Reference OMP back end (or the restatement) on a bounded sample: sort of 2^26 uint32."""
+def _timed(fn, warmups, reps):
+    for _ in range(warmups):
+        fn()
+    ts = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        fn()
+        ts.append(time.perf_counter() - t0)
+    ts.sort()
+    return ts[0], ts[len(ts) // 2]
+
+
+def cpu_baseline(sort_keys, c1_values):
+    """The reference's OpenMP device system (or the restatement) on the host cores, on the
+    configuration itself: the very keys and values the GPU legs used (downloaded from the
+    device), 2^28 elements each; 1 warm-up + 2 timed sorts, 1 warm-up + 5 timed reduces and
+    scans; minimum and median.  The other rows' figures are on 2^24-element samples."""
     from oracle import cpu as ocpu
     from thrust_amd import datagen
     cores = len(os.sched_getaffinity(0))
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
-    n = 1 << 26
-    keys = datagen.c2_uint32(n)
     if ocpu.ref_available("omp"):
         impl, kind = ocpu.Reference("omp"), "reference"
     else:
         if not os.path.exists(ocpu.ORACLE_LIB):
             ocpu.build(with_ref=False)
         impl, kind = ocpu.Oracle(), "port"
-    best = None
-    for _ in range(2):
-        k = keys.copy()
-        t0 = time.perf_counter()
-        out = impl.sort_keys(k)
-        dt = time.perf_counter() - t0
-        best = dt if best is None else min(best, dt)
-    if not np.all(out[:-1] <= out[1:]):
+    n = sort_keys.size
+    out = {}
+    t_min, t_med = _timed(lambda: out.update(s=impl.sort_keys(sort_keys)), 1, 2)
+    if not np.all(out["s"][:-1] <= out["s"][1:]):
         raise SystemExit("bench: CPU baseline output is not sorted")
-    x = datagen.c1_int32(1 << 26)
-    t0 = time.perf_counter(); impl.reduce(x); t_red = time.perf_counter() - t0
-    t0 = time.perf_counter(); impl.inclusive_scan(x); t_scan = time.perf_counter() - t0
+    del out
+    r_min, r_med = _timed(lambda: impl.reduce(c1_values), 1, 5)
+    s_min, s_med = _timed(lambda: impl.inclusive_scan(c1_values), 1, 5)
     # the other rows of the path on 2^24-element samples of their configurations (GB/s of the
-    # same algorithmic bytes the GPU figures use; one call each after building the inputs)
+    # same algorithmic bytes the GPU figures use; 1 warm-up + 2 timed calls, minimum)
     m = 1 << 24
 
     def gbs(nbytes, fn):
-        t0 = time.perf_counter()
-        fn()
-        return round(nbytes / (time.perf_counter() - t0) / 1e9, 3)
+        return round(nbytes / _timed(fn, 1, 2)[0] / 1e9, 3)
     ck, cv = datagen.c4_segments(m, 8)
     runs = int(ck[-1]) + 1
     f = datagen.c5_float32(m)
@@ -153,15 +160,18 @@ def cpu_baseline():
         "copy_if_half_GBps": gbs(6.0 * m, lambda: impl.copy_if(f, ocpu.LT, 0.5)),
         "stable_partition_half_GBps": gbs(8.0 * m, lambda: impl.stable_partition(f.copy(), ocpu.LT, 0.5)),
         "merge_by_key_GBps": gbs(16.0 * m, lambda: impl.merge_by_key(ka, kb, va, vb)),
-        "inclusive_scan_by_key_GBps": gbs(12.0 * m, lambda: impl.inclusive_scan_by_key(ck, cv)),
-        "set_union_GBps": gbs(8.0 * m, lambda: impl.set_operation(3, ka, kb)),
     }
     return {
-        "value": n / best / 1e9, "unit": "Gkeys/s", "cores": cores, "kind": kind,
+        "value": round(n / t_med / 1e9, 4), "unit": "Gkeys/s", "cores": cores, "kind": kind,
+        "sample": f"thrust::sort of the same 2^{n.bit_length() - 1} uint32 keys the GPU sorted (the whole "
+                  "configuration), 1 warm-up + 2 timed calls, median; each call includes one copy of the "
+                  "input made by the binding",
+        "sort_s": {"min": round(t_min, 3), "median": round(t_med, 3)},
+        "reduce_i32_2p28": {"GBps": round(4.0 * c1_values.size / r_med / 1e9, 2),
+                            "ms_min": round(r_min * 1e3, 2), "ms_median": round(r_med * 1e3, 2)},
+        "inclusive_scan_i32_2p28": {"GBps": round(8.0 * c1_values.size / s_med / 1e9, 2),
+                                    "ms_min": round(s_min * 1e3, 2), "ms_median": round(s_med * 1e3, 2)},
         "rows_2p24": rows,
-        "sample": "thrust::sort of 2^26 uint32 (same generator as the GPU run's key space), best of 2, "
-                  "timing includes one copy of the input made by the binding",
-        "reduce_GBps": 4.0 * x.size / t_red / 1e9, "inclusive_scan_GBps": 8.0 * x.size / t_scan / 1e9,
         "note": "OMP back end: sort = per-thread LSD radix + serial pairwise merges; "
                 "inclusive_scan is single-threaded by construction",
     }
@@ -173,6 +183,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the verified rows of the other configurations (C2 float, C3, C4, C5)")
     args = ap.parse_args()
     if args.gpus != 1:
         raise SystemExit("bench.py: this build measures one GPU only (the device system is "
@@ -186,9 +198,15 @@ def main():
         raise SystemExit("bench.py needs a GPU")
     capi.load()  # raises if the HIP library is missing: there is no fallback
 
-    ms_sort, pass_ms, kernels_ms = bench_sort(torch, capi, args.steps, args.warmup)
-    ms_reduce, ms_scan = bench_c1(torch, capi, args.steps, args.warmup)
+    want_host = not args.no_cpu_baseline
+    ms_sort, pass_ms, kernels_ms, host_keys = bench_sort(torch, capi, args.steps, args.warmup, want_host)
     torch.cuda.empty_cache()
+    ms_reduce, ms_scan, host_c1 = bench_c1(torch, capi, args.steps, args.warmup, want_host)
+    torch.cuda.empty_cache()
+    config_rows = None
+    if not args.no_configs:
+        from thrust_amd import bench_configs
+        config_rows = bench_configs.run_all(torch, capi)
 
     n = N_SORT
     gkeys = n / ms_sort / 1e6
@@ -220,8 +238,10 @@ def main():
                      "frac": round(pass_gbs / HBM_PEAK_GBS, 4), "traffic": PASS_TRAFFIC_BYTES,
                      "launch_ms": round(pass_ms, 4)},
     }
+    if config_rows is not None:
+        line["configs"] = config_rows
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline()
+        line["cpu_baseline"] = cpu_baseline(host_keys, host_c1)
     print(json.dumps(line))
 
 

@@ -123,6 +123,39 @@ def test_config3_key_distributions(dev, oracle_seq, kind):
     assert np.array_equal(dk.numpy(), rk) and np.array_equal(dv.numpy(), rv)
 
 
+@pytest.mark.parametrize("kind", ["full", "low16", "skew90"])
+def test_config3_full_size_properties(dev, kind):
+    """Config 3 at its own size, N = 2^27 uint64 keys with uint32 values = original index
+    (testing/stable_sort_by_key.cu:99-116 at the configuration's size).  Checked on the device:
+    keys ascending, the values a permutation of 0..n-1, every value still carrying its key
+    (keys_in[values_out] == keys_out) and values ascending inside every run of equal keys.
+    Together these fix the output completely: it is the stable sort of the input."""
+    import torch
+    n = 1 << 27
+    k = datagen.c3_uint64(n, kind)
+    keys_in = torch.from_numpy(k.view(np.int64)).cuda()
+    del k
+    dk = dev.DeviceArray(n, dev.U64, keys_in.view(torch.uint8).clone())
+    dv = dev.DeviceArray(n, dev.U32, torch.arange(n, dtype=torch.int32, device="cuda").view(torch.uint8))
+    dev.sort_pairs(dk, dv)
+    ko = dk.storage.view(torch.int64)
+    vo = dv.storage.view(torch.int32).to(torch.int64)  # indices below 2^27: non-negative
+    flip = torch.tensor(-(1 << 63), dtype=torch.int64, device="cuda")
+    ordered = ko ^ flip  # unsigned order as signed order
+    assert bool((ordered[1:] >= ordered[:-1]).all().item()), kind
+    seen = torch.zeros(n, dtype=torch.bool, device="cuda")
+    seen[vo] = True
+    assert bool(seen.all().item()), kind
+    assert bool((keys_in[vo] == ko).all().item()), kind
+    same = ko[1:] == ko[:-1]
+    assert bool((vo[1:][same] > vo[:-1][same]).all().item()), kind
+    if kind == "low16":
+        assert int(ko.max().item()) <= 0xFFFF
+    if kind == "skew90":
+        frac = float((ko == datagen.C3_CONSTANT).sum().item()) / n
+        assert 0.89 < frac < 0.91
+
+
 def test_config2_full_size_properties(dev):
     """Config 2 at N=2^28: sortedness, multiset preservation (histogram of all bytes and a
     64-bit sum/xor checksum) for uint32; the float32 case is checked on its encoded bits."""

@@ -1,210 +1,204 @@
-#!/usr/bin/env python3
-"""Timings of the benchmark configurations beside the headline one, on one GPU.
+"""The benchmark configurations beside the headline one: each is run on the device at its own
+size, its result is verified there against an independent torch computation, and the whole
+call (every kernel it launches, launch gaps included) is timed with events on the launch
+stream.  bench.py imports this module and prints the rows inside its JSON line.
 
-For each configuration the device-side time of one call is reported as the sum of the
-library's own per-kernel event timers (inputs resident in HBM, temp storage sized once),
-with the algorithmic bytes of the call and the resulting fraction of the 8 TB/s HBM peak:
-
-  C2  sort of 2^28 float32 keys
-  C3  sort_by_key of 2^27 uint64 keys + uint32 values: full range / low 16 bits / 90 % one key
-  C4  reduce_by_key and unique_by_key over 2^28 (int32 key, float32 value), mean run 8 / 1000
+  C2  sort of 2^28 float32 keys (1 % of +-0.0 and denormals)
+  C3  stable sort_by_key of 2^27 uint64 keys + uint32 values: full range / low 16 bits / 90 % one key
+  C4  reduce_by_key, unique_by_key and unique over 2^28 (int32 key, float32 value), mean run 8 / 1000
   C5  copy_if and stable_partition of 2^28 float32 at 50 % / 5 % selectivity,
-      merge and merge_by_key of two sorted ranges of 2^27 uint32 (+ uint32 values)
-  C6  callers on either side of the path: count_if, inner_product, transform_reduce and
-      the transform scans over 2^28 int32 / float32, inclusive and exclusive scan_by_key
-      over 2^28 (int32 key, float32 value)
+      merge_by_key and merge of two sorted ranges of 2^27 uint32 (+ uint32 values)
 
-  C7  the four set operations on two sorted ranges of 2^27 uint32 with runs of about four
-      and two equal keys (bytes: both inputs read, the result written)
-  C8  the stable comparison sort (merge sort) of 2^28 uint32 keys and of 2^27 uint64 keys
-      with uint32 values (bytes: one block sort and ceil(log2(n / 4096)) merge passes, each
-      reading and writing every element)
-
-Inputs are generated on the device from a seeded generator.  Usage:
-  python3 thrust_amd/bench_configs.py [c2] [c3] [c4] [c5] [c6] [c7] [c8]
+Bytes are the algorithmic ones of each call (what must be read and written once).
 """
-import os
-import sys
-
 import numpy as np
 
-sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+from . import datagen_device as gen
 
 HBM_PEAK_GBS = 8000.0
-REPS = 5
 
 
-def main():
-    import torch
-    from thrust_amd import capi
-    if not torch.cuda.is_available():
-        raise SystemExit("bench_configs.py needs a GPU")
-    capi.load()
-    which = [a.lower() for a in sys.argv[1:]] or ["c2", "c3", "c4", "c5", "c6", "c7", "c8"]
-    g = torch.Generator(device="cuda")
-    g.manual_seed(1)
+def _dev(capi, torch, t, code):
+    items = t.numel() * t.element_size() // np.dtype(capi.NP_DTYPES[code]).itemsize
+    return capi.DeviceArray(items, code, t.view(torch.uint8))
 
-    def dev(t, code):
-        items = t.numel() * t.element_size() // np.dtype(capi.NP_DTYPES[code]).itemsize
-        return capi.DeviceArray(items, code, t.view(torch.uint8))
 
-    def run(name, fn, nbytes, setup=None, extra=""):
+_PAD = {}
+
+
+def _time_calls(torch, fn, reps, setup=None):
+    """Median and minimum device time of fn() in ms; setup() runs before each call, untimed.
+    fn must not synchronise.  The device is kept busy with a fill while the host prepares
+    the call, so that the first event is not reached before the call has been enqueued."""
+    if "buf" not in _PAD:
+        _PAD["buf"] = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    if setup:
+        setup()
+    fn()  # sizes temp storage, warms up
+    torch.cuda.synchronize()
+    times = []
+    for _ in range(reps):
         if setup:
             setup()
-        fn()  # sizes temp storage, warms up
-        torch.cuda.synchronize()
-        capi.profile_enable(True)
-        for _ in range(REPS):
-            if setup:
-                setup()
-            fn()
-        torch.cuda.synchronize()
-        prof = capi.profile_collect()
-        capi.profile_enable(False)
-        ms = sum(v[1] for v in prof.values()) / REPS
-        kernels = "  ".join(f"{k}={v[1] / REPS:.3f}" for k, v in prof.items())
-        gbs = nbytes / ms / 1e6
-        print(f"{name:44s} {ms:8.3f} ms {gbs:8.0f} GB/s {gbs / HBM_PEAK_GBS * 100:5.1f}%  {extra}  [{kernels}]",
-              flush=True)
+        _PAD["buf"].zero_()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        fn()
+        b.record()
+        b.synchronize()
+        times.append(a.elapsed_time(b))
+    times.sort()
+    return times[len(times) // 2], times[0]
 
+
+def _row(ms_med, ms_min, nbytes, **extra):
+    gbs = nbytes / ms_med / 1e6
+    row = {"ms": round(ms_med, 4), "ms_min": round(ms_min, 4), "GBps": round(gbs, 1),
+           "pct_of_peak": round(gbs / HBM_PEAK_GBS * 100, 2), "bytes": int(nbytes), "verified": True}
+    row.update(extra)
+    return row
+
+
+def _fail(what):
+    raise SystemExit(f"bench: {what} failed its result check")
+
+
+def run_c2_float(torch, capi, reps):
     n = 1 << 28
-    if "c2" in which:
-        f = (torch.rand(n, device="cuda", generator=g) * 2e6 - 1e6).float()
-        src, work, t = dev(f, capi.F32), capi.DeviceArray(n, capi.F32), capi.Temp()
-        run("C2 sort f32 2^28", lambda: capi.sort_keys(work, temp=t), 36 * n,
-            setup=lambda: work.storage.copy_(src.storage), extra="36 B/key")
-        del f, src, work, t
-    if "c3" in which:
-        m = 1 << 27
-        for kind in ("full", "low16", "skew90"):
-            r = torch.randint(-(1 << 62), 1 << 62, (m,), dtype=torch.int64, device="cuda", generator=g) * 2 \
-                + torch.randint(0, 2, (m,), dtype=torch.int64, device="cuda", generator=g)
-            if kind == "low16":
-                r = r & 0xFFFF
-            if kind == "skew90":
-                pick = torch.randint(0, 10, (m,), device="cuda", generator=g)
-                r = torch.where(pick != 0, torch.full_like(r, 0x0123456789ABCDEF), r)
-            v = torch.arange(m, dtype=torch.int32, device="cuda")
-            sk, sv = dev(r, capi.U64), dev(v, capi.U32)
-            wk, wv, t = capi.DeviceArray(m, capi.U64), capi.DeviceArray(m, capi.U32), capi.Temp()
+    f = gen.c2_float32(torch, n)
+    src, work, t = _dev(capi, torch, f, capi.F32), capi.DeviceArray(n, capi.F32), capi.Temp()
+    med, mn = _time_calls(torch, lambda: capi.sort_keys(work, temp=t), reps,
+                          setup=lambda: work.storage.copy_(src.storage))
+    out = work.storage.view(torch.int32)
+    # radix order of floats: flip all bits of negatives, the sign bit of the others
+    enc = lambda b: torch.where(b < 0, ~b, b ^ (-(1 << 31))).to(torch.int64) & 0xFFFFFFFF
+    e = enc(out)
+    if not bool((e[1:] >= e[:-1]).all().item()):
+        _fail("C2 float32 sort (order)")
+    if int(e.sum().item()) != int(enc(f.view(torch.int32)).sum().item()):
+        _fail("C2 float32 sort (checksum)")
+    return {"c2_sort_f32_2p28": _row(med, mn, 36 * n, Gkeys_per_s=round(n / med / 1e6, 2), model="36 B/key")}
 
-            def setup():
-                wk.storage.copy_(sk.storage)
-                wv.storage.copy_(sv.storage)
-            # model: histogram read + 8 passes reading and writing 12 B per pair
-            run(f"C3 sort_by_key u64+u32 2^27 {kind}", lambda: capi.sort_pairs(wk, wv, temp=t), 200 * m,
-                setup=setup, extra="200 B/pair when all 8 passes run")
-            del r, v, sk, sv, wk, wv, t
-    if "c4" in which:
-        for mean in (8, 1000):
-            nseg = int(n / mean * 1.2) + 1000
-            u = torch.rand(nseg, device="cuda", generator=g, dtype=torch.float64).clamp_(1e-12, 1.0)
-            lens = (torch.floor(torch.log(u) / np.log1p(-1.0 / mean)) + 1).long()
-            keys = torch.repeat_interleave(torch.arange(nseg, device="cuda", dtype=torch.int32), lens)[:n].contiguous()
-            if keys.numel() != n:
-                raise SystemExit("bench_configs: segment generator came up short")
-            runs = int(keys[-1].item()) + 1
-            vals = torch.rand(n, device="cuda", generator=g)
-            dk, dv = dev(keys, capi.I32), dev(vals, capi.F32)
-            ko, vo, t = capi.DeviceArray(n, capi.I32), capi.DeviceArray(n, capi.F32), capi.Temp()
-            run(f"C4 reduce_by_key mean run {mean}",
-                lambda: capi.reduce_by_key(dk, dv, temp=t, keys_out=ko, values_out=vo), 8 * n + 8 * runs)
-            run(f"C4 unique_by_key mean run {mean}",
-                lambda: capi.unique_by_key(dk, dv, keys_out=ko, values_out=vo, temp=t), 8 * n + 8 * runs)
-            run(f"C4 unique (keys only) mean run {mean}",
-                lambda: capi.unique(dk, out=ko, temp=t), 4 * n + 4 * runs)
-            del keys, vals, dk, dv, ko, vo, t, u, lens
-    if "c5" in which:
-        x = torch.rand(n, device="cuda", generator=g)
-        dx, out, work = dev(x, capi.F32), capi.DeviceArray(n, capi.F32), capi.DeviceArray(n, capi.F32)
-        t, tp = capi.Temp(), capi.Temp()
-        for thr in (0.5, 0.05):
-            _, cnt = capi.copy_if(dx, capi.LT, thr, out=out, temp=t)
-            run(f"C5 copy_if x<{thr}", lambda: capi.copy_if(dx, capi.LT, thr, out=out, temp=t), 4 * n + 4 * cnt)
-            run(f"C5 stable_partition x<{thr}", lambda: capi.stable_partition(work, capi.LT, thr, temp=tp), 8 * n,
-                setup=lambda: work.storage.copy_(dx.storage))
-        del x, dx, out, work, t, tp
-        m = 1 << 27
 
-        def sorted_u32():
-            r = torch.randint(-(1 << 31), 1 << 31, (m,), dtype=torch.int32, device="cuda", generator=g)
-            return torch.sort(r.to(torch.int64) & 0xFFFFFFFF)[0].to(torch.int32)
-        ka, kb = sorted_u32(), sorted_u32()
-        va = torch.arange(m, dtype=torch.int32, device="cuda")
-        vb = va + m
-        a = [dev(z, capi.U32) for z in (ka, kb, va, vb)]
-        ko, vo, t, t2 = capi.DeviceArray(2 * m, capi.U32), capi.DeviceArray(2 * m, capi.U32), capi.Temp(), capi.Temp()
-        run("C5 merge_by_key 2 x 2^27 u32+u32",
-            lambda: capi.merge_by_key(*a, temp=t, keys_out=ko, values_out=vo), 16 * 2 * m)
-        run("C5 merge 2 x 2^27 u32", lambda: capi.merge(a[0], a[1], out=ko, temp=t2), 8 * 2 * m)
-        del ka, kb, va, vb, a, ko, vo, t, t2
-    if "c6" in which:
-        x = torch.randint(0, 1001, (n,), dtype=torch.int32, device="cuda", generator=g)
-        dx, t = dev(x, capi.I32), capi.Temp()
-        run("C6 count_if i32 x<500", lambda: capi.count_if(dx, capi.LT, 500, temp=t), 4 * n)
-        f1 = torch.rand(n, device="cuda", generator=g)
-        f2 = torch.rand(n, device="cuda", generator=g)
-        d1, d2, t2, out1 = dev(f1, capi.F32), dev(f2, capi.F32), capi.Temp(), capi.DeviceArray(1, capi.F32)
-        run("C6 inner_product f32", lambda: capi.inner_product(d1, d2, init=0.0, temp=t2, out=out1), 8 * n)
-        t3, t4, so, so_i = capi.Temp(), capi.Temp(), capi.DeviceArray(n, capi.F32), capi.DeviceArray(n, capi.I32)
-        run("C6 transform_reduce f32 square, plus",
-            lambda: capi.transform_reduce(d1, capi.SQUARE, init=0.0, temp=t3, out=out1), 4 * n)
-        run("C6 transform_inclusive_scan f32 negate, plus",
-            lambda: capi.transform_inclusive_scan(d1, capi.NEGATE, out=so, temp=t4), 8 * n)
-        run("C6 transform_exclusive_scan i32 square, plus",
-            lambda: capi.transform_exclusive_scan(dx, capi.SQUARE, init=3, out=so_i, temp=t4), 8 * n)
-        del x, dx, f1, f2, d1, d2, t, t2, t3, t4, so, so_i
-        mean = 8
-        nseg = int(n / mean * 1.2) + 1000
-        u = torch.rand(nseg, device="cuda", generator=g, dtype=torch.float64).clamp_(1e-12, 1.0)
-        lens = (torch.floor(torch.log(u) / np.log1p(-1.0 / mean)) + 1).long()
-        keys = torch.repeat_interleave(torch.arange(nseg, device="cuda", dtype=torch.int32), lens)[:n].contiguous()
-        vals = torch.rand(n, device="cuda", generator=g)
-        dk, dv, vo, t = dev(keys, capi.I32), dev(vals, capi.F32), capi.DeviceArray(n, capi.F32), capi.Temp()
-        run("C6 inclusive_scan_by_key mean run 8", lambda: capi.inclusive_scan_by_key(dk, dv, out=vo, temp=t), 12 * n)
-        run("C6 exclusive_scan_by_key mean run 8",
-            lambda: capi.exclusive_scan_by_key(dk, dv, init=0.0, out=vo, temp=t), 12 * n)
-    if "c7" in which:
-        m = 1 << 27
-
-        def sorted_keys(distinct):
-            r = torch.randint(0, distinct, (m,), dtype=torch.int32, device="cuda", generator=g)
-            return torch.sort(r)[0]
-        ka, kb = sorted_keys(m // 4), sorted_keys(m // 2)
-        da, db = dev(ka, capi.U32), dev(kb, capi.U32)
-        out, t = capi.DeviceArray(2 * m, capi.U32), capi.Temp()
-        names = ("set_difference", "set_intersection", "set_symmetric_difference", "set_union")
-        for op, name in enumerate(names):
-            _, cnt = capi.set_operation(op, da, db, out=out, temp=t)
-            run(f"C7 {name} 2 x 2^27 u32", lambda: capi.set_operation(op, da, db, out=out, temp=t),
-                4 * (2 * m + cnt), extra=f"{cnt} out")
-        va = torch.arange(m, dtype=torch.int32, device="cuda")
-        dva, dvb, vo, t2 = dev(va, capi.U32), dev(va + m, capi.U32), capi.DeviceArray(2 * m, capi.U32), capi.Temp()
-        _, _, cnt = capi.set_operation_by_key(3, da, db, dva, dvb, keys_out=out, values_out=vo, temp=t2)
-        run("C7 set_union_by_key 2 x 2^27 u32+u32",
-            lambda: capi.set_operation_by_key(3, da, db, dva, dvb, keys_out=out, values_out=vo, temp=t2),
-            4 * (2 * m + cnt) + 8 * cnt, extra=f"{cnt} out")
-        del ka, kb, da, db, out, t, va, dva, dvb, vo, t2
-    if "c8" in which:
-        def passes(count):
-            return 1 + int(np.ceil(np.log2(max(1.0, count / 4096))))
-        r = torch.randint(-(1 << 31), 1 << 31, (n,), dtype=torch.int32, device="cuda", generator=g)
-        src, work, t = dev(r, capi.U32), capi.DeviceArray(n, capi.U32), capi.Temp()
-        run("C8 comparison sort u32 2^28", lambda: capi.merge_sort_keys(work, temp=t), passes(n) * 8 * n,
-            setup=lambda: work.storage.copy_(src.storage), extra=f"{passes(n)} x 8 B/key")
-        del r, src, work, t
-        m = 1 << 27
-        r = torch.randint(-(1 << 62), 1 << 62, (m,), dtype=torch.int64, device="cuda", generator=g)
-        v = torch.arange(m, dtype=torch.int32, device="cuda")
-        sk, sv = dev(r, capi.U64), dev(v, capi.U32)
+def run_c3(torch, capi, reps):
+    m = 1 << 27
+    rows = {}
+    for kind in ("full", "low16", "skew90"):
+        keys = gen.c3_uint64(torch, m, kind)
+        vals = torch.arange(m, dtype=torch.int32, device="cuda")
+        sk, sv = _dev(capi, torch, keys, capi.U64), _dev(capi, torch, vals, capi.U32)
         wk, wv, t = capi.DeviceArray(m, capi.U64), capi.DeviceArray(m, capi.U32), capi.Temp()
 
         def setup():
             wk.storage.copy_(sk.storage)
             wv.storage.copy_(sv.storage)
-        run("C8 comparison sort_by_key u64+u32 2^27", lambda: capi.merge_sort_pairs(wk, wv, temp=t),
-            passes(m) * 24 * m, setup=setup, extra=f"{passes(m)} x 24 B/pair")
+        med, mn = _time_calls(torch, lambda: capi.sort_pairs(wk, wv, temp=t), reps, setup=setup)
+        ko = wk.storage.view(torch.int64)
+        vo = wv.storage.view(torch.int32).to(torch.int64)
+        o = ko ^ (-(1 << 63))
+        same = ko[1:] == ko[:-1]
+        ok = bool((o[1:] >= o[:-1]).all().item()) and bool((keys[vo] == ko).all().item()) \
+            and bool((vo[1:][same] > vo[:-1][same]).all().item())
+        if not ok:
+            _fail(f"C3 sort_by_key {kind}")
+        rows[f"c3_sort_by_key_u64_u32_2p27_{kind}"] = _row(
+            med, mn, 200 * m, Gpairs_per_s=round(m / med / 1e6, 2),
+            model="200 B/pair: histogram read + 8 passes x 24 B; passes over a constant digit are skipped")
+        del keys, vals, sk, sv, wk, wv, t, ko, vo, o, same
+    return rows
 
 
-if __name__ == "__main__":
-    main()
+def run_c4(torch, capi, reps):
+    n = 1 << 28
+    rows = {}
+    for mean in (8, 1000):
+        keys, vals = gen.c4_segments(torch, n, mean)
+        runs = int(keys[-1].item()) + 1
+        dk, dv = _dev(capi, torch, keys, capi.I32), _dev(capi, torch, vals, capi.F32)
+        ko, vo, t = capi.DeviceArray(n, capi.I32), capi.DeviceArray(n, capi.F32), capi.Temp()
+        starts = torch.searchsorted(keys, torch.arange(runs, dtype=torch.int32, device="cuda"))
+        want_keys = torch.arange(runs, dtype=torch.int32, device="cuda")
+
+        res = {}
+        med, mn = _time_calls(torch, lambda: res.update(r=capi.reduce_by_key(dk, dv, temp=t, keys_out=ko, values_out=vo, read_count=False)), reps)
+        cnt = int(res["r"][-1].numpy()[0])
+        sums = torch.zeros(runs, dtype=torch.float64, device="cuda").index_add_(0, keys.to(torch.int64), vals.to(torch.float64))
+        got = vo.storage.view(torch.float32)[:runs].to(torch.float64)
+        rel = ((got - sums).abs() / sums.abs().clamp_min(1e-30)).max().item()
+        if cnt != runs or not torch.equal(ko.storage.view(torch.int32)[:runs], want_keys) or rel > 1e-5:
+            _fail(f"C4 reduce_by_key mean {mean} (count {cnt} vs {runs}, rel {rel:.2e})")
+        rows[f"c4_reduce_by_key_mean{mean}"] = _row(med, mn, 8 * n + 8 * runs, runs=runs, max_rel_err_vs_f64=float(f"{rel:.3e}"))
+
+        med, mn = _time_calls(torch, lambda: res.update(r=capi.unique_by_key(dk, dv, keys_out=ko, values_out=vo, temp=t, read_count=False)), reps)
+        cnt = int(res["r"][-1].numpy()[0])
+        if cnt != runs or not torch.equal(ko.storage.view(torch.int32)[:runs], want_keys) \
+                or not torch.equal(vo.storage.view(torch.float32)[:runs], vals[starts]):
+            _fail(f"C4 unique_by_key mean {mean}")
+        rows[f"c4_unique_by_key_mean{mean}"] = _row(med, mn, 8 * n + 8 * runs, runs=runs)
+
+        med, mn = _time_calls(torch, lambda: res.update(r=capi.unique(dk, out=ko, temp=t, read_count=False)), reps)
+        cnt = int(res["r"][-1].numpy()[0])
+        if cnt != runs or not torch.equal(ko.storage.view(torch.int32)[:runs], want_keys):
+            _fail(f"C4 unique mean {mean}")
+        rows[f"c4_unique_keys_mean{mean}"] = _row(med, mn, 4 * n + 4 * runs, runs=runs)
+        del keys, vals, dk, dv, ko, vo, t, starts, want_keys, sums, got
+    return rows
+
+
+def run_c5(torch, capi, reps):
+    n = 1 << 28
+    rows = {}
+    x = gen.c5_float32(torch, n)
+    dx, out, work = _dev(capi, torch, x, capi.F32), capi.DeviceArray(n, capi.F32), capi.DeviceArray(n, capi.F32)
+    t, tp = capi.Temp(), capi.Temp()
+    for thr, tag in ((0.5, "50pct"), (0.05, "5pct")):
+        thr32 = float(np.float32(thr))
+        mask = x < thr32
+        want_true = x[mask]
+        cnt_want = want_true.numel()
+        res = {}
+        med, mn = _time_calls(torch, lambda: res.update(r=capi.copy_if(dx, capi.LT, thr, out=out, temp=t, read_count=False)), reps)
+        cnt = int(res["r"][-1].numpy()[0])
+        if cnt != cnt_want or not torch.equal(out.storage.view(torch.float32)[:cnt], want_true):
+            _fail(f"C5 copy_if {tag}")
+        rows[f"c5_copy_if_{tag}"] = _row(med, mn, 4 * n + 4 * cnt, selected=cnt)
+
+        med, mn = _time_calls(torch, lambda: res.update(r=(capi.stable_partition(work, capi.LT, thr, temp=tp, read_count=False),)), reps,
+                              setup=lambda: work.storage.copy_(dx.storage))
+        cnt = int(res["r"][-1].numpy()[0])
+        got = work.storage.view(torch.float32)
+        if cnt != cnt_want or not torch.equal(got[:cnt], want_true) or not torch.equal(got[cnt:], x[~mask]):
+            _fail(f"C5 stable_partition {tag}")
+        rows[f"c5_stable_partition_{tag}"] = _row(med, mn, 8 * n, selected=cnt)
+        del mask, want_true, got
+    del x, dx, out, work, t, tp
+
+    m = 1 << 27
+    (ka, va), (kb, vb) = gen.c5_merge_inputs(torch, m)
+    vb = vb + m  # payloads of the second range are told apart from the first's
+    a = [_dev(capi, torch, z, capi.U32) for z in (ka, kb, va, vb)]
+    ko, vo, t, t2 = capi.DeviceArray(2 * m, capi.U32), capi.DeviceArray(2 * m, capi.U32), capi.Temp(), capi.Temp()
+    # a stable sort of (first range, second range) is the merge with ties from the first range first
+    both = torch.cat([ka, kb]).to(torch.int64) & 0xFFFFFFFF
+    want_k, order = torch.sort(both, stable=True)
+    want_v = torch.cat([va, vb])[order]
+    med, mn = _time_calls(torch, lambda: capi.merge_by_key(*a, temp=t, keys_out=ko, values_out=vo), reps)
+    if not torch.equal(ko.storage.view(torch.int32).to(torch.int64) & 0xFFFFFFFF, want_k) \
+            or not torch.equal(vo.storage.view(torch.int32), want_v):
+        _fail("C5 merge_by_key")
+    rows["c5_merge_by_key_2x2p27"] = _row(med, mn, 16 * 2 * m)
+    med, mn = _time_calls(torch, lambda: capi.merge(a[0], a[1], out=ko, temp=t2), reps)
+    if not torch.equal(ko.storage.view(torch.int32).to(torch.int64) & 0xFFFFFFFF, want_k):
+        _fail("C5 merge")
+    rows["c5_merge_2x2p27"] = _row(med, mn, 8 * 2 * m)
+    return rows
+
+
+def run_all(torch, capi, reps=5):
+    rows = {}
+    for part in (run_c2_float, run_c3, run_c4, run_c5):
+        rows.update(part(torch, capi, reps))
+        torch.cuda.empty_cache()
+    _PAD.clear()
+    torch.cuda.empty_cache()
+    return rows

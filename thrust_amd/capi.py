@@ -234,12 +234,12 @@ def transform_reduce(x, unary, op=PLUS, init=0, temp=None, out=None):
     return out
 
 
-def count_if(x, cmp, threshold=0, temp=None):
+def count_if(x, cmp, threshold=0, temp=None, read_count=True):
     num = DeviceArray(1, U64)
     tv = _scalar(x.dtype, threshold)
     _run("thrust_amd_count_if", temp, lambda fn, t, b: fn(
         t, b, x.ptr, x.n, x.dtype, cmp, tv.ctypes.data, num.ptr, stream_ptr()))
-    return _count(num)
+    return _count(num, read_count)
 
 
 def inner_product(a, b_, init=0, temp=None, out=None):
@@ -328,11 +328,13 @@ def merge_sort_pairs(keys, values, descending=False, temp=None):
         t, b, keys.ptr, values.ptr, keys.n, keys.dtype, values.itemsize, int(descending), stream_ptr()))
 
 
-def _count(dev_u64):
-    return int(dev_u64.numpy()[0])
+def _count(dev_u64, read=True):
+    """The uint64 result count: read back (blocks) or, with read=False, left on the device
+    for callers that must not synchronise inside a timed region."""
+    return int(dev_u64.numpy()[0]) if read else dev_u64
 
 
-def copy_if(x, cmp, threshold=0, stencil=None, out=None, temp=None):
+def copy_if(x, cmp, threshold=0, stencil=None, out=None, temp=None, read_count=True):
     out = out or DeviceArray(x.n, x.dtype)
     num = DeviceArray(1, U64)
     tested = stencil if stencil is not None else x
@@ -340,10 +342,10 @@ def copy_if(x, cmp, threshold=0, stencil=None, out=None, temp=None):
     _run("thrust_amd_copy_if", temp, lambda fn, t, b: fn(
         t, b, x.ptr, stencil.ptr if stencil is not None else None, out.ptr, num.ptr, x.n,
         x.itemsize, tested.dtype, cmp, tv.ctypes.data, stream_ptr()))
-    return out, _count(num)
+    return out, _count(num, read_count)
 
 
-def partition_copy(x, cmp, threshold=0, stencil=None, temp=None):
+def partition_copy(x, cmp, threshold=0, stencil=None, temp=None, read_count=True):
     out_t, out_f = DeviceArray(x.n, x.dtype), DeviceArray(x.n, x.dtype)
     num = DeviceArray(1, U64)
     tested = stencil if stencil is not None else x
@@ -351,45 +353,45 @@ def partition_copy(x, cmp, threshold=0, stencil=None, temp=None):
     _run("thrust_amd_partition_copy", temp, lambda fn, t, b: fn(
         t, b, x.ptr, stencil.ptr if stencil is not None else None, out_t.ptr, out_f.ptr, num.ptr,
         x.n, x.itemsize, tested.dtype, cmp, tv.ctypes.data, stream_ptr()))
-    return out_t, out_f, _count(num)
+    return out_t, out_f, _count(num, read_count)
 
 
-def stable_partition(x, cmp, threshold=0, stencil=None, temp=None):
+def stable_partition(x, cmp, threshold=0, stencil=None, temp=None, read_count=True):
     num = DeviceArray(1, U64)
     tested = stencil if stencil is not None else x
     tv = _scalar(tested.dtype, threshold)
     _run("thrust_amd_stable_partition", temp, lambda fn, t, b: fn(
         t, b, x.ptr, stencil.ptr if stencil is not None else None, num.ptr, x.n, x.itemsize,
         tested.dtype, cmp, tv.ctypes.data, stream_ptr()))
-    return _count(num)
+    return _count(num, read_count)
 
 
-def unique(x, out=None, temp=None):
+def unique(x, out=None, temp=None, read_count=True):
     out = out or DeviceArray(x.n, x.dtype)
     num = DeviceArray(1, U64)
     _run("thrust_amd_unique", temp, lambda fn, t, b: fn(
         t, b, x.ptr, out.ptr, num.ptr, x.n, x.dtype, stream_ptr()))
-    return out, _count(num)
+    return out, _count(num, read_count)
 
 
-def unique_by_key(keys, values, keys_out=None, values_out=None, temp=None):
+def unique_by_key(keys, values, keys_out=None, values_out=None, temp=None, read_count=True):
     keys_out = keys_out or DeviceArray(keys.n, keys.dtype)
     values_out = values_out or DeviceArray(values.n, values.dtype)
     num = DeviceArray(1, U64)
     _run("thrust_amd_unique_by_key", temp, lambda fn, t, b: fn(
         t, b, keys.ptr, values.ptr, keys_out.ptr, values_out.ptr, num.ptr, keys.n, keys.dtype,
         values.itemsize, stream_ptr()))
-    return keys_out, values_out, _count(num)
+    return keys_out, values_out, _count(num, read_count)
 
 
-def reduce_by_key(keys, values, op=PLUS, temp=None, keys_out=None, values_out=None):
+def reduce_by_key(keys, values, op=PLUS, temp=None, keys_out=None, values_out=None, read_count=True):
     keys_out = keys_out or DeviceArray(keys.n, keys.dtype)
     values_out = values_out or DeviceArray(values.n, values.dtype)
     num = DeviceArray(1, U64)
     _run("thrust_amd_reduce_by_key", temp, lambda fn, t, b: fn(
         t, b, keys.ptr, values.ptr, keys_out.ptr, values_out.ptr, num.ptr, keys.n, keys.dtype,
         values.dtype, op, stream_ptr()))
-    return keys_out, values_out, _count(num)
+    return keys_out, values_out, _count(num, read_count)
 
 
 def merge(a, b_, descending=False, out=None, temp=None):
@@ -399,23 +401,23 @@ def merge(a, b_, descending=False, out=None, temp=None):
     return out
 
 
-def set_operation(op, a, b_, descending=False, out=None, temp=None):
+def set_operation(op, a, b_, descending=False, out=None, temp=None, read_count=True):
     """Returns (out, length); out holds a.n + b.n elements unless the caller passes one."""
     out = out or DeviceArray(a.n + b_.n, a.dtype)
     num = DeviceArray(1, U64)
     _run("thrust_amd_set_operation", temp, lambda fn, t, b: fn(
         t, b, op, a.ptr, a.n, b_.ptr, b_.n, out.ptr, num.ptr, a.dtype, int(descending), stream_ptr()))
-    return out, _count(num)
+    return out, _count(num, read_count)
 
 
-def set_operation_by_key(op, ka, kb, va, vb, descending=False, temp=None, keys_out=None, values_out=None):
+def set_operation_by_key(op, ka, kb, va, vb, descending=False, temp=None, keys_out=None, values_out=None, read_count=True):
     keys_out = keys_out or DeviceArray(ka.n + kb.n, ka.dtype)
     values_out = values_out or DeviceArray(ka.n + kb.n, va.dtype)
     num = DeviceArray(1, U64)
     _run("thrust_amd_set_operation_by_key", temp, lambda fn, t, b: fn(
         t, b, op, ka.ptr, ka.n, kb.ptr, kb.n, va.ptr, vb.ptr if vb is not None else None, keys_out.ptr,
         values_out.ptr, num.ptr, ka.dtype, va.itemsize, int(descending), stream_ptr()))
-    return keys_out, values_out, _count(num)
+    return keys_out, values_out, _count(num, read_count)
 
 
 def merge_by_key(ka, kb, va, vb, descending=False, temp=None, keys_out=None, values_out=None):
