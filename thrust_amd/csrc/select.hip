@@ -30,23 +30,23 @@ namespace ta {
 
 enum SelectFlagMode { FLAG_PRED = 0, FLAG_HEAD = 1, FLAG_BYTE = 2 };
 
-// Two shapes.  Without a payload and with elements of up to four bytes, 16 elements per
-// lane keep the kernel within 64 registers, so two 1024-thread workgroups share a CU and
-// one loads while the other waits for its prefix: that beats a larger tile (measured:
-// copy_if of 2^28 float32 0.40 ms against 0.45 ms with 32 elements per lane).  Every other
-// combination needs more registers than that anyway and takes a larger tile (192 bytes of
-// input per lane, at most 32 elements: narrow elements are unpacked into a register each),
-// because every tile draws a ticket from one counter and waits for the prefix to travel
-// to it, and both costs are per tile (unique_by_key of int32 + float32: 0.63 -> 0.57 ms;
-// 512-thread workgroups for these shapes were slower, 0.63 ms).
-constexpr int SELECT_BLOCK = 1024;
-constexpr int SELECT_LEAN_ITEMS = 16;
-// The head-flag form of the lean shape needs fewer registers per element (no threshold
-// compare, one flag source) and takes 20 elements per lane within the same 64 registers:
-// unique of 2^28 int32 0.46 -> 0.39 ms.  The predicate form at 20 spills 28 registers and
-// loses (copy_if 0.41 -> 0.55 ms).
-constexpr int SELECT_LEAN_HEAD_ITEMS = 20;
-constexpr int SELECT_LANE_BYTES = 192;
+// Two shapes.  What bounds this kernel is not arithmetic but how many bytes a CU holds while
+// its tiles wait for their prefix: a tile stays in registers from its load until every earlier
+// tile has published its count, and the memory system is only busy while loads are in flight.
+// Measured on 2^28 float32 (copy_if at 50 % / 5 %): 1024 threads x 16 elements, two workgroups
+// per CU (64 registers): 0.43 / 0.36 ms; 512 threads x 64 elements, two workgroups per CU
+// (128 registers, twice the bytes per CU): 0.38 / 0.31 ms; 32 or 48 elements, three or four
+// smaller workgroups per CU, 1024 x 32..64: all slower.  So: without a payload and with
+// elements of up to four bytes, 512 threads x 64 elements (56 in the head-flag form, whose
+// previous-element compare needs a few registers more: unique of 2^28 int32 0.39 -> 0.28 ms).
+// With a payload, 1024 threads and 256 bytes of input per lane (at most 32 elements: narrow
+// elements are unpacked into a register each), one workgroup per CU: unique_by_key of
+// int32 + float32 0.54 -> 0.50 ms against 192 bytes per lane.
+constexpr int SELECT_BLOCK = 1024;       // with a payload
+constexpr int SELECT_LEAN_BLOCK = 512;   // without
+constexpr int SELECT_LEAN_ITEMS = 64;
+constexpr int SELECT_LEAN_HEAD_ITEMS = 56;
+constexpr int SELECT_LANE_BYTES = 256;
 constexpr int SELECT_MIN_ITEMS = 8;   // sizes the descriptor array
 constexpr int SELECT_MAX_ITEMS = 32;
 
@@ -54,10 +54,8 @@ template <typename T, typename U, bool HAS_PAYLOAD, int MODE>
 struct SelectShape {
   static constexpr int VEC = Vec16<T>::N;
   static constexpr bool LEAN = !HAS_PAYLOAD && sizeof(T) <= 4;
-  static constexpr int BLOCK = SELECT_BLOCK;
-  // 8 = registers for two lean workgroups per CU (a few spilled registers in the head-flag
-  // form cost less than the second workgroup brings)
-  static constexpr int WAVES_PER_SIMD = LEAN ? 8 : 4;  // registers for two lean workgroups per CU
+  static constexpr int BLOCK = LEAN ? SELECT_LEAN_BLOCK : SELECT_BLOCK;
+  static constexpr int WAVES_PER_SIMD = 4;  // 128 registers: two lean workgroups per CU, or one with a payload
   static constexpr int BY_BYTES = SELECT_LANE_BYTES / (int)(sizeof(T) + (HAS_PAYLOAD ? sizeof(U) : 0));
   static constexpr int WANTED =
       LEAN ? (MODE == FLAG_HEAD ? SELECT_LEAN_HEAD_ITEMS : SELECT_LEAN_ITEMS)
