@@ -274,6 +274,17 @@ TA_DEVICE T wave_inclusive_scan(T v, Op op) {
 TA_DEVICE int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
 
 // Comparison against a threshold chosen at run time (thrust_amd_cmp codes).
+template <int CMP, typename T>
+TA_DEVICE bool apply_cmp_code(T x, T t) {
+  if constexpr (CMP == THRUST_AMD_LT) return x < t;
+  else if constexpr (CMP == THRUST_AMD_LE) return x <= t;
+  else if constexpr (CMP == THRUST_AMD_GT) return x > t;
+  else if constexpr (CMP == THRUST_AMD_GE) return x >= t;
+  else if constexpr (CMP == THRUST_AMD_EQ) return x == t;
+  else if constexpr (CMP == THRUST_AMD_NE) return x != t;
+  else return x != (T)0;
+}
+
 template <typename T>
 TA_DEVICE bool apply_cmp(int cmp, T x, T t) {
   const bool negate = (cmp & THRUST_AMD_CMP_NOT) != 0;  // uniform: the logical negation of the code
@@ -288,6 +299,21 @@ TA_DEVICE bool apply_cmp(int cmp, T x, T t) {
     default: r = x != (T)0; break;
   }
   return r != negate;
+}
+
+// Calls f(integral_constant<int, CODE>) for the comparison code inside `cmp` (without its
+// negation bit): one uniform branch for a whole tile instead of one per element.
+template <typename F>
+TA_DEVICE void with_cmp_code(int cmp, F&& f) {
+  switch (cmp & ~THRUST_AMD_CMP_NOT) {
+    case THRUST_AMD_LT: f(std::integral_constant<int, THRUST_AMD_LT>{}); break;
+    case THRUST_AMD_LE: f(std::integral_constant<int, THRUST_AMD_LE>{}); break;
+    case THRUST_AMD_GT: f(std::integral_constant<int, THRUST_AMD_GT>{}); break;
+    case THRUST_AMD_GE: f(std::integral_constant<int, THRUST_AMD_GE>{}); break;
+    case THRUST_AMD_EQ: f(std::integral_constant<int, THRUST_AMD_EQ>{}); break;
+    case THRUST_AMD_NE: f(std::integral_constant<int, THRUST_AMD_NE>{}); break;
+    default: f(std::integral_constant<int, THRUST_AMD_NONZERO>{}); break;
+  }
 }
 
 // ------------------------------------------------------------------ search
