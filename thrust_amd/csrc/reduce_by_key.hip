@@ -54,7 +54,8 @@ __global__ __launch_bounds__(256) void rbk_init_kernel(uint64_t* __restrict__ wo
 // tile needs ONE wave scan of pairs per wave.  (Lanes of a wave then read 16-byte pieces
 // 64 bytes apart; the four loads of a lane cover its cache lines completely.)
 template <typename K, typename V, typename Op>
-__global__ __launch_bounds__(RBK_BLOCK, 4) void rbk_kernel(RbkArgs<K, V> a) {
+__global__ __launch_bounds__((RbkItems<K, V>::block), 4) void rbk_kernel(RbkArgs<K, V> a) {
+  constexpr int RBK_BLOCK = RbkItems<K, V>::block;
   constexpr int VEC = Vec16<K>::N;
   constexpr int CHUNKS = RbkItems<K, V>::value / VEC >= 1 ? RbkItems<K, V>::value / VEC : 1;
   constexpr int ITEMS = CHUNKS * VEC;
@@ -218,7 +219,8 @@ static int rbk_run(void* temp, size_t* temp_bytes, const void* keys_in, const vo
                    hipStream_t stream) {
   constexpr int VEC = Vec16<K>::N;
   constexpr int CHUNKS = RbkItems<K, V>::value / VEC >= 1 ? RbkItems<K, V>::value / VEC : 1;
-  constexpr uint64_t TILE = (uint64_t)RBK_BLOCK * CHUNKS * VEC;
+  constexpr int BLOCK = RbkItems<K, V>::block;
+  constexpr uint64_t TILE = (uint64_t)BLOCK * CHUNKS * VEC;
   using Pair = SegPair<typename SegValue<V>::type>;
   constexpr int W = TileWords<Pair>::W;
   const uint64_t tiles = (n + TILE - 1) / TILE;
@@ -250,7 +252,7 @@ static int rbk_run(void* temp, size_t* temp_bytes, const void* keys_in, const vo
             a.status, words, a.ticket, d_num_runs);
   TA_CHECK_LAUNCH();
   if (n == 0) return 0;
-  TA_LAUNCH("reduce_by_key", stream, (rbk_kernel<K, V, Op>), dim3((uint32_t)tiles), dim3(RBK_BLOCK), a);
+  TA_LAUNCH("reduce_by_key", stream, (rbk_kernel<K, V, Op>), dim3((uint32_t)tiles), dim3(BLOCK), a);
   TA_CHECK_LAUNCH();
   return 0;
 }

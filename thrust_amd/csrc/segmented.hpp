@@ -18,12 +18,15 @@ constexpr int RBK_BLOCK = 1024;
 constexpr int SBK_BLOCK = 512;
 constexpr int RBK_ITEMS = 16;  // elements per lane
 
-// reduce_by_key with keys and values of up to four bytes takes 20 elements per lane: the
-// largest tile that still fits 128 registers (0.69 -> 0.66 ms and 0.63 -> 0.61 ms at 2^28 pairs;
-// 24 spill and lose again); wider elements stay at 16.
+// reduce_by_key with keys and values of up to four bytes: 512 threads x 28 elements per lane,
+// two workgroups per CU (127 registers) -- more bytes per CU wait for their prefix at a time
+// than with one workgroup of 1024 x 20 (0.65 -> 0.61 ms and 0.61 -> 0.57 ms at 2^28 pairs,
+// mean run 8 / 1000; 1024 x 24 spills and loses).  Wider elements stay at 1024 x 16.
 template <typename K, typename V>
 struct RbkItems {
-  static constexpr int value = (sizeof(K) <= 4 && sizeof(V) <= 4) ? 20 : RBK_ITEMS;
+  static constexpr bool NARROW = sizeof(K) <= 4 && sizeof(V) <= 4;
+  static constexpr int value = NARROW ? 28 : RBK_ITEMS;
+  static constexpr int block = NARROW ? 512 : RBK_BLOCK;
 };
 
 template <typename V>
