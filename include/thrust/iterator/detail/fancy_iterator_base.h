@@ -58,6 +58,9 @@ template <typename T> inline T* device_view(T* p) { return p; }
 template <typename T> inline T* device_view(const device_ptr<T>& p) { return p.get(); }
 template <typename It>
 inline auto device_view(const It& it) -> decltype(it.device_view()) { return it.device_view(); }
+// an iterator type of the user's own travels as it is
+template <typename It>
+inline typename std::enable_if<is_user_device_iterator<It>::value, It>::type device_view(const It& it) { return it; }
 template <typename It>
 struct device_view_of { typedef decltype(device_view(std::declval<const It&>())) type; };
 

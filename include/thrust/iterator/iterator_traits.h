@@ -8,10 +8,25 @@
 
 namespace thrust {
 
+// thrust::iterator_traits: std::iterator_traits unless a user specialises it for an iterator
+// type of their own (the reference's tests do so for iterators that only define what an
+// algorithm needs, testing/scan.cu:586-594).
 template <typename It>
-struct iterator_value { typedef typename std::iterator_traits<It>::value_type type; };
+struct iterator_traits : std::iterator_traits<It> {};
+
+namespace detail {
+template <typename Traits, typename = void>
+struct difference_of { typedef std::ptrdiff_t type; };
+template <typename Traits>
+struct difference_of<Traits, typename std::enable_if<!std::is_void<typename Traits::difference_type>::value>::type> {
+  typedef typename Traits::difference_type type;
+};
+}  // namespace detail
+
 template <typename It>
-struct iterator_difference { typedef typename std::iterator_traits<It>::difference_type type; };
+struct iterator_value { typedef typename thrust::iterator_traits<It>::value_type type; };
+template <typename It>
+struct iterator_difference { typedef typename detail::difference_of<thrust::iterator_traits<It> >::type type; };
 
 // The system an iterator belongs to: device_ptr -> device system, anything else -> host.
 template <typename It>
@@ -28,6 +43,25 @@ template <typename T> struct is_device_iterator<device_ptr<T> > : std::true_type
 struct fancy_iterator_marker {};
 template <typename It>
 struct is_fancy_iterator : std::is_base_of<fancy_iterator_marker, It> {};
+// ... and those that take writes (discard_iterator) from this as well.
+struct fancy_output_marker {};
+template <typename It>
+struct is_fancy_output_iterator : std::is_base_of<fancy_output_marker, It> {};
+
+// An iterator type of the user's own, handed to kernels by value under a device policy: a
+// class that is none of the library's iterators and that std::iterator_traits does not know
+// (so not a container's iterator either).  Its operator[] and the assignment to what that
+// returns must be callable in device code.
+template <typename It, typename = void>
+struct is_std_iterator : std::false_type {};
+template <typename It>
+struct is_std_iterator<It, typename std::enable_if<!std::is_void<typename std::iterator_traits<It>::iterator_category>::value>::type>
+    : std::true_type {};
+template <typename It>
+struct is_user_device_iterator
+    : std::integral_constant<bool, std::is_class<It>::value && std::is_trivially_copyable<It>::value &&
+                                       !is_device_iterator<It>::value && !is_fancy_iterator<It>::value &&
+                                       !is_std_iterator<It>::value> {};
 
 // Raw address of the element an iterator points at.  Device iterators are device_ptr or,
 // under an explicit device policy, plain pointers; host iterators must be contiguous

@@ -205,13 +205,13 @@ Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T i
 // units).  A is the accumulator's type, as in the library path.
 template <bool EXCLUSIVE, typename A, typename D, typename In, typename Out, typename Op>
 Out scan_generic(execution_policy<D>& exec, In first, In last, Out result, A init, Op op) {
-  static_assert(is_device_input<In>::value &&
-                    (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value),
-                "scan on the device system needs device_ptr / device_vector iterators or raw device pointers "
-                "(fancy iterators as input only)");
+  static_assert(is_device_input<In>::value && is_device_output<Out>::value,
+                "scan on the device system needs device_ptr / device_vector iterators, raw device pointers, fancy "
+                "iterators, or for the output an iterator type that kernels can take by value");
 #if defined(__HIPCC__)
   namespace gk = thrust::system::hip::generic;
   typedef typename thrust::detail::device_view_of<In>::type View;
+  typedef typename thrust::detail::device_view_of<Out>::type OutView;
   typedef typename iterator_value<Out>::type U;
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
@@ -253,13 +253,13 @@ Out scan_generic(execution_policy<D>& exec, In first, In last, Out result, A ini
   throw_on_error(launch_status(), "scan: kernel launch");
   for (int k = levels - 1; k >= 1; --k) {
     // in place: a workgroup reads its tile into registers before it writes
-    hipLaunchKernelGGL((gk::scan_tiles_kernel<false, const A*, A, A, Op>), dim3((unsigned)count[k]), dim3(gk::BLOCK), 0,
+    hipLaunchKernelGGL((gk::scan_tiles_kernel<false, const A*, A, A, A*, Op>), dim3((unsigned)count[k]), dim3(gk::BLOCK), 0,
                        (hipStream_t)stream, (const A*)level[k - 1], level[k - 1], count[k - 1], op, init,
                        (const A*)level[k]);
     throw_on_error(launch_status(), "scan: kernel launch");
   }
-  hipLaunchKernelGGL((gk::scan_tiles_kernel<EXCLUSIVE, View, A, U, Op>), dim3((unsigned)tiles), dim3(gk::BLOCK), 0,
-                     (hipStream_t)stream, thrust::detail::device_view(first), thrust::detail::raw(result), n, op, init,
+  hipLaunchKernelGGL((gk::scan_tiles_kernel<EXCLUSIVE, View, A, U, OutView, Op>), dim3((unsigned)tiles), dim3(gk::BLOCK), 0,
+                     (hipStream_t)stream, thrust::detail::device_view(first), thrust::detail::device_view(result), n, op, init,
                      (const A*)tile_total);
   throw_on_error(launch_status(), "scan: kernel launch");
   synchronize(stream, "scan: synchronize");
@@ -293,13 +293,19 @@ template <typename D, typename In, typename Out, typename Op>
 Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op op) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
   typedef typename iterator_value<Out>::type U;
-  return detail::inclusive_scan(exec, first, last, result, op, detail::scans_in_library<V, U, V, Op>());
+  // the library's kernels write arrays; any other output (an iterator type of the caller's own,
+  // discard_iterator) is written by the generic kernels, which take it by value
+  typedef std::integral_constant<bool, detail::scans_in_library<V, U, V, Op>::value &&
+                                           (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value)> in_library;
+  return detail::inclusive_scan(exec, first, last, result, op, in_library());
 }
 template <typename D, typename In, typename Out, typename T, typename Op>
 Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T init, Op op) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
   typedef typename iterator_value<Out>::type U;
-  return detail::exclusive_scan(exec, first, last, result, init, op, detail::scans_in_library<V, U, T, Op>());
+  typedef std::integral_constant<bool, detail::scans_in_library<V, U, T, Op>::value &&
+                                           (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value)> in_library;
+  return detail::exclusive_scan(exec, first, last, result, init, op, in_library());
 }
 
 namespace detail {

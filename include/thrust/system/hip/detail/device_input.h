@@ -27,7 +27,9 @@ struct is_device_input
 // Where kernels that take iterators by value may write: device memory, or a zip of such.
 template <typename It>
 struct is_device_output
-    : std::integral_constant<bool, std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value> {};
+    : std::integral_constant<bool, std::is_pointer<It>::value || thrust::detail::is_device_iterator<It>::value ||
+                                       thrust::detail::is_user_device_iterator<It>::value ||
+                                       thrust::detail::is_fancy_output_iterator<It>::value> {};
 
 template <>
 struct is_device_output<thrust::zip_iterator<thrust::tuple<> > > : std::true_type {};

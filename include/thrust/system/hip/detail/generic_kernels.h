@@ -259,8 +259,9 @@ __global__ __launch_bounds__(BLOCK) void scan_tile_prefix_kernel(T* tile_total, 
 //   inclusive:  out[i] = x0 + ... + xi                    (init is not used)
 //   exclusive:  out[i] = init + x0 + ... + x(i-1)
 // out may be the input itself: a tile is read completely before any of it is written.
-template <bool EXCLUSIVE, typename View, typename T, typename U, typename Op>
-__global__ __launch_bounds__(BLOCK) void scan_tiles_kernel(View first, U* out, uint64_t n, Op op, T init,
+// out: a pointer, or any iterator that kernels can take by value (out[i] = value)
+template <bool EXCLUSIVE, typename View, typename T, typename U, typename OutView, typename Op>
+__global__ __launch_bounds__(BLOCK) void scan_tiles_kernel(View first, OutView out, uint64_t n, Op op, T init,
                                                            const T* tile_prefix) {
   THRUST_AMD_SCAN_SHARED(T)
   const uint64_t tile_base = (uint64_t)blockIdx.x * S::TILE;

@@ -14,6 +14,7 @@
 #include <thrust/host_vector.h>
 #include <thrust/inner_product.h>
 #include <thrust/iterator/constant_iterator.h>
+#include <thrust/iterator/discard_iterator.h>
 #include <thrust/iterator/counting_iterator.h>
 #include <thrust/iterator/permutation_iterator.h>
 #include <thrust/iterator/transform_iterator.h>
@@ -408,6 +409,84 @@ static void TestReduceWithBigIndexes() {
   ASSERT_TRUE(sum == (long long)((unsigned long long)n * (unsigned long long)(n - 1) / 2));
 }
 
+// testing/scan.cu:563-663 and testing/copy.cu:713-781: ranges of 2^30 .. 2^33 elements that exist
+// only as an iterator, written through an iterator of the test's own that remembers whether
+// the one expected value came by.  Nothing is stored: only the 64-bit indexing is on trial.
+struct only_set_when_expected_it {
+  long long expected;
+  bool* flag;
+  __host__ __device__ only_set_when_expected_it operator++() const { return *this; }
+  __host__ __device__ only_set_when_expected_it operator*() const { return *this; }
+  template <typename Difference>
+  __host__ __device__ only_set_when_expected_it operator+(Difference) const { return *this; }
+  template <typename Difference>
+  __host__ __device__ only_set_when_expected_it operator+=(Difference) const { return *this; }
+  template <typename Index>
+  __host__ __device__ only_set_when_expected_it operator[](Index) const { return *this; }
+  __device__ void operator=(long long value) const {
+    if (value == expected) *flag = true;
+  }
+};
+namespace thrust {
+template <>
+struct iterator_traits<only_set_when_expected_it> {
+  typedef long long value_type;
+  typedef only_set_when_expected_it reference;
+};
+}  // namespace thrust
+
+static void TestScanAndCopyWithBigIndexes() {
+  g_test = "ScanAndCopyWithBigIndexes";
+  thrust::device_vector<bool> flag(1);
+  for (int magnitude = 30; magnitude <= 33; ++magnitude) {
+    const long long n = 1ll << magnitude;
+    thrust::constant_iterator<long long> ones(1);
+    flag[0] = false;
+    only_set_when_expected_it last_of_inclusive = {n, thrust::raw_pointer_cast(flag.data())};
+    thrust::inclusive_scan(thrust::device, ones, ones + n, last_of_inclusive);
+    ASSERT_TRUE((bool)flag[0]);
+    flag[0] = false;
+    only_set_when_expected_it last_of_exclusive = {n - 1, thrust::raw_pointer_cast(flag.data())};
+    thrust::exclusive_scan(thrust::device, ones, ones + n, last_of_exclusive, 0ll);
+    ASSERT_TRUE((bool)flag[0]);
+    flag[0] = false;
+    thrust::counting_iterator<long long> index(0);
+    only_set_when_expected_it last_index = {n - 1, thrust::raw_pointer_cast(flag.data())};
+    thrust::copy(thrust::device, index, index + n, last_index);
+    ASSERT_TRUE((bool)flag[0]);
+  }
+  // a value that never comes by leaves the flag alone
+  flag[0] = false;
+  thrust::constant_iterator<long long> ones(1);
+  only_set_when_expected_it never = {-5, thrust::raw_pointer_cast(flag.data())};
+  thrust::inclusive_scan(thrust::device, ones, ones + (1ll << 20), never);
+  ASSERT_TRUE(!(bool)flag[0]);
+}
+
+// thrust::discard_iterator as the output nobody wants, and an operator of another type than
+// the elements: inclusive_scan of floats with plus<int> keeps the first element as it is and
+// adds the others as integers (testing/scan.cu:257-262).
+static void TestDiscardAndForeignOperator() {
+  g_test = "DiscardIterator";
+  {
+    thrust::device_vector<int> d(hv<int>({1, 3, -2, 4, -5}));
+    thrust::discard_iterator<> sink;
+    auto end = thrust::inclusive_scan(thrust::device, d.begin(), d.end(), sink);
+    ASSERT_TRUE(end - sink == 5);
+    auto end2 = thrust::copy(thrust::device, thrust::counting_iterator<int>(0), thrust::counting_iterator<int>(1000), sink);
+    ASSERT_TRUE(end2 - sink == 1000);
+  }
+  g_test = "ScanMixedTypesForeignOperator";
+  {
+    thrust::device_vector<float> in(hv<float>({1.5f, 2.5f, 3.5f, 4.5f})), out(4);
+    thrust::inclusive_scan(in.begin(), in.end(), out.begin(), thrust::plus<int>());
+    ASSERT_TRUE(same(to_host(out), hv<float>({1.5f, 3.0f, 6.0f, 10.0f})));
+    thrust::host_vector<float> hin = in, hout(4);
+    thrust::inclusive_scan(hin.begin(), hin.end(), hout.begin(), thrust::plus<int>());
+    ASSERT_TRUE(same(hout, hv<float>({1.5f, 3.0f, 6.0f, 10.0f})));
+  }
+}
+
 static void TestKnownAnswers() {
   g_test = "GatherSimple";
   {
@@ -600,6 +679,8 @@ static void Differential() {
 int main() {
   TestKnownAnswers();
   TestReduceWithBigIndexes();
+  TestScanAndCopyWithBigIndexes();
+  TestDiscardAndForeignOperator();
   Differential();
   TestUserOperators();
   TestWideElements();
