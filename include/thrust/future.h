@@ -14,6 +14,7 @@
 // .after(...); else a new stream of its own.  The work starts only after every dependency
 // has finished; a dependency stays usable (its stream is shared, not taken away).
 #pragma once
+#include <atomic>
 #include <cstddef>
 #include <memory>
 #include <utility>
@@ -27,10 +28,19 @@ namespace system {
 namespace hip {
 
 namespace detail {
+// enqueued counts the pieces of work the library has put on the stream, synced how many of
+// them a host-side wait has seen finished: an event whose number is not above `synced` is
+// complete without asking the runtime (which, after a wait on an idle stream's event, can go
+// on answering "not ready" for a stream that has been synchronised).
 struct stream_state {
   void* stream;
   bool owned;
-  stream_state(void* s, bool o) : stream(s), owned(o) {}
+  std::atomic<unsigned long long> enqueued, synced;
+  stream_state(void* s, bool o) : stream(s), owned(o), enqueued(0), synced(0) {}
+  void mark_synced(unsigned long long upto) {
+    unsigned long long seen = synced.load();
+    while (seen < upto && !synced.compare_exchange_weak(seen, upto)) {}
+  }
   ~stream_state() {
     if (owned && stream) {
       (void)thrust_amd_stream_synchronize(stream);
@@ -44,6 +54,7 @@ struct stream_state {
 // their registration, the stream last.
 struct keep_alive {
   std::shared_ptr<stream_state> stream;
+  unsigned long long ticket = 0;  // the work's number on its stream (stream_state::enqueued)
   std::vector<std::shared_ptr<void> > resources;
   ~keep_alive() {
     while (!resources.empty()) resources.pop_back();
@@ -82,21 +93,36 @@ class unique_eager_event {
   bool valid_stream() const { return stream_.valid(); }
   unique_stream& stream() { return stream_; }
   const unique_stream& stream() const { return stream_; }
+  // Once the work has been seen complete it stays complete, whatever is enqueued on the
+  // (shared) stream afterwards; the runtime is only asked while that is not yet known.
   bool ready() const {
-    if (!valid_stream()) return true;
+    if (!valid_stream() || complete()) return true;
     int done = 0;
     detail::throw_on_error(thrust_amd_stream_query(stream_.native_handle(), &done), "stream query failed");
+    if (done) done_ = true;
     return done != 0;
   }
   void wait() const {
-    if (valid_stream())
-      detail::throw_on_error(thrust_amd_stream_synchronize(stream_.native_handle()), "waiting for asynchronous work failed");
+    if (!valid_stream() || complete()) return;
+    const std::shared_ptr<detail::stream_state>& st = stream_.state();
+    const unsigned long long upto = st->enqueued.load();  // everything enqueued before the wait
+    detail::throw_on_error(thrust_amd_stream_synchronize(stream_.native_handle()), "waiting for asynchronous work failed");
+    st->mark_synced(upto);
+    done_ = true;
   }
   const std::shared_ptr<detail::keep_alive>& keep() const { return keep_; }
 
  protected:
   std::shared_ptr<detail::keep_alive> keep_;
   unique_stream stream_;
+  mutable bool done_ = false;
+
+ private:
+  bool complete() const {
+    if (done_) return true;
+    if (keep_ && keep_->ticket != 0 && keep_->ticket <= stream_.state()->synced.load()) done_ = true;
+    return done_;
+  }
 };
 
 template <typename T>
@@ -191,6 +217,7 @@ inline async_context make_context(void* on_stream, bool has_stream, const depend
   if (has_stream) ctx.keep->stream = std::make_shared<stream_state>(on_stream, false);
   else if (deps && !deps->items.empty()) ctx.keep->stream = deps->items.front()->stream;
   else ctx.keep->stream = unique_stream::create().state();
+  ctx.keep->ticket = ++ctx.keep->stream->enqueued;
   if (deps)
     for (const auto& d : deps->items) {
       wait_for(ctx.stream(), d);
@@ -251,6 +278,20 @@ template <typename... Events>
 inline void when_all_wait(const Events&... events) {
   const int dummy[] = {0, (events.wait(), 0)...};
   (void)dummy;
+}
+
+// when_all(a, b, ...): an event that is complete once every event or future given is
+// (thrust/system/cuda/detail/future.inl:1350-1362).  No work is enqueued: the result lives on
+// the first argument's stream, which is made to wait for the others on the device, and keeps
+// alive what they keep alive.  With no arguments the event is complete at once.
+template <typename... Events>
+inline device_event when_all(const Events&... events) {
+  system::hip::dependency_list deps;
+  const int dummy[] = {0, (deps.add(events), 0)...};
+  (void)dummy;
+  if (deps.items.empty()) return device_event();
+  system::hip::detail::async_context ctx = system::hip::detail::make_context(nullptr, false, &deps);
+  return device_event(ctx.keep);
 }
 
 }  // namespace thrust

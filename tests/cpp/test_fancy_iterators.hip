@@ -13,6 +13,9 @@
 #include <thrust/gather.h>
 #include <thrust/host_vector.h>
 #include <thrust/inner_product.h>
+#include <thrust/async/for_each.h>
+#include <thrust/async/transform.h>
+#include <thrust/future.h>
 #include <thrust/iterator/constant_iterator.h>
 #include <thrust/iterator/discard_iterator.h>
 #include <thrust/iterator/counting_iterator.h>
@@ -487,6 +490,47 @@ static void TestDiscardAndForeignOperator() {
   }
 }
 
+// thrust::async::for_each / transform with functors of the test's own, and when_all
+// (testing/async_for_each.cu:20-60, testing/async_transform.cu:30-90: the asynchronous result
+// equals the synchronous algorithm's; the event is waited for before the data is read).
+struct add_seven { __host__ __device__ void operator()(int& x) const { x += 7; } };
+struct times_three { __host__ __device__ long long operator()(int x) const { return 3ll * x; } };
+static void TestAsyncForEachTransformWhenAll() {
+  g_test = "AsyncForEachTransformWhenAll";
+  for (size_t n : {(size_t)0, (size_t)1, (size_t)1000, ((size_t)1 << 20) + 3}) {
+    thrust::host_vector<int> h(n);
+    for (size_t i = 0; i < n; ++i) h[i] = (int)(i * 2654435761u >> 8);
+    thrust::device_vector<int> a = h, b = h;
+    thrust::device_vector<long long> out(n);
+    thrust::device_event e1 = thrust::async::for_each(a.begin(), a.end(), add_seven());
+    thrust::device_event e2 = thrust::async::transform(thrust::device, b.begin(), b.end(), out.begin(), times_three());
+    thrust::device_event both = thrust::when_all(e1, e2);
+    both.wait();
+    ASSERT_TRUE(both.ready());
+    ASSERT_TRUE(e1.ready());
+    e2.wait();
+    ASSERT_TRUE(e2.ready());
+    thrust::host_vector<int> ha = a;
+    thrust::host_vector<long long> ho = out;
+    bool ok = true;
+    for (size_t i = 0; i < n; ++i) ok = ok && ha[i] == h[i] + 7 && ho[i] == 3ll * h[i];
+    ASSERT_TRUE(ok);
+    // chained: the transform starts after the for_each it depends on, on the same stream
+    thrust::device_event e3 = thrust::async::for_each(a.begin(), a.end(), add_seven());
+    void* s3 = e3.stream().native_handle();
+    thrust::device_event e4 = thrust::async::transform(thrust::device.after(e3), a.begin(), a.end(), out.begin(), times_three());
+    ASSERT_TRUE(e4.stream().native_handle() == s3);
+    e4.wait();
+    ho = out;
+    ok = true;
+    for (size_t i = 0; i < n; ++i) ok = ok && ho[i] == 3ll * (h[i] + 14);
+    ASSERT_TRUE(ok);
+  }
+  thrust::device_event none = thrust::when_all();
+  ASSERT_TRUE(none.ready());
+  none.wait();
+}
+
 static void TestKnownAnswers() {
   g_test = "GatherSimple";
   {
@@ -681,6 +725,7 @@ int main() {
   TestReduceWithBigIndexes();
   TestScanAndCopyWithBigIndexes();
   TestDiscardAndForeignOperator();
+  TestAsyncForEachTransformWhenAll();
   Differential();
   TestUserOperators();
   TestWideElements();

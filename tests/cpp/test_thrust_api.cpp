@@ -25,7 +25,11 @@
 #include <thrust/inner_product.h>
 #include <thrust/merge.h>
 #include <thrust/mr/allocator.h>
+#include <thrust/mr/disjoint_pool.h>
+#include <thrust/mr/disjoint_sync_pool.h>
+#include <thrust/mr/new.h>
 #include <thrust/mr/pool.h>
+#include <thrust/mr/sync_pool.h>
 #include <thrust/partition.h>
 #include <thrust/reduce.h>
 #include <thrust/remove.h>
@@ -37,12 +41,14 @@
 #include <thrust/unique.h>
 #include <thrust/universal_vector.h>
 
+#include <atomic>
 #include <cstdint>
 #include <cstdio>
 #include <cstring>
 #include <functional>
 #include <limits>
 #include <string>
+#include <thread>
 #include <vector>
 
 static int g_failed = 0, g_checks = 0;
@@ -1241,6 +1247,87 @@ static void TestTempArenaOutlivesStream() {
   ASSERT_TRUE(thrust_amd_temp_bytes_held() == 0);
 }
 
+// The other pool resources: the disjoint pool (bookkeeping in host memory, blocks carved from
+// chunks), and the two mutex-guarded wrappers shared by several host threads
+// (testing/mr_disjoint_pool.cu and testing/mr_pool.cu check the same behaviour: reuse of
+// returned blocks, chunk growth, oversized blocks, release).
+static void TestPoolResources() {
+  g_test = "DisjointPool";
+  typedef thrust::mr::disjoint_unsynchronized_pool_resource<thrust::device_memory_resource> Disjoint;
+  thrust::device_memory_resource upstream;
+  thrust::mr::new_delete_resource book;
+  {
+    Disjoint pool(&upstream, &book);
+    // 16 blocks of 256 bytes per first chunk: 17 allocations take two chunks
+    std::vector<thrust::device_ptr<void> > blocks;
+    for (int i = 0; i < 17; ++i) blocks.push_back(pool.allocate(200));
+    ASSERT_TRUE(pool.chunks() == 2 && pool.upstream_allocations() == 2);
+    bool distinct = true, aligned = true;
+    for (size_t i = 0; i < blocks.size(); ++i) {
+      aligned = aligned && (reinterpret_cast<std::uintptr_t>(blocks[i].get()) % 256 == 0);
+      for (size_t j = 0; j < i; ++j) distinct = distinct && blocks[i].get() != blocks[j].get();
+    }
+    ASSERT_TRUE(distinct && aligned);
+    // a returned block is the next one handed out for its size
+    pool.deallocate(blocks[5], 200);
+    thrust::device_ptr<void> again = pool.allocate(256);
+    ASSERT_TRUE(again.get() == blocks[5].get() && pool.upstream_allocations() == 2);
+    // the blocks are device memory: fill one and read it back
+    thrust::device_ptr<int> ints(static_cast<int*>(blocks[3].get()));
+    thrust::fill(ints, ints + 50, 7);
+    ASSERT_TRUE(thrust::reduce(ints, ints + 50) == 350);
+    // oversized blocks are cached and reused for requests of a similar size
+    thrust::device_ptr<void> big = pool.allocate((size_t)3 << 20);
+    const size_t calls = pool.upstream_allocations();
+    pool.deallocate(big, (size_t)3 << 20);
+    ASSERT_TRUE(pool.cached_oversized_blocks() == 1);
+    thrust::device_ptr<void> big2 = pool.allocate((size_t)2 << 20);
+    ASSERT_TRUE(big2.get() == big.get() && pool.upstream_allocations() == calls);
+    pool.deallocate(big2, (size_t)2 << 20);
+    for (auto& b : blocks) pool.deallocate(b, 200);
+    pool.release();
+    ASSERT_TRUE(pool.chunks() == 0 && pool.cached_oversized_blocks() == 0);
+    // vectors and temporary storage from the pool
+    typedef thrust::mr::allocator<int, Disjoint> Alloc;
+    Alloc alloc(&pool);
+    thrust::host_vector<int> h = random_integers<int>(5000, 21, 0), hs = h;
+    std::sort(hs.begin(), hs.end());
+    {
+      thrust::device_vector<int, Alloc> v(h.begin(), h.end(), alloc);
+      thrust::sort(thrust::device(&pool), v.begin(), v.end());
+      ASSERT_EQUAL_VEC(to_host(v), hs);
+    }
+    const size_t before = pool.upstream_allocations();
+    {
+      thrust::device_vector<int, Alloc> v(h.begin(), h.end(), alloc);
+      thrust::sort(thrust::device(&pool), v.begin(), v.end());
+      ASSERT_EQUAL_VEC(to_host(v), hs);
+    }
+    ASSERT_TRUE(pool.upstream_allocations() == before);  // everything came from the pool's chunks
+  }
+  g_test = "SynchronizedPools";
+  {
+    thrust::mr::synchronized_pool_resource<thrust::device_memory_resource> sync(&upstream);
+    thrust::mr::disjoint_synchronized_pool_resource<thrust::device_memory_resource> dsync(&upstream, &book);
+    std::atomic<int> bad(0);
+    auto worker = [&](int id) {
+      for (int round = 0; round < 200; ++round) {
+        const size_t bytes = 256 + 64 * (size_t)((id * 7 + round) % 9);
+        thrust::device_ptr<void> a = sync.allocate(bytes), b = dsync.allocate(bytes);
+        if (!a.get() || !b.get() || a.get() == b.get()) ++bad;
+        sync.deallocate(a, bytes);
+        dsync.deallocate(b, bytes);
+      }
+    };
+    std::thread t0(worker, 0), t1(worker, 1), t2(worker, 2), t3(worker, 3);
+    t0.join(); t1.join(); t2.join(); t3.join();
+    ASSERT_TRUE(bad.load() == 0);
+    ASSERT_TRUE(sync.upstream_allocations() <= 4 * 4 && dsync.upstream_allocations() <= 8);
+    sync.release();
+    dsync.release();
+  }
+}
+
 static void TestMemoryResources() {
   g_test = "MemoryResources";
   typedef thrust::mr::unsynchronized_pool_resource<thrust::device_memory_resource> Pool;
@@ -1352,6 +1439,7 @@ int main() {
   TestAsyncAlgorithms();
   TestTempArenaOutlivesStream();
   TestMemoryResources();
+  TestPoolResources();
   TestUniversalVector();
   std::printf("%s: %d checks, %d failed\n", g_failed ? "FAILED" : "PASSED", g_checks, g_failed);
   return g_failed ? 1 : 0;

@@ -22,11 +22,7 @@ namespace ta {
 // Tile shapes (threads x 16-byte vectors per lane).  The per-tile cost of the ticket
 // (a same-address atomic retires every ~12 ns on MI355X) and of the look-back makes large
 // tiles win once there are enough of them to fill 256 CUs; small inputs use small tiles.
-#ifndef TA_SCAN_LARGE_BLOCK
-#define TA_SCAN_LARGE_BLOCK 1024
-#define TA_SCAN_LARGE_CHUNKS 12
-#endif
-struct ScanShapeLarge { static constexpr int BLOCK = TA_SCAN_LARGE_BLOCK, CHUNKS = TA_SCAN_LARGE_CHUNKS; };
+struct ScanShapeLarge { static constexpr int BLOCK = 1024, CHUNKS = 12; };
 struct ScanShapeSmall { static constexpr int BLOCK = 256, CHUNKS = 4; };
 constexpr uint64_t SCAN_LARGE_MIN_BYTES = (uint64_t)32 << 20;
 
