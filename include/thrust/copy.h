@@ -243,7 +243,6 @@ Out copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred)
 template <typename D, typename In, typename St, typename Out, typename Pred>
 Out copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result, Pred pred) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
   static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
                 "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
   return detail::copy_if_impl(exec, first, last, stencil, true, result, pred, false);

@@ -74,11 +74,10 @@ pair<KOut, VOut> reduce_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, KOu
   typedef typename iterator_value<VIt>::type V;
   if (kf == kl) return thrust::make_pair(ko, vo);
   K run_key = *kf;
-  K prev = run_key;
   V acc = *vf;
   for (++kf, ++vf; kf != kl; ++kf, ++vf) {
     const K k = *kf;
-    if (pred(prev, k)) {
+    if (pred(run_key, k)) {  // against the key that opened the run, not the previous one
       acc = op(acc, *vf);
     } else {
       *ko = run_key; ++ko;
@@ -86,7 +85,6 @@ pair<KOut, VOut> reduce_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, KOu
       run_key = k;
       acc = *vf;
     }
-    prev = k;
   }
   *ko = run_key; ++ko;
   *vo = acc; ++vo;
@@ -100,7 +98,6 @@ namespace hip {
 namespace detail {
 template <typename D, typename It, typename T, typename Op>
 T reduce(execution_policy<D>& exec, It first, It last, T init, Op, std::true_type) {
-  typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   device_input<It> source(stream, temp_source_of(exec), first, n);

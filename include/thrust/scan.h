@@ -181,7 +181,6 @@ Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op,
 
 template <typename D, typename In, typename Out, typename T, typename Op>
 Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T init, Op, std::true_type) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
   typedef typename iterator_value<Out>::type U;
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);

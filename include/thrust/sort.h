@@ -11,6 +11,8 @@
 // translation unit compiled by a plain host compiler stops there with a message.
 #pragma once
 #include <algorithm>
+#include <cstdint>
+#include <cstring>
 #include <numeric>
 #include <tuple>
 #include <vector>
@@ -65,18 +67,66 @@ void stable_sort_by_key(thrust::execution_policy<D>& exec, KIt kf, KIt kl, VIt v
 }  // namespace detail
 
 namespace cpp {
+namespace detail {
+// The reference's host system sorts arithmetic keys under thrust::less / thrust::greater with
+// its radix sort (thrust/system/detail/sequential/sort.inl:139-148), i.e. by the keys' radix
+// encoding (stable_radix_sort.inl:52-130): floating-point keys are ordered by their bits, -0.0
+// before +0.0 and NaNs beyond the infinities of their sign, where operator< would call them
+// equivalent or unordered.  rank() is that encoding; for integers it is the key itself.
+template <typename K>
+inline K rank(K k, std::false_type) { return k; }
+inline std::uint32_t rank(float k, std::true_type) {
+  std::uint32_t b;
+  std::memcpy(&b, &k, sizeof b);
+  return b ^ ((b >> 31) ? 0xFFFFFFFFu : 0x80000000u);
+}
+inline std::uint64_t rank(double k, std::true_type) {
+  std::uint64_t b;
+  std::memcpy(&b, &k, sizeof b);
+  return b ^ ((b >> 63) ? ~std::uint64_t(0) : (std::uint64_t(1) << 63));
+}
+template <typename K>
+struct has_bit_rank : std::integral_constant<bool, std::is_same<K, float>::value || std::is_same<K, double>::value> {};
+
+// CODE: 0 = thrust::less<K>, 1 = thrust::greater<K> on an arithmetic K, < 0 anything else
+template <int CODE, typename K, typename Comp>
+struct key_order {
+  Comp comp;
+  bool operator()(const K& a, const K& b) const { return comp(a, b); }
+};
+template <typename K, typename Comp>
+struct key_order<0, K, Comp> {
+  Comp comp;
+  bool operator()(const K& a, const K& b) const { return rank(a, has_bit_rank<K>()) < rank(b, has_bit_rank<K>()); }
+};
+template <typename K, typename Comp>
+struct key_order<1, K, Comp> {
+  Comp comp;
+  bool operator()(const K& a, const K& b) const { return rank(b, has_bit_rank<K>()) < rank(a, has_bit_rank<K>()); }
+};
+template <typename K, typename Comp>
+key_order<(!std::is_arithmetic<K>::value ? -1
+           : std::is_same<Comp, thrust::less<K> >::value ? 0
+           : std::is_same<Comp, thrust::greater<K> >::value ? 1 : -1), K, Comp>
+order_of(Comp comp) {
+  return {comp};
+}
+}  // namespace detail
+
 template <typename D, typename It, typename Comp>
 void stable_sort(execution_policy<D>&, It first, It last, Comp comp) {
-  std::stable_sort(first, last, comp);
+  typedef typename std::remove_const<typename iterator_value<It>::type>::type K;
+  std::stable_sort(first, last, detail::order_of<K>(comp));
 }
 template <typename D, typename KIt, typename VIt, typename Comp>
 void stable_sort_by_key(execution_policy<D>&, KIt kf, KIt kl, VIt vf, Comp comp) {
   typedef typename iterator_value<KIt>::type K;
   typedef typename iterator_value<VIt>::type V;
   const std::size_t n = (std::size_t)(kl - kf);
+  const auto before = detail::order_of<K>(comp);
   std::vector<std::size_t> order(n);
   std::iota(order.begin(), order.end(), std::size_t(0));
-  std::stable_sort(order.begin(), order.end(), [&](std::size_t a, std::size_t b) { return comp(kf[a], kf[b]); });
+  std::stable_sort(order.begin(), order.end(), [&](std::size_t a, std::size_t b) { return before(kf[a], kf[b]); });
   std::vector<K> k(n);
   std::vector<V> v(n);
   for (std::size_t i = 0; i < n; ++i) { k[i] = kf[order[i]]; v[i] = vf[order[i]]; }

@@ -320,8 +320,10 @@ class Reference(_Base):
     prefix = "ref_"
     threaded = False
 
-    def __init__(self, kind):
-        super().__init__(REF_LIBS[kind])
+    def __init__(self, kind, path=None):
+        """path: another build of ref_driver.cpp with the same exports (the tests compile it
+        against this repository's own headers to check their host system)."""
+        super().__init__(path or REF_LIBS[kind])
         self.kind = kind
 
     # The real mixed-type calls, int32 <-> float32 only: these run the reference's own type

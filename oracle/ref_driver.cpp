@@ -7,6 +7,12 @@
 // interface as thrust_oracle.c, so that tests can compare the restatement with the
 // real thing and write golden vectors, and the benchmark can time the reference's
 // OMP path as CPU baseline.  Built only into oracle/_ref/, which is not committed.
+//
+// The same file also compiles against any other implementation of the same API: with
+// -DDRIVER_POLICY=thrust::host -DDRIVER_HOST_POINTERS every call below runs on the host
+// system of whichever <thrust/...> headers are first on the include path, over raw
+// pointers.  The tests build it that way against this repository's own headers to compare
+// their host system with the reference's, call for call.
 #include <thrust/copy.h>
 #include <thrust/count.h>
 #include <thrust/device_ptr.h>
@@ -32,8 +38,16 @@
 
 namespace {
 
+#ifndef DRIVER_POLICY
+#define DRIVER_POLICY thrust::device
+#endif
+#ifdef DRIVER_HOST_POINTERS
+template <typename T> T* dp(void* p) { return (T*)p; }
+template <typename T> const T* dp(const void* p) { return (const T*)p; }
+#else
 template <typename T> thrust::device_ptr<T> dp(void* p) { return thrust::device_pointer_cast((T*)p); }
 template <typename T> thrust::device_ptr<const T> dp(const void* p) { return thrust::device_pointer_cast((const T*)p); }
+#endif
 
 template <typename F>
 int with_dtype(int dtype, F&& f) {
@@ -101,13 +115,17 @@ cmp_pred<T> make_pred(int cmp, const void* thr) {
 }  // namespace
 
 // 1 = OMP device system, 0 = CPP
+#if defined(THRUST_DEVICE_SYSTEM) && defined(THRUST_DEVICE_SYSTEM_OMP) && !defined(DRIVER_HOST_POINTERS)
 REF_API int ref_is_omp(void) { return THRUST_DEVICE_SYSTEM == THRUST_DEVICE_SYSTEM_OMP; }
+#else
+REF_API int ref_is_omp(void) { return 0; }
+#endif
 
 REF_API int ref_reduce(const void* in, uint64_t n, int dtype, int op, const void* init, void* out) {
   return with_dtype(dtype, [&](auto z) {
     using T = decltype(z);
     return with_op<T>(op, [&](auto o) {
-      *(T*)out = thrust::reduce(thrust::device, dp<T>(in), dp<T>(in) + n, *(const T*)init, o);
+      *(T*)out = thrust::reduce(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, *(const T*)init, o);
       return 0;
     });
   });
@@ -117,7 +135,7 @@ REF_API int ref_inclusive_scan(const void* in, void* out, uint64_t n, int dtype,
   return with_dtype(dtype, [&](auto z) {
     using T = decltype(z);
     return with_op<T>(op, [&](auto o) {
-      thrust::inclusive_scan(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), o);
+      thrust::inclusive_scan(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, dp<T>(out), o);
       return 0;
     });
   });
@@ -128,7 +146,7 @@ REF_API int ref_exclusive_scan(const void* in, void* out, uint64_t n, int dtype,
   return with_dtype(dtype, [&](auto z) {
     using T = decltype(z);
     return with_op<T>(op, [&](auto o) {
-      thrust::exclusive_scan(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), *(const T*)init, o);
+      thrust::exclusive_scan(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, dp<T>(out), *(const T*)init, o);
       return 0;
     });
   });
@@ -137,8 +155,8 @@ REF_API int ref_exclusive_scan(const void* in, void* out, uint64_t n, int dtype,
 REF_API int ref_sort_keys(void* keys, uint64_t n, int dtype, int descending) {
   return with_dtype(dtype, [&](auto z) {
     using T = decltype(z);
-    if (descending) thrust::sort(thrust::device, dp<T>(keys), dp<T>(keys) + n, thrust::greater<T>());
-    else thrust::sort(thrust::device, dp<T>(keys), dp<T>(keys) + n);
+    if (descending) thrust::sort(DRIVER_POLICY, dp<T>(keys), dp<T>(keys) + n, thrust::greater<T>());
+    else thrust::sort(DRIVER_POLICY, dp<T>(keys), dp<T>(keys) + n);
     return 0;
   });
 }
@@ -150,9 +168,9 @@ REF_API int ref_sort_pairs(void* keys, void* values, uint64_t n, int dtype, uint
     return with_bytes(value_bytes, [&](auto vz) {
       using V = decltype(vz);
       if (descending)
-        thrust::stable_sort_by_key(thrust::device, dp<T>(keys), dp<T>(keys) + n, dp<V>(values), thrust::greater<T>());
+        thrust::stable_sort_by_key(DRIVER_POLICY, dp<T>(keys), dp<T>(keys) + n, dp<V>(values), thrust::greater<T>());
       else
-        thrust::stable_sort_by_key(thrust::device, dp<T>(keys), dp<T>(keys) + n, dp<V>(values));
+        thrust::stable_sort_by_key(DRIVER_POLICY, dp<T>(keys), dp<T>(keys) + n, dp<V>(values));
       return 0;
     });
   });
@@ -174,12 +192,12 @@ template <typename T> struct user_less_div {  // testing/stable_sort.cu:43-47 wi
 template <typename T, typename C>
 void comparison_sort(void* keys, void* values, uint64_t n, uint64_t value_bytes, C comp) {
   if (!values) {
-    thrust::stable_sort(thrust::device, dp<T>(keys), dp<T>(keys) + n, comp);
+    thrust::stable_sort(DRIVER_POLICY, dp<T>(keys), dp<T>(keys) + n, comp);
     return;
   }
   with_bytes(value_bytes, [&](auto vz) {
     using V = decltype(vz);
-    thrust::stable_sort_by_key(thrust::device, dp<T>(keys), dp<T>(keys) + n, dp<V>(values), comp);
+    thrust::stable_sort_by_key(DRIVER_POLICY, dp<T>(keys), dp<T>(keys) + n, dp<V>(values), comp);
     return 0;
   });
 }
@@ -202,9 +220,9 @@ REF_API int ref_merge(const void* a, uint64_t na, const void* b, uint64_t nb, vo
   return with_dtype(dtype, [&](auto z) {
     using T = decltype(z);
     if (descending)
-      thrust::merge(thrust::device, dp<T>(a), dp<T>(a) + na, dp<T>(b), dp<T>(b) + nb, dp<T>(out), thrust::greater<T>());
+      thrust::merge(DRIVER_POLICY, dp<T>(a), dp<T>(a) + na, dp<T>(b), dp<T>(b) + nb, dp<T>(out), thrust::greater<T>());
     else
-      thrust::merge(thrust::device, dp<T>(a), dp<T>(a) + na, dp<T>(b), dp<T>(b) + nb, dp<T>(out));
+      thrust::merge(DRIVER_POLICY, dp<T>(a), dp<T>(a) + na, dp<T>(b), dp<T>(b) + nb, dp<T>(out));
     return 0;
   });
 }
@@ -217,10 +235,10 @@ REF_API int ref_merge_by_key(const void* ka, uint64_t na, const void* kb, uint64
     return with_bytes(value_bytes, [&](auto vz) {
       using V = decltype(vz);
       if (descending)
-        thrust::merge_by_key(thrust::device, dp<T>(ka), dp<T>(ka) + na, dp<T>(kb), dp<T>(kb) + nb,
+        thrust::merge_by_key(DRIVER_POLICY, dp<T>(ka), dp<T>(ka) + na, dp<T>(kb), dp<T>(kb) + nb,
                              dp<V>(va), dp<V>(vb), dp<T>(kout), dp<V>(vout), thrust::greater<T>());
       else
-        thrust::merge_by_key(thrust::device, dp<T>(ka), dp<T>(ka) + na, dp<T>(kb), dp<T>(kb) + nb,
+        thrust::merge_by_key(DRIVER_POLICY, dp<T>(ka), dp<T>(ka) + na, dp<T>(kb), dp<T>(kb) + nb,
                              dp<V>(va), dp<V>(vb), dp<T>(kout), dp<V>(vout));
       return 0;
     });
@@ -233,12 +251,12 @@ REF_API int ref_copy_if(const void* in, const void* stencil, void* out, uint64_t
     using T = decltype(z);
     const cmp_pred<T> pred = make_pred<T>(cmp, threshold);
     if (!stencil) {
-      *num = thrust::copy_if(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), pred) - dp<T>(out);
+      *num = thrust::copy_if(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, dp<T>(out), pred) - dp<T>(out);
       return 0;
     }
     return with_bytes(item_bytes, [&](auto vz) {
       using V = decltype(vz);
-      *num = thrust::copy_if(thrust::device, dp<V>(in), dp<V>(in) + n, dp<T>(stencil), dp<V>(out), pred) - dp<V>(out);
+      *num = thrust::copy_if(DRIVER_POLICY, dp<V>(in), dp<V>(in) + n, dp<T>(stencil), dp<V>(out), pred) - dp<V>(out);
       return 0;
     });
   });
@@ -251,13 +269,13 @@ REF_API int ref_partition_copy(const void* in, const void* stencil, void* out_tr
     using T = decltype(z);
     const cmp_pred<T> pred = make_pred<T>(cmp, threshold);
     if (!stencil) {
-      *num_true = thrust::stable_partition_copy(thrust::device, dp<T>(in), dp<T>(in) + n,
+      *num_true = thrust::stable_partition_copy(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n,
                                                 dp<T>(out_true), dp<T>(out_false), pred).first - dp<T>(out_true);
       return 0;
     }
     return with_bytes(item_bytes, [&](auto vz) {
       using V = decltype(vz);
-      *num_true = thrust::stable_partition_copy(thrust::device, dp<V>(in), dp<V>(in) + n, dp<T>(stencil),
+      *num_true = thrust::stable_partition_copy(DRIVER_POLICY, dp<V>(in), dp<V>(in) + n, dp<T>(stencil),
                                                 dp<V>(out_true), dp<V>(out_false), pred).first - dp<V>(out_true);
       return 0;
     });
@@ -271,12 +289,12 @@ REF_API int ref_stable_partition(void* data, const void* stencil, uint64_t* num_
     using T = decltype(z);
     const cmp_pred<T> pred = make_pred<T>(cmp, threshold);
     if (!stencil) {
-      *num_true = thrust::stable_partition(thrust::device, dp<T>(data), dp<T>(data) + n, pred) - dp<T>(data);
+      *num_true = thrust::stable_partition(DRIVER_POLICY, dp<T>(data), dp<T>(data) + n, pred) - dp<T>(data);
       return 0;
     }
     return with_bytes(item_bytes, [&](auto vz) {
       using V = decltype(vz);
-      *num_true = thrust::stable_partition(thrust::device, dp<V>(data), dp<V>(data) + n, dp<T>(stencil), pred) - dp<V>(data);
+      *num_true = thrust::stable_partition(DRIVER_POLICY, dp<V>(data), dp<V>(data) + n, dp<T>(stencil), pred) - dp<V>(data);
       return 0;
     });
   });
@@ -285,8 +303,8 @@ REF_API int ref_stable_partition(void* data, const void* stencil, uint64_t* num_
 REF_API int ref_unique(const void* in, void* out, uint64_t* num, uint64_t n, int dtype) {
   return with_dtype(dtype, [&](auto z) {
     using T = decltype(z);
-    if (in == out) *num = thrust::unique(thrust::device, dp<T>(out), dp<T>(out) + n) - dp<T>(out);
-    else *num = thrust::unique_copy(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out)) - dp<T>(out);
+    if (in == out) *num = thrust::unique(DRIVER_POLICY, dp<T>(out), dp<T>(out) + n) - dp<T>(out);
+    else *num = thrust::unique_copy(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, dp<T>(out)) - dp<T>(out);
     return 0;
   });
 }
@@ -299,9 +317,9 @@ REF_API int ref_unique_by_key(const void* keys_in, const void* values_in, void* 
     return with_bytes(value_bytes, [&](auto vz) {
       using V = decltype(vz);
       if (keys_in == keys_out)
-        *num = thrust::unique_by_key(thrust::device, dp<T>(keys_out), dp<T>(keys_out) + n, dp<V>(values_out)).first - dp<T>(keys_out);
+        *num = thrust::unique_by_key(DRIVER_POLICY, dp<T>(keys_out), dp<T>(keys_out) + n, dp<V>(values_out)).first - dp<T>(keys_out);
       else
-        *num = thrust::unique_by_key_copy(thrust::device, dp<T>(keys_in), dp<T>(keys_in) + n, dp<V>(values_in),
+        *num = thrust::unique_by_key_copy(DRIVER_POLICY, dp<T>(keys_in), dp<T>(keys_in) + n, dp<V>(values_in),
                                           dp<T>(keys_out), dp<V>(values_out)).first - dp<T>(keys_out);
       return 0;
     });
@@ -317,7 +335,7 @@ REF_API int ref_reduce_by_key(const void* keys_in, const void* values_in, void* 
     using K = decltype(kz);
     using V = decltype(vz);
     return with_op<V>(op, [&](auto o) {
-      *num_runs = thrust::reduce_by_key(thrust::device, dp<K>(keys_in), dp<K>(keys_in) + n, dp<V>(values_in),
+      *num_runs = thrust::reduce_by_key(DRIVER_POLICY, dp<K>(keys_in), dp<K>(keys_in) + n, dp<V>(values_in),
                                         dp<K>(keys_out), dp<V>(values_out), thrust::equal_to<K>(), o).first - dp<K>(keys_out);
       return 0;
     });
@@ -345,7 +363,7 @@ REF_API int ref_count_if(const void* in, uint64_t n, int dtype, int cmp, const v
                          uint64_t* count) {
   return with_dtype(dtype, [&](auto z) {
     using T = decltype(z);
-    *count = (uint64_t)thrust::count_if(thrust::device, dp<T>(in), dp<T>(in) + n, make_pred<T>(cmp, threshold));
+    *count = (uint64_t)thrust::count_if(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, make_pred<T>(cmp, threshold));
     return 0;
   });
 }
@@ -354,7 +372,7 @@ REF_API int ref_inner_product(const void* a, const void* b, uint64_t n, int dtyp
                               void* out) {
   return with_dtype(dtype, [&](auto z) {
     using T = decltype(z);
-    *(T*)out = thrust::inner_product(thrust::device, dp<T>(a), dp<T>(a) + n, dp<T>(b), *(const T*)init);
+    *(T*)out = thrust::inner_product(DRIVER_POLICY, dp<T>(a), dp<T>(a) + n, dp<T>(b), *(const T*)init);
     return 0;
   });
 }
@@ -366,16 +384,16 @@ REF_API int ref_convert(const void* in, int in_dtype, void* out, int out_dtype, 
     using TI = decltype(zi);
     return with_dtype(out_dtype, [&](auto zo) {
       using TO = decltype(zo);
-      thrust::copy(thrust::device, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out));  // converting copy
+      thrust::copy(DRIVER_POLICY, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out));  // converting copy
       return 0;
     });
   });
 }
 REF_API int ref_reduce_mixed(const void* in, int in_dtype, uint64_t n, int init_dtype, const void* init, void* out) {
   if (in_dtype == THRUST_AMD_F32 && init_dtype == THRUST_AMD_I32)
-    *(int32_t*)out = thrust::reduce(thrust::device, dp<float>(in), dp<float>(in) + n, *(const int32_t*)init);
+    *(int32_t*)out = thrust::reduce(DRIVER_POLICY, dp<float>(in), dp<float>(in) + n, *(const int32_t*)init);
   else if (in_dtype == THRUST_AMD_I32 && init_dtype == THRUST_AMD_F32)
-    *(float*)out = thrust::reduce(thrust::device, dp<int32_t>(in), dp<int32_t>(in) + n, *(const float*)init);
+    *(float*)out = thrust::reduce(DRIVER_POLICY, dp<int32_t>(in), dp<int32_t>(in) + n, *(const float*)init);
   else
     return -1;
   return 0;
@@ -387,11 +405,11 @@ REF_API int ref_scan_mixed(const void* in, int in_dtype, void* out, uint64_t n, 
   auto run = [&](auto zi, auto zo) {
     using TI = decltype(zi);
     using TO = decltype(zo);
-    if (exclusive < 0) thrust::inclusive_scan(thrust::device, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out));
+    if (exclusive < 0) thrust::inclusive_scan(DRIVER_POLICY, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out));
     else if (init_dtype == THRUST_AMD_I32)
-      thrust::exclusive_scan(thrust::device, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out), *(const int32_t*)init);
+      thrust::exclusive_scan(DRIVER_POLICY, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out), *(const int32_t*)init);
     else
-      thrust::exclusive_scan(thrust::device, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out), *(const float*)init);
+      thrust::exclusive_scan(DRIVER_POLICY, dp<TI>(in), dp<TI>(in) + n, dp<TO>(out), *(const float*)init);
     return 0;
   };
   if (in_dtype == THRUST_AMD_F32) return run((float)0, (int32_t)0);
@@ -406,11 +424,11 @@ uint64_t run_set_operation(int op, const void* a, uint64_t na, const void* b, ui
   auto a0 = dp<K>(a), b0 = dp<K>(b);
   auto o0 = dp<K>(out);
   switch (op) {
-    case THRUST_AMD_SET_DIFFERENCE: return thrust::set_difference(thrust::device, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
-    case THRUST_AMD_SET_INTERSECTION: return thrust::set_intersection(thrust::device, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
+    case THRUST_AMD_SET_DIFFERENCE: return thrust::set_difference(DRIVER_POLICY, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
+    case THRUST_AMD_SET_INTERSECTION: return thrust::set_intersection(DRIVER_POLICY, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
     case THRUST_AMD_SET_SYMMETRIC_DIFFERENCE:
-      return thrust::set_symmetric_difference(thrust::device, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
-    default: return thrust::set_union(thrust::device, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
+      return thrust::set_symmetric_difference(DRIVER_POLICY, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
+    default: return thrust::set_union(DRIVER_POLICY, a0, a0 + na, b0, b0 + nb, o0, comp) - o0;
   }
 }
 template <typename K, typename V, typename C>
@@ -422,12 +440,12 @@ uint64_t run_set_operation_by_key(int op, const void* ka, uint64_t na, const voi
   auto vo = dp<V>(vout);
   switch (op) {
     case THRUST_AMD_SET_DIFFERENCE:
-      return thrust::set_difference_by_key(thrust::device, a0, a0 + na, b0, b0 + nb, v1, v2, ko, vo, comp).first - ko;
+      return thrust::set_difference_by_key(DRIVER_POLICY, a0, a0 + na, b0, b0 + nb, v1, v2, ko, vo, comp).first - ko;
     case THRUST_AMD_SET_INTERSECTION:
-      return thrust::set_intersection_by_key(thrust::device, a0, a0 + na, b0, b0 + nb, v1, ko, vo, comp).first - ko;
+      return thrust::set_intersection_by_key(DRIVER_POLICY, a0, a0 + na, b0, b0 + nb, v1, ko, vo, comp).first - ko;
     case THRUST_AMD_SET_SYMMETRIC_DIFFERENCE:
-      return thrust::set_symmetric_difference_by_key(thrust::device, a0, a0 + na, b0, b0 + nb, v1, v2, ko, vo, comp).first - ko;
-    default: return thrust::set_union_by_key(thrust::device, a0, a0 + na, b0, b0 + nb, v1, v2, ko, vo, comp).first - ko;
+      return thrust::set_symmetric_difference_by_key(DRIVER_POLICY, a0, a0 + na, b0, b0 + nb, v1, v2, ko, vo, comp).first - ko;
+    default: return thrust::set_union_by_key(DRIVER_POLICY, a0, a0 + na, b0, b0 + nb, v1, v2, ko, vo, comp).first - ko;
   }
 }
 }  // namespace
@@ -487,7 +505,7 @@ REF_API int ref_transform_reduce(const void* in, uint64_t n, int dtype, int unar
     using T = decltype(z);
     return with_unary<T>(unary, [&](auto u) {
       return with_op<T>(op, [&](auto o) {
-        *(T*)out = thrust::transform_reduce(thrust::device, dp<T>(in), dp<T>(in) + n, u, *(const T*)init, o);
+        *(T*)out = thrust::transform_reduce(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, u, *(const T*)init, o);
         return 0;
       });
     });
@@ -500,7 +518,7 @@ REF_API int ref_transform_inclusive_scan(const void* in, void* out, uint64_t n, 
     using T = decltype(z);
     return with_unary<T>(unary, [&](auto u) {
       return with_op<T>(op, [&](auto o) {
-        thrust::transform_inclusive_scan(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), u, o);
+        thrust::transform_inclusive_scan(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, dp<T>(out), u, o);
         return 0;
       });
     });
@@ -513,7 +531,7 @@ REF_API int ref_transform_exclusive_scan(const void* in, void* out, uint64_t n, 
     using T = decltype(z);
     return with_unary<T>(unary, [&](auto u) {
       return with_op<T>(op, [&](auto o) {
-        thrust::transform_exclusive_scan(thrust::device, dp<T>(in), dp<T>(in) + n, dp<T>(out), u, *(const T*)init, o);
+        thrust::transform_exclusive_scan(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, dp<T>(out), u, *(const T*)init, o);
         return 0;
       });
     });
@@ -549,7 +567,7 @@ REF_API int ref_inclusive_scan_by_key(const void* keys, const void* values, void
     using K = decltype(kz);
     using V = decltype(vz);
     return with_op<V>(op, [&](auto o) {
-      thrust::inclusive_scan_by_key(thrust::device, dp<K>(keys), dp<K>(keys) + n, dp<V>(values), dp<V>(out),
+      thrust::inclusive_scan_by_key(DRIVER_POLICY, dp<K>(keys), dp<K>(keys) + n, dp<V>(values), dp<V>(out),
                                     thrust::equal_to<K>(), o);
       return 0;
     });
@@ -562,7 +580,7 @@ REF_API int ref_exclusive_scan_by_key(const void* keys, const void* values, void
     using K = decltype(kz);
     using V = decltype(vz);
     return with_op<V>(op, [&](auto o) {
-      thrust::exclusive_scan_by_key(thrust::device, dp<K>(keys), dp<K>(keys) + n, dp<V>(values), dp<V>(out),
+      thrust::exclusive_scan_by_key(DRIVER_POLICY, dp<K>(keys), dp<K>(keys) + n, dp<V>(values), dp<V>(out),
                                     *(const V*)init, thrust::equal_to<K>(), o);
       return 0;
     });

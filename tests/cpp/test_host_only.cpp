@@ -1,0 +1,74 @@
+// Host-system behaviour that needs no GPU: run by tests/test_host_system.py on any machine.
+// Each expectation is what the reference's sequential system produces for the same call.
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+#include <thrust/execution_policy.h>
+#include <thrust/functional.h>
+#include <thrust/host_vector.h>
+#include <thrust/reduce.h>
+#include <thrust/sort.h>
+
+static int g_checks = 0, g_fail = 0;
+#define CHECK(c)                                                          \
+  do {                                                                    \
+    ++g_checks;                                                           \
+    if (!(c)) { ++g_fail; std::printf("FAILED %s:%d: %s\n", __FILE__, __LINE__, #c); } \
+  } while (0)
+
+struct within_one {
+  bool operator()(int a, int b) const { return std::abs(a - b) <= 1; }
+};
+
+// thrust/system/detail/sequential/reduce_by_key.h:61-87: a run lasts while pred(first key of
+// the run, key) holds.  A predicate that is not transitive tells this from a comparison of
+// neighbours: 1 2 3 4 is two runs (1 2 | 3 4), not one.
+static void TestReduceByKeyComparesWithTheRunsFirstKey() {
+  thrust::host_vector<int> keys(std::vector<int>{1, 2, 3, 4, 4, 6, 7, 8});
+  thrust::host_vector<int> vals(std::vector<int>{1, 10, 100, 1000, 10000, 100000, 1000000, 10000000});
+  thrust::host_vector<int> ko(8), vo(8);
+  auto ends = thrust::reduce_by_key(thrust::host, keys.begin(), keys.end(), vals.begin(), ko.begin(), vo.begin(),
+                                    within_one(), thrust::plus<int>());
+  CHECK(ends.first - ko.begin() == 4);
+  CHECK(ko[0] == 1 && vo[0] == 11);
+  CHECK(ko[1] == 3 && vo[1] == 11100);
+  CHECK(ko[2] == 6 && vo[2] == 1100000);
+  CHECK(ko[3] == 8 && vo[3] == 10000000);
+}
+
+// thrust/system/detail/sequential/sort.inl:139-148: less<K> / greater<K> on arithmetic keys take
+// the radix sort, which orders floats by their bits; any other comparator takes the merge
+// sort, for which -0.0 and +0.0 are equivalent and keep their order.
+static void TestFloatZerosUnderLessAndUnderAUserComparator() {
+  const float pz = 0.0f, nz = -0.0f;
+  thrust::host_vector<float> k(std::vector<float>{pz, nz, 1.0f, pz, nz, -1.0f});
+  thrust::host_vector<int> v(std::vector<int>{0, 1, 2, 3, 4, 5});
+  thrust::host_vector<float> k1 = k;
+  thrust::host_vector<int> v1 = v;
+  thrust::stable_sort_by_key(thrust::host, k1.begin(), k1.end(), v1.begin(), thrust::less<float>());
+  const int want_less[] = {5, 1, 4, 0, 3, 2};
+  for (int i = 0; i < 6; ++i) CHECK(v1[i] == want_less[i]);
+  CHECK(std::signbit(k1[1]) && std::signbit(k1[2]) && !std::signbit(k1[3]) && !std::signbit(k1[4]));
+
+  thrust::host_vector<float> k2 = k;
+  thrust::host_vector<int> v2 = v;
+  thrust::stable_sort_by_key(thrust::host, k2.begin(), k2.end(), v2.begin(), thrust::greater<float>());
+  const int want_greater[] = {2, 0, 3, 1, 4, 5};
+  for (int i = 0; i < 6; ++i) CHECK(v2[i] == want_greater[i]);
+
+  thrust::host_vector<float> k3 = k;
+  thrust::host_vector<int> v3 = v;
+  thrust::stable_sort_by_key(thrust::host, k3.begin(), k3.end(), v3.begin(),
+                             [](float a, float b) { return a < b; });
+  const int want_user[] = {5, 0, 1, 3, 4, 2};
+  for (int i = 0; i < 6; ++i) CHECK(v3[i] == want_user[i]);
+}
+
+int main() {
+  TestReduceByKeyComparesWithTheRunsFirstKey();
+  TestFloatZerosUnderLessAndUnderAUserComparator();
+  std::printf("%d checks, %d failed\n", g_checks, g_fail);
+  return g_fail ? 1 : 0;
+}

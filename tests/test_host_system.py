@@ -1,0 +1,258 @@
+"""The front end's host system (thrust::host over raw pointers: include/thrust/*.h, namespace
+system::cpp) against the reference's sequential CPP system, call for call.
+
+oracle/ref_driver.cpp is the one driver source: oracle/Makefile compiles it against the
+reference's headers (oracle/_ref/libref_cpp.so), tests/cpp/Makefile compiles it against this
+repository's headers with the host policy (tests/cpp/bin/libfront_host.so).  Where the real
+reference library was not built, the C restatement with one thread stands in for it
+(tests/test_oracle.py pins the restatement against the real reference and the fixtures).
+Everything is compared bit for bit; no GPU is touched.
+"""
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from oracle import cpu
+from thrust_amd import datagen
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+FRONT_LIB = os.path.join(HERE, "cpp", "bin", "libfront_host.so")
+
+
+@pytest.fixture(scope="module")
+def front():
+    # make rebuilds only when a header or the driver changed (about 40 s then)
+    subprocess.run(["make", "-C", os.path.join(HERE, "cpp"), FRONT_LIB], check=True, capture_output=True)
+    return cpu.Reference("cpp", path=FRONT_LIB)
+
+
+@pytest.fixture(scope="module")
+def want():
+    if cpu.ref_available("cpp"):
+        return cpu.Reference("cpp")
+    if not os.path.exists(cpu.ORACLE_LIB):
+        cpu.build(with_ref=False)
+    return cpu.Oracle(nthreads=1)
+
+
+def same(a, b):
+    if isinstance(a, tuple):
+        assert len(a) == len(b)
+        for x, y in zip(a, b):
+            same(x, y)
+        return
+    a, b = np.asarray(a), np.asarray(b)
+    assert a.dtype == b.dtype and a.shape == b.shape
+    assert a.tobytes() == b.tobytes()
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+def floats_with_specials(n, seed, dtype=np.float32):
+    """Finite values, both zeros, denormals, infinities and NaNs of both signs."""
+    r = rng(seed)
+    x = (r.standard_normal(n) * 100).astype(dtype)
+    tiny = np.finfo(dtype).smallest_subnormal
+    specials = np.array([0.0, -0.0, tiny, -tiny, np.inf, -np.inf, np.nan, -np.nan, 1.0, -1.0], dtype)
+    where = r.integers(0, n, n // 8)
+    x[where] = specials[r.integers(0, specials.size, where.size)]
+    return x
+
+
+SIZES = [0, 1, 2, 63, 1000, 40001]
+INT_TYPES = [np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64]
+
+
+@pytest.mark.parametrize("n", SIZES)
+@pytest.mark.parametrize("dtype", INT_TYPES + [np.float32, np.float64])
+def test_reduce_and_scans(front, want, dtype, n):
+    r = rng(n + 1)
+    if np.issubdtype(dtype, np.integer):
+        x = r.integers(0, 100, n).astype(dtype)
+    else:
+        x = r.random(n).astype(dtype)
+    for op in (cpu.PLUS, cpu.MIN, cpu.MAX):
+        same(front.reduce(x, op, 3), want.reduce(x, op, 3))
+        same(front.inclusive_scan(x, op), want.inclusive_scan(x, op))
+        same(front.exclusive_scan(x, 5, op), want.exclusive_scan(x, 5, op))
+
+
+def test_config1_values(front, want):
+    x = datagen.c1_int32(1 << 20)
+    same(front.reduce(x), want.reduce(x))
+    same(front.inclusive_scan(x), want.inclusive_scan(x))
+    same(front.exclusive_scan(x, 0), want.exclusive_scan(x, 0))
+
+
+@pytest.mark.parametrize("descending", [False, True])
+@pytest.mark.parametrize("n", SIZES)
+@pytest.mark.parametrize("dtype", INT_TYPES)
+def test_sort_integers(front, want, dtype, n, descending):
+    info = np.iinfo(dtype)
+    keys = rng(n).integers(info.min, info.max, n, dtype=dtype, endpoint=True)
+    keys[: n // 3] = keys[n // 2: n // 2 + n // 3]  # duplicates
+    same(front.sort_keys(keys, descending), want.sort_keys(keys, descending))
+    vals = np.arange(n, dtype=np.uint32)
+    same(front.sort_pairs(keys, vals, descending), want.sort_pairs(keys, vals, descending))
+
+
+@pytest.mark.parametrize("descending", [False, True])
+@pytest.mark.parametrize("dtype", [np.float32, np.float64])
+def test_sort_floats_orders_zeros_and_nans_as_the_reference(front, want, dtype, descending):
+    """The reference sorts arithmetic keys under less/greater by their radix encoding
+    (thrust/system/detail/sequential/stable_primitive_sort.inl:33-66,
+    stable_radix_sort.inl:52-130): -0.0 before +0.0, NaNs at the ends by sign."""
+    keys = floats_with_specials(20000, 7, dtype)
+    same(front.sort_keys(keys, descending), want.sort_keys(keys, descending))
+    vals = np.arange(keys.size, dtype=np.uint64)
+    same(front.sort_pairs(keys, vals, descending), want.sort_pairs(keys, vals, descending))
+
+
+def test_config2_and_config3_inputs(front, want):
+    k = datagen.c2_uint32(1 << 18)
+    same(front.sort_keys(k), want.sort_keys(k))
+    f = datagen.c2_float32(1 << 18)
+    same(front.sort_keys(f), want.sort_keys(f))
+    for kind in ("full", "low16", "skew90"):
+        k64 = datagen.c3_uint64(1 << 17, kind)
+        v = np.arange(k64.size, dtype=np.uint32)
+        same(front.sort_pairs(k64, v), want.sort_pairs(k64, v))
+
+
+@pytest.mark.parametrize("comparator,param", [(cpu.CMP_SORT_LESS, 0), (cpu.CMP_SORT_GREATER, 0), (cpu.CMP_SORT_LESS_DIV, 10)])
+@pytest.mark.parametrize("dtype", [np.int32, np.uint8, np.float32])
+def test_sort_with_user_comparators(front, want, dtype, comparator, param):
+    r = rng(11)
+    keys = r.integers(0, 100, 30000).astype(dtype)
+    vals = np.arange(keys.size, dtype=np.uint32)
+    same(front.comparison_sort(keys, None, comparator, param), want.comparison_sort(keys, None, comparator, param))
+    same(front.comparison_sort(keys, vals, comparator, param), want.comparison_sort(keys, vals, comparator, param))
+
+
+@pytest.mark.parametrize("mean", [1, 8, 1000])
+def test_config4_by_key_family(front, want, mean):
+    keys, vals = datagen.c4_segments(200000, mean)
+    same(front.reduce_by_key(keys, vals), want.reduce_by_key(keys, vals))
+    same(front.unique_by_key(keys, vals), want.unique_by_key(keys, vals))
+    same(front.unique(keys), want.unique(keys))
+    same(front.inclusive_scan_by_key(keys, vals), want.inclusive_scan_by_key(keys, vals))
+    same(front.exclusive_scan_by_key(keys, vals, 2), want.exclusive_scan_by_key(keys, vals, 2))
+    for op in (cpu.MIN, cpu.MAX):
+        same(front.reduce_by_key(keys, vals, op), want.reduce_by_key(keys, vals, op))
+
+
+def test_by_key_runs_of_float_keys_with_nans(front, want):
+    """NaN == NaN is false: every NaN key is a run of its own; -0.0 == +0.0 joins runs."""
+    keys = np.array([0.0, -0.0, 1.0, np.nan, np.nan, 2.0, 2.0, -0.0, 0.0, np.nan], np.float32)
+    vals = np.arange(1, keys.size + 1, dtype=np.int32)
+    same(front.reduce_by_key(keys, vals), want.reduce_by_key(keys, vals))
+    same(front.unique_by_key(keys, vals.view(np.uint32)), want.unique_by_key(keys, vals.view(np.uint32)))
+    same(front.unique(keys), want.unique(keys))
+    same(front.inclusive_scan_by_key(keys, vals), want.inclusive_scan_by_key(keys, vals))
+
+
+@pytest.mark.parametrize("n", [0, 1, 5, 70000])
+@pytest.mark.parametrize("key_dtype,value_dtype", [(np.int32, np.float32), (np.uint64, np.int64), (np.uint32, np.float64), (np.int64, np.int32)])
+def test_by_key_family_types(front, want, key_dtype, value_dtype, n):
+    r = rng(n + 3)
+    keys = np.cumsum(r.integers(0, 2, n)).astype(key_dtype)
+    vals = r.integers(0, 50, n).astype(value_dtype)
+    same(front.reduce_by_key(keys, vals), want.reduce_by_key(keys, vals))
+    same(front.inclusive_scan_by_key(keys, vals), want.inclusive_scan_by_key(keys, vals))
+    same(front.exclusive_scan_by_key(keys, vals, 1), want.exclusive_scan_by_key(keys, vals, 1))
+
+
+@pytest.mark.parametrize("threshold", [0.5, 0.05, -1.0, 2.0])
+def test_config5_selection(front, want, threshold):
+    x = datagen.c5_float32(150000)
+    same(front.copy_if(x, cpu.LT, threshold), want.copy_if(x, cpu.LT, threshold))
+    same(front.partition_copy(x, cpu.LT, threshold), want.partition_copy(x, cpu.LT, threshold))
+    same(front.stable_partition(x, cpu.LT, threshold), want.stable_partition(x, cpu.LT, threshold))
+    same(front.count_if(x, cpu.LT, threshold), want.count_if(x, cpu.LT, threshold))
+
+
+@pytest.mark.parametrize("cmp", [cpu.LT, cpu.LE, cpu.GT, cpu.GE, cpu.EQ, cpu.NE, cpu.NONZERO])
+def test_selection_predicates_and_stencils(front, want, cmp):
+    x = floats_with_specials(30000, 5)
+    same(front.copy_if(x, cmp, 0.0), want.copy_if(x, cmp, 0.0))
+    same(front.stable_partition(x, cmp, 0.0), want.stable_partition(x, cmp, 0.0))
+    stencil = rng(9).integers(-3, 4, x.size).astype(np.int32)
+    items = np.arange(x.size, dtype=np.uint64)
+    same(front.copy_if(items, cmp, 1, stencil), want.copy_if(items, cmp, 1, stencil))
+    same(front.partition_copy(items, cmp, 1, stencil), want.partition_copy(items, cmp, 1, stencil))
+    same(front.stable_partition(items, cmp, 1, stencil), want.stable_partition(items, cmp, 1, stencil))
+
+
+@pytest.mark.parametrize("descending", [False, True])
+def test_config5_merges(front, want, descending):
+    (ka, va), (kb, vb) = datagen.c5_merge_inputs(60000)
+    vb = vb + np.uint32(ka.size)
+    if descending:
+        ka, va, kb, vb = ka[::-1].copy(), va[::-1].copy(), kb[::-1].copy(), vb[::-1].copy()
+    same(front.merge(ka, kb, descending), want.merge(ka, kb, descending))
+    same(front.merge_by_key(ka, kb, va, vb, descending), want.merge_by_key(ka, kb, va, vb, descending))
+    empty = ka[:0]
+    same(front.merge(ka, empty, descending), want.merge(ka, empty, descending))
+    same(front.merge(empty, kb, descending), want.merge(empty, kb, descending))
+
+
+def test_merge_of_float_ties_keeps_the_first_range_first(front, want):
+    a = np.array([-1.0, -0.0, 0.0, 3.0], np.float32)
+    b = np.array([-2.0, 0.0, -0.0, 3.0, 4.0], np.float32)
+    same(front.merge(a, b), want.merge(a, b))
+    va, vb = np.arange(4, dtype=np.uint32), np.arange(10, 15, dtype=np.uint32)
+    same(front.merge_by_key(a, b, va, vb), want.merge_by_key(a, b, va, vb))
+
+
+@pytest.mark.parametrize("descending", [False, True])
+@pytest.mark.parametrize("op", [cpu.SET_DIFFERENCE, cpu.SET_INTERSECTION, cpu.SET_SYMMETRIC_DIFFERENCE, cpu.SET_UNION])
+def test_set_operations(front, want, op, descending):
+    r = rng(op + 20)
+    a = np.sort(r.integers(0, 3000, 20000).astype(np.int32))
+    b = np.sort(r.integers(0, 3000, 15000).astype(np.int32))
+    if descending:
+        a, b = a[::-1].copy(), b[::-1].copy()
+    same(front.set_operation(op, a, b, descending), want.set_operation(op, a, b, descending))
+    va, vb = np.arange(a.size, dtype=np.uint32), np.arange(b.size, dtype=np.uint32) + np.uint32(1 << 20)
+    same(front.set_operation_by_key(op, a, b, va, vb, descending), want.set_operation_by_key(op, a, b, va, vb, descending))
+
+
+@pytest.mark.parametrize("unary", [cpu.IDENTITY, cpu.NEGATE, cpu.SQUARE])
+@pytest.mark.parametrize("dtype", [np.int32, np.float32, np.int64])
+def test_transformed_reductions_and_scans(front, want, dtype, unary):
+    x = rng(4).integers(-20, 20, 50000).astype(dtype)
+    same(front.transform_reduce(x, unary, cpu.PLUS, 1), want.transform_reduce(x, unary, cpu.PLUS, 1))
+    same(front.transform_inclusive_scan(x, unary), want.transform_inclusive_scan(x, unary))
+    same(front.transform_exclusive_scan(x, unary, 2), want.transform_exclusive_scan(x, unary, 2))
+    same(front.inner_product(x, x, 3), want.inner_product(x, x, 3))
+
+
+def test_mixed_element_types(front, want):
+    """The accumulator of reduce has the type of init; a scan without init accumulates in the
+    input's type and converts on output, one with init in init's type
+    (thrust/system/detail/sequential/scan.h:42-107)."""
+    xf = (rng(2).random(3000) * 10).astype(np.float32)
+    xi = rng(3).integers(-9, 9, 3000).astype(np.int32)
+    same(front.reduce_as(xf, np.int32(0)), want.reduce_as(xf, np.int32(0)))
+    same(front.reduce_as(xi, np.float32(0.5)), want.reduce_as(xi, np.float32(0.5)))
+    same(front.inclusive_scan_as(xf, np.int32), want.inclusive_scan_as(xf, np.int32))
+    same(front.inclusive_scan_as(xi, np.float32), want.inclusive_scan_as(xi, np.float32))
+    same(front.exclusive_scan_as(xf, np.int32(1), np.int32), want.exclusive_scan_as(xf, np.int32(1), np.int32))
+    same(front.exclusive_scan_as(xf, np.float32(1.5), np.int32), want.exclusive_scan_as(xf, np.float32(1.5), np.int32))
+    same(front.exclusive_scan_as(xi, np.float32(0.25), np.float32), want.exclusive_scan_as(xi, np.float32(0.25), np.float32))
+    same(front.convert(xf, np.int32), want.convert(xf, np.int32))
+    same(front.convert(xi, np.float64), want.convert(xi, np.float64))
+
+
+def test_host_only_program():
+    """tests/cpp/test_host_only.cpp: reduce_by_key with a predicate that is not transitive, and
+    where -0.0 lands under less, greater and a comparator of the caller's own."""
+    prog = os.path.join(HERE, "cpp", "bin", "test_host_only")
+    subprocess.run(["make", "-C", os.path.join(HERE, "cpp"), prog], check=True, capture_output=True)
+    res = subprocess.run([prog], capture_output=True, text=True, timeout=60)
+    assert res.returncode == 0, res.stdout + res.stderr
+    assert " 0 failed" in res.stdout
