@@ -13,6 +13,9 @@
 #include <thrust/iterator/transform_iterator.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#if defined(__HIPCC__)
+#include <thrust/system/hip/detail/generic_select.h>
+#endif
 
 namespace thrust {
 
@@ -137,6 +140,17 @@ template <typename Pred, typename T, bool = is_abi_type<T>::value>
 struct selects_in_kernel : std::integral_constant<bool, unary_pred<Pred, T>::supported> {};
 template <typename Pred, typename T>
 struct selects_in_kernel<Pred, T, false> : std::false_type {};
+// 0: a recognised predicate, evaluated by the library's kernel from a comparison code
+// 1: any other predicate on a type the compaction kernel can hold: the kernel is instantiated
+//    for the predicate in this translation unit (hipcc) and evaluates it in registers
+// 2: the predicate is evaluated into one byte per element first (tested types of other sizes)
+template <typename Pred, typename S>
+struct selection_route
+    : std::integral_constant<int, selects_in_kernel<Pred, S>::value ? 0
+#if defined(__HIPCC__)
+                                  : is_kernel_item<S>::value ? 1
+#endif
+                                                             : 2> {};
 }  // namespace detail
 
 template <typename D, typename In, typename Out>
@@ -213,10 +227,29 @@ class tested_stream<St, Pred, false> {
   device_input<thrust::transform_iterator<as_flag<Pred>, St> > flags_;
 };
 
-template <typename D, typename In, typename St, typename Out, typename Pred>
-Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, bool has_stencil, Out result, Pred pred,
-                 bool negate) {
+#if defined(__HIPCC__)
+// route 1: the predicate runs inside the compaction kernel
+template <typename D, typename In, typename St, typename HasStencil, typename Out, typename Pred>
+Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, HasStencil, Out result, Pred pred,
+                 bool negate, std::integral_constant<int, 1>) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  device_input<In> source(stream, temp_source_of(exec), first, n);
+  device_input<St> tested(stream, temp_source_of(exec), stencil, HasStencil::value ? n : 0);
+  const uint64_t cnt = generic_selection<HasStencil::value>(
+      stream, temp_source_of(exec), (const T*)source.ptr(), (const S*)tested.ptr(), thrust::detail::raw(result),
+      (T*)nullptr, false, n, pred, negate, "copy_if failed");
+  return result + cnt;
+}
+#endif
+template <typename D, typename In, typename St, typename HasStencil, typename Out, typename Pred, int ROUTE>
+Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, HasStencil, Out result, Pred pred,
+                 bool negate, std::integral_constant<int, ROUTE>) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  const bool has_stencil = HasStencil::value;
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
@@ -231,6 +264,12 @@ Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, bool 
       negate);
   return result + cnt;
 }
+template <typename D, typename In, typename St, typename HasStencil, typename Out, typename Pred>
+Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, HasStencil has_stencil, Out result,
+                 Pred pred, bool negate) {
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  return copy_if_impl(exec, first, last, stencil, has_stencil, result, pred, negate, selection_route<Pred, S>());
+}
 }  // namespace detail
 
 template <typename D, typename In, typename Out, typename Pred>
@@ -238,14 +277,14 @@ Out copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred)
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
   static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
                 "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  return detail::copy_if_impl(exec, first, last, first, false, result, pred, false);
+  return detail::copy_if_impl(exec, first, last, first, std::false_type(), result, pred, false);
 }
 template <typename D, typename In, typename St, typename Out, typename Pred>
 Out copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result, Pred pred) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
   static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
                 "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  return detail::copy_if_impl(exec, first, last, stencil, true, result, pred, false);
+  return detail::copy_if_impl(exec, first, last, stencil, std::true_type(), result, pred, false);
 }
 }  // namespace hip
 }  // namespace system

@@ -249,6 +249,23 @@ host_vector<T, Alloc>& host_vector<T, Alloc>::operator=(const device_vector<T, D
   return *this;
 }
 
+template <typename T, typename Alloc>
+template <typename U>
+host_vector<T, Alloc>::host_vector(device_ptr<U> first, device_ptr<U> last) : base((std::size_t)(last - first)) {
+  typedef typename std::remove_const<U>::type V;
+  const std::size_t n = this->size();
+  if (n == 0) return;
+  if (std::is_same<V, T>::value) {
+    system::hip::detail::throw_on_error(
+        thrust_amd_memcpy(this->data(), first.get(), n * sizeof(V), THRUST_AMD_D2H, nullptr), "host_vector copy");
+  } else {
+    std::vector<V> staged(n);
+    system::hip::detail::throw_on_error(
+        thrust_amd_memcpy(staged.data(), first.get(), n * sizeof(V), THRUST_AMD_D2H, nullptr), "host_vector copy");
+    for (std::size_t i = 0; i < n; ++i) (*this)[i] = static_cast<T>(staged[i]);
+  }
+}
+
 template <typename T, typename DA, typename DB>
 inline bool operator==(const device_vector<T, DA>& a, const device_vector<T, DB>& b) {
   return host_vector<T>(a) == host_vector<T>(b);

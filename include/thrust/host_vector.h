@@ -8,6 +8,7 @@ namespace thrust {
 
 template <typename T> class device_allocator;
 template <typename T, typename Alloc> class device_vector;
+template <typename T> class device_ptr;
 
 template <typename T, typename Alloc = std::allocator<T> >
 class host_vector : public std::vector<T, Alloc> {
@@ -25,6 +26,9 @@ class host_vector : public std::vector<T, Alloc> {
   host_vector(const device_vector<T, DA>& d);             // defined in device_vector.h
   template <typename DA>
   host_vector& operator=(const device_vector<T, DA>& d);  // defined in device_vector.h
+  // a range of device memory: one copy for the whole range, not one per element
+  template <typename U>
+  host_vector(device_ptr<U> first, device_ptr<U> last);   // defined in device_vector.h
 };
 
 }  // namespace thrust

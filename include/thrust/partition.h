@@ -49,10 +49,51 @@ pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In l
 
 namespace hip {
 namespace detail {
-template <typename D, typename It, typename St, typename Pred>
-It stable_partition_impl(execution_policy<D>& exec, It first, It last, St stencil, bool has_stencil, Pred pred) {
+#if defined(__HIPCC__)
+// a user's predicate: it runs inside the compaction kernel, instantiated here
+template <typename D, typename It, typename St, typename HasStencil, typename Pred>
+It stable_partition_impl(execution_policy<D>& exec, It first, It last, St stencil, HasStencil, Pred pred,
+                         std::integral_constant<int, 1>) {
+  typedef typename iterator_value<It>::type T;
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  static_assert(is_abi_item<T>::value, "stable_partition on the device system: items of 1, 2, 4 or 8 bytes");
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return first;
+  device_input<St> tested(stream, temp_source_of(exec), stencil, HasStencil::value ? n : 0);
+  T* data = thrust::detail::raw(first);
+  const uint64_t cnt = generic_selection<HasStencil::value>(stream, temp_source_of(exec), (const T*)data,
+                                                            (const S*)tested.ptr(), data, (T*)nullptr, true, n, pred,
+                                                            false, "stable_partition failed");
+  synchronize(stream, "stable_partition: synchronize");
+  return first + cnt;
+}
+template <typename D, typename In, typename St, typename HasStencil, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy_impl(execution_policy<D>& exec, In first, In last, St stencil, HasStencil,
+                                            Out1 out_true, Out2 out_false, Pred pred, std::integral_constant<int, 1>) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  static_assert(is_abi_item<T>::value && std::is_same<typename iterator_value<Out1>::type, T>::value &&
+                    std::is_same<typename iterator_value<Out2>::type, T>::value,
+                "partition_copy on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return thrust::make_pair(out_true, out_false);
+  device_input<In> source(stream, temp_source_of(exec), first, n);
+  device_input<St> tested(stream, temp_source_of(exec), stencil, HasStencil::value ? n : 0);
+  const uint64_t cnt = generic_selection<HasStencil::value>(
+      stream, temp_source_of(exec), (const T*)source.ptr(), (const S*)tested.ptr(), thrust::detail::raw(out_true),
+      thrust::detail::raw(out_false), false, n, pred, false, "partition_copy failed");
+  synchronize(stream, "partition_copy: synchronize");
+  return thrust::make_pair(out_true + cnt, out_false + (n - cnt));
+}
+#endif
+template <typename D, typename It, typename St, typename HasStencil, typename Pred, int ROUTE>
+It stable_partition_impl(execution_policy<D>& exec, It first, It last, St stencil, HasStencil, Pred pred,
+                         std::integral_constant<int, ROUTE>) {
   typedef typename iterator_value<It>::type T;
   static_assert(is_abi_item<T>::value, "stable_partition on the device system: items of 1, 2, 4 or 8 bytes");
+  const bool has_stencil = HasStencil::value;
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return first;
@@ -66,9 +107,12 @@ It stable_partition_impl(execution_policy<D>& exec, It first, It last, St stenci
   synchronize(stream, "stable_partition: synchronize");
   return first + cnt;
 }
-template <typename D, typename In, typename St, typename Out1, typename Out2, typename Pred>
-pair<Out1, Out2> stable_partition_copy_impl(execution_policy<D>& exec, In first, In last, St stencil, bool has_stencil,
-                                            Out1 out_true, Out2 out_false, Pred pred) {
+template <typename D, typename In, typename St, typename HasStencil, typename Out1, typename Out2, typename Pred,
+          int ROUTE>
+pair<Out1, Out2> stable_partition_copy_impl(execution_policy<D>& exec, In first, In last, St stencil, HasStencil,
+                                            Out1 out_true, Out2 out_false, Pred pred,
+                                            std::integral_constant<int, ROUTE>) {
+  const bool has_stencil = HasStencil::value;
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
   static_assert(is_abi_item<T>::value && std::is_same<typename iterator_value<Out1>::type, T>::value &&
                     std::is_same<typename iterator_value<Out2>::type, T>::value,
@@ -88,25 +132,37 @@ pair<Out1, Out2> stable_partition_copy_impl(execution_policy<D>& exec, In first,
   synchronize(stream, "partition_copy: synchronize");
   return thrust::make_pair(out_true + cnt, out_false + (n - cnt));
 }
+template <typename D, typename It, typename St, typename HasStencil, typename Pred>
+It stable_partition_impl(execution_policy<D>& exec, It first, It last, St stencil, HasStencil has_stencil, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  return stable_partition_impl(exec, first, last, stencil, has_stencil, pred, selection_route<Pred, S>());
+}
+template <typename D, typename In, typename St, typename HasStencil, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy_impl(execution_policy<D>& exec, In first, In last, St stencil,
+                                            HasStencil has_stencil, Out1 out_true, Out2 out_false, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<St>::type>::type S;
+  return stable_partition_copy_impl(exec, first, last, stencil, has_stencil, out_true, out_false, pred,
+                                    selection_route<Pred, S>());
+}
 }  // namespace detail
 
 template <typename D, typename It, typename Pred>
 It stable_partition(execution_policy<D>& exec, It first, It last, Pred pred) {
-  return detail::stable_partition_impl(exec, first, last, first, false, pred);
+  return detail::stable_partition_impl(exec, first, last, first, std::false_type(), pred);
 }
 template <typename D, typename It, typename St, typename Pred>
 It stable_partition(execution_policy<D>& exec, It first, It last, St stencil, Pred pred) {
-  return detail::stable_partition_impl(exec, first, last, stencil, true, pred);
+  return detail::stable_partition_impl(exec, first, last, stencil, std::true_type(), pred);
 }
 template <typename D, typename In, typename Out1, typename Out2, typename Pred>
 pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In last, Out1 out_true, Out2 out_false,
                                        Pred pred) {
-  return detail::stable_partition_copy_impl(exec, first, last, first, false, out_true, out_false, pred);
+  return detail::stable_partition_copy_impl(exec, first, last, first, std::false_type(), out_true, out_false, pred);
 }
 template <typename D, typename In, typename St, typename Out1, typename Out2, typename Pred>
 pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In last, St stencil, Out1 out_true,
                                        Out2 out_false, Pred pred) {
-  return detail::stable_partition_copy_impl(exec, first, last, stencil, true, out_true, out_false, pred);
+  return detail::stable_partition_copy_impl(exec, first, last, stencil, std::true_type(), out_true, out_false, pred);
 }
 }  // namespace hip
 }  // namespace system

@@ -23,6 +23,7 @@
 #include <thrust/pair.h>
 #include <thrust/scan.h>
 #include <thrust/system/hip/detail/device_input.h>
+#include <thrust/system/hip/detail/generic_select.h>
 
 namespace thrust {
 namespace system {
@@ -112,12 +113,8 @@ Out unique_copy_generic(execution_policy<D>& exec, In first, In last, Out result
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
   device_input<In> source(stream, temp_source_of(exec), first, n);
-  temp_storage flags(stream, temp_source_of(exec));
-  flags.ensure((std::size_t)n);
-  unsigned char* head = static_cast<unsigned char*>(flags.ptr());
-  launch_run_flags(exec, source.ptr(), n, pred, head, nullptr);
-  const uint64_t cnt = select_by_flags(stream, temp_source_of(exec), source.ptr(), head, thrust::detail::raw(result), n,
-                                       sizeof(T), "unique failed");
+  const uint64_t cnt = generic_unique(stream, temp_source_of(exec), (const T*)source.ptr(), thrust::detail::raw(result),
+                                      n, pred, "unique failed");
   return result + cnt;
 }
 
@@ -134,15 +131,9 @@ pair<KOut, VOut> unique_by_key_copy_generic(execution_policy<D>& exec, KIn kf, K
   if (n == 0) return thrust::make_pair(ko, vo);
   device_input<KIn> keys(stream, temp_source_of(exec), kf, n);
   device_input<VIn> values(stream, temp_source_of(exec), vf, n);
-  temp_storage flags(stream, temp_source_of(exec));
-  flags.ensure((std::size_t)n);
-  unsigned char* head = static_cast<unsigned char*>(flags.ptr());
-  launch_run_flags(exec, keys.ptr(), n, pred, head, nullptr);
-  // the flags are made, so the two compactions may overwrite their inputs (in-place forms)
-  const uint64_t cnt = select_by_flags(stream, temp_source_of(exec), values.ptr(), head, thrust::detail::raw(vo), n,
-                                       sizeof(V), "unique_by_key failed");
-  (void)select_by_flags(stream, temp_source_of(exec), keys.ptr(), head, thrust::detail::raw(ko), n, sizeof(K),
-                        "unique_by_key failed");
+  const uint64_t cnt = generic_unique_by_key(stream, temp_source_of(exec), (const K*)keys.ptr(), (const V*)values.ptr(),
+                                             thrust::detail::raw(ko), thrust::detail::raw(vo), n, pred,
+                                             "unique_by_key failed");
   return thrust::make_pair(ko + cnt, vo + cnt);
 }
 

@@ -720,6 +720,162 @@ static void Differential() {
   }
 }
 
+// Predicates, stencils and element structs of several widths through the selection kernel that is
+// instantiated for them: every form against the host system on the same input, at sizes of
+// several tiles, with most, half, few and none of the elements selected (the in-place partition
+// sweeps from either end depending on that).
+struct point {
+  int x;
+  float w;
+  __host__ __device__ bool operator==(const point& o) const { return x == o.x && w == o.w; }
+};
+struct quad {  // a 16-byte stencil element
+  int a, b, c, d;
+};
+struct below {
+  int limit;
+  __host__ __device__ bool operator()(int v) const { return v < limit; }
+};
+struct point_below {
+  int limit;
+  __host__ __device__ bool operator()(const point& p) const { return p.x < limit; }
+};
+struct quad_sum_below {
+  int limit;
+  __host__ __device__ bool operator()(const quad& q) const { return q.a + q.b + q.c + q.d < limit; }
+};
+struct byte_is_odd {
+  __host__ __device__ bool operator()(unsigned char b) const { return (b & 1) != 0; }
+};
+struct double_below {
+  double limit;
+  __host__ __device__ bool operator()(double v) const { return v < limit; }
+};
+struct same_point_x {
+  __host__ __device__ bool operator()(const point& a, const point& b) const { return a.x / 4 == b.x / 4; }
+};
+
+template <typename T, typename S, typename Pred>
+static void CheckSelectionForms(const thrust::host_vector<T>& h, const thrust::host_vector<S>& hs, Pred pred) {
+  const size_t n = h.size();
+  const thrust::device_vector<T> d(h);
+  const thrust::device_vector<S> ds(hs);
+  thrust::host_vector<T> ho(n), hf(n);
+  thrust::device_vector<T> dout(n), dfalse(n);
+  {  // copy_if / remove_copy_if by stencil
+    auto he = thrust::copy_if(h.begin(), h.end(), hs.begin(), ho.begin(), pred);
+    auto de = thrust::copy_if(d.begin(), d.end(), ds.begin(), dout.begin(), pred);
+    ASSERT_TRUE(de - dout.begin() == he - ho.begin());
+    ASSERT_TRUE(same(thrust::host_vector<T>(dout.begin(), de), thrust::host_vector<T>(ho.begin(), he)));
+    he = thrust::remove_copy_if(h.begin(), h.end(), hs.begin(), ho.begin(), pred);
+    de = thrust::remove_copy_if(d.begin(), d.end(), ds.begin(), dout.begin(), pred);
+    ASSERT_TRUE(de - dout.begin() == he - ho.begin());
+    ASSERT_TRUE(same(thrust::host_vector<T>(dout.begin(), de), thrust::host_vector<T>(ho.begin(), he)));
+  }
+  {  // partition_copy by stencil
+    auto hr = thrust::partition_copy(h.begin(), h.end(), hs.begin(), ho.begin(), hf.begin(), pred);
+    auto dr = thrust::partition_copy(d.begin(), d.end(), ds.begin(), dout.begin(), dfalse.begin(), pred);
+    ASSERT_TRUE(dr.first - dout.begin() == hr.first - ho.begin() && dr.second - dfalse.begin() == hr.second - hf.begin());
+    ASSERT_TRUE(same(thrust::host_vector<T>(dout.begin(), dr.first), thrust::host_vector<T>(ho.begin(), hr.first)));
+    ASSERT_TRUE(same(thrust::host_vector<T>(dfalse.begin(), dr.second), thrust::host_vector<T>(hf.begin(), hr.second)));
+  }
+  {  // stable_partition and remove_if in place, by stencil
+    thrust::host_vector<T> hp(h);
+    thrust::device_vector<T> dp(d);
+    auto hm = thrust::stable_partition(hp.begin(), hp.end(), hs.begin(), pred);
+    auto dm = thrust::stable_partition(dp.begin(), dp.end(), ds.begin(), pred);
+    ASSERT_TRUE(dm - dp.begin() == hm - hp.begin());
+    ASSERT_TRUE(same(to_host(dp), hp));
+    hp = h;
+    dp = d;
+    auto hend = thrust::remove_if(hp.begin(), hp.end(), hs.begin(), pred);
+    auto dend = thrust::remove_if(dp.begin(), dp.end(), ds.begin(), pred);
+    ASSERT_TRUE(dend - dp.begin() == hend - hp.begin());
+    ASSERT_TRUE(same(thrust::host_vector<T>(dp.begin(), dend), thrust::host_vector<T>(hp.begin(), hend)));
+  }
+}
+template <typename T, typename Pred>
+static void CheckSelectionOnTheElements(const thrust::host_vector<T>& h, Pred pred) {
+  const size_t n = h.size();
+  const thrust::device_vector<T> d(h);
+  thrust::host_vector<T> ho(n), hf(n);
+  thrust::device_vector<T> dout(n), dfalse(n);
+  auto he = thrust::copy_if(h.begin(), h.end(), ho.begin(), pred);
+  auto de = thrust::copy_if(d.begin(), d.end(), dout.begin(), pred);
+  ASSERT_TRUE(de - dout.begin() == he - ho.begin());
+  ASSERT_TRUE(same(thrust::host_vector<T>(dout.begin(), de), thrust::host_vector<T>(ho.begin(), he)));
+  auto hr = thrust::partition_copy(h.begin(), h.end(), ho.begin(), hf.begin(), pred);
+  auto dr = thrust::partition_copy(d.begin(), d.end(), dout.begin(), dfalse.begin(), pred);
+  ASSERT_TRUE(dr.first - dout.begin() == hr.first - ho.begin() && dr.second - dfalse.begin() == hr.second - hf.begin());
+  ASSERT_TRUE(same(thrust::host_vector<T>(dout.begin(), dr.first), thrust::host_vector<T>(ho.begin(), hr.first)));
+  ASSERT_TRUE(same(thrust::host_vector<T>(dfalse.begin(), dr.second), thrust::host_vector<T>(hf.begin(), hr.second)));
+  thrust::host_vector<T> hp(h);
+  thrust::device_vector<T> dp(d);
+  auto hm = thrust::stable_partition(hp.begin(), hp.end(), pred);
+  auto dm = thrust::stable_partition(dp.begin(), dp.end(), pred);
+  ASSERT_TRUE(dm - dp.begin() == hm - hp.begin());
+  ASSERT_TRUE(same(to_host(dp), hp));
+  hp = h;
+  dp = d;
+  auto hend = thrust::remove_if(hp.begin(), hp.end(), pred);
+  auto dend = thrust::remove_if(dp.begin(), dp.end(), pred);
+  ASSERT_TRUE(dend - dp.begin() == hend - hp.begin());
+  ASSERT_TRUE(same(thrust::host_vector<T>(dp.begin(), dend), thrust::host_vector<T>(hp.begin(), hend)));
+}
+
+static void TestUserPredicateSelectionShapes() {
+  for (size_t n : {(size_t)1, (size_t)777, (size_t)40000, (size_t)300001, ((size_t)1 << 20) + 3}) {
+    const thrust::host_vector<int> h = random_values<int>(n, 21, 1000);
+    thrust::host_vector<point> hpnt(n);
+    thrust::host_vector<quad> hq(n);
+    thrust::host_vector<unsigned char> hb(n);
+    thrust::host_vector<double> hd(n);
+    thrust::host_vector<short> hsh(n);
+    for (size_t i = 0; i < n; ++i) {
+      hpnt[i].x = (int)(mix(i + 5) % 1000);
+      hpnt[i].w = (float)i;
+      hq[i] = quad{(int)(mix(i) % 250), (int)(mix(i + 1) % 250), (int)(mix(i + 2) % 250), (int)(mix(i + 3) % 250)};
+      hb[i] = (unsigned char)(mix(i + 9) % 256);
+      hd[i] = (double)(mix(i + 11) % 1000) / 7.0;
+      hsh[i] = (short)(mix(i + 13) % 1000);
+    }
+    for (int limit : {0, 30, 500, 970, 1000}) {
+      g_test = "selection with a user predicate on the elements";
+      CheckSelectionOnTheElements(h, below{limit});
+      CheckSelectionOnTheElements(hpnt, point_below{limit});
+      g_test = "selection with a user predicate on a stencil";
+      CheckSelectionForms(hpnt, h, below{limit});          // 8-byte items, 4-byte stencil
+      CheckSelectionForms(hsh, hq, quad_sum_below{limit});  // 2-byte items, 16-byte stencil
+      CheckSelectionForms(hd, hpnt, point_below{limit});    // 8-byte items, 8-byte struct stencil
+    }
+    g_test = "selection with stencils of one and eight bytes";
+    CheckSelectionForms(h, hb, byte_is_odd());
+    CheckSelectionForms(hb, hd, double_below{40.0});
+    g_test = "unique on structs with a user equality";
+    {
+      thrust::host_vector<point> hs2(hpnt);
+      for (size_t i = 0; i < n; ++i) hs2[i].x = (int)(i / 3 + mix(i / 5) % 3);
+      thrust::device_vector<point> ds2(hs2), dout(n);
+      thrust::host_vector<point> hout(n);
+      auto he = thrust::unique_copy(hs2.begin(), hs2.end(), hout.begin(), same_point_x());
+      auto de = thrust::unique_copy(ds2.begin(), ds2.end(), dout.begin(), same_point_x());
+      ASSERT_TRUE(de - dout.begin() == he - hout.begin());
+      ASSERT_TRUE(same(thrust::host_vector<point>(dout.begin(), de), thrust::host_vector<point>(hout.begin(), he)));
+      thrust::host_vector<short> hv(hsh), hvo(n);
+      thrust::device_vector<short> dv(hsh), dvo(n);
+      auto hu = thrust::unique_by_key_copy(hs2.begin(), hs2.end(), hv.begin(), hout.begin(), hvo.begin(), same_point_x());
+      auto du = thrust::unique_by_key_copy(ds2.begin(), ds2.end(), dv.begin(), dout.begin(), dvo.begin(), same_point_x());
+      ASSERT_TRUE(du.first - dout.begin() == hu.first - hout.begin());
+      ASSERT_TRUE(same(thrust::host_vector<point>(dout.begin(), du.first), thrust::host_vector<point>(hout.begin(), hu.first)));
+      ASSERT_TRUE(same(thrust::host_vector<short>(dvo.begin(), du.second), thrust::host_vector<short>(hvo.begin(), hu.second)));
+      auto hin = thrust::unique(hs2.begin(), hs2.end(), same_point_x());
+      auto din = thrust::unique(ds2.begin(), ds2.end(), same_point_x());
+      ASSERT_TRUE(din - ds2.begin() == hin - hs2.begin());
+      ASSERT_TRUE(same(thrust::host_vector<point>(ds2.begin(), din), thrust::host_vector<point>(hs2.begin(), hin)));
+    }
+  }
+}
+
 int main() {
   TestKnownAnswers();
   TestReduceWithBigIndexes();
@@ -727,6 +883,7 @@ int main() {
   TestDiscardAndForeignOperator();
   TestAsyncForEachTransformWhenAll();
   Differential();
+  TestUserPredicateSelectionShapes();
   TestUserOperators();
   TestWideElements();
   TestUserPredicatesByKey();

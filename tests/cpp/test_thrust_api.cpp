@@ -1206,6 +1206,26 @@ static void TestUniversalVector() {  // testing/universal_memory.cu:25-82: one p
 // an event per block, never the stream.  async::reduce runs on a stream of its own and gives
 // its temporary storage back on that stream; dropping the future destroys the stream; the
 // synchronous reduce of the same size on the null stream then picks that very block up.
+// thrust/detail/vector_base.inl:165-180 in the reference: a host_vector built from a range of
+// device iterators copies the range in one piece (here: a million elements in far less time
+// than a million single reads would take), converting the elements if the types differ.
+static void TestHostVectorFromDeviceRange() {
+  g_test = "host_vector from a device range";
+  const size_t n = 1u << 20;
+  thrust::host_vector<int> src(n);
+  for (size_t i = 0; i < n; ++i) src[i] = (int)i + 7;
+  thrust::device_vector<int> d(src);
+  thrust::host_vector<int> h(d.begin() + 5, d.end() - 3);
+  ASSERT_TRUE(h.size() == n - 8);
+  bool ok = true;
+  for (size_t i = 0; i < h.size(); ++i) ok = ok && h[i] == (int)(i + 12);
+  ASSERT_TRUE(ok);
+  thrust::host_vector<long long> wide(d.begin(), d.begin() + 100);
+  ASSERT_TRUE(wide.size() == 100 && wide[0] == 7 && wide[99] == 106);
+  thrust::host_vector<int> none(d.begin(), d.begin());
+  ASSERT_TRUE(none.empty());
+}
+
 static void TestTempArenaOutlivesStream() {
   g_test = "TempArenaOutlivesStream";
   ASSERT_TRUE(thrust_amd_temp_trim() == 0);  // nothing cached: the next block is the only one
@@ -1440,6 +1460,7 @@ int main() {
   TestTempArenaOutlivesStream();
   TestMemoryResources();
   TestPoolResources();
+  TestHostVectorFromDeviceRange();
   TestUniversalVector();
   std::printf("%s: %d checks, %d failed\n", g_failed ? "FAILED" : "PASSED", g_checks, g_failed);
   return g_failed ? 1 : 0;
