@@ -35,6 +35,13 @@ struct binary_function { typedef A1 first_argument_type; typedef A2 second_argum
 THRUST_AMD_BINARY_FUNCTOR(plus, T, lhs + rhs)
 THRUST_AMD_BINARY_FUNCTOR(minus, T, lhs - rhs)
 THRUST_AMD_BINARY_FUNCTOR(multiplies, T, lhs * rhs)
+THRUST_AMD_BINARY_FUNCTOR(divides, T, lhs / rhs)
+THRUST_AMD_BINARY_FUNCTOR(modulus, T, lhs % rhs)
+THRUST_AMD_BINARY_FUNCTOR(bit_and, T, lhs & rhs)
+THRUST_AMD_BINARY_FUNCTOR(bit_or, T, lhs | rhs)
+THRUST_AMD_BINARY_FUNCTOR(bit_xor, T, lhs ^ rhs)
+THRUST_AMD_BINARY_FUNCTOR(logical_and, bool, lhs && rhs)
+THRUST_AMD_BINARY_FUNCTOR(logical_or, bool, lhs || rhs)
 THRUST_AMD_BINARY_FUNCTOR(equal_to, bool, lhs == rhs)
 THRUST_AMD_BINARY_FUNCTOR(not_equal_to, bool, lhs != rhs)
 THRUST_AMD_BINARY_FUNCTOR(less, bool, lhs < rhs)
@@ -63,6 +70,58 @@ struct logical_not {
   typedef bool result_type;
   constexpr bool operator()(const T& x) const { return !x; }
 };
+template <>
+struct logical_not<void> {
+  template <typename A>
+  constexpr bool operator()(const A& x) const { return !x; }
+};
+// project1st / project2nd return one of their two arguments (thrust/functional.h:1307-1401 in
+// the reference); not1 / not2 negate a predicate (thrust/functional.h:1407-1493).
+template <typename T1 = void, typename T2 = void>
+struct project1st {
+  typedef T1 first_argument_type;
+  typedef T2 second_argument_type;
+  typedef T1 result_type;
+  constexpr const T1& operator()(const T1& lhs, const T2&) const { return lhs; }
+};
+template <>
+struct project1st<void, void> {
+  template <typename A, typename B>
+  constexpr const A& operator()(const A& lhs, const B&) const { return lhs; }
+};
+template <typename T1 = void, typename T2 = void>
+struct project2nd {
+  typedef T1 first_argument_type;
+  typedef T2 second_argument_type;
+  typedef T2 result_type;
+  constexpr const T2& operator()(const T1&, const T2& rhs) const { return rhs; }
+};
+template <>
+struct project2nd<void, void> {
+  template <typename A, typename B>
+  constexpr const B& operator()(const A&, const B& rhs) const { return rhs; }
+};
+template <typename Predicate>
+struct unary_negate {
+  typedef bool result_type;
+  Predicate pred;
+  explicit constexpr unary_negate(const Predicate& p) : pred(p) {}
+  template <typename A>
+  constexpr bool operator()(const A& x) const { return !pred(x); }
+};
+template <typename Predicate>
+constexpr unary_negate<Predicate> not1(const Predicate& pred) { return unary_negate<Predicate>(pred); }
+template <typename Predicate>
+struct binary_negate {
+  typedef bool result_type;
+  Predicate pred;
+  explicit constexpr binary_negate(const Predicate& p) : pred(p) {}
+  template <typename A, typename B>
+  constexpr bool operator()(const A& x, const B& y) const { return !pred(x, y); }
+};
+template <typename Predicate>
+constexpr binary_negate<Predicate> not2(const Predicate& pred) { return binary_negate<Predicate>(pred); }
+
 template <typename T = void>
 struct negate {
   typedef T argument_type;

@@ -1,18 +1,23 @@
-// unique, unique_by_key and reduce_by_key for a user's key predicate, operator or element
-// structs (hipcc translation units).  They are put together from pieces that exist already:
+// unique, unique_by_key, reduce_by_key and scan_by_key for a user's key predicate, operator or
+// element structs (hipcc translation units).
 //
-//   run flags   one kernel, instantiated for the predicate: head[i] = i == 0 || !pred(k[i-1], k[i])
-//               and tail[i] = i == n-1 || !pred(k[i], k[i+1]), one byte each
-//               (thrust/detail/range/head_flags.h:130-160, tail_flags.h in the reference)
-//   selection   the library's compaction kernel with those bytes as its stencil: the keys at the
-//               heads, the values at the heads (unique_by_key) or at the tails (reduce_by_key)
-//   sums        reduce_by_key scans (head, value) pairs with the segmented form of the operator
-//               through the generic in-order scan, exactly the reference's formulation
-//               (thrust/system/detail/generic/reduce_by_key.inl:50-136); the pairs are made as
-//               the scan reads them and only the values are written; the value at a run's
-//               tail is the run's sum
-//
-// Keys and values are moved by the selection kernel as items of 1, 2, 4 or 8 bytes.
+//   unique, unique_by_key   the single-pass compaction kernel, instantiated for the predicate
+//                           (thrust/system/hip/detail/generic_select.h)
+//   reduce_by_key           the single-pass segmented reduction, instantiated for the predicate and
+//                           the operator (thrust/system/hip/detail/reduce_by_key_kernels.h), when
+//                           the sums have the values' own type and keys and values are items of
+//                           up to 8 bytes
+//   otherwise, and for scan_by_key, a composition of pieces:
+//     run flags   one kernel, instantiated for the predicate: head[i] = i == 0 || !pred(k[i-1], k[i])
+//                 and tail[i] = i == n-1 || !pred(k[i], k[i+1]), one byte each
+//                 (thrust/detail/range/head_flags.h:130-160, tail_flags.h in the reference)
+//     sums        (head, value) pairs scanned with the segmented form of the operator through
+//                 the generic in-order scan, the reference's formulation
+//                 (thrust/system/detail/generic/reduce_by_key.inl:50-136); the pairs are made as
+//                 the scan reads them and only the values are written; the value at a run's
+//                 tail is the run's sum
+//     selection   the library's compaction kernel with the flag bytes as its stencil: the keys at
+//                 the heads, the sums at the tails
 #pragma once
 #if !defined(__HIPCC__)
 #error "thrust/system/hip/detail/generic_by_key.h is HIP code: compile this translation unit with hipcc"
@@ -24,6 +29,7 @@
 #include <thrust/scan.h>
 #include <thrust/system/hip/detail/device_input.h>
 #include <thrust/system/hip/detail/generic_select.h>
+#include <thrust/system/hip/detail/reduce_by_key_kernels.h>
 
 namespace thrust {
 namespace system {
@@ -137,11 +143,54 @@ pair<KOut, VOut> unique_by_key_copy_generic(execution_policy<D>& exec, KIn kf, K
   return thrust::make_pair(ko + cnt, vo + cnt);
 }
 
+// Keys and values the single-pass kernel takes as they are: keys of up to 8 bytes, values of the
+// output's own type, 4 or 8 bytes wide (or a narrow integer, which travels widened).
+template <typename K, typename VI, typename V>
+struct reduces_by_key_in_one_pass
+    : std::integral_constant<bool, is_kernel_item<K>::value && sizeof(K) <= 8 && std::is_same<VI, V>::value &&
+                                       is_kernel_item<V>::value &&
+                                       (sizeof(V) == 4 || sizeof(V) == 8 || std::is_same<V, int8_t>::value ||
+                                        std::is_same<V, uint8_t>::value || std::is_same<V, int16_t>::value ||
+                                        std::is_same<V, uint16_t>::value)> {};
+
+// The single-pass kernel, instantiated for the caller's key equality and operator.
+template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key_one_pass(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo, Pred pred,
+                                        Op op) {
+  namespace seg = ::thrust::system::hip::segmented;
+  typedef typename std::remove_const<typename iterator_value<KIn>::type>::type K;
+  typedef typename iterator_value<VOut>::type V;
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(kl - kf);
+  device_input<KIn> keys(stream, temp_source_of(exec), kf, n);
+  device_input<VIn> values(stream, temp_source_of(exec), vf, n);
+  const seg::RbkTemp<K, V> lay(n);
+  temp_storage temp(stream, temp_source_of(exec));
+  temp.ensure(lay.total + 256);
+  char* base = static_cast<char*>(temp.ptr());
+  uint64_t* d_num = reinterpret_cast<uint64_t*>(base + lay.total);
+  seg::RbkArgs<K, V, Pred, Op> a = seg::make_rbk_args<K, V>(pred, op);
+  a.keys = (const K*)keys.ptr();
+  a.values = (const V*)values.ptr();
+  a.keys_out = thrust::detail::raw(ko);
+  a.values_out = thrust::detail::raw(vo);
+  a.d_num_runs = d_num;
+  a.n = n;
+  throw_on_error(seg::rbk_launch(base, a, (hipStream_t)stream), "reduce_by_key failed");
+  const uint64_t runs = read_scalar<uint64_t>(d_num, stream, "reduce_by_key failed");
+  return thrust::make_pair(ko + runs, vo + runs);
+}
+
 template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred, typename Op>
 pair<KOut, VOut> reduce_by_key_generic(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo, Pred pred,
                                        Op op) {
   typedef typename std::remove_const<typename iterator_value<KIn>::type>::type K;
   typedef typename iterator_value<VOut>::type V;  // sums have the output's value type
+  typedef typename std::remove_const<typename iterator_value<VIn>::type>::type VI;
+  if constexpr (reduces_by_key_in_one_pass<K, VI, V>::value && std::is_same<typename iterator_value<KOut>::type, K>::value) {
+    // the kernel counts runs in 32 bits; beyond that the composition below takes over
+    if ((uint64_t)(kl - kf) < 0xffffffffull) return reduce_by_key_one_pass(exec, kf, kl, vf, ko, vo, pred, op);
+  }
   static_assert(is_abi_item<K>::value && std::is_same<typename iterator_value<KOut>::type, K>::value &&
                     is_abi_item<V>::value,
                 "reduce_by_key on the device system: keys and sums of 1, 2, 4 or 8 bytes, same key type in and out");

@@ -313,6 +313,84 @@ static void TestUserPredicatesByKey() {
   }
 }
 
+// reduce_by_key through the single-pass kernel instantiated for the caller's functors: operators
+// without an identity that are not commutative (so any change of order or a stray operand
+// shows), struct values, struct keys, narrow values, and runs from one element to several tiles.
+struct span {  // the range of positions a run covers, and how many elements it has
+  int first, last;
+  __host__ __device__ bool operator==(const span& o) const { return first == o.first && last == o.last; }
+};
+struct join_spans {  // associative, not commutative, no identity
+  __host__ __device__ span operator()(const span& a, const span& b) const { return span{a.first, b.last}; }
+};
+struct take_right {
+  __host__ __device__ unsigned operator()(unsigned, unsigned b) const { return b; }
+};
+struct affine {  // x -> a x + b over the integers modulo 2^32; composition is associative, not commutative
+  unsigned a, b;
+  __host__ __device__ bool operator==(const affine& o) const { return a == o.a && b == o.b; }
+};
+struct compose_affine {
+  __host__ __device__ affine operator()(const affine& f, const affine& g) const { return affine{g.a * f.a, g.a * f.b + g.b}; }
+};
+struct wide_key {
+  int group;
+  int noise;
+  __host__ __device__ bool operator==(const wide_key& o) const { return group == o.group && noise == o.noise; }
+};
+struct same_group {
+  __host__ __device__ bool operator()(const wide_key& a, const wide_key& b) const { return a.group == b.group; }
+};
+struct short_max {
+  __host__ __device__ short operator()(short a, short b) const { return a < b ? b : a; }
+};
+
+template <typename K, typename V, typename Eq, typename Op>
+static void CheckReduceByKey(const thrust::host_vector<K>& hk, const thrust::host_vector<V>& hval, Eq eq, Op op) {
+  const size_t n = hk.size();
+  const thrust::device_vector<K> dk(hk);
+  const thrust::device_vector<V> dval(hval);
+  thrust::host_vector<K> hko(n);
+  thrust::host_vector<V> hvo(n);
+  thrust::device_vector<K> dko(n);
+  thrust::device_vector<V> dvo(n);
+  auto hr = thrust::reduce_by_key(hk.begin(), hk.end(), hval.begin(), hko.begin(), hvo.begin(), eq, op);
+  auto dr = thrust::reduce_by_key(dk.begin(), dk.end(), dval.begin(), dko.begin(), dvo.begin(), eq, op);
+  const size_t runs = hr.first - hko.begin();
+  ASSERT_TRUE((size_t)(dr.first - dko.begin()) == runs && (size_t)(dr.second - dvo.begin()) == runs);
+  ASSERT_TRUE(same(thrust::host_vector<K>(dko.begin(), dko.begin() + runs), thrust::host_vector<K>(hko.begin(), hko.begin() + runs)));
+  ASSERT_TRUE(same(thrust::host_vector<V>(dvo.begin(), dvo.begin() + runs), thrust::host_vector<V>(hvo.begin(), hvo.begin() + runs)));
+}
+
+static void TestReduceByKeyWithUserFunctors() {
+  g_test = "reduce_by_key with user functors in the single-pass kernel";
+  for (size_t n : {(size_t)1, (size_t)2, (size_t)100, (size_t)14336, (size_t)14337, (size_t)100000, ((size_t)1 << 20) + 11}) {
+    for (size_t mean_run : {(size_t)1, (size_t)3, (size_t)700, (size_t)50000, n + 1}) {
+      thrust::host_vector<int> hk(n);
+      thrust::host_vector<wide_key> hw(n);
+      thrust::host_vector<span> hspan(n);
+      thrust::host_vector<unsigned> hu(n);
+      thrust::host_vector<affine> haff(n);
+      thrust::host_vector<short> hsh(n);
+      int group = 0;
+      for (size_t i = 0; i < n; ++i) {
+        if (i && mix(i * 7 + mean_run) % mean_run == 0) ++group;
+        hk[i] = group;
+        hw[i] = wide_key{group, (int)(mix(i) % 5)};
+        hspan[i] = span{(int)i, (int)i};
+        hu[i] = (unsigned)mix(i + 3);
+        haff[i] = affine{(unsigned)(mix(i) | 1u), (unsigned)mix(i + 17)};
+        hsh[i] = (short)(mix(i + 23) % 30000);
+      }
+      CheckReduceByKey(hk, hspan, thrust::equal_to<int>(), join_spans());
+      CheckReduceByKey(hk, hu, thrust::equal_to<int>(), take_right());
+      CheckReduceByKey(hw, haff, same_group(), compose_affine());
+      CheckReduceByKey(hw, hu, same_group(), thrust::bit_xor<unsigned>());
+      CheckReduceByKey(hk, hsh, thrust::equal_to<int>(), short_max());
+    }
+  }
+}
+
 struct add_first_two_into_third {  // the functor of examples/arbitrary_transformation.cu
   template <typename Tuple>
   __host__ __device__ void operator()(Tuple t) const { thrust::get<2>(t) = thrust::get<0>(t) + thrust::get<1>(t); }
@@ -887,6 +965,7 @@ int main() {
   TestUserOperators();
   TestWideElements();
   TestUserPredicatesByKey();
+  TestReduceByKeyWithUserFunctors();
   TestZipIterator();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
   std::printf(g_failed ? "FAILED\n" : "PASSED\n");

@@ -66,7 +66,27 @@ static void TestFloatZerosUnderLessAndUnderAUserComparator() {
   for (int i = 0; i < 6; ++i) CHECK(v3[i] == want_user[i]);
 }
 
+// thrust/functional.h:420-1493 in the reference: the arithmetic, bitwise and logical functors,
+// the projections and the negators, here through host algorithms.
+static void TestFunctors() {
+  thrust::host_vector<unsigned> x(std::vector<unsigned>{12, 10, 7, 5});
+  CHECK(thrust::reduce(thrust::host, x.begin(), x.end(), 0u, thrust::bit_xor<unsigned>()) == (12u ^ 10u ^ 7u ^ 5u));
+  CHECK(thrust::reduce(thrust::host, x.begin(), x.end(), ~0u, thrust::bit_and<unsigned>()) == (12u & 10u & 7u & 5u));
+  CHECK(thrust::reduce(thrust::host, x.begin(), x.end(), 0u, thrust::bit_or<unsigned>()) == 15u);
+  CHECK(thrust::divides<int>()(17, 5) == 3 && thrust::modulus<int>()(17, 5) == 2);
+  CHECK(thrust::divides<>()(9.0, 2) == 4.5);
+  CHECK(thrust::logical_and<int>()(3, 0) == false && thrust::logical_or<int>()(3, 0) == true);
+  CHECK(thrust::logical_not<>()(0) == true);
+  CHECK((thrust::project1st<int, double>()(4, 2.5) == 4) && (thrust::project2nd<int, double>()(4, 2.5) == 2.5));
+  CHECK(thrust::project2nd<>()(4, 'c') == 'c');
+  CHECK(thrust::reduce(thrust::host, x.begin(), x.end(), 99u, thrust::project2nd<unsigned, unsigned>()) == 5u);
+  CHECK(thrust::not2(within_one())(1, 2) == false && thrust::not2(within_one())(1, 3) == true);
+  struct is_odd { bool operator()(unsigned v) const { return v & 1u; } };
+  CHECK(thrust::not1(is_odd())(12u) == true && thrust::not1(is_odd())(7u) == false);
+}
+
 int main() {
+  TestFunctors();
   TestReduceByKeyComparesWithTheRunsFirstKey();
   TestFloatZerosUnderLessAndUnderAUserComparator();
   std::printf("%d checks, %d failed\n", g_checks, g_fail);
