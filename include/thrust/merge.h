@@ -9,6 +9,8 @@
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
 #if defined(__HIPCC__)
+#include <thrust/system/hip/detail/generic_select.h>
+#include <thrust/system/hip/detail/merge_kernels.h>
 #include <thrust/system/hip/detail/merge_sort_kernels.h>
 #endif
 
@@ -131,6 +133,34 @@ void merge_generic(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1
   void* stream = stream_of(exec);
   const uint64_t na = (uint64_t)(kl1 - kf1), nb = (uint64_t)(kl2 - kf2), n = na + nb;
   if (n == 0) return;
+  // keys (and values) of up to 8 bytes: the merge-path kernels of the library, instantiated for
+  // the comparator, read the two ranges where they lie (fancy iterators are written out first)
+  if constexpr (is_kernel_item<K>::value && sizeof(K) <= 8 && is_kernel_item<V>::value && sizeof(V) <= 8 &&
+                std::is_same<typename std::remove_const<typename iterator_value<K2>::type>::type, K>::value) {
+    namespace mg = thrust::system::hip::merging;
+    device_input<K1> a(stream, temp_source_of(exec), kf1, na);
+    device_input<K2> b(stream, temp_source_of(exec), kf2, nb);
+    temp_storage temp(stream, temp_source_of(exec));
+    temp.ensure(mg::merge_temp_bytes(n));
+    int rc;
+    if (has_values) {
+      typedef typename std::remove_const<typename iterator_value<V1>::type>::type Va;
+      typedef typename std::remove_const<typename iterator_value<V2>::type>::type Vb;
+      static_assert(std::is_same<Va, Vb>::value, "merge_by_key on the device system: one value type for both ranges");
+      device_input<V1> va(stream, temp_source_of(exec), vf1, na);
+      device_input<V2> vb(stream, temp_source_of(exec), vf2, nb);
+      rc = mg::merge_launch<K, Va, true>(static_cast<uint64_t*>(temp.ptr()), (const K*)a.ptr(), na, (const K*)b.ptr(), nb,
+                                         (const Va*)va.ptr(), (const Va*)vb.ptr(), thrust::detail::raw(ko),
+                                         (Va*)thrust::detail::raw(vo), comp, (hipStream_t)stream);
+    } else {
+      rc = mg::merge_launch<K, uint32_t, false>(static_cast<uint64_t*>(temp.ptr()), (const K*)a.ptr(), na,
+                                                (const K*)b.ptr(), nb, (const uint32_t*)nullptr, (const uint32_t*)nullptr,
+                                                thrust::detail::raw(ko), (uint32_t*)nullptr, comp, (hipStream_t)stream);
+    }
+    throw_on_error(rc, "merge failed");
+    synchronize(stream, "merge: synchronize");
+    return;
+  }
   const uint64_t tiles = (n + ms::TILE - 1) / ms::TILE;
   const std::size_t key_bytes = ((std::size_t)n * sizeof(K) + 255) / 256 * 256;
   const std::size_t val_bytes = has_values ? ((std::size_t)n * sizeof(V) + 255) / 256 * 256 : 0;

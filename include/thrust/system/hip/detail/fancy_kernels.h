@@ -49,7 +49,7 @@ __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void scatter_kernel(ViewIn in, V
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[map[i]] = in[i];
 }
 
-inline int launch_status() { return (int)hipGetLastError(); }
+inline int launch_status() { return (int)hipPeekAtLastError(); }
 
 }  // namespace detail
 }  // namespace hip

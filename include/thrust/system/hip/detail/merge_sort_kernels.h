@@ -373,20 +373,20 @@ int sort(void* temp, size_t* temp_bytes, K* keys, V* vals, uint64_t n, Comp comp
   THRUST_AMD_MERGE_SORT_LAUNCH("merge_sort_block", stream, (block_sort_kernel<K, V, HAS_VALUES, Comp>),
                                dim3((uint32_t)lay.tiles), dim3(BLOCK), (const K*)keys, (const V*)vals, key_buf[cur],
                                val_buf[cur], n, comp);
-  hipError_t err = hipGetLastError();
+  hipError_t err = hipPeekAtLastError();
   if (err != hipSuccess) return (int)err;
   uint64_t run = TILE;
   for (int p = 0; p < passes; ++p) {
     THRUST_AMD_MERGE_SORT_LAUNCH("merge_sort_partition", stream, (merge_partition_kernel<K, Comp>),
                                  dim3((uint32_t)((lay.tiles + 255) / 256)), dim3(256), (const K*)key_buf[cur], n, run,
                                  lay.tiles, comp, split);
-    err = hipGetLastError();
+    err = hipPeekAtLastError();
     if (err != hipSuccess) return (int)err;
     THRUST_AMD_MERGE_SORT_LAUNCH("merge_sort_pass", stream, (merge_pass_kernel<K, V, HAS_VALUES, Comp>),
                                  dim3((uint32_t)lay.tiles), dim3(BLOCK), (const K*)key_buf[cur],
                                  (const V*)val_buf[cur], key_buf[cur ^ 1], val_buf[cur ^ 1], n, run, lay.tiles,
                                  (const uint64_t*)split, comp);
-    err = hipGetLastError();
+    err = hipPeekAtLastError();
     if (err != hipSuccess) return (int)err;
     cur ^= 1;
     run *= 2;
@@ -404,12 +404,12 @@ int merge_two(const K* both, const V* both_values, uint64_t na, uint64_t n, K* o
   if (tiles > 0x7fffffffull) return (int)hipErrorInvalidValue;
   THRUST_AMD_MERGE_SORT_LAUNCH("merge_sort_partition", stream, (merge_partition_kernel<K, Comp, true>),
                                dim3((uint32_t)((tiles + 255) / 256)), dim3(256), both, n, na, tiles, comp, split);
-  hipError_t err = hipGetLastError();
+  hipError_t err = hipPeekAtLastError();
   if (err != hipSuccess) return (int)err;
   THRUST_AMD_MERGE_SORT_LAUNCH("merge_sort_pass", stream, (merge_pass_kernel<K, V, HAS_VALUES, Comp, true>),
                                dim3((uint32_t)tiles), dim3(BLOCK), both, both_values, out, out_values, n, na, tiles,
                                (const uint64_t*)split, comp);
-  return (int)hipGetLastError();
+  return (int)hipPeekAtLastError();
 }
 
 }  // namespace merge_sort

@@ -151,22 +151,4 @@ TA_DEVICE void with_cmp_code(int cmp, F&& f) {
   }
 }
 
-// ------------------------------------------------------------------ search
-// First index in [lo, hi] at which a monotone predicate turns false (pred is true on a
-// prefix of [lo, hi) and false after it; the result is hi when it is true throughout).
-// Plain bisection: for the tile-boundary searches over whole inputs, probing more points
-// per round (eight-way per lane, or 64-way per wave) was measured 2x and 5x slower -- the
-// lanes of a wave search distant diagonals, every probe is its own cache line and page,
-// and the extra probes cost more than the saved rounds.
-template <typename Pred>
-TA_DEVICE uint64_t partition_point(uint64_t lo, uint64_t hi, Pred pred) {
-  while (lo < hi) {
-    const uint64_t mid = (lo + hi) >> 1;
-    if (pred(mid)) lo = mid + 1;
-    else hi = mid;
-  }
-  return lo;
-}
-
-
 }  // namespace ta
