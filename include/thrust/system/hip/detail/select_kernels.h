@@ -90,10 +90,14 @@ struct SelectShape {
   static constexpr bool LEAN_TWO = LEAN && TWO;
   static constexpr int BLOCK = LEAN ? SELECT_LEAN_BLOCK : SELECT_BLOCK;
   static constexpr int WAVES_PER_SIMD = 4;  // 128 registers: two lean workgroups per CU, or one with a payload
-  static constexpr int BY_BYTES = SELECT_LANE_BYTES / (int)(sizeof(T) + (HAS_PAYLOAD ? sizeof(U) : 0));
+  // registers count, not bytes: an element narrower than four bytes still takes a register once unpacked
+  static constexpr int BY_BYTES = SELECT_LANE_BYTES / (int)((sizeof(T) < 4 ? 4 : sizeof(T)) + (HAS_PAYLOAD ? (sizeof(U) < 4 ? 4 : sizeof(U)) : 0));
+  // 8-byte elements without a payload: 24 instead of 32 (16 vectors' worth of flags and ranks beside
+  // 64 data registers and 64-bit comparisons spilled)
+  static constexpr int WIDE_ALONE = (!HAS_PAYLOAD && sizeof(T) == 8) ? 24 : SELECT_MAX_ITEMS;
   static constexpr int WANTED =
       LEAN_TWO ? SELECT_LEAN_TWO_ITEMS : LEAN ? (MODE == FLAG_HEAD ? SELECT_LEAN_HEAD_ITEMS : SELECT_LEAN_ITEMS)
-           : (BY_BYTES < SELECT_MIN_ITEMS ? SELECT_MIN_ITEMS : (BY_BYTES > SELECT_MAX_ITEMS ? SELECT_MAX_ITEMS : BY_BYTES));
+           : (BY_BYTES < SELECT_MIN_ITEMS ? SELECT_MIN_ITEMS : (BY_BYTES > WIDE_ALONE ? WIDE_ALONE : BY_BYTES));
   static constexpr int CHUNKS = WANTED / VEC >= 1 ? WANTED / VEC : 1;
   static constexpr uint32_t TILE = (uint32_t)BLOCK * CHUNKS * VEC;
   // LDS of one wave for the write-out: four 16-byte vectors per lane, or one chunk of the

@@ -14,10 +14,10 @@ pytestmark = pytest.mark.gpu
 BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "cpp", "bin")
 
 
-def _run(name, timeout=300):
+def _run(name, *args, timeout=300):
     path = os.path.join(BIN, name)
     assert os.path.exists(path), f"{path} is not built (python -c 'import __graft_entry__ as g; g.build()')"
-    r = subprocess.run([path], capture_output=True, text=True, timeout=timeout)
+    r = subprocess.run([path, *args], capture_output=True, text=True, timeout=timeout)
     print(r.stdout[-4000:])
     print(r.stderr[-2000:])
     assert r.returncode == 0, r.stdout[-4000:]
@@ -44,3 +44,12 @@ def test_fancy_iterators_and_user_functors_compiled_with_hipcc():
     # counting / constant / transform / permutation iterators as inputs, transform, for_each, sequence, gather, scatter
     out = _run("test_fancy_iterators")
     assert "PASSED" in out
+
+
+@pytest.mark.parametrize("log2_n", ["12", "22"])
+def test_user_functors_and_library_functors_give_the_same_output(log2_n):
+    # every algorithm once with a functor of the caller's own (kernels instantiated in the test's translation unit) and
+    # once with the library's (kernels of libthrust_amd.so): sizes and contents must agree; the times it prints are
+    # informative only
+    out = _run("test_user_functor_paths", log2_n)
+    assert "PASSED" in out and "0 mismatches" in out

@@ -69,6 +69,27 @@ def test_copy_if_stencil(dev, oracle, item, sdtype):
         assert cnt == ref.size and np.array_equal(out.numpy(cnt), ref)
 
 
+@pytest.mark.parametrize("sdtype", [np.int8, np.uint8, np.int16, np.uint16, np.int32, np.uint32, np.int64, np.uint64,
+                                    np.float32, np.float64])
+def test_stencil_forms_for_every_stencil_type_and_item_width(dev, oracle, sdtype):
+    """copy_if and partition_copy by stencil run one kernel per (stencil type, item width, one or two
+    outputs): each of them once, on a ragged size of several tiles, with every comparison code."""
+    n = 100003
+    st = _vals(n, sdtype, 23)
+    ds = dev.DeviceArray.from_numpy(st)
+    thr = 0.5 if np.dtype(sdtype).kind == "f" else 100
+    for item in (np.uint8, np.uint16, np.uint32, np.uint64):
+        x = _vals(n, item, 29)
+        d = dev.DeviceArray.from_numpy(x)
+        for cmp in (dev.LT, dev.LE, dev.GT, dev.GE, dev.EQ, dev.NE, dev.NONZERO):
+            out, cnt = dev.copy_if(d, cmp, thr, stencil=ds)
+            ref = oracle.copy_if(x, cmp, thr, stencil=st)
+            assert cnt == ref.size and np.array_equal(out.numpy(cnt), ref), (sdtype, item, cmp)
+        ot, of, cnt = dev.partition_copy(d, dev.LT, thr, stencil=ds)
+        rt, rf = oracle.partition_copy(x, dev.LT, thr, stencil=st)
+        assert cnt == rt.size and np.array_equal(ot.numpy(cnt), rt) and np.array_equal(of.numpy(n - cnt), rf), (sdtype, item)
+
+
 @pytest.mark.parametrize("dtype", [np.float32, np.uint8, np.uint64])
 def test_copy_if_in_place(dev, oracle, dtype):
     """out aliases in, the form remove_if uses (thrust/system/cuda/detail/remove.h:54-66): a

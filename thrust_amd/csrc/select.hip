@@ -6,41 +6,9 @@
 #include "dispatch.hpp"
 #include "launch.hpp"
 
-#include "../../include/thrust/system/hip/detail/select_kernels.h"
+#include "select_flaggers.hpp"
 
 namespace ta {
-using namespace ::thrust::system::hip::select;
-
-// The flags of the C interface: a comparison code and a threshold chosen at run time (one
-// uniform branch per tile picks the comparison), the bytes of a flag array, and "differs
-// from its predecessor" for unique.
-template <typename T>
-struct CmpFlagger {
-  int cmp;
-  T threshold;
-  template <typename Body>
-  TA_DEVICE void per_tile(Body&& body) const {
-    const bool flip = (cmp & THRUST_AMD_CMP_NOT) != 0;
-    const T thr = threshold;
-    with_cmp_code(cmp, [&](auto code) {
-      constexpr int CMP = decltype(code)::value;
-      body([thr](const T& x) { return apply_cmp_code<CMP>(x, thr); }, flip);
-    });
-  }
-};
-struct ByteFlagger {
-  template <typename Body>
-  TA_DEVICE void per_tile(Body&& body) const {
-    body([](uint8_t x) { return x != 0; }, false);
-  }
-};
-template <typename T>
-struct DiffersFlagger {
-  template <typename Body>
-  TA_DEVICE void per_tile(Body&& body) const {
-    body([](const T& before, const T& x) { return !(before == x); }, false);
-  }
-};
 
 // Stencil forms: flags[i] = stencil[i] CMP threshold as one byte each.
 template <typename T>
@@ -106,7 +74,14 @@ static int select_by_predicate(void* temp, size_t* temp_bytes, const void* in, c
       return 0;
     });
   }
-  // stencil form: byte flags first, then compaction of the items under those flags
+  // stencil form, separate outputs: one pass, the stencil is tested in its own type and the
+  // items travel as the payload (select_stencil.hip)
+  if (!in_place)
+    return select_by_stencil(temp, temp_bytes, in, stencil, out_true, out_false, d_num, n, item_bytes, stencil_dtype,
+                             cmp, threshold, stream);
+  // stencil form in place: byte flags first (the sweep may run from either end, and the
+  // items of a tile are parked or written over before the stencil's turn would come),
+  // then compaction of the items under those flags
   return with_item_bytes(item_bytes, [&](auto ut) {
     using U = typename decltype(ut)::type;
     const size_t flag_bytes = align_up((size_t)n, 256);
