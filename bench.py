@@ -203,9 +203,12 @@ def main():
     capi.load()  # raises if the HIP library is missing: there is no fallback
 
     want_host = not args.no_cpu_baseline
-    ms_sort, pass_ms, kernels_ms, host_keys = bench_sort(torch, capi, args.steps, args.warmup, want_host)
-    torch.cuda.empty_cache()
+    # reduce / scan first, on memory the process has not used before: device memory that was freed and
+    # allocated again can come back in smaller physical pieces, and a pure read then runs 3 % slower
+    # (0.182 against 0.177 ms for the same kernel on the same virtual address, measured)
     ms_reduce, ms_scan, host_c1 = bench_c1(torch, capi, args.steps, args.warmup, want_host)
+    torch.cuda.empty_cache()
+    ms_sort, pass_ms, kernels_ms, host_keys = bench_sort(torch, capi, args.steps, args.warmup, want_host)
     torch.cuda.empty_cache()
     config_rows = None
     if not args.no_configs:

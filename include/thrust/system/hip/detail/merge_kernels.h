@@ -53,7 +53,12 @@ __global__ __launch_bounds__(256) void merge_partition_kernel(const T* __restric
   const uint64_t total = na + nb;
   uint64_t diag = t * MERGE_TILE;
   if (diag > total) diag = total;
-  a_split[t] = merge_path<T>(a, na, b, nb, diag, comp);
+  // the merge-path search of merge_path() below, over the whole ranges: probes shared between threads
+  a_split[t] = aligned_partition_point(diag > nb ? diag - nb : 0, diag < na ? diag : na, [&](uint64_t mid) {
+    const T ka = a[mid];
+    const T kb = b[diag - 1 - mid];
+    return !comp(kb, ka);
+  });
 }
 
 // Slot of output element e in the LDS exchange buffer: one spare slot after every

@@ -223,8 +223,21 @@ __global__ __launch_bounds__(256) void merge_partition_kernel(const K* keys, uin
   const PairOfRuns p = pair_of<LONE>(t, run, n);
   const K* a = keys + p.a_begin;
   const K* b = keys + p.b_begin;
-  split[t] = merge_path<uint64_t>([&](uint64_t x) { return a[x]; }, p.na, [&](uint64_t x) { return b[x]; }, p.nb,
-                                  p.out0, comp);
+  // The merge-path search over the whole pair of runs, probing at every step the index of its
+  // interval that is a multiple of the largest power of two: as many steps as a bisection at
+  // worst, but the first steps of all threads of a pair probe the same few elements, which come
+  // from the caches instead of each being a miss of its own.
+  const uint64_t diag = p.out0;
+  uint64_t lo = diag > p.nb ? diag - p.nb : 0;
+  uint64_t hi = diag < p.na ? diag : p.na;
+  while (lo < hi) {
+    const uint64_t last = hi - 1;
+    const uint64_t differ = lo ^ last;
+    const uint64_t mid = differ ? (last & ~((1ull << (63 - __builtin_clzll(differ))) - 1ull)) : lo;
+    if (!comp(b[diag - 1 - mid], a[mid])) lo = mid + 1;
+    else hi = mid;
+  }
+  split[t] = lo;
 }
 
 template <typename K, typename V, bool HAS_VALUES, typename Comp, bool LONE = false>

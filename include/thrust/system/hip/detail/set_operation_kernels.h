@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void set_partition_kernel(const T* __restrict_
   const uint64_t total = na + nb;
   uint64_t diag = t * tile_size;
   if (diag > total) diag = total;
-  const uint64_t as = partition_point(diag > nb ? diag - nb : 0, diag < na ? diag : na, [&](uint64_t mid) {
+  const uint64_t as = aligned_partition_point(diag > nb ? diag - nb : 0, diag < na ? diag : na, [&](uint64_t mid) {
     return !comp(b[diag - 1 - mid], a[mid]);
   });
   split[t] = as;
@@ -95,10 +95,10 @@ __global__ __launch_bounds__(256) void set_partition_kernel(const T* __restrict_
   if (as < na && (bs >= nb || !comp(b[bs], a[as]))) x = a[as];
   else x = b[bs];
   // first index whose element is not before x / is after x, in each range
-  const uint64_t lb_a = partition_point(0, na, [&](uint64_t i) { return comp(a[i], x); });
-  const uint64_t ub_a = partition_point(lb_a, na, [&](uint64_t i) { return !comp(x, a[i]); });
-  const uint64_t lb_b = partition_point(0, nb, [&](uint64_t i) { return comp(b[i], x); });
-  const uint64_t ub_b = partition_point(lb_b, nb, [&](uint64_t i) { return !comp(x, b[i]); });
+  const uint64_t lb_a = aligned_partition_point(0, na, [&](uint64_t i) { return comp(a[i], x); });
+  const uint64_t ub_a = aligned_partition_point(lb_a, na, [&](uint64_t i) { return !comp(x, a[i]); });
+  const uint64_t lb_b = aligned_partition_point(0, nb, [&](uint64_t i) { return comp(b[i], x); });
+  const uint64_t ub_b = aligned_partition_point(lb_b, nb, [&](uint64_t i) { return !comp(x, b[i]); });
   key[t] = x;
   run[3 * t + 0] = lb_a + lb_b;
   run[3 * t + 1] = ub_a + lb_b;
