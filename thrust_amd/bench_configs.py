@@ -8,6 +8,11 @@ stream.  bench.py imports this module and prints the rows inside its JSON line.
   C4  reduce_by_key, unique_by_key and unique over 2^28 (int32 key, float32 value), mean run 8 / 1000
   C5  copy_if and stable_partition of 2^28 float32 at 50 % / 5 % selectivity,
       merge_by_key and merge of two sorted ranges of 2^27 uint32 (+ uint32 values)
+and the entry points beside the named path (rows "next_*"):
+  C6  count_if, inner_product, transform_reduce, transform_exclusive_scan over 2^28, inclusive_scan_by_key
+      over the C4 input with mean run 8
+  C7  set_union and set_intersection of the two sorted C5 ranges
+  C8  the comparison sort (merge sort) of 2^28 uint32 keys and of 2^27 uint64 keys with uint32 values
 
 Bytes are the algorithmic ones of each call (what must be read and written once).
 """
@@ -23,15 +28,17 @@ def _dev(capi, torch, t, code):
     return capi.DeviceArray(items, code, t.view(torch.uint8))
 
 
-_PAD = {}
+def _hold_device(torch):
+    """Keeps the device busy for a few hundred microseconds without touching memory, so that the
+    host can enqueue the whole call before the opening event is reached.  (A large fill did the
+    same job but left a gigabyte of dirty cache lines whose write-back ran into the timed call:
+    30-40 us on every row, 60 us on the read-only ones.)"""
+    torch.cuda._sleep(800_000)
 
 
 def _time_calls(torch, fn, reps, setup=None):
     """Median and minimum device time of fn() in ms; setup() runs before each call, untimed.
-    fn must not synchronise.  The device is kept busy with a fill while the host prepares
-    the call, so that the first event is not reached before the call has been enqueued."""
-    if "buf" not in _PAD:
-        _PAD["buf"] = torch.empty(1 << 30, dtype=torch.uint8, device="cuda")
+    fn must not synchronise."""
     if setup:
         setup()
     fn()  # sizes temp storage, warms up
@@ -40,7 +47,7 @@ def _time_calls(torch, fn, reps, setup=None):
     for _ in range(reps):
         if setup:
             setup()
-        _PAD["buf"].zero_()
+        _hold_device(torch)
         a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
         a.record()
         fn()
@@ -194,11 +201,121 @@ def run_c5(torch, capi, reps):
     return rows
 
 
+def run_c6(torch, capi, reps):
+    n = 1 << 28
+    rows = {}
+    xi = gen.c1_int32(torch, n)
+    di, t = _dev(capi, torch, xi, capi.I32), capi.Temp()
+    res = {}
+    med, mn = _time_calls(torch, lambda: res.update(r=capi.count_if(di, capi.LT, 500, temp=t, read_count=False)), reps)
+    if int(res["r"].numpy()[0]) != int((xi < 500).sum().item()):
+        _fail("C6 count_if")
+    rows["next_c6_count_if_i32"] = _row(med, mn, 4 * n)
+    oi, t2 = capi.DeviceArray(n, capi.I32), capi.Temp()
+    med, mn = _time_calls(torch, lambda: capi.transform_exclusive_scan(di, capi.SQUARE, 0, out=oi, temp=t2), reps)
+    sq = xi.to(torch.int64)
+    sq = sq * sq
+    want = torch.cumsum(sq, 0) - sq  # exclusive; values stay far below 2^63
+    if not torch.equal(oi.storage.view(torch.int32).to(torch.int64) & 0xFFFFFFFF, want & 0xFFFFFFFF):
+        _fail("C6 transform_exclusive_scan")
+    rows["next_c6_transform_exclusive_scan_i32_square"] = _row(med, mn, 8 * n)
+    del xi, di, oi, sq, want
+
+    xf, yf = gen.c5_float32(torch, n), gen.c5_float32(torch, n, seed=7)
+    df, dy, o1, t = _dev(capi, torch, xf, capi.F32), _dev(capi, torch, yf, capi.F32), capi.DeviceArray(1, capi.F32), capi.Temp()
+    exact = float((xf.to(torch.float64) * yf.to(torch.float64)).sum().item())
+    med, mn = _time_calls(torch, lambda: capi.inner_product(df, dy, 0, temp=t, out=o1), reps)
+    if abs(float(o1.numpy()[0]) - exact) > 1e-5 * exact:
+        _fail("C6 inner_product")
+    rows["next_c6_inner_product_f32"] = _row(med, mn, 8 * n)
+    del yf, dy
+    exact = float((xf.to(torch.float64) ** 2).sum().item())
+    t = capi.Temp()
+    med, mn = _time_calls(torch, lambda: capi.transform_reduce(df, capi.SQUARE, capi.PLUS, 0, temp=t, out=o1), reps)
+    if abs(float(o1.numpy()[0]) - exact) > 1e-5 * exact:
+        _fail("C6 transform_reduce")
+    rows["next_c6_transform_reduce_f32_square"] = _row(med, mn, 4 * n)
+    del xf, df
+
+    keys, vals = gen.c4_segments(torch, n, 8)
+    dk, dv = _dev(capi, torch, keys, capi.I32), _dev(capi, torch, vals, capi.F32)
+    out, t = capi.DeviceArray(n, capi.F32), capi.Temp()
+    med, mn = _time_calls(torch, lambda: capi.inclusive_scan_by_key(dk, dv, out=out, temp=t), reps)
+    # float64 running sums that start over at every run: the cumulative sum minus its value before the run
+    cs = torch.cumsum(vals.to(torch.float64), 0)
+    runs = int(keys[-1].item()) + 1
+    starts = torch.searchsorted(keys, torch.arange(runs, dtype=torch.int32, device="cuda"))
+    before = torch.where(starts > 0, cs[(starts - 1).clamp_min(0)], torch.zeros_like(cs[:1]))
+    want = cs - before[keys.to(torch.int64)]
+    if float((out.storage.view(torch.float32).to(torch.float64) - want).abs().max().item()) > 1e-4:
+        _fail("C6 inclusive_scan_by_key")
+    rows["next_c6_inclusive_scan_by_key_mean8"] = _row(med, mn, 12 * n)
+    return rows
+
+
+def _multiplicities(torch, sorted_u, uniq):
+    return torch.searchsorted(sorted_u, uniq, right=True) - torch.searchsorted(sorted_u, uniq)
+
+
+def run_c7(torch, capi, reps):
+    m = 1 << 27
+    (ka, _), (kb, _) = gen.c5_merge_inputs(torch, m)
+    a, b = _dev(capi, torch, ka, capi.U32), _dev(capi, torch, kb, capi.U32)
+    out = capi.DeviceArray(2 * m, capi.U32)
+    ua, ub = ka.to(torch.int64) & 0xFFFFFFFF, kb.to(torch.int64) & 0xFFFFFFFF
+    uniq = torch.unique(torch.cat([ua, ub]))
+    ca, cb = _multiplicities(torch, ua, uniq), _multiplicities(torch, ub, uniq)
+    rows = {}
+    for op, name, want in ((capi.SET_UNION, "set_union", torch.maximum(ca, cb)),
+                           (capi.SET_INTERSECTION, "set_intersection", torch.minimum(ca, cb))):
+        t, res = capi.Temp(), {}
+        med, mn = _time_calls(torch, lambda: res.update(r=capi.set_operation(op, a, b, out=out, temp=t, read_count=False)), reps)
+        cnt = int(res["r"][-1].numpy()[0])
+        got = out.storage.view(torch.int32)[:cnt].to(torch.int64) & 0xFFFFFFFF
+        # the multiset definition: every key as often as the rule says, in order
+        if cnt != int(want.sum().item()) or not bool((got[1:] >= got[:-1]).all().item()) \
+                or not torch.equal(_multiplicities(torch, got, uniq), want):
+            _fail(f"C7 {name}")
+        rows[f"next_c7_{name}_2x2p27"] = _row(med, mn, 4 * (2 * m + cnt), kept=cnt)
+    return rows
+
+
+def run_c8(torch, capi, reps):
+    n = 1 << 28
+    src = gen.c2_uint32(torch, n)
+    s, work, t = _dev(capi, torch, src, capi.U32), capi.DeviceArray(n, capi.U32), capi.Temp()
+    med, mn = _time_calls(torch, lambda: capi.merge_sort_keys(work, temp=t), reps,
+                          setup=lambda: work.storage.copy_(s.storage))
+    out = work.storage.view(torch.int32).to(torch.int64) & 0xFFFFFFFF
+    if not bool((out[1:] >= out[:-1]).all().item()) or int(out.sum().item()) != int((src.to(torch.int64) & 0xFFFFFFFF).sum().item()):
+        _fail("C8 merge sort of keys")
+    passes = 16  # ceil(log2(2^28 / 4096))
+    rows = {"next_c8_merge_sort_u32_2p28": _row(med, mn, (1 + passes) * 8 * n, Gkeys_per_s=round(n / med / 1e6, 2),
+                                                model="(1 + 16 merge passes) x 8 B/key")}
+    del src, s, work, t, out
+    m = 1 << 27
+    keys = gen.c3_uint64(torch, m, "full")
+    vals = torch.arange(m, dtype=torch.int32, device="cuda")
+    sk, sv = _dev(capi, torch, keys, capi.U64), _dev(capi, torch, vals, capi.U32)
+    wk, wv, t = capi.DeviceArray(m, capi.U64), capi.DeviceArray(m, capi.U32), capi.Temp()
+
+    def setup():
+        wk.storage.copy_(sk.storage)
+        wv.storage.copy_(sv.storage)
+    med, mn = _time_calls(torch, lambda: capi.merge_sort_pairs(wk, wv, temp=t), reps, setup=setup)
+    ko, vo = wk.storage.view(torch.int64), wv.storage.view(torch.int32).to(torch.int64)
+    o = ko ^ (-(1 << 63))
+    if not bool((o[1:] >= o[:-1]).all().item()) or not bool((keys[vo] == ko).all().item()):
+        _fail("C8 merge sort of pairs")
+    passes = 15
+    rows["next_c8_merge_sort_by_key_u64_u32_2p27"] = _row(med, mn, (1 + passes) * 24 * m, Gpairs_per_s=round(m / med / 1e6, 2),
+                                                          model="(1 + 15 merge passes) x 24 B/pair")
+    return rows
+
+
 def run_all(torch, capi, reps=5):
     rows = {}
-    for part in (run_c2_float, run_c3, run_c4, run_c5):
+    for part in (run_c2_float, run_c3, run_c4, run_c5, run_c6, run_c7, run_c8):
         rows.update(part(torch, capi, reps))
         torch.cuda.empty_cache()
-    _PAD.clear()
-    torch.cuda.empty_cache()
     return rows
