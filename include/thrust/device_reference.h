@@ -1,0 +1,3 @@
+// thrust/device_reference.h of the reference: here the declarations live in thrust/device_ptr.h.
+#pragma once
+#include <thrust/device_ptr.h>

@@ -5,6 +5,10 @@
 #include <cstdlib>
 #include <vector>
 
+#include <thrust/device_free.h>
+#include <thrust/device_malloc.h>
+#include <thrust/device_reference.h>
+#include <thrust/distance.h>
 #include <thrust/execution_policy.h>
 #include <thrust/functional.h>
 #include <thrust/host_vector.h>
@@ -85,8 +89,16 @@ static void TestFunctors() {
   CHECK(thrust::not1(is_odd())(12u) == true && thrust::not1(is_odd())(7u) == false);
 }
 
+static void TestDistance() {
+  thrust::host_vector<int> v(17);
+  CHECK(thrust::distance(v.begin(), v.end()) == 17);
+  thrust::device_ptr<int> p(nullptr);
+  CHECK(thrust::distance(p, p + 5) == 5);
+}
+
 int main() {
   TestFunctors();
+  TestDistance();
   TestReduceByKeyComparesWithTheRunsFirstKey();
   TestFloatZerosUnderLessAndUnderAUserComparator();
   std::printf("%d checks, %d failed\n", g_checks, g_fail);
