@@ -15,6 +15,8 @@
 #include <thrust/system/hip/detail/device_input.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/generic_kernels.h>
+#include <thrust/system/hip/detail/generic_select.h>
+#include <thrust/system/hip/detail/scan_kernels.h>
 #endif
 
 namespace thrust {
@@ -270,14 +272,57 @@ Out scan_generic(execution_policy<D>& exec, In first, In last, Out result, A ini
   return result;
 #endif
 }
+#if defined(__HIPCC__)
+// Elements of 4 or 8 bytes, the same type in, out and in the accumulator, written to device
+// memory: the single-pass scan (scan_kernels.h), instantiated for the operator.  Everything
+// else (wider structs, converting scans, outputs that are not memory) takes scan_generic.
+template <typename A, typename In, typename Out>
+struct scans_in_one_pass
+    : std::integral_constant<bool, is_kernel_item<A>::value && (sizeof(A) == 4 || sizeof(A) == 8) &&
+                                       std::is_same<typename std::remove_const<typename iterator_value<In>::type>::type, A>::value &&
+                                       std::is_same<typename iterator_value<Out>::type, A>::value &&
+                                       (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value)> {};
+template <bool EXCLUSIVE, typename A, typename D, typename In, typename Out, typename Op>
+Out scan_one_pass(execution_policy<D>& exec, In first, In last, Out result, A init, Op op) {
+  namespace sc = thrust::system::hip::scanning;
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  device_input<In> source(stream, temp_source_of(exec), first, n);
+  temp_storage temp(stream, temp_source_of(exec));
+  temp.ensure(sc::scan_temp_bytes<A>(n));
+  throw_on_error(sc::ordered_scan_launch<EXCLUSIVE>(static_cast<char*>(temp.ptr()), (const A*)source.ptr(),
+                                                    (A*)thrust::detail::raw(result), n, init, op, (hipStream_t)stream),
+                 "scan failed");
+  synchronize(stream, "scan: synchronize");
+  return result + n;
+}
+template <bool EXCLUSIVE, typename A, typename D, typename In, typename Out, typename Op>
+Out scan_user(execution_policy<D>& exec, In first, In last, Out result, A init, Op op, std::true_type) {
+  return scan_one_pass<EXCLUSIVE, A>(exec, first, last, result, init, op);
+}
+#endif
+template <bool EXCLUSIVE, typename A, typename D, typename In, typename Out, typename Op>
+Out scan_user(execution_policy<D>& exec, In first, In last, Out result, A init, Op op, std::false_type) {
+  return scan_generic<EXCLUSIVE, A>(exec, first, last, result, init, op);
+}
+template <typename A, typename In, typename Out>
+struct scan_user_route
+#if defined(__HIPCC__)
+    : scans_in_one_pass<A, In, Out> {
+};
+#else
+    : std::false_type {
+};
+#endif
 template <typename D, typename In, typename Out, typename Op>
 Out inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Op op, std::false_type) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
-  return scan_generic<false, V>(exec, first, last, result, V(), op);
+  return scan_user<false, V>(exec, first, last, result, V(), op, scan_user_route<V, In, Out>());
 }
 template <typename D, typename In, typename Out, typename T, typename Op>
 Out exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, T init, Op op, std::false_type) {
-  return scan_generic<true, T>(exec, first, last, result, init, op);
+  return scan_user<true, T>(exec, first, last, result, init, op, scan_user_route<T, In, Out>());
 }
 
 // library path: arithmetic input, output and accumulator with plus / minimum / maximum of the accumulator's type

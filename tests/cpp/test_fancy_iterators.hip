@@ -197,6 +197,38 @@ static void TestUserOperators() {
   }
 }
 
+// Ranges of more than 32 MiB take the large tile shape of the single-pass scan (1024 threads x 12
+// vectors): the same checks there, for an operator that does not commute on 8-byte elements and
+// for one of thrust/functional.h on 4-byte elements.
+static void TestUserOperatorScansOfLargeRanges() {
+  g_test = "scans of large ranges with user operators";
+  {
+    const size_t n = ((size_t)1 << 23) + 12345;
+    thrust::host_vector<Affine> h(n), want(n);
+    for (size_t i = 0; i < n; ++i) h[i] = Affine{(unsigned)(mix(i) | 1u), (unsigned)mix(i + 99)};
+    thrust::device_vector<Affine> d(h), out(n);
+    thrust::inclusive_scan(h.begin(), h.end(), want.begin(), compose());
+    thrust::inclusive_scan(d.begin(), d.end(), out.begin(), compose());
+    ASSERT_TRUE(same(to_host(out), want));
+    const Affine init = {5u, 11u};
+    thrust::exclusive_scan(h.begin(), h.end(), want.begin(), init, compose());
+    thrust::exclusive_scan(d.begin(), d.end(), d.begin(), init, compose());  // in place
+    ASSERT_TRUE(same(to_host(d), want));
+  }
+  {
+    const size_t n = ((size_t)1 << 23) + 7;
+    const thrust::host_vector<unsigned> h = random_values<unsigned>(n, 41, 1u << 31);
+    thrust::host_vector<unsigned> want(n);
+    thrust::device_vector<unsigned> d(h), out(n);
+    thrust::inclusive_scan(h.begin(), h.end(), want.begin(), thrust::multiplies<unsigned>());
+    thrust::inclusive_scan(d.begin(), d.end(), out.begin(), thrust::multiplies<unsigned>());
+    ASSERT_TRUE(same(to_host(out), want));
+    thrust::exclusive_scan(h.begin(), h.end(), want.begin(), 3u, bit_xor_op());
+    thrust::exclusive_scan(d.begin(), d.end(), out.begin(), 3u, bit_xor_op());
+    ASSERT_TRUE(same(to_host(out), want));
+  }
+}
+
 struct same_tens {  // the key predicate of testing/reduce_by_key.cu:60-112 and unique.cu:125-142
   __host__ __device__ bool operator()(int a, int b) const { return a / 10 == b / 10; }
 };
@@ -963,6 +995,7 @@ int main() {
   Differential();
   TestUserPredicateSelectionShapes();
   TestUserOperators();
+  TestUserOperatorScansOfLargeRanges();
   TestWideElements();
   TestUserPredicatesByKey();
   TestReduceByKeyWithUserFunctors();
