@@ -7,7 +7,9 @@
 //                           the operator (thrust/system/hip/detail/reduce_by_key_kernels.h), when
 //                           the sums have the values' own type and keys and values are items of
 //                           up to 8 bytes
-//   otherwise, and for scan_by_key, a composition of pieces:
+//   scan_by_key             the single-pass segmented scan (thrust/system/hip/detail/scan_by_key_kernels.h)
+//                           under the same conditions, written to device memory
+//   otherwise a composition of pieces:
 //     run flags   one kernel, instantiated for the predicate: head[i] = i == 0 || !pred(k[i-1], k[i])
 //                 and tail[i] = i == n-1 || !pred(k[i], k[i+1]), one byte each
 //                 (thrust/detail/range/head_flags.h:130-160, tail_flags.h in the reference)
@@ -30,6 +32,7 @@
 #include <thrust/system/hip/detail/device_input.h>
 #include <thrust/system/hip/detail/generic_select.h>
 #include <thrust/system/hip/detail/reduce_by_key_kernels.h>
+#include <thrust/system/hip/detail/scan_by_key_kernels.h>
 
 namespace thrust {
 namespace system {
@@ -239,6 +242,42 @@ __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void shifted_seg_pairs_kernel(Vi
   }
 }
 
+// The single-pass segmented scan, instantiated for the caller's key equality and operator: keys of
+// up to 8 bytes, values, accumulator and output of one type (4 or 8 bytes, or a narrow integer),
+// written to device memory.
+template <typename K, typename VI, typename A, typename Out>
+struct scans_by_key_in_one_pass
+    : std::integral_constant<bool, reduces_by_key_in_one_pass<K, VI, A>::value &&
+                                       std::is_same<typename iterator_value<Out>::type, A>::value &&
+                                       (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value)> {};
+template <bool EXCLUSIVE, typename D, typename KIt, typename VIt, typename Out, typename A, typename Pred, typename Op>
+Out scan_by_key_one_pass(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, A init, Pred pred, Op op) {
+  namespace seg = ::thrust::system::hip::segmented;
+  typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(kl - kf);
+  device_input<KIt> keys(stream, temp_source_of(exec), kf, n);
+  device_input<VIt> values(stream, temp_source_of(exec), vf, n);
+  const A* in = (const A*)values.ptr();
+  A* out = (A*)thrust::detail::raw(result);
+  // the exclusive form reads values[i-1] across tile borders: in place it scans a copy of the values
+  temp_storage copy(stream, temp_source_of(exec));
+  if (EXCLUSIVE && (const A*)out == in) {
+    copy.ensure((std::size_t)n * sizeof(A));
+    throw_on_error(thrust_amd_memcpy(copy.ptr(), in, n * sizeof(A), THRUST_AMD_D2D, stream),
+                   "exclusive_scan_by_key: copy of the values");
+    in = static_cast<const A*>(copy.ptr());
+  }
+  const seg::SbkTemp<K, A> lay(n);
+  temp_storage temp(stream, temp_source_of(exec));
+  temp.ensure(lay.total);
+  throw_on_error(seg::sbk_launch(static_cast<char*>(temp.ptr()), (const K*)keys.ptr(), in, out, n, EXCLUSIVE, init, pred, op,
+                                 (hipStream_t)stream),
+                 "scan_by_key failed");
+  synchronize(stream, "scan_by_key: synchronize");
+  return result + n;
+}
+
 template <bool EXCLUSIVE, typename D, typename KIt, typename VIt, typename Out, typename A, typename Pred, typename Op>
 Out scan_by_key_generic(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, A init, Pred pred, Op op) {
   static_assert(is_device_input<KIt>::value && is_device_input<VIt>::value && is_device_output<Out>::value,
@@ -246,6 +285,14 @@ Out scan_by_key_generic(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out r
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(kl - kf);
   if (n == 0) return result;
+  {
+    typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
+    typedef typename std::remove_const<typename iterator_value<VIt>::type>::type VI;
+    if constexpr (scans_by_key_in_one_pass<K, VI, A, Out>::value) {
+      // the kernel counts run beginnings in 32 bits; beyond that the composition below takes over
+      if (n < 0xffffffffull) return scan_by_key_one_pass<EXCLUSIVE>(exec, kf, kl, vf, result, init, pred, op);
+    }
+  }
   temp_storage flags(stream, temp_source_of(exec));
   flags.ensure((std::size_t)n);
   unsigned char* head = static_cast<unsigned char*>(flags.ptr());

@@ -392,10 +392,22 @@ static void CheckReduceByKey(const thrust::host_vector<K>& hk, const thrust::hos
   ASSERT_TRUE((size_t)(dr.first - dko.begin()) == runs && (size_t)(dr.second - dvo.begin()) == runs);
   ASSERT_TRUE(same(thrust::host_vector<K>(dko.begin(), dko.begin() + runs), thrust::host_vector<K>(hko.begin(), hko.begin() + runs)));
   ASSERT_TRUE(same(thrust::host_vector<V>(dvo.begin(), dvo.begin() + runs), thrust::host_vector<V>(hvo.begin(), hvo.begin() + runs)));
+  // the segmented scans over the same runs: inclusive, exclusive with an init, exclusive in place
+  if (n == 0) return;
+  thrust::inclusive_scan_by_key(hk.begin(), hk.end(), hval.begin(), hvo.begin(), eq, op);
+  thrust::inclusive_scan_by_key(dk.begin(), dk.end(), dval.begin(), dvo.begin(), eq, op);
+  ASSERT_TRUE(same(to_host(dvo), hvo));
+  const V init = hval[n / 2];
+  thrust::exclusive_scan_by_key(hk.begin(), hk.end(), hval.begin(), hvo.begin(), init, eq, op);
+  thrust::exclusive_scan_by_key(dk.begin(), dk.end(), dval.begin(), dvo.begin(), init, eq, op);
+  ASSERT_TRUE(same(to_host(dvo), hvo));
+  thrust::device_vector<V> din(dval);
+  thrust::exclusive_scan_by_key(dk.begin(), dk.end(), din.begin(), din.begin(), init, eq, op);
+  ASSERT_TRUE(same(to_host(din), hvo));
 }
 
 static void TestReduceByKeyWithUserFunctors() {
-  g_test = "reduce_by_key with user functors in the single-pass kernel";
+  g_test = "reduce_by_key and scan_by_key with user functors in the single-pass kernels";
   for (size_t n : {(size_t)1, (size_t)2, (size_t)100, (size_t)14336, (size_t)14337, (size_t)100000, ((size_t)1 << 20) + 11}) {
     for (size_t mean_run : {(size_t)1, (size_t)3, (size_t)700, (size_t)50000, n + 1}) {
       thrust::host_vector<int> hk(n);

@@ -180,6 +180,20 @@ int main(int argc, char** argv) {
   expect(runs == runs2 && same_prefix(out, out2, runs) && same_prefix(vout, vout2, runs), "reduce_by_key");
   pair_line("reduce_by_key, mean run 8", tu, tl, 8.0 * n + 8.0 * runs);
   std::printf("  (%zu runs)\n", runs);
+  tu = best_ms([&] { thrust::inclusive_scan_by_key(y.begin(), y.end(), vals.begin(), out.begin(), my_equal(), my_plus()); });
+  tl = best_ms([&] {
+    thrust::inclusive_scan_by_key(y.begin(), y.end(), vals.begin(), out2.begin(), thrust::equal_to<unsigned>(),
+                                  thrust::plus<unsigned>());
+  });
+  expect(same_prefix(out, out2, n), "inclusive_scan_by_key");
+  pair_line("inclusive_scan_by_key, mean run 8", tu, tl, 12.0 * n);
+  tu = best_ms([&] { thrust::exclusive_scan_by_key(y.begin(), y.end(), vals.begin(), out.begin(), 7u, my_equal(), my_plus()); });
+  tl = best_ms([&] {
+    thrust::exclusive_scan_by_key(y.begin(), y.end(), vals.begin(), out2.begin(), 7u, thrust::equal_to<unsigned>(),
+                                  thrust::plus<unsigned>());
+  });
+  expect(same_prefix(out, out2, n), "exclusive_scan_by_key");
+  pair_line("exclusive_scan_by_key, mean run 8", tu, tl, 12.0 * n);
 
   // two sorted ranges of n / 2 with duplicates in and across them
   const size_t m = n / 2;

@@ -10,6 +10,4 @@
 namespace ta {
 using namespace ::thrust::system::hip::segmented;
 
-constexpr int SBK_BLOCK = 512;  // scan_by_key: two workgroups of 512 per CU
-
 }  // namespace ta
