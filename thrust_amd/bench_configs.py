@@ -1,7 +1,8 @@
 """The benchmark configurations beside the headline one: each is run on the device at its own
 size, its result is verified there against an independent torch computation, and the whole
 call (every kernel it launches, launch gaps included) is timed with events on the launch
-stream.  bench.py imports this module and prints the rows inside its JSON line.
+stream (three warm-ups, then the median and the minimum of 20 calls).  bench.py imports this module and
+prints the rows inside its JSON line.
 
   C2  sort of 2^28 float32 keys (1 % of +-0.0 and denormals)
   C3  stable sort_by_key of 2^27 uint64 keys + uint32 values: full range / low 16 bits / 90 % one key
@@ -39,9 +40,10 @@ def _hold_device(torch):
 def _time_calls(torch, fn, reps, setup=None):
     """Median and minimum device time of fn() in ms; setup() runs before each call, untimed.
     fn must not synchronise."""
-    if setup:
-        setup()
-    fn()  # sizes temp storage, warms up
+    for _ in range(3):  # the first call sizes the temporary storage; three warm-ups in all
+        if setup:
+            setup()
+        fn()
     torch.cuda.synchronize()
     times = []
     for _ in range(reps):
@@ -313,9 +315,10 @@ def run_c8(torch, capi, reps):
     return rows
 
 
-def run_all(torch, capi, reps=5):
+def run_all(torch, capi, reps=20):
     rows = {}
     for part in (run_c2_float, run_c3, run_c4, run_c5, run_c6, run_c7, run_c8):
+        # (no empty_cache between the parts: while the driver clears gigabytes of freed memory in the
+        # background, everything that is bound by bandwidth runs about 3 % slower for a few seconds)
         rows.update(part(torch, capi, reps))
-        torch.cuda.empty_cache()
     return rows
