@@ -9,12 +9,15 @@
 #include <algorithm>
 #include <vector>
 
+#include <thrust/host_vector.h>
 #include <thrust/functional.h>
 #include <thrust/iterator/transform_iterator.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#include <thrust/system/hip/detail/staged_output.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/generic_select.h>
+#include <thrust/system/hip/detail/any_range_selection.h>
 #endif
 
 namespace thrust {
@@ -37,6 +40,12 @@ inline void copy_raw(const T* src, bool src_device, T* dst, bool dst_device, std
   }
 }
 
+// result + n for the iterators that were written through their address
+template <typename Out>
+inline Out advanced(Out result, std::size_t n, std::true_type) { return result + n; }
+template <typename Out>
+inline Out advanced(Out result, std::size_t, std::false_type) { return result; }
+
 // Fancy iterators have no address: element by element through the iterators themselves
 // (host code; device_ptr ends go through their host-side proxies).
 template <typename In, typename Out>
@@ -49,29 +58,39 @@ template <typename In, typename Out>
 inline typename std::enable_if<!is_fancy_iterator<In>::value && !is_fancy_iterator<Out>::value, Out>::type copy_dispatch(
     In first, In last, Out result, bool in_device, bool out_device, void* stream, bool blocking = true) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  typedef typename iterator_value<Out>::type U;
+  // (pure output iterators such as std::back_insert_iterator name no value type)
+  typedef typename std::conditional<std::is_void<typename iterator_value<Out>::type>::value, T,
+                                    typename iterator_value<Out>::type>::type U;
   const std::size_t n = (std::size_t)std::distance(first, last);
   if (n == 0) return result;
   if (!in_device && !out_device) return std::copy(first, last, result);
-  static_assert(std::is_trivially_copyable<T>::value, "thrust::copy involving the device needs trivially copyable elements");
+  static_assert(std::is_trivially_copy_constructible<T>::value,
+                "thrust::copy involving the device needs trivially copy-constructible elements");
+  // addresses of the ends that have one (a device end always has)
+  typedef std::integral_constant<bool, is_device_iterator<In>::value || std::is_pointer<In>::value ||
+                                           is_contiguous_host_iterator<In>::value> in_has_address;
+  typedef std::integral_constant<bool, is_device_iterator<Out>::value || std::is_pointer<Out>::value ||
+                                           is_contiguous_host_iterator<Out>::value> out_has_address;
+  const T* in_raw = raw_if<const T>(first, in_has_address());
+  U* out_raw = raw_if<U>(result, out_has_address());
   if (std::is_same<T, U>::value && (in_device || is_contiguous_host_iterator<In>::value) &&
       (out_device || is_contiguous_host_iterator<Out>::value)) {
-    copy_raw<T>(raw(first), in_device, reinterpret_cast<T*>(raw(result)), out_device, n, stream, blocking);
+    copy_raw<T>(in_raw, in_device, reinterpret_cast<T*>(out_raw), out_device, n, stream, blocking);
   } else if (in_device) {
     // device -> host with conversion or a non-contiguous destination: stage on the host
-    std::vector<T> staged(n);
-    copy_raw<T>(raw(first), true, staged.data(), false, n, stream);
+    staging_vector<T> staged(n);
+    copy_raw<T>(in_raw, true, staged.data(), false, n, stream);
     if (out_device) {
-      std::vector<U> converted(staged.begin(), staged.end());
-      copy_raw<U>(converted.data(), false, reinterpret_cast<U*>(raw(result)), true, n, stream);
+      staging_vector<U> converted(staged.begin(), staged.end());
+      copy_raw<U>(converted.data(), false, out_raw, true, n, stream);
     } else {
-      std::copy(staged.begin(), staged.end(), result);
+      return std::copy(staged.begin(), staged.end(), result);
     }
   } else {
-    std::vector<U> staged(first, last);
-    copy_raw<U>(staged.data(), false, reinterpret_cast<U*>(raw(result)), true, n, stream);
+    staging_vector<U> staged(first, last);
+    copy_raw<U>(staged.data(), false, out_raw, true, n, stream);
   }
-  return result + n;
+  return advanced(result, n, out_has_address());
 }
 }  // namespace detail
 
@@ -132,7 +151,7 @@ Out copy(execution_policy<D>& exec, In first, In last, Out result, std::true_typ
 // a user predicate as one byte per element, for the stencil form of the selection kernels
 template <typename Pred>
 struct as_flag {
-  Pred pred;
+  mutable Pred pred;  // a caller's predicate need not be const-callable
   template <typename V>
   __host__ __device__ unsigned char operator()(const V& x) const { return pred(x) ? 1 : 0; }
 };
@@ -272,19 +291,45 @@ Out copy_if_impl(execution_policy<D>& exec, In first, In last, St stencil, HasSt
 }
 }  // namespace detail
 
+namespace detail {
+// Items of 1, 2, 4 or 8 bytes into an array of the same type: the compaction kernels.  Anything
+// else (wider elements, a zip or discard iterator as output, another output type): the
+// three-pass selection through the iterators themselves.
+template <typename D, typename In, typename St, typename HasStencil, typename Out, typename Pred>
+Out copy_if_any(execution_policy<D>& exec, In first, In last, St stencil, HasStencil has_stencil, Out result, Pred pred,
+                bool negate, std::true_type) {
+  return copy_if_impl(exec, first, last, stencil, has_stencil, result, pred, negate);
+}
+template <typename D, typename In, typename St, typename HasStencil, typename Out, typename Pred>
+Out copy_if_any(execution_policy<D>& exec, In first, In last, St stencil, HasStencil, Out result, Pred pred, bool negate,
+                std::false_type) {
+#if defined(__HIPCC__)
+  const uint64_t n = (uint64_t)(last - first);
+  return result + select_any_range<false>(exec, first, n, stencil, result, result, pred, negate, "copy_if failed");
+#else
+  static_assert(fancy_needs_hipcc<Pred>::value,
+                "thrust::copy_if / remove_copy_if on the device system: items other than 1, 2, 4 or 8 bytes, and outputs "
+                "that are not arrays of the input's type, are handled by kernels instantiated for the iterators; "
+                "compile this translation unit with hipcc");
+  return result;
+#endif
+}
+template <typename D, typename In, typename St, typename HasStencil, typename Out, typename Pred>
+Out copy_if_any(execution_policy<D>& exec, In first, In last, St stencil, HasStencil has_stencil, Out result, Pred pred,
+                bool negate) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  return copy_if_any(exec, first, last, stencil, has_stencil, result, pred, negate,
+                     std::integral_constant<bool, is_abi_item<T>::value && is_array_of<T, Out>::value>());
+}
+}  // namespace detail
+
 template <typename D, typename In, typename Out, typename Pred>
 Out copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
-                "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  return detail::copy_if_impl(exec, first, last, first, std::false_type(), result, pred, false);
+  return detail::copy_if_any(exec, first, last, first, std::false_type(), result, pred, false);
 }
 template <typename D, typename In, typename St, typename Out, typename Pred>
 Out copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result, Pred pred) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
-                "thrust::copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  return detail::copy_if_impl(exec, first, last, stencil, std::true_type(), result, pred, false);
+  return detail::copy_if_any(exec, first, last, stencil, std::true_type(), result, pred, false);
 }
 }  // namespace hip
 }  // namespace system

@@ -5,7 +5,7 @@
 // construction from a size, a size and a value, a host range, a std::vector / host_vector
 // or another device_vector; begin/end/data/size/resize/clear/swap; operator[] / front /
 // back through device_reference; assignment across systems.  Elements must be trivially
-// copyable: storage is raw device memory, filled and copied by the device system.  Storage
+// copy-constructible and destructible: storage is raw device memory, filled and copied by the device system.  Storage
 // comes from Alloc (default thrust::device_allocator<T>: the device system's malloc); any
 // allocator whose allocate(n) yields a device_ptr<T> or a raw device pointer will do, e.g.
 // thrust::mr::allocator<T, Pool> over a pool resource (thrust/mr/pool.h).
@@ -26,8 +26,10 @@ namespace thrust {
 
 template <typename T, typename Alloc = device_allocator<T> >
 class device_vector {
-  static_assert(std::is_trivially_copyable<T>::value,
-                "thrust::device_vector: elements must be trivially copyable");
+  // (a type may still define its own assignment: elements are never assigned on the device
+  // side of this class, only copied as bytes)
+  static_assert(std::is_trivially_copy_constructible<T>::value && std::is_trivially_destructible<T>::value,
+                "thrust::device_vector: elements must be trivially copy-constructible and destructible");
 
  public:
   typedef T value_type;
@@ -57,6 +59,10 @@ class device_vector {
   }
   template <typename A>
   device_vector(const std::vector<T, A>& h, const Alloc& alloc = Alloc()) : device_vector(alloc) {
+    assign_std_vector(h, std::is_same<T, bool>());
+  }
+  // host_vector<bool>: an array of bool
+  device_vector(const detail::contiguous_vector<T>& h, const Alloc& alloc = Alloc()) : device_vector(alloc) {
     assign_host(h.data(), h.size());
   }
   template <typename InputIterator,
@@ -76,6 +82,10 @@ class device_vector {
   }
   template <typename A>
   device_vector& operator=(const std::vector<T, A>& h) {
+    assign_std_vector(h, std::is_same<T, bool>());
+    return *this;
+  }
+  device_vector& operator=(const detail::contiguous_vector<T>& h) {
     assign_host(h.data(), h.size());
     return *this;
   }
@@ -224,9 +234,14 @@ class device_vector {
   // host range (any input iterator)
   template <typename It>
   void assign_range(It first, It last, long) {
-    std::vector<T> staged(first, last);
+    detail::staging_vector<T> staged(first, last);
     assign_host(staged.data(), staged.size());
   }
+  template <typename A>
+  void assign_std_vector(const std::vector<T, A>& h, std::false_type) { assign_host(h.data(), h.size()); }
+  // std::vector<bool> is bit-packed: through an array of bool
+  template <typename A>
+  void assign_std_vector(const std::vector<T, A>& h, std::true_type) { assign_range(h.begin(), h.end(), 0L); }
 
   T* data_;
   size_type size_, capacity_;
@@ -259,7 +274,7 @@ host_vector<T, Alloc>::host_vector(device_ptr<U> first, device_ptr<U> last) : ba
     system::hip::detail::throw_on_error(
         thrust_amd_memcpy(this->data(), first.get(), n * sizeof(V), THRUST_AMD_D2H, nullptr), "host_vector copy");
   } else {
-    std::vector<V> staged(n);
+    detail::staging_vector<V> staged(n);
     system::hip::detail::throw_on_error(
         thrust_amd_memcpy(staged.data(), first.get(), n * sizeof(V), THRUST_AMD_D2H, nullptr), "host_vector copy");
     for (std::size_t i = 0; i < n; ++i) (*this)[i] = static_cast<T>(staged[i]);

@@ -75,12 +75,24 @@ inline auto raw(It it) -> typename std::enable_if<
   // never dereferences: callers pass begin() of a non-empty contiguous range or use n == 0
   return std::addressof(*it);
 }
+// (std::vector<bool> is bit-packed: its iterators point at no array of bool; a pure output
+// iterator names no value type at all)
+template <typename It, typename V>
+struct is_vector_iterator_of
+    : std::integral_constant<bool, std::is_same<It, typename std::vector<V>::iterator>::value ||
+                                       std::is_same<It, typename std::vector<V>::const_iterator>::value> {};
+template <typename It> struct is_vector_iterator_of<It, bool> : std::false_type {};
+template <typename It> struct is_vector_iterator_of<It, void> : std::false_type {};
 template <typename It>
 struct is_contiguous_host_iterator
-    : std::integral_constant<bool,
-          std::is_pointer<It>::value ||
-          std::is_same<It, typename std::vector<typename std::iterator_traits<It>::value_type>::iterator>::value ||
-          std::is_same<It, typename std::vector<typename std::iterator_traits<It>::value_type>::const_iterator>::value> {};
+    : std::integral_constant<bool, std::is_pointer<It>::value ||
+                                       is_vector_iterator_of<It, typename std::iterator_traits<It>::value_type>::value> {};
+// raw(it) where the iterator has an address to give, a null pointer of the same type where it
+// has none (for branches that are compiled for every iterator but only run for contiguous ones)
+template <typename T, typename It>
+inline T* raw_if(It it, std::true_type) { return const_cast<T*>(raw(it)); }
+template <typename T, typename It>
+inline T* raw_if(It, std::false_type) { return nullptr; }
 
 template <typename T>
 struct is_execution_policy : std::is_base_of<thrust::detail::execution_policy_marker,

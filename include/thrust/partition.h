@@ -146,23 +146,83 @@ pair<Out1, Out2> stable_partition_copy_impl(execution_policy<D>& exec, In first,
 }
 }  // namespace detail
 
+namespace detail {
+// Items of 1, 2, 4 or 8 bytes in arrays of one type: the compaction kernels.  Anything else
+// (wider elements, zip or discard iterators, another output type): the three-pass selection
+// through the iterators themselves.
+template <typename D, typename It, typename St, typename HasStencil, typename Pred>
+It stable_partition_any(execution_policy<D>& exec, It first, It last, St stencil, HasStencil has_stencil, Pred pred,
+                        std::true_type) {
+  return stable_partition_impl(exec, first, last, stencil, has_stencil, pred);
+}
+template <typename D, typename In, typename St, typename HasStencil, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy_any(execution_policy<D>& exec, In first, In last, St stencil,
+                                           HasStencil has_stencil, Out1 out_true, Out2 out_false, Pred pred,
+                                           std::true_type) {
+  return stable_partition_copy_impl(exec, first, last, stencil, has_stencil, out_true, out_false, pred);
+}
+template <typename D, typename It, typename St, typename HasStencil, typename Pred>
+It stable_partition_any(execution_policy<D>& exec, It first, It last, St stencil, HasStencil, Pred pred,
+                        std::false_type) {
+#if defined(__HIPCC__)
+  return first + partition_any_range(exec, first, (uint64_t)(last - first), stencil, pred, "stable_partition failed");
+#else
+  static_assert(fancy_needs_hipcc<Pred>::value,
+                "thrust::partition / stable_partition on the device system: items other than 1, 2, 4 or 8 bytes and "
+                "ranges that are not arrays are handled by kernels instantiated for the iterators; compile this "
+                "translation unit with hipcc");
+  return first;
+#endif
+}
+template <typename D, typename In, typename St, typename HasStencil, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy_any(execution_policy<D>& exec, In first, In last, St stencil, HasStencil,
+                                           Out1 out_true, Out2 out_false, Pred pred, std::false_type) {
+#if defined(__HIPCC__)
+  const uint64_t n = (uint64_t)(last - first);
+  const uint64_t cnt = select_any_range<true>(exec, first, n, stencil, out_true, out_false, pred, false,
+                                              "partition_copy failed");
+  return thrust::make_pair(out_true + cnt, out_false + (n - cnt));
+#else
+  static_assert(fancy_needs_hipcc<Pred>::value,
+                "thrust::partition_copy / stable_partition_copy on the device system: items other than 1, 2, 4 or 8 "
+                "bytes and outputs that are not arrays of the input's type are handled by kernels instantiated for "
+                "the iterators; compile this translation unit with hipcc");
+  return thrust::make_pair(out_true, out_false);
+#endif
+}
+template <typename D, typename It, typename St, typename HasStencil, typename Pred>
+It stable_partition_any(execution_policy<D>& exec, It first, It last, St stencil, HasStencil has_stencil, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<It>::type>::type T;
+  return stable_partition_any(exec, first, last, stencil, has_stencil, pred,
+                              std::integral_constant<bool, is_abi_item<T>::value && is_array_of<T, It>::value>());
+}
+template <typename D, typename In, typename St, typename HasStencil, typename Out1, typename Out2, typename Pred>
+pair<Out1, Out2> stable_partition_copy_any(execution_policy<D>& exec, In first, In last, St stencil,
+                                           HasStencil has_stencil, Out1 out_true, Out2 out_false, Pred pred) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  return stable_partition_copy_any(
+      exec, first, last, stencil, has_stencil, out_true, out_false, pred,
+      std::integral_constant<bool, is_abi_item<T>::value && is_array_of<T, Out1>::value && is_array_of<T, Out2>::value>());
+}
+}  // namespace detail
+
 template <typename D, typename It, typename Pred>
 It stable_partition(execution_policy<D>& exec, It first, It last, Pred pred) {
-  return detail::stable_partition_impl(exec, first, last, first, std::false_type(), pred);
+  return detail::stable_partition_any(exec, first, last, first, std::false_type(), pred);
 }
 template <typename D, typename It, typename St, typename Pred>
 It stable_partition(execution_policy<D>& exec, It first, It last, St stencil, Pred pred) {
-  return detail::stable_partition_impl(exec, first, last, stencil, std::true_type(), pred);
+  return detail::stable_partition_any(exec, first, last, stencil, std::true_type(), pred);
 }
 template <typename D, typename In, typename Out1, typename Out2, typename Pred>
 pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In last, Out1 out_true, Out2 out_false,
                                        Pred pred) {
-  return detail::stable_partition_copy_impl(exec, first, last, first, std::false_type(), out_true, out_false, pred);
+  return detail::stable_partition_copy_any(exec, first, last, first, std::false_type(), out_true, out_false, pred);
 }
 template <typename D, typename In, typename St, typename Out1, typename Out2, typename Pred>
 pair<Out1, Out2> stable_partition_copy(execution_policy<D>& exec, In first, In last, St stencil, Out1 out_true,
                                        Out2 out_false, Pred pred) {
-  return detail::stable_partition_copy_impl(exec, first, last, stencil, std::true_type(), out_true, out_false, pred);
+  return detail::stable_partition_copy_any(exec, first, last, stencil, std::true_type(), out_true, out_false, pred);
 }
 }  // namespace hip
 }  // namespace system

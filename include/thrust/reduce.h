@@ -9,6 +9,8 @@
 #include <thrust/pair.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#include <thrust/system/hip/detail/staged_output.h>
+#include <thrust/copy.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/generic_kernels.h>
 #include <thrust/system/hip/detail/generic_by_key.h>
@@ -223,13 +225,36 @@ pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf
 }
 }  // namespace detail
 
+namespace detail {
 template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
-pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred pred, Op op) {
+pair<KOut, VOut> reduce_by_key_staged(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred pred,
+                                      Op op, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
   typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
-  return detail::reduce_by_key(exec, kf, kl, vf, ko, vo, pred, op,
-                               detail::reduces_by_key_in_library<K, V, typename iterator_value<KOut>::type,
-                                                                 typename iterator_value<VOut>::type, Pred, Op>());
+  return reduce_by_key(exec, kf, kl, vf, ko, vo, pred, op,
+                       reduces_by_key_in_library<K, V, typename iterator_value<KOut>::type,
+                                                 typename iterator_value<VOut>::type, Pred, Op>());
+}
+// an output that is not an array in memory: into temporary storage, then through the iterator
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key_staged(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred pred,
+                                      Op op, std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
+  const uint64_t n = (uint64_t)(kl - kf);
+  output_stage<KOut, K> keys_out(stream_of(exec), temp_source_of(exec), ko, n);
+  output_stage<VOut, V> sums_out(stream_of(exec), temp_source_of(exec), vo, n);
+  const auto ends = reduce_by_key_staged(exec, kf, kl, vf, keys_out.begin(), sums_out.begin(), pred, op, std::true_type());
+  const uint64_t runs = (uint64_t)(ends.first - keys_out.begin());
+  return thrust::make_pair(keys_out.finish(exec, runs), sums_out.finish(exec, runs));
+}
+}  // namespace detail
+
+template <typename D, typename KIt, typename VIt, typename KOut, typename VOut, typename Pred, typename Op>
+pair<KOut, VOut> reduce_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, KOut ko, VOut vo, Pred pred, Op op) {
+  return detail::reduce_by_key_staged(
+      exec, kf, kl, vf, ko, vo, pred, op,
+      std::integral_constant<bool, detail::is_memory_iterator<KOut>::value && detail::is_memory_iterator<VOut>::value>());
 }
 }  // namespace hip
 }  // namespace system

@@ -66,17 +66,11 @@ It remove_if(execution_policy<D>& exec, It first, It last, Pred pred) {
 namespace hip {
 template <typename D, typename In, typename Out, typename Pred>
 Out remove_copy_if(execution_policy<D>& exec, In first, In last, Out result, Pred pred) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
-                "thrust::remove_copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  return detail::copy_if_impl(exec, first, last, first, std::false_type(), result, pred, true);
+  return detail::copy_if_any(exec, first, last, first, std::false_type(), result, pred, true);
 }
 template <typename D, typename In, typename St, typename Out, typename Pred>
 Out remove_copy_if(execution_policy<D>& exec, In first, In last, St stencil, Out result, Pred pred) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  static_assert(detail::is_abi_item<T>::value && std::is_same<typename iterator_value<Out>::type, T>::value,
-                "thrust::remove_copy_if on the device system: items of 1, 2, 4 or 8 bytes, same type in and out");
-  return detail::copy_if_impl(exec, first, last, stencil, std::true_type(), result, pred, true);
+  return detail::copy_if_any(exec, first, last, stencil, std::true_type(), result, pred, true);
 }
 // in place: the compaction kernel writes a tile only after every earlier tile has been read
 template <typename D, typename It, typename Pred>

@@ -38,8 +38,14 @@ template <> struct dtype_of<double> { static const int value = THRUST_AMD_F64; }
 
 template <typename T>
 struct is_abi_type : std::integral_constant<bool, (dtype_of<T>::value >= 0)> {};
+// Moved as bytes: copying the object representation is copy construction, and nothing needs to
+// run when a copy goes away.  (The type may still define an assignment of its own; elements
+// are never assigned to, only constructed from bytes.)
 template <typename T>
-struct is_abi_item : std::integral_constant<bool, std::is_trivially_copyable<T>::value &&
+struct is_bytewise_movable : std::integral_constant<bool, std::is_trivially_copy_constructible<T>::value &&
+                                                          std::is_trivially_destructible<T>::value> {};
+template <typename T>
+struct is_abi_item : std::integral_constant<bool, is_bytewise_movable<T>::value &&
                                                   (sizeof(T) == 1 || sizeof(T) == 2 || sizeof(T) == 4 || sizeof(T) == 8)> {};
 
 // ---- functor types -> codes

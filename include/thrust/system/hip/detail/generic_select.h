@@ -42,7 +42,10 @@ struct run_flagger {
   }
 };
 
-// what the kernel can hold in registers and load as (parts of) 16-byte vectors
+// What the kernel can hold in registers and load as (parts of) 16-byte vectors.  Trivially
+// copyable in full: the kernel assigns elements to registers and to staging memory that no
+// constructor has run on, which a type with an assignment operator of its own may not survive
+// (such a type has its predicate evaluated into flags first and is then moved as bytes).
 template <typename S>
 struct is_kernel_item
     : std::integral_constant<bool, std::is_trivially_copyable<S>::value && std::is_default_constructible<S>::value &&

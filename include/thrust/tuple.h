@@ -20,7 +20,7 @@ template <>
 class tuple<> {
  public:
   __host__ __device__ tuple() {}
-  __host__ __device__ tuple(const tuple&) {}
+  tuple(const tuple&) = default;
   __host__ __device__ const tuple& operator=(const tuple&) const { return *this; }
   __host__ __device__ bool equal(const tuple&) const { return true; }
   __host__ __device__ bool less(const tuple&) const { return false; }
@@ -34,7 +34,9 @@ class tuple<H, T...> {
 
   struct cons_tag {};
   __host__ __device__ tuple() : head(), tail() {}
-  __host__ __device__ tuple(const tuple& o) : head(o.head), tail(o.tail) {}
+  // (defaulted: a tuple of plain values is copied as its bytes are, also by device code that
+  // moves elements without knowing their type)
+  tuple(const tuple& o) = default;
   // from the first element and the tuple of the others
   template <typename HH>
   __host__ __device__ tuple(cons_tag, HH&& h, const tuple<T...>& t) : head(static_cast<HH&&>(h)), tail(t) {}

@@ -9,6 +9,8 @@
 #include <thrust/pair.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#include <thrust/system/hip/detail/staged_output.h>
+#include <thrust/copy.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/generic_by_key.h>
 #endif
@@ -167,17 +169,51 @@ pair<KOut, VOut> unique_by_key_copy(execution_policy<D>& exec, KIn kf, KIn kl, V
 }
 }  // namespace detail
 
+namespace detail {
+template <typename D, typename In, typename Out, typename Pred>
+Out unique_copy_staged(execution_policy<D>& exec, In first, In last, Out result, Pred pred, std::true_type) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  return unique_copy(exec, first, last, result, pred, uniques_in_library<T, typename iterator_value<Out>::type, Pred>());
+}
+template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred>
+pair<KOut, VOut> unique_by_key_copy_staged(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo,
+                                           Pred pred, std::true_type) {
+  typedef typename std::remove_const<typename iterator_value<KIn>::type>::type K;
+  return unique_by_key_copy(exec, kf, kl, vf, ko, vo, pred,
+                            uniques_in_library<K, typename iterator_value<KOut>::type, Pred>());
+}
+// an output that is not an array in memory: into temporary storage, then through the iterator
+template <typename D, typename In, typename Out, typename Pred>
+Out unique_copy_staged(execution_policy<D>& exec, In first, In last, Out result, Pred pred, std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
+  output_stage<Out, T> out(stream_of(exec), temp_source_of(exec), result, (uint64_t)(last - first));
+  const auto end = unique_copy_staged(exec, first, last, out.begin(), pred, std::true_type());
+  return out.finish(exec, (uint64_t)(end - out.begin()));
+}
+template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred>
+pair<KOut, VOut> unique_by_key_copy_staged(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo,
+                                           Pred pred, std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<KIn>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<VIn>::type>::type V;
+  const uint64_t n = (uint64_t)(kl - kf);
+  output_stage<KOut, K> keys_out(stream_of(exec), temp_source_of(exec), ko, n);
+  output_stage<VOut, V> values_out(stream_of(exec), temp_source_of(exec), vo, n);
+  const auto ends = unique_by_key_copy_staged(exec, kf, kl, vf, keys_out.begin(), values_out.begin(), pred, std::true_type());
+  const uint64_t runs = (uint64_t)(ends.first - keys_out.begin());
+  return thrust::make_pair(keys_out.finish(exec, runs), values_out.finish(exec, runs));
+}
+}  // namespace detail
+
 template <typename D, typename In, typename Out, typename Pred>
 Out unique_copy(execution_policy<D>& exec, In first, In last, Out result, Pred pred) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type T;
-  return detail::unique_copy(exec, first, last, result, pred,
-                             detail::uniques_in_library<T, typename iterator_value<Out>::type, Pred>());
+  return detail::unique_copy_staged(exec, first, last, result, pred,
+                                    std::integral_constant<bool, detail::is_memory_iterator<Out>::value>());
 }
 template <typename D, typename KIn, typename VIn, typename KOut, typename VOut, typename Pred>
 pair<KOut, VOut> unique_by_key_copy(execution_policy<D>& exec, KIn kf, KIn kl, VIn vf, KOut ko, VOut vo, Pred pred) {
-  typedef typename std::remove_const<typename iterator_value<KIn>::type>::type K;
-  return detail::unique_by_key_copy(exec, kf, kl, vf, ko, vo, pred,
-                                    detail::uniques_in_library<K, typename iterator_value<KOut>::type, Pred>());
+  return detail::unique_by_key_copy_staged(
+      exec, kf, kl, vf, ko, vo, pred,
+      std::integral_constant<bool, detail::is_memory_iterator<KOut>::value && detail::is_memory_iterator<VOut>::value>());
 }
 }  // namespace hip
 }  // namespace system

@@ -53,3 +53,11 @@ def test_user_functors_and_library_functors_give_the_same_output(log2_n):
     # informative only
     out = _run("test_user_functor_paths", log2_n)
     assert "PASSED" in out and "0 mismatches" in out
+
+
+def test_reference_cases_with_unusual_inputs_and_outputs():
+    # bool keys, std::vector / std::list / vector<bool> sources, discard_iterator outputs of the by-key and partition
+    # families, zip iterators as partitioned range and as stencil, predicates that return numbers, table-driven
+    # operators, elements of 4 to 256 bytes under the default plus
+    out = _run("test_reference_cases")
+    assert "PASSED" in out
