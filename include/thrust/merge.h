@@ -8,6 +8,8 @@
 #include <thrust/pair.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#include <thrust/system/hip/detail/staged_output.h>
+#include <thrust/copy.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/generic_select.h>
 #include <thrust/system/hip/detail/merge_kernels.h>
@@ -209,20 +211,58 @@ template <typename K, typename K2, typename KO, typename Comp>
 struct merges_in_library<K, K2, KO, Comp, false> : std::false_type {};
 }  // namespace detail
 
+namespace detail {
 template <typename D, typename In1, typename In2, typename Out, typename Comp>
-Out merge(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+Out merge_staged(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp,
+                 std::true_type) {
   typedef typename std::remove_const<typename iterator_value<In1>::type>::type K;
   typedef typename std::remove_const<typename iterator_value<In2>::type>::type K2;
-  return detail::merge(exec, first1, last1, first2, last2, result, comp,
-                       detail::merges_in_library<K, K2, typename iterator_value<Out>::type, Comp>());
+  return merge(exec, first1, last1, first2, last2, result, comp,
+               merges_in_library<K, K2, typename iterator_value<Out>::type, Comp>());
+}
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
+pair<KOut, VOut> merge_by_key_staged(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko,
+                                     VOut vo, Comp comp, std::true_type) {
+  typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<K2>::type>::type Kb;
+  return merge_by_key(exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp,
+                      merges_in_library<K, Kb, typename iterator_value<KOut>::type, Comp>());
+}
+// an output that is not an array in memory (discard_iterator, a zip): into temporary storage,
+// then through the iterator
+template <typename D, typename In1, typename In2, typename Out, typename Comp>
+Out merge_staged(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp,
+                 std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<In1>::type>::type K;
+  const uint64_t n = (uint64_t)(last1 - first1) + (uint64_t)(last2 - first2);
+  output_stage<Out, K> out(stream_of(exec), temp_source_of(exec), result, n);
+  merge_staged(exec, first1, last1, first2, last2, out.begin(), comp, std::true_type());
+  return out.finish(exec, n);
+}
+template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
+pair<KOut, VOut> merge_by_key_staged(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko,
+                                     VOut vo, Comp comp, std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<V1>::type>::type V;
+  const uint64_t n = (uint64_t)(kl1 - kf1) + (uint64_t)(kl2 - kf2);
+  output_stage<KOut, K> keys_out(stream_of(exec), temp_source_of(exec), ko, n);
+  output_stage<VOut, V> values_out(stream_of(exec), temp_source_of(exec), vo, n);
+  merge_by_key_staged(exec, kf1, kl1, kf2, kl2, vf1, vf2, keys_out.begin(), values_out.begin(), comp, std::true_type());
+  return thrust::make_pair(keys_out.finish(exec, n), values_out.finish(exec, n));
+}
+}  // namespace detail
+
+template <typename D, typename In1, typename In2, typename Out, typename Comp>
+Out merge(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+  return detail::merge_staged(exec, first1, last1, first2, last2, result, comp,
+                              std::integral_constant<bool, detail::is_memory_iterator<Out>::value>());
 }
 template <typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut, typename Comp>
 pair<KOut, VOut> merge_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2, KOut ko,
                               VOut vo, Comp comp) {
-  typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
-  typedef typename std::remove_const<typename iterator_value<K2>::type>::type Kb;
-  return detail::merge_by_key(exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp,
-                              detail::merges_in_library<K, Kb, typename iterator_value<KOut>::type, Comp>());
+  return detail::merge_by_key_staged(
+      exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp,
+      std::integral_constant<bool, detail::is_memory_iterator<KOut>::value && detail::is_memory_iterator<VOut>::value>());
 }
 }  // namespace hip
 }  // namespace system

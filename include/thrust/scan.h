@@ -13,6 +13,7 @@
 #include <thrust/functional.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#include <thrust/system/hip/detail/staged_output.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/generic_kernels.h>
 #include <thrust/system/hip/detail/generic_select.h>
@@ -478,17 +479,21 @@ template <typename D, typename KIt, typename VIt, typename Out, typename Pred, t
 Out inclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, Pred pred, Op op) {
   typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
   typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
-  return detail::inclusive_scan_by_key(
-      exec, kf, kl, vf, result, pred, op,
-      detail::scans_by_key_in_library<K, V, typename iterator_value<Out>::type, V, Pred, Op>());
+  // the library's kernels read and write arrays; fancy inputs and outputs that are not memory
+  // (discard_iterator, a zip) go through the kernels instantiated for the iterators
+  typedef std::integral_constant<bool, detail::scans_by_key_in_library<K, V, typename iterator_value<Out>::type, V, Pred, Op>::value &&
+                                           detail::is_memory_iterator<KIt>::value && detail::is_memory_iterator<VIt>::value &&
+                                           detail::is_memory_iterator<Out>::value> in_library;
+  return detail::inclusive_scan_by_key(exec, kf, kl, vf, result, pred, op, in_library());
 }
 template <typename D, typename KIt, typename VIt, typename Out, typename T, typename Pred, typename Op>
 Out exclusive_scan_by_key(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out result, T init, Pred pred, Op op) {
   typedef typename std::remove_const<typename iterator_value<KIt>::type>::type K;
   typedef typename std::remove_const<typename iterator_value<VIt>::type>::type V;
-  return detail::exclusive_scan_by_key(
-      exec, kf, kl, vf, result, init, pred, op,
-      detail::scans_by_key_in_library<K, V, typename iterator_value<Out>::type, T, Pred, Op>());
+  typedef std::integral_constant<bool, detail::scans_by_key_in_library<K, V, typename iterator_value<Out>::type, T, Pred, Op>::value &&
+                                           detail::is_memory_iterator<KIt>::value && detail::is_memory_iterator<VIt>::value &&
+                                           detail::is_memory_iterator<Out>::value> in_library;
+  return detail::exclusive_scan_by_key(exec, kf, kl, vf, result, init, pred, op, in_library());
 }
 }  // namespace hip
 }  // namespace system

@@ -17,6 +17,8 @@
 #include <thrust/pair.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#include <thrust/system/hip/detail/staged_output.h>
+#include <thrust/copy.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/generic_set_operations.h>
 #endif
@@ -126,10 +128,27 @@ inline Out set_operation(execution_policy<D>& exec, In1 first1, In1 last1, In2 f
 }
 
 template <int OP, typename D, typename In1, typename In2, typename Out, typename Comp>
-inline Out set_operation(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+inline Out set_operation_staged(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result,
+                                Comp comp, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<In1>::type>::type K;
   return set_operation<OP>(exec, first1, last1, first2, last2, result, comp,
                            set_operation_in_library<K, In2, Out, Comp>());
+}
+// an output that is not an array in memory (discard_iterator, a zip): into temporary storage,
+// then through the iterator
+template <int OP, typename D, typename In1, typename In2, typename Out, typename Comp>
+inline Out set_operation_staged(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result,
+                                Comp comp, std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<In1>::type>::type K;
+  const uint64_t capacity = (uint64_t)(last1 - first1) + (uint64_t)(last2 - first2);
+  output_stage<Out, K> out(stream_of(exec), temp_source_of(exec), result, capacity);
+  const auto end = set_operation_staged<OP>(exec, first1, last1, first2, last2, out.begin(), comp, std::true_type());
+  return out.finish(exec, (uint64_t)(end - out.begin()));
+}
+template <int OP, typename D, typename In1, typename In2, typename Out, typename Comp>
+inline Out set_operation(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, In2 last2, Out result, Comp comp) {
+  return set_operation_staged<OP>(exec, first1, last1, first2, last2, result, comp,
+                                  std::integral_constant<bool, is_memory_iterator<Out>::value>());
 }
 
 template <int OP, typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut,
@@ -176,11 +195,33 @@ inline pair<KOut, VOut> set_operation_by_key(execution_policy<D>& exec, K1 kf1, 
 
 template <int OP, typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut,
           typename Comp>
-inline pair<KOut, VOut> set_operation_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2,
-                                             KOut ko, VOut vo, Comp comp) {
+inline pair<KOut, VOut> set_operation_by_key_staged(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1,
+                                                    V2 vf2, KOut ko, VOut vo, Comp comp, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
   return set_operation_by_key<OP>(exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp,
                                   set_operation_in_library<K, K2, KOut, Comp>());
+}
+template <int OP, typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut,
+          typename Comp>
+inline pair<KOut, VOut> set_operation_by_key_staged(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1,
+                                                    V2 vf2, KOut ko, VOut vo, Comp comp, std::false_type) {
+  typedef typename std::remove_const<typename iterator_value<K1>::type>::type K;
+  typedef typename std::remove_const<typename iterator_value<V1>::type>::type V;
+  const uint64_t capacity = (uint64_t)(kl1 - kf1) + (uint64_t)(kl2 - kf2);
+  output_stage<KOut, K> keys_out(stream_of(exec), temp_source_of(exec), ko, capacity);
+  output_stage<VOut, V> values_out(stream_of(exec), temp_source_of(exec), vo, capacity);
+  const auto ends = set_operation_by_key_staged<OP>(exec, kf1, kl1, kf2, kl2, vf1, vf2, keys_out.begin(),
+                                                    values_out.begin(), comp, std::true_type());
+  const uint64_t count = (uint64_t)(ends.first - keys_out.begin());
+  return thrust::make_pair(keys_out.finish(exec, count), values_out.finish(exec, count));
+}
+template <int OP, typename D, typename K1, typename K2, typename V1, typename V2, typename KOut, typename VOut,
+          typename Comp>
+inline pair<KOut, VOut> set_operation_by_key(execution_policy<D>& exec, K1 kf1, K1 kl1, K2 kf2, K2 kl2, V1 vf1, V2 vf2,
+                                             KOut ko, VOut vo, Comp comp) {
+  return set_operation_by_key_staged<OP>(
+      exec, kf1, kl1, kf2, kl2, vf1, vf2, ko, vo, comp,
+      std::integral_constant<bool, is_memory_iterator<KOut>::value && is_memory_iterator<VOut>::value>());
 }
 }  // namespace detail
 }  // namespace hip

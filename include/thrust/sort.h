@@ -20,6 +20,8 @@
 #include <thrust/functional.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
+#include <thrust/iterator/counting_iterator.h>
+#include <thrust/iterator/permutation_iterator.h>
 #if defined(__HIPCC__)
 #include <thrust/system/hip/detail/merge_sort_kernels.h>
 #endif
@@ -178,20 +180,83 @@ void sort_pairs(void* stream, temp_source source, K* keys, V* values, uint64_t n
   });
 }
 #if defined(__HIPCC__)
+// The merge sort holds tiles of keys and values in registers and LDS: key and value together
+// may take 32 bytes.  Wider elements are sorted through their positions: the merge sort orders
+// 32-bit indices by the keys they point at (which stay where they are), and the keys and
+// values are gathered into that order afterwards.  The reference's merge sort moves the wide
+// elements themselves in every pass (thrust/system/cuda/detail/sort.h:1005-1200).
+constexpr std::size_t MERGE_SORT_ITEM_BYTES = 32;
 template <typename K, typename Comp>
-void sort_keys(void* stream, temp_source source, K* keys, uint64_t n, Comp comp, std::false_type) {
+struct compares_positions {
+  const K* keys;
+  mutable Comp comp;  // a caller's comparator need not be const-callable
+  __host__ __device__ bool operator()(uint32_t a, uint32_t b) const { return comp(keys[a], keys[b]) ? true : false; }
+};
+template <typename T>
+inline void gather_in_place(void* stream, const temp_source& source, T* data, const uint32_t* order, uint64_t n) {
+  temp_storage gathered(stream, source);
+  gathered.ensure((std::size_t)n * sizeof(T));
+  T* out = static_cast<T*>(gathered.ptr());
+  materialize(stream, thrust::make_permutation_iterator((const T*)data, order), out, n);
+  throw_on_error(thrust_amd_memcpy(data, out, n * sizeof(T), THRUST_AMD_D2D, stream), "sort: copy of the gathered elements");
+  synchronize(stream, "sort: synchronize");  // `gathered` returns to the arena when this function ends
+}
+// positions 0 .. n-1 ordered by keys[position] under comp, stable
+template <typename K, typename Comp>
+inline void sort_positions(void* stream, const temp_source& source, const K* keys, uint32_t* order, uint64_t n, Comp comp) {
+  if (n >= 0xffffffffull) throw thrust::system::system_error((int)hipErrorInvalidValue, "sort of wide elements: positions are 32-bit");
+  materialize(stream, thrust::counting_iterator<uint32_t>(0), order, n);
+  temp_storage temp(stream, source);
+  const compares_positions<K, Comp> by_key = {keys, comp};
+  run(temp, 0, "sort (comparison path, wide elements) failed", [&](void* t, std::size_t* b) {
+    return thrust::system::hip::merge_sort::sort<uint32_t, unsigned, false>(t, b, order, (unsigned*)nullptr, n, by_key,
+                                                                            (hipStream_t)stream);
+  });
+  synchronize(stream, "sort: synchronize");
+}
+
+template <typename K, typename Comp>
+void sort_keys_comparing(void* stream, temp_source source, K* keys, uint64_t n, Comp comp, std::true_type /*fits*/) {
   temp_storage temp(stream, source);
   run(temp, 0, "sort (comparison path) failed", [&](void* t, std::size_t* b) {
     return thrust::system::hip::merge_sort::sort<K, unsigned, false>(t, b, keys, (unsigned*)nullptr, n, comp,
                                                                      (hipStream_t)stream);
   });
 }
+template <typename K, typename Comp>
+void sort_keys_comparing(void* stream, temp_source source, K* keys, uint64_t n, Comp comp, std::false_type) {
+  temp_storage positions(stream, source);
+  positions.ensure((std::size_t)n * sizeof(uint32_t));
+  uint32_t* order = static_cast<uint32_t*>(positions.ptr());
+  sort_positions(stream, source, (const K*)keys, order, n, comp);
+  gather_in_place(stream, source, keys, order, n);
+}
+template <typename K, typename Comp>
+void sort_keys(void* stream, temp_source source, K* keys, uint64_t n, Comp comp, std::false_type) {
+  sort_keys_comparing(stream, source, keys, n, comp,
+                      std::integral_constant<bool, sizeof(K) <= MERGE_SORT_ITEM_BYTES>());
+}
+
 template <typename K, typename V, typename Comp>
-void sort_pairs(void* stream, temp_source source, K* keys, V* values, uint64_t n, Comp comp, std::false_type) {
+void sort_pairs_comparing(void* stream, temp_source source, K* keys, V* values, uint64_t n, Comp comp, std::true_type) {
   temp_storage temp(stream, source);
   run(temp, 0, "sort_by_key (comparison path) failed", [&](void* t, std::size_t* b) {
     return thrust::system::hip::merge_sort::sort<K, V, true>(t, b, keys, values, n, comp, (hipStream_t)stream);
   });
+}
+template <typename K, typename V, typename Comp>
+void sort_pairs_comparing(void* stream, temp_source source, K* keys, V* values, uint64_t n, Comp comp, std::false_type) {
+  temp_storage positions(stream, source);
+  positions.ensure((std::size_t)n * sizeof(uint32_t));
+  uint32_t* order = static_cast<uint32_t*>(positions.ptr());
+  sort_positions(stream, source, (const K*)keys, order, n, comp);
+  gather_in_place(stream, source, keys, order, n);
+  gather_in_place(stream, source, values, order, n);
+}
+template <typename K, typename V, typename Comp>
+void sort_pairs(void* stream, temp_source source, K* keys, V* values, uint64_t n, Comp comp, std::false_type) {
+  sort_pairs_comparing(stream, source, keys, values, n, comp,
+                       std::integral_constant<bool, sizeof(K) + sizeof(V) <= MERGE_SORT_ITEM_BYTES>());
 }
 #else
 template <typename K, typename Comp>

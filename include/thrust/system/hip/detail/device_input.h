@@ -8,6 +8,7 @@
 // translation unit compiled with hipcc.
 #pragma once
 #include <thrust/iterator/detail/fancy_iterator_base.h>
+#include <thrust/iterator/permutation_iterator.h>
 #include <thrust/iterator/zip_iterator.h>
 #include <thrust/system/hip/detail/backend.h>
 #if defined(__HIPCC__)
@@ -37,6 +38,11 @@ template <typename H, typename... T>
 struct is_device_output<thrust::zip_iterator<thrust::tuple<H, T...> > >
     : std::integral_constant<bool, is_device_output<H>::value &&
                                        is_device_output<thrust::zip_iterator<thrust::tuple<T...> > >::value> {};
+
+// a permutation of something writable, through indices that can be read
+template <typename E, typename I>
+struct is_device_output<thrust::permutation_iterator<E, I> >
+    : std::integral_constant<bool, is_device_output<E>::value && is_device_input<I>::value> {};
 
 template <typename It>
 struct fancy_needs_hipcc : std::false_type {};

@@ -2,12 +2,17 @@
 //
 // The scans of thrust/scan.h over unary_op(x) instead of x.  The running value has the
 // type unary_op returns (inclusive form) or the type of init (exclusive form)
-// (thrust/system/detail/generic/transform_scan.inl:37-97).  On the device system unary_op
-// is one of thrust::identity / negate / square on the element type and binary_op one of
-// plus / minimum / maximum; result may be the input range.
+// (thrust/system/detail/generic/transform_scan.inl:37-97).  On the device system
+// thrust::identity / negate / square with plus / minimum / maximum over arrays of one
+// arithmetic type run in the library's scan kernel; any other function, operator, iterator or
+// mix of types is the scan of a transform iterator (translation units compiled with hipcc).
+// result may be the input range.
 #pragma once
 #include <thrust/functional.h>
+#include <thrust/iterator/transform_iterator.h>
+#include <thrust/scan.h>
 #include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/staged_output.h>
 
 namespace thrust {
 
@@ -50,54 +55,93 @@ Out transform_exclusive_scan(execution_policy<D>&, In first, In last, Out result
 
 namespace hip {
 namespace detail {
+// library path: arrays of one arithmetic type in and out, identity / negate / square, plus /
+// minimum / maximum
+template <typename In, typename Out, typename T, typename Fn, typename Op,
+          bool = is_abi_type<typename std::remove_const<typename iterator_value<In>::type>::type>::value>
+struct transform_scans_in_library
+    : std::integral_constant<
+          bool, is_memory_iterator<In>::value && is_memory_iterator<Out>::value &&
+                    std::is_same<typename std::remove_const<typename iterator_value<In>::type>::type, T>::value &&
+                    std::is_same<typename iterator_value<Out>::type, T>::value &&
+                    (unary_code<Fn, typename std::remove_const<typename iterator_value<In>::type>::type>::value >= 0) &&
+                    (binop_code<Op, typename std::remove_const<typename iterator_value<In>::type>::type>::value >= 0)> {};
 template <typename In, typename Out, typename T, typename Fn, typename Op>
-struct transform_scan_checks {
+struct transform_scans_in_library<In, Out, T, Fn, Op, false> : std::false_type {};
+
+template <typename D, typename In, typename Out, typename Fn, typename Op>
+Out transform_inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Fn, Op, std::true_type) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
-  static_assert((std::is_pointer<In>::value || thrust::detail::is_device_iterator<In>::value) &&
-                    (std::is_pointer<Out>::value || thrust::detail::is_device_iterator<Out>::value),
-                "transform scans on the device system need device_ptr / device_vector iterators or raw device pointers");
-  static_assert(is_abi_type<V>::value && std::is_same<V, T>::value &&
-                    std::is_same<typename iterator_value<Out>::type, V>::value,
-                "transform scans on the device system: input, output and init must share one arithmetic type");
-  static_assert(unary_code<Fn, V>::value >= 0,
-                "transform scans on the device system support thrust::identity, thrust::negate and thrust::square");
-  static_assert(binop_code<Op, V>::value >= 0,
-                "transform scans on the device system support thrust::plus, thrust::minimum and thrust::maximum");
-};
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  temp_storage temp(stream, temp_source_of(exec));
+  run(temp, 0, "transform_inclusive_scan failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_transform_inclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
+                                               dtype_of<V>::value, unary_code<Fn, V>::value, binop_code<Op, V>::value,
+                                               stream);
+  });
+  synchronize(stream, "transform_inclusive_scan: synchronize");
+  return result + n;
+}
+template <typename D, typename In, typename Out, typename Fn, typename T, typename Op>
+Out transform_exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Fn, T init, Op, std::true_type) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  void* stream = stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+  temp_storage temp(stream, temp_source_of(exec));
+  run(temp, 0, "transform_exclusive_scan failed", [&](void* t, std::size_t* b) {
+    return thrust_amd_transform_exclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
+                                               dtype_of<V>::value, unary_code<Fn, V>::value, binop_code<Op, V>::value,
+                                               &init, stream);
+  });
+  synchronize(stream, "transform_exclusive_scan: synchronize");
+  return result + n;
+}
+// Everything else is the scan of a transform iterator, as the reference's generic layer states
+// it (thrust/system/detail/generic/transform_scan.inl:37-97): any function, any operator, fancy
+// inputs, outputs of another type or that are not memory.
+template <typename D, typename In, typename Out, typename Fn, typename Op>
+Out transform_inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Fn unary_op, Op binary_op,
+                             std::false_type) {
+#if defined(__HIPCC__)
+  return thrust::inclusive_scan(exec, thrust::make_transform_iterator(first, unary_op),
+                                thrust::make_transform_iterator(last, unary_op), result, binary_op);
+#else
+  static_assert(fancy_needs_hipcc<Fn>::value,
+                "transform scans on the device system: functions other than thrust::identity / negate / square, operators "
+                "other than thrust::plus / minimum / maximum, fancy iterators and mixed element types run in kernels "
+                "instantiated for them; compile this translation unit with hipcc");
+  return result;
+#endif
+}
+template <typename D, typename In, typename Out, typename Fn, typename T, typename Op>
+Out transform_exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Fn unary_op, T init, Op binary_op,
+                             std::false_type) {
+#if defined(__HIPCC__)
+  return thrust::exclusive_scan(exec, thrust::make_transform_iterator(first, unary_op),
+                                thrust::make_transform_iterator(last, unary_op), result, init, binary_op);
+#else
+  static_assert(fancy_needs_hipcc<Fn>::value,
+                "transform scans on the device system: functions other than thrust::identity / negate / square, operators "
+                "other than thrust::plus / minimum / maximum, fancy iterators and mixed element types run in kernels "
+                "instantiated for them; compile this translation unit with hipcc");
+  return result;
+#endif
+}
 }  // namespace detail
 
 template <typename D, typename In, typename Out, typename Fn, typename Op>
-Out transform_inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Fn, Op) {
+Out transform_inclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Fn unary_op, Op binary_op) {
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
-  (void)sizeof(detail::transform_scan_checks<In, Out, V, Fn, Op>);
-  void* stream = detail::stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return result;
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
-  detail::run(temp, 0, "transform_inclusive_scan failed", [&](void* t, std::size_t* b) {
-    return thrust_amd_transform_inclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
-                                               detail::dtype_of<V>::value, detail::unary_code<Fn, V>::value,
-                                               detail::binop_code<Op, V>::value, stream);
-  });
-  detail::synchronize(stream, "transform_inclusive_scan: synchronize");
-  return result + n;
+  return detail::transform_inclusive_scan(exec, first, last, result, unary_op, binary_op,
+                                          detail::transform_scans_in_library<In, Out, V, Fn, Op>());
 }
-
 template <typename D, typename In, typename Out, typename Fn, typename T, typename Op>
-Out transform_exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Fn, T init, Op) {
-  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
-  (void)sizeof(detail::transform_scan_checks<In, Out, T, Fn, Op>);
-  void* stream = detail::stream_of(exec);
-  const uint64_t n = (uint64_t)(last - first);
-  if (n == 0) return result;
-  detail::temp_storage temp(stream, detail::temp_source_of(exec));
-  detail::run(temp, 0, "transform_exclusive_scan failed", [&](void* t, std::size_t* b) {
-    return thrust_amd_transform_exclusive_scan(t, b, thrust::detail::raw(first), thrust::detail::raw(result), n,
-                                               detail::dtype_of<V>::value, detail::unary_code<Fn, V>::value,
-                                               detail::binop_code<Op, V>::value, &init, stream);
-  });
-  detail::synchronize(stream, "transform_exclusive_scan: synchronize");
-  return result + n;
+Out transform_exclusive_scan(execution_policy<D>& exec, In first, In last, Out result, Fn unary_op, T init, Op binary_op) {
+  return detail::transform_exclusive_scan(exec, first, last, result, unary_op, init, binary_op,
+                                          detail::transform_scans_in_library<In, Out, T, Fn, Op>());
 }
 }  // namespace hip
 }  // namespace system

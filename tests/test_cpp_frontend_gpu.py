@@ -61,3 +61,12 @@ def test_reference_cases_with_unusual_inputs_and_outputs():
     # operators, elements of 4 to 256 bytes under the default plus
     out = _run("test_reference_cases")
     assert "PASSED" in out
+
+
+def test_reference_cases_of_sorts_scans_merges_and_set_operations():
+    # sorts through permutation iterators and of keys / values up to 1 KiB, keys that use few bits; scan_by_key with
+    # head-flag predicates, transform-iterator values, mixed types, discard output, wide values; merges and set operations
+    # into discard iterators, descending, on equal ranges and multisets; remove_copy into zip / discard outputs; transform
+    # scans from structs, counting iterators and with thrust::identity<> / maximum<>
+    out = _run("test_reference_cases_sorts_scans")
+    assert "PASSED" in out
