@@ -23,13 +23,18 @@ template <typename T>
 class device_reference {
  public:
   typedef typename std::remove_const<T>::type value_type;
+  typedef device_ptr<T> pointer;
   explicit device_reference(T* p) : ptr_(p) {}
+  explicit device_reference(const device_ptr<T>& p);  // defined below device_ptr
   device_reference(const device_reference&) = default;
+  // a reference to const from a reference to non-const
+  template <typename U, typename = typename std::enable_if<std::is_same<const U, T>::value>::type>
+  device_reference(const device_reference<U>& o) : ptr_((&o).get()) {}
 
   operator value_type() const {
     value_type v;
     system::hip::detail::throw_on_error(
-        thrust_amd_memcpy(&v, ptr_, sizeof(value_type), THRUST_AMD_D2H, nullptr), "device_reference read");
+        thrust_amd_memcpy(static_cast<void*>(&v), ptr_, sizeof(value_type), THRUST_AMD_D2H, nullptr), "device_reference read");
     return v;
   }
   device_reference& operator=(const value_type& v) {
@@ -39,7 +44,18 @@ class device_reference {
     return *this;
   }
   device_reference& operator=(const device_reference& other) { return *this = (value_type)other; }
+  // from a reference to another element type: converted on the way
+  template <typename U>
+  device_reference& operator=(const device_reference<U>& other) {
+    return *this = static_cast<value_type>((typename device_reference<U>::value_type)other);
+  }
   device_ptr<T> operator&() const { return device_ptr<T>(ptr_); }
+  // exchanges the two referents
+  void swap(device_reference& other) {
+    const value_type mine = *this, theirs = other;
+    *this = theirs;
+    other = mine;
+  }
 #define THRUST_AMD_REF_COMPOUND(OP)                               \
   device_reference& operator OP##=(const value_type& v) {         \
     value_type t = *this;                                         \
@@ -47,13 +63,28 @@ class device_reference {
     return *this = t;                                             \
   }
   THRUST_AMD_REF_COMPOUND(+) THRUST_AMD_REF_COMPOUND(-) THRUST_AMD_REF_COMPOUND(*) THRUST_AMD_REF_COMPOUND(/)
+  THRUST_AMD_REF_COMPOUND(%) THRUST_AMD_REF_COMPOUND(<<) THRUST_AMD_REF_COMPOUND(>>) THRUST_AMD_REF_COMPOUND(&)
+  THRUST_AMD_REF_COMPOUND(|) THRUST_AMD_REF_COMPOUND(^)
 #undef THRUST_AMD_REF_COMPOUND
   device_reference& operator++() { return *this += value_type(1); }
   device_reference& operator--() { return *this -= value_type(1); }
+  value_type operator++(int) {
+    const value_type before = *this;
+    *this = before + value_type(1);
+    return before;
+  }
+  value_type operator--(int) {
+    const value_type before = *this;
+    *this = before - value_type(1);
+    return before;
+  }
 
  private:
   T* ptr_;
 };
+// thrust::swap of two references exchanges what they refer to (the references are proxies, taken by value)
+template <typename T>
+inline void swap(device_reference<T> a, device_reference<T> b) { a.swap(b); }
 
 template <typename T>
 class device_ptr {
@@ -82,10 +113,17 @@ class device_ptr {
   device_ptr operator++(int) { device_ptr t(*this); ++ptr_; return t; }
   device_ptr& operator--() { --ptr_; return *this; }
   device_ptr operator--(int) { device_ptr t(*this); --ptr_; return t; }
-  device_ptr& operator+=(difference_type n) { ptr_ += n; return *this; }
-  device_ptr& operator-=(difference_type n) { ptr_ -= n; return *this; }
-  device_ptr operator+(difference_type n) const { return device_ptr(ptr_ + n); }
-  device_ptr operator-(difference_type n) const { return device_ptr(ptr_ - n); }
+  device_ptr& operator=(std::nullptr_t) { ptr_ = nullptr; return *this; }
+  // (templates on the integer type: an unsigned or 64-bit offset would otherwise be ambiguous
+  // between the offset form and the conversion of the offset to a pointer difference)
+  template <typename I, typename = typename std::enable_if<std::is_integral<I>::value>::type>
+  device_ptr& operator+=(I n) { ptr_ += (difference_type)n; return *this; }
+  template <typename I, typename = typename std::enable_if<std::is_integral<I>::value>::type>
+  device_ptr& operator-=(I n) { ptr_ -= (difference_type)n; return *this; }
+  template <typename I, typename = typename std::enable_if<std::is_integral<I>::value>::type>
+  device_ptr operator+(I n) const { return device_ptr(ptr_ + (difference_type)n); }
+  template <typename I, typename = typename std::enable_if<std::is_integral<I>::value>::type>
+  device_ptr operator-(I n) const { return device_ptr(ptr_ - (difference_type)n); }
   difference_type operator-(const device_ptr& o) const { return ptr_ - o.ptr_; }
   bool operator==(const device_ptr& o) const { return ptr_ == o.ptr_; }
   bool operator!=(const device_ptr& o) const { return ptr_ != o.ptr_; }
@@ -93,10 +131,18 @@ class device_ptr {
   bool operator>(const device_ptr& o) const { return ptr_ > o.ptr_; }
   bool operator<=(const device_ptr& o) const { return ptr_ <= o.ptr_; }
   bool operator>=(const device_ptr& o) const { return ptr_ >= o.ptr_; }
+  bool operator==(std::nullptr_t) const { return ptr_ == nullptr; }
+  bool operator!=(std::nullptr_t) const { return ptr_ != nullptr; }
 
  private:
   T* ptr_;
 };
+template <typename T>
+inline bool operator==(std::nullptr_t, const device_ptr<T>& p) { return p.get() == nullptr; }
+template <typename T>
+inline bool operator!=(std::nullptr_t, const device_ptr<T>& p) { return p.get() != nullptr; }
+template <typename T>
+inline device_reference<T>::device_reference(const device_ptr<T>& p) : ptr_(p.get()) {}
 
 template <>
 class device_ptr<void> {

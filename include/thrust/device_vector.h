@@ -10,8 +10,10 @@
 // allocator whose allocate(n) yields a device_ptr<T> or a raw device pointer will do, e.g.
 // thrust::mr::allocator<T, Pool> over a pool resource (thrust/mr/pool.h).
 #pragma once
+#include <algorithm>
 #include <cstring>
 #include <new>
+#include <stdexcept>
 #include <cstddef>
 #include <iterator>
 #include <type_traits>
@@ -42,6 +44,8 @@ class device_vector {
   typedef device_ptr<const T> const_iterator;
   typedef device_reference<T> reference;
   typedef device_reference<const T> const_reference;
+  typedef std::reverse_iterator<iterator> reverse_iterator;
+  typedef std::reverse_iterator<const_iterator> const_reverse_iterator;
 
   device_vector() : data_(nullptr), size_(0), capacity_(0), alloc_() {}
   explicit device_vector(const Alloc& alloc) : data_(nullptr), size_(0), capacity_(0), alloc_(alloc) {}
@@ -103,6 +107,12 @@ class device_vector {
   const_iterator end() const { return const_iterator(data_ + size_); }
   const_iterator cbegin() const { return begin(); }
   const_iterator cend() const { return end(); }
+  reverse_iterator rbegin() { return reverse_iterator(end()); }
+  reverse_iterator rend() { return reverse_iterator(begin()); }
+  const_reverse_iterator rbegin() const { return const_reverse_iterator(end()); }
+  const_reverse_iterator rend() const { return const_reverse_iterator(begin()); }
+  const_reverse_iterator crbegin() const { return rbegin(); }
+  const_reverse_iterator crend() const { return rend(); }
   pointer data() { return pointer(data_); }
   const_pointer data() const { return const_pointer(data_); }
   size_type size() const { return size_; }
@@ -113,6 +123,17 @@ class device_vector {
   const_reference operator[](size_type i) const { return const_reference(data_ + i); }
   reference front() { return reference(data_); }
   reference back() { return reference(data_ + size_ - 1); }
+  const_reference front() const { return const_reference(data_); }
+  const_reference back() const { return const_reference(data_ + size_ - 1); }
+  reference at(size_type i) {
+    if (i >= size_) throw std::out_of_range("thrust::device_vector::at");
+    return reference(data_ + i);
+  }
+  const_reference at(size_type i) const {
+    if (i >= size_) throw std::out_of_range("thrust::device_vector::at");
+    return const_reference(data_ + i);
+  }
+  size_type max_size() const { return (~size_type(0)) / sizeof(T); }
 
   allocator_type get_allocator() const { return alloc_; }
   void reserve(size_type n) {
@@ -159,6 +180,32 @@ class device_vector {
     ++size_;
   }
   void pop_back() { --size_; }
+  iterator erase(iterator position) { return erase(position, position + 1); }
+  // Inserts before `position`; returns the first inserted element.  The elements behind the
+  // insertion point move through a temporary copy (device memory cannot be shifted onto itself).
+  iterator insert(iterator position, const T& value) { return insert(position, (size_type)1, value); }
+  iterator insert(iterator position, size_type n, const T& value) {
+    const size_type at = (size_type)(position - begin());
+    open_gap(at, n);
+    if (n) {
+      device_vector fill(n, value);
+      copy_raw(data_ + at, fill.data_, n, THRUST_AMD_D2D);
+      sync();
+    }
+    return begin() + at;
+  }
+  template <typename InputIterator,
+            typename = typename std::iterator_traits<InputIterator>::iterator_category>
+  iterator insert(iterator position, InputIterator first, InputIterator last) {
+    const size_type at = (size_type)(position - begin());
+    device_vector added(first, last);  // (also when the range lies in this vector)
+    open_gap(at, added.size());
+    if (added.size()) {
+      copy_raw(data_ + at, added.data_, added.size(), THRUST_AMD_D2D);
+      sync();
+    }
+    return begin() + at;
+  }
   iterator erase(iterator first, iterator last) {
     const size_type tail = end() - last;
     if (tail && first != last) {
@@ -203,6 +250,20 @@ class device_vector {
   static void copy_raw(T* dst, const T* src, size_type n, int kind) {
     system::hip::detail::throw_on_error(thrust_amd_memcpy(dst, src, n * sizeof(T), kind, nullptr),
                                         "device_vector copy");
+  }
+  // Makes room for n elements at index `at`: the tail moves n places back, the size grows by n.
+  // The capacity grows only when it has to, and then to exactly the new size.
+  void open_gap(size_type at, size_type n) {
+    if (n == 0) return;
+    const size_type tail = size_ - at;
+    device_vector moved;
+    if (tail) moved.assign_device(data_ + at, tail);
+    if (size_ + n > capacity_) reserve(size_ + n);
+    if (tail) {
+      copy_raw(data_ + at + n, moved.data_, tail, THRUST_AMD_D2D);
+      sync();
+    }
+    size_ += n;
   }
   void release() {
     free_raw(data_, capacity_);
@@ -281,16 +342,38 @@ host_vector<T, Alloc>::host_vector(device_ptr<U> first, device_ptr<U> last) : ba
   }
 }
 
+// Comparisons between device_vector, host_vector and std::vector, in either order
+// (thrust/detail/vector_base.inl:1190-1320): the device side is copied to the host once.
 template <typename T, typename DA, typename DB>
 inline bool operator==(const device_vector<T, DA>& a, const device_vector<T, DB>& b) {
+  if (a.size() != b.size()) return false;
   return host_vector<T>(a) == host_vector<T>(b);
 }
 template <typename T, typename DA, typename A>
 inline bool operator==(const device_vector<T, DA>& a, const std::vector<T, A>& b) {
-  host_vector<T> h(a);
-  return h.size() == b.size() && std::equal(h.begin(), h.end(), b.begin());
+  if (a.size() != b.size()) return false;
+  const host_vector<T> h(a);
+  return std::equal(h.begin(), h.end(), b.begin());
 }
 template <typename T, typename DA, typename A>
 inline bool operator==(const std::vector<T, A>& a, const device_vector<T, DA>& b) { return b == a; }
+template <typename T, typename DA>
+inline bool operator==(const device_vector<T, DA>& a, const detail::contiguous_vector<T>& b) {
+  if (a.size() != b.size()) return false;
+  const host_vector<T> h(a);
+  return std::equal(h.begin(), h.end(), b.begin());
+}
+template <typename T, typename DA>
+inline bool operator==(const detail::contiguous_vector<T>& a, const device_vector<T, DA>& b) { return b == a; }
+template <typename T, typename DA, typename DB>
+inline bool operator!=(const device_vector<T, DA>& a, const device_vector<T, DB>& b) { return !(a == b); }
+template <typename T, typename DA, typename A>
+inline bool operator!=(const device_vector<T, DA>& a, const std::vector<T, A>& b) { return !(a == b); }
+template <typename T, typename DA, typename A>
+inline bool operator!=(const std::vector<T, A>& a, const device_vector<T, DA>& b) { return !(b == a); }
+template <typename T, typename DA>
+inline bool operator!=(const device_vector<T, DA>& a, const detail::contiguous_vector<T>& b) { return !(a == b); }
+template <typename T, typename DA>
+inline bool operator!=(const detail::contiguous_vector<T>& a, const device_vector<T, DA>& b) { return !(b == a); }
 
 }  // namespace thrust

@@ -103,12 +103,28 @@ It for_each(execution_policy<D>& exec, It first, It last, F f) {
 #endif
   return last;
 }
+namespace detail {
+// an array of arithmetic elements of the type of init: the library's kernel (no hipcc needed)
 template <typename D, typename It, typename T>
-void sequence(execution_policy<D>& exec, It first, It last, T init, T step) {
-  const detail::sequence_value<T> value = {init, step};
+void sequence(execution_policy<D>& exec, It first, It last, T init, T step, std::true_type) {
+  throw_on_error(thrust_amd_sequence(thrust::detail::raw(first), (uint64_t)(last - first), dtype_of<T>::value, &init,
+                                     &step, stream_of(exec)),
+                 "sequence failed");
+  synchronize(stream_of(exec), "sequence: synchronize");
+}
+// anything else: the values are computed by a transform iterator and copied through the output
+template <typename D, typename It, typename T>
+void sequence(execution_policy<D>& exec, It first, It last, T init, T step, std::false_type) {
+  const sequence_value<T> value = {init, step};
   thrust::counting_iterator<unsigned long long> zero(0);
   thrust::copy(exec, thrust::make_transform_iterator(zero, value),
                thrust::make_transform_iterator(zero + (last - first), value), first);
+}
+}  // namespace detail
+template <typename D, typename It, typename T>
+void sequence(execution_policy<D>& exec, It first, It last, T init, T step) {
+  detail::sequence(exec, first, last, init, step,
+                   std::integral_constant<bool, detail::is_abi_type<T>::value && detail::is_array_of<T, It>::value>());
 }
 template <typename D, typename MapIt, typename In, typename Out>
 Out gather(execution_policy<D>& exec, MapIt map_first, MapIt map_last, In input, Out result) {

@@ -151,6 +151,13 @@ int thrust_amd_stream_synchronize(void* stream);
 int thrust_amd_convert(const void* in, int in_dtype, void* out, int out_dtype, uint64_t n,
                        void* stream);
 
+/* out[i] = (T)(init + step * (T)i) for i in [0, n), T the element type named by dtype; init
+ * and step point at host values of that type.  Replaces thrust::sequence -> thrust::tabulate
+ * with compute_sequence_value (thrust/system/detail/generic/sequence.inl:56-85) for arrays of
+ * arithmetic elements, so that code compiled by a plain host compiler can fill its inputs. */
+int thrust_amd_sequence(void* out, uint64_t n, int dtype, const void* init, const void* step,
+                        void* stream);
+
 /* Streams and events for callers that overlap work (the asynchronous algorithms of the
  * front end).  A stream created here is independent of the null stream; an event is
  * recorded on one stream and another stream can be made to wait for it without blocking

@@ -120,3 +120,30 @@ def test_convert_rejects_bad_arguments(dev):
     assert lib.thrust_amd_convert(d.ptr, 0, d.ptr, -1, 16, dev.stream_ptr()) != 0
     assert lib.thrust_amd_convert(None, 0, d.ptr, 0, 16, dev.stream_ptr()) != 0
     assert lib.thrust_amd_convert(None, 0, None, 0, 0, dev.stream_ptr()) == 0
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_sequence_every_type(dev, dtype):
+    # thrust::sequence(first, last, init, step): element i is (T)(init + step * (T)i)
+    # (thrust/system/detail/generic/sequence.inl:56-85; testing/sequence.cu:43-76 for the literal cases)
+    t = np.dtype(dtype)
+    cases = [(0, 1), (10, 2), (3, 7)] if t.kind != "f" else [(0.0, 1.0), (10.0, 2.0), (0.1, 0.3), (-1.5, 1e-3)]
+    if t.kind == "i":
+        cases.append((-5, -3))
+    for n in (0, 1, 5, 63, 4097, 100003):
+        i = np.arange(n, dtype=np.uint64).astype(t)  # (T)i: wraps for the narrow types
+        for init, step in cases:
+            with np.errstate(over="ignore"):
+                if t.kind == "f":
+                    want = t.type(init) + t.type(step) * i  # every operation rounded to T, no fused multiply-add
+                else:
+                    wide = np.int64 if t.kind == "i" else np.uint64
+                    want = (wide(init) + wide(step) * i.astype(wide)).astype(t)
+            got = dev.sequence(n, dev.DTYPE_OF_NP[t], init, step).numpy()
+            assert got.dtype == want.dtype and got.tobytes() == want.tobytes(), (dtype, n, init, step)
+    got = dev.sequence(5, dev.DTYPE_OF_NP[t], 10, 2).numpy()
+    assert list(got) == [10, 12, 14, 16, 18]
+    lib = dev.load()
+    assert lib.thrust_amd_sequence(None, 0, dev.DTYPE_OF_NP[t], None, None, dev.stream_ptr()) == 0
+    assert lib.thrust_amd_sequence(None, 4, dev.DTYPE_OF_NP[t], None, None, dev.stream_ptr()) != 0
+    assert lib.thrust_amd_sequence(got.ctypes.data, 4, 99, got.ctypes.data, got.ctypes.data, dev.stream_ptr()) != 0

@@ -29,6 +29,13 @@ def test_thrust_api_known_answers_and_differential():
     assert "PASSED" in out
 
 
+def test_containers_and_pointers_as_the_reference_tests_use_them():
+    # host_vector / device_vector (construction, assignment across systems, insert, erase, resize, reserve, comparisons
+    # with std::vector in either order, reverse iterators, large elements), device_ptr, device_reference
+    out = _run("test_containers")
+    assert "PASSED" in out
+
+
 def test_c_abi_from_plain_c():
     out = _run("test_thrust_c11")
     assert "PASS" in out

@@ -51,6 +51,7 @@ SIGNATURES = {
     "thrust_amd_profile_enable": (_int, [_int]),
     "thrust_amd_profile_collect": (_int, [_c.c_char_p, _sz, _szp]),
     "thrust_amd_convert": (_int, [_vp, _int, _vp, _int, _u64, _vp]),
+    "thrust_amd_sequence": (_int, [_vp, _u64, _int, _vp, _vp, _vp]),
     "thrust_amd_stream_create": (_int, [ctypes.POINTER(_vp)]),
     "thrust_amd_stream_destroy": (_int, [_vp]),
     "thrust_amd_stream_query": (_int, [_vp, ctypes.POINTER(_int)]),
@@ -223,6 +224,13 @@ def reduce(x, op=PLUS, init=0, temp=None, out=None):
 def convert(x, out_dtype, out=None):
     out = out or DeviceArray(x.n, out_dtype)
     check(load().thrust_amd_convert(x.ptr, x.dtype, out.ptr, out_dtype, x.n, stream_ptr()), "thrust_amd_convert")
+    return out
+
+
+def sequence(n, dtype, init=0, step=1, out=None):
+    out = out or DeviceArray(n, dtype)
+    iv, sv = _scalar(dtype, init), _scalar(dtype, step)
+    check(load().thrust_amd_sequence(out.ptr, n, dtype, iv.ctypes.data, sv.ctypes.data, stream_ptr()), "thrust_amd_sequence")
     return out
 
 

@@ -209,6 +209,39 @@ TA_EXPORT int thrust_amd_convert(const void* in, int in_dtype, void* out, int ou
   });
 }
 
+namespace ta {
+// The product is rounded before the sum, as in the reference's host back ends (no fused
+// multiply-add), so that floating-point sequences agree with them bit for bit.
+template <typename T>
+__global__ __launch_bounds__(256) void sequence_kernel(T* out, uint64_t n, T init, T step) {
+#pragma clang fp contract(off)
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
+    out[i] = static_cast<T>(init + step * static_cast<T>(i));
+}
+}  // namespace ta
+
+TA_EXPORT int thrust_amd_sequence(void* out, uint64_t n, int dtype, const void* init, const void* step,
+                                  void* stream) {
+  using namespace ta;
+  if (!valid_dtype(dtype)) return (int)hipErrorInvalidValue;
+  if (n == 0) return 0;
+  if (!out || !init || !step) return (int)hipErrorInvalidValue;
+  return with_dtype(dtype, [&](auto tt) {
+    using T = typename decltype(tt)::type;
+    T first, by;
+    __builtin_memcpy(&first, init, sizeof(T));
+    __builtin_memcpy(&by, step, sizeof(T));
+    uint64_t blocks = (n + 255) / 256;
+    const uint64_t cap = (uint64_t)1 << 20;
+    if (blocks > cap) blocks = cap;
+    TA_LAUNCH("sequence", (hipStream_t)stream, (sequence_kernel<T>), dim3((uint32_t)blocks), dim3(256),
+              static_cast<T*>(out), n, first, by);
+    TA_CHECK_LAUNCH();
+    return 0;
+  });
+}
+
 // ------------------------------------------------------------------ temp arena
 // Blocks are rounded up to size classes (powers of two from 4 KiB to 64 MiB, then
 // multiples of 64 MiB -- a 2^28-key radix sort needs ~1.2 GiB and must not round to
