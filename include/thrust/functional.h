@@ -11,6 +11,7 @@
 //   unary transforms   identity, negate, square          (transform_reduce, transform scans)
 #pragma once
 #include <thrust/detail/config.h>
+#include <thrust/detail/placeholder_expressions.h>
 
 namespace thrust {
 
@@ -147,18 +148,22 @@ struct square<void> {
 };
 
 namespace detail {
-// `x CMP value` as a unary predicate; CMP is a thrust_amd_cmp code (0 LT .. 5 NE).
+// `x CMP value` as a unary predicate; CMP is a thrust_amd_cmp code (0 LT .. 5 NE).  It is what
+// `_1 CMP value` builds: the one placeholder expression the library's own selection kernels
+// take (as a comparison code and a threshold), and a node like any other inside larger
+// expressions (`_1 > 2 && _1 < 9`).
 #if defined(__GNUC__)
 #pragma GCC diagnostic push
 #pragma GCC diagnostic ignored "-Wsign-compare"  // the expression is the caller's, conversions included
 #endif
 template <int CMP, typename T>
-struct compare_with {
+struct compare_with : lambda::actor_base {
   T value;
+  constexpr explicit compare_with(const T& v) : value(v) {}
   // evaluated on the argument as it is, under the usual arithmetic conversions, as the
-  // reference's placeholder expression `_1 < t` does
-  template <typename A>
-  constexpr bool operator()(const A& x) const {
+  // reference's placeholder expression `_1 < t` does (further arguments are ignored)
+  template <typename A, typename... Rest>
+  constexpr bool operator()(const A& x, Rest&&...) const {
     return CMP == 0 ? x < value : CMP == 1 ? x <= value : CMP == 2 ? x > value
          : CMP == 3 ? x >= value : CMP == 4 ? x == value : x != value;
   }
@@ -166,20 +171,15 @@ struct compare_with {
 #if defined(__GNUC__)
 #pragma GCC diagnostic pop
 #endif
-struct placeholder1 {};
-}  // namespace detail
 
-// Placeholder expressions of the form `_1 < t` (and <=, >, >=, ==, !=), the shape the
-// reference's own code uses for simple predicates (thrust/functional.h placeholders).
-namespace placeholders {
-static const thrust::detail::placeholder1 _1;
-}
-namespace detail {
+namespace lambda {
+// `_1 CMP value` and `value CMP _1` with a plain value (more specialised than the general
+// operators of placeholder_expressions.h, so these are chosen)
 #define THRUST_AMD_PLACEHOLDER_CMP(OP, CODE, SWAPPED)                                                  \
-  template <typename T>                                                                                \
-  constexpr compare_with<CODE, T> operator OP(placeholder1, const T& v) { return compare_with<CODE, T>{v}; } \
-  template <typename T>                                                                                \
-  constexpr compare_with<SWAPPED, T> operator OP(const T& v, placeholder1) { return compare_with<SWAPPED, T>{v}; }
+  template <typename T, typename = typename std::enable_if<!is_actor<T>::value>::type>                 \
+  constexpr compare_with<CODE, T> operator OP(argument<0>, const T& v) { return compare_with<CODE, T>(v); } \
+  template <typename T, typename = typename std::enable_if<!is_actor<T>::value>::type>                 \
+  constexpr compare_with<SWAPPED, T> operator OP(const T& v, argument<0>) { return compare_with<SWAPPED, T>(v); }
 THRUST_AMD_PLACEHOLDER_CMP(<, 0, 2)
 THRUST_AMD_PLACEHOLDER_CMP(<=, 1, 3)
 THRUST_AMD_PLACEHOLDER_CMP(>, 2, 0)
@@ -187,6 +187,21 @@ THRUST_AMD_PLACEHOLDER_CMP(>=, 3, 1)
 THRUST_AMD_PLACEHOLDER_CMP(==, 4, 4)
 THRUST_AMD_PLACEHOLDER_CMP(!=, 5, 5)
 #undef THRUST_AMD_PLACEHOLDER_CMP
+}  // namespace lambda
 }  // namespace detail
+
+// thrust::placeholders::_1 .. _10 (thrust/functional.h:1430-1520 of the reference)
+namespace placeholders {
+static const thrust::detail::lambda::argument<0> _1 = {};
+static const thrust::detail::lambda::argument<1> _2 = {};
+static const thrust::detail::lambda::argument<2> _3 = {};
+static const thrust::detail::lambda::argument<3> _4 = {};
+static const thrust::detail::lambda::argument<4> _5 = {};
+static const thrust::detail::lambda::argument<5> _6 = {};
+static const thrust::detail::lambda::argument<6> _7 = {};
+static const thrust::detail::lambda::argument<7> _8 = {};
+static const thrust::detail::lambda::argument<8> _9 = {};
+static const thrust::detail::lambda::argument<9> _10 = {};
+}  // namespace placeholders
 
 }  // namespace thrust

@@ -37,6 +37,14 @@ __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void for_each_kernel(View first,
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) f(first[i]);
 }
 
+// (the functor receives the element itself, so a functor that modifies its argument -- `++_1`
+// -- changes the input, as it does in the reference)
+template <typename View, typename OutView, typename F>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform1_kernel(View in, OutView out, uint64_t n, F f) {
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[i] = f(in[i]);
+}
+
 template <typename ViewA, typename ViewB, typename OutView, typename F>
 __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform2_kernel(ViewA a, ViewB b, OutView out, uint64_t n, F f) {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;

@@ -58,7 +58,23 @@ struct sequence_value {  // element i of thrust::sequence(first, last, init, ste
 
 template <typename D, typename In, typename Out, typename F>
 Out transform(execution_policy<D>& exec, In first, In last, Out result, F f) {
-  return thrust::copy(exec, thrust::make_transform_iterator(first, f), thrust::make_transform_iterator(last, f), result);
+  static_assert(detail::is_device_input<In>::value && detail::is_device_output<Out>::value,
+                "thrust::transform on the device system reads device or fancy iterators and writes device memory");
+  void* stream = detail::stream_of(exec);
+  const uint64_t n = (uint64_t)(last - first);
+  if (n == 0) return result;
+#if defined(__HIPCC__)
+  hipLaunchKernelGGL((detail::transform1_kernel<typename thrust::detail::device_view_of<In>::type,
+                                                typename thrust::detail::device_view_of<Out>::type, F>),
+                     dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
+                     thrust::detail::device_view(first), thrust::detail::device_view(result), n, f);
+  detail::throw_on_error(detail::launch_status(), "transform: kernel launch");
+  detail::synchronize(stream, "transform: synchronize");
+#else
+  static_assert(detail::fancy_needs_hipcc<F>::value,
+                "thrust::transform on the device system runs the functor in a kernel; compile this translation unit with hipcc");
+#endif
+  return result + n;
 }
 template <typename D, typename In1, typename In2, typename Out, typename F>
 Out transform(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, Out result, F f) {

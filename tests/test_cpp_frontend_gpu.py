@@ -77,3 +77,10 @@ def test_reference_cases_of_sorts_scans_merges_and_set_operations():
     # scans from structs, counting iterators and with thrust::identity<> / maximum<>
     out = _run("test_reference_cases_sorts_scans")
     assert "PASSED" in out
+
+
+def test_placeholder_expressions_as_functors():
+    # thrust::placeholders: arithmetic, bitwise, logical, relational, compound assignment and increment forms through
+    # thrust::transform on both systems, and as predicates / operators of count_if, copy_if, partition, reduce, inner_product
+    out = _run("test_placeholders")
+    assert "PASSED" in out
