@@ -287,12 +287,14 @@ THRUST_AMD_DEVICE uint32_t tile_try_load(const uint64_t* slot, P& payload) {
 // waited on, and those have started, so the spin terminates without assuming any
 // workgroup scheduling order.  `id` must be a true identity of op.  Returns, in all
 // lanes, the fold of all tiles before `tile`.
-template <typename P, typename Op>
+template <typename P, int WINDOW = 8, typename Op>
 THRUST_AMD_DEVICE P tile_lookback(const uint64_t* status_base, uint32_t tile, Op op, P id) {
   constexpr int W = TileWords<P>::W;
-  // Descriptors inspected per round: the nearest 8.  A wider window reads more cache lines
-  // per round and, with many tiles in flight, costs more than it saves.
-  constexpr int WIN = 8;
+  // Descriptors inspected per round: the nearest WINDOW.  A wider window reads more cache lines
+  // per round and, with many tiles in flight, mostly costs more than it saves: 8 measured best
+  // for the scans and the selection kernels, 16 for reduce_by_key (whose tiles have little left
+  // to do once their prefix is known: 0.617 -> 0.600 ms at 2^28 pairs).
+  constexpr int WIN = WINDOW;
   const int lane = lane_id();
   P running = id;
   int64_t base = (int64_t)tile - 1;

@@ -418,12 +418,37 @@ THRUST_AMD_DEVICE void select_tile(const SelectArgs<T, U, Flagger>& a, SelectSha
   // ---- selected elements before this tile
   constexpr int W = TileWords<uint64_t>::W;
   uint64_t* my_slot = a.status + (size_t)tile * W;
+  if (wave == 0 && lane == 0) tile_publish<uint64_t>(my_slot, tile == 0 ? TS_INCLUSIVE : TS_PARTIAL, (uint64_t)tile_cnt);
+
+  // A tile that keeps few elements (one output, forward sweep) gathers them in LDS at their place
+  // inside the tile while its prefix is on its way, and has only a coalesced copy left to do when
+  // it arrives.  The workgroup's write-out regions together serve as the gathering area.
+  constexpr uint32_t STAGE_TOTAL = (uint32_t)WAVES * Shape::STAGE_BYTES;
+  // (a multiple of 16 elements, so that the payload's part starts on a 16-byte boundary)
+  constexpr uint32_t GATHER_CAP = (STAGE_TOTAL / (uint32_t)(sizeof(T) + (HAS_PAYLOAD ? sizeof(U) : 0))) & ~15u;
+  T* gather_tested = reinterpret_cast<T*>(sh.stage);
+  U* gather_payload = reinterpret_cast<U*>(sh.stage + (size_t)GATHER_CAP * sizeof(T));
+  const bool gathered = !TWO && !REV && tile_cnt <= GATHER_CAP;
+  if constexpr (!TWO && !REV) {
+    if (gathered) {
+#pragma unroll
+      for (int j = 0; j < CHUNKS; ++j) {
+        uint32_t r = wave_prefix + lane_excl[j];
+#pragma unroll
+        for (int i = 0; i < VEC; ++i) {
+          if ((fl[j] >> i) & 1u) {
+            if (a.tested_true) gather_tested[r] = x[j].v[i];
+            if constexpr (HAS_PAYLOAD) gather_payload[r] = y[j].v[i];
+            ++r;
+          }
+        }
+      }
+    }
+  }
+
   if (wave == 0) {
     uint64_t excl = 0;
-    if (tile == 0) {
-      if (lane == 0) tile_publish<uint64_t>(my_slot, TS_INCLUSIVE, (uint64_t)tile_cnt);
-    } else {
-      if (lane == 0) tile_publish<uint64_t>(my_slot, TS_PARTIAL, (uint64_t)tile_cnt);
+    if (tile != 0) {
       excl = tile_lookback<uint64_t>(a.status, tile, OpPlus{}, (uint64_t)0);
       if (lane == 0) tile_publish<uint64_t>(my_slot, TS_INCLUSIVE, excl + tile_cnt);
     }
@@ -433,6 +458,16 @@ THRUST_AMD_DEVICE void select_tile(const SelectArgs<T, U, Flagger>& a, SelectSha
     }
   }
   __syncthreads();
+  if constexpr (!TWO && !REV) {
+    if (gathered) {
+      const uint64_t base = sh.prefix;
+      if (a.tested_true)
+        for (uint32_t e = threadIdx.x; e < tile_cnt; e += Shape::BLOCK) a.tested_true[base + e] = gather_tested[e];
+      if constexpr (HAS_PAYLOAD)
+        for (uint32_t e = threadIdx.x; e < tile_cnt; e += Shape::BLOCK) a.payload_true[base + e] = gather_payload[e];
+      return;
+    }
+  }
   // the wave's selected elements start at prefix + wave_prefix of the first output; a
   // rejected element at tile offset e with r selected elements before it in the tile
   // lands at (tile_base - prefix) + e - r of the second output
