@@ -325,6 +325,25 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     }
   }
 
+  // The values start their way now, so that they have arrived by the time the keys have left:
+  // loaded only after the look-back, their latency was the longest part of what a tile still
+  // had to do once its offsets were known.
+  V v[HAS_VALUES ? ITEMS : 1];
+  if constexpr (HAS_VALUES) {
+    if (valid == (uint32_t)TILE) {
+      // whole tile: no predicates, so that all loads are in flight together (a predicated
+      // load makes the compiler wait for it before issuing the next one)
+#pragma unroll
+      for (int r = 0; r < ITEMS; ++r) v[r] = vals_in[tile_base + span + r * WAVE];
+    } else {
+#pragma unroll
+      for (int r = 0; r < ITEMS; ++r) {
+        const uint32_t pos = span + r * WAVE;
+        v[r] = (pos < valid) ? vals_in[tile_base + pos] : V{};
+      }
+    }
+  }
+
   // ---- rank inside the wave by digit
   // Per digit bit: v_bfe_i32 (lane's bit as 0 / -1), one ballot, and two v_bitop3 folding
   // "same bit as mine" into the 64-bit peer mask.  The wave-private counter is read, then
@@ -478,19 +497,6 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     }
   }
   if constexpr (HAS_VALUES) {
-    V v[ITEMS];
-    if (valid == (uint32_t)TILE) {
-      // whole tile: no predicates, so that all loads are in flight together (a predicated
-      // load makes the compiler wait for it before issuing the next one)
-#pragma unroll
-      for (int r = 0; r < ITEMS; ++r) v[r] = vals_in[tile_base + span + r * WAVE];
-    } else {
-#pragma unroll
-      for (int r = 0; r < ITEMS; ++r) {
-        const uint32_t pos = span + r * WAVE;
-        v[r] = (pos < valid) ? vals_in[tile_base + pos] : V{};
-      }
-    }
     __syncthreads();  // keys have been read out of the exchange buffer
 #pragma unroll
     for (int r = 0; r < ITEMS; ++r) s_vals[(rank2[r / 2] >> (16 * (r % 2))) & 0xffffu] = v[r];
