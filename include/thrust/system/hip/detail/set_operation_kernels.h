@@ -55,19 +55,6 @@ struct SetShape {
   static constexpr int WAVES_PER_SIMD = ITEM > 4 ? 3 : 4;
 };
 
-// Number of elements taken from A among the first `diag` elements of the merged order.
-template <typename T, typename PA, typename PB, typename Comp>
-THRUST_AMD_DEVICE uint64_t set_merge_path(PA a, uint64_t na, PB b, uint64_t nb, uint64_t diag, Comp& comp) {
-  uint64_t lo = diag > nb ? diag - nb : 0;
-  uint64_t hi = diag < na ? diag : na;
-  while (lo < hi) {
-    const uint64_t mid = (lo + hi) >> 1;
-    if (!comp(b[diag - 1 - mid], a[mid])) lo = mid + 1;
-    else hi = mid;
-  }
-  return lo;
-}
-
 // Per tile boundary t (t = 0 .. tiles), found by one thread: split[t] = elements of A before
 // merged position t * tile_size; for boundaries inside the merged order, key[t] = the
 // element at that position and run[3t .. 3t+2] = merged positions where its run starts,
@@ -118,12 +105,17 @@ __global__ __launch_bounds__(256) void set_init_kernel(uint64_t* __restrict__ wo
   }
 }
 
-// Two positions scanned together: the run start in the high half, the B-part start in the low.
-struct OpMaxPair {
-  THRUST_AMD_DEVICE uint64_t operator()(uint64_t x, uint64_t y) const {
-    const uint32_t xh = (uint32_t)(x >> 32), yh = (uint32_t)(y >> 32);
-    const uint32_t xl = (uint32_t)x, yl = (uint32_t)y;
-    return ((uint64_t)(xh > yh ? xh : yh) << 32) | (xl > yl ? xl : yl);
+// Two tile-local positions that travel through a max-scan together, 16 bits each.
+struct OpMaxPair16 {
+  THRUST_AMD_DEVICE uint32_t operator()(uint32_t x, uint32_t y) const {
+    typedef unsigned short pair16 __attribute__((ext_vector_type(2)));
+    pair16 a, b;
+    __builtin_memcpy(&a, &x, 4);
+    __builtin_memcpy(&b, &y, 4);
+    const pair16 m = __builtin_elementwise_max(a, b);
+    uint32_t r;
+    __builtin_memcpy(&r, &m, 4);
+    return r;
   }
 };
 
@@ -146,6 +138,42 @@ THRUST_AMD_DEVICE V set_block_exclusive(V v, Op op, V id, V* buf, V* total) {
   return op(prefix, before);
 }
 
+// Two scans of position pairs behind one barrier: `before` = the fold of `fwd` over the
+// threads before this one, `after` = the fold of `bwd` over the threads after it, `all` =
+// the fold of `fwd` over the workgroup.  0 is the identity.
+template <int WAVES>
+THRUST_AMD_DEVICE void set_block_both_ways(uint32_t fwd, uint32_t bwd, uint32_t* buf_fwd, uint32_t* buf_bwd,
+                                           uint32_t& before, uint32_t& after, uint32_t& all) {
+  const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
+  const OpMaxPair16 op;
+  const int mirror = (WAVE - 1 - lane) * 4;
+  const uint32_t incl_f = wave_inclusive_scan(fwd, op, 0u);
+  const uint32_t incl_b = wave_inclusive_scan((uint32_t)__builtin_amdgcn_ds_bpermute(mirror, (int)bwd), op, 0u);
+  if (lane == WAVE - 1) {
+    buf_fwd[wave] = incl_f;
+    buf_bwd[wave] = incl_b;
+  }
+  const uint32_t excl_f = dpp_move<0x138 /* wave_shr:1 */>(0u, incl_f);
+  const uint32_t excl_b =
+      (uint32_t)__builtin_amdgcn_ds_bpermute(mirror, (int)dpp_move<0x138 /* wave_shr:1 */>(0u, incl_b));
+  __syncthreads();
+  uint32_t prefix = 0, total = 0, suffix = 0;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    if (w == wave) prefix = total;
+    total = op(total, buf_fwd[w]);
+    if (w > wave) suffix = op(suffix, buf_bwd[w]);
+  }
+  before = op(prefix, excl_f);
+  after = op(suffix, excl_b);
+  all = total;
+}
+
+// all ones when bit `o` of `bits` is set, else zero
+THRUST_AMD_DEVICE int32_t set_bit_mask(uint32_t bits, int o) { return (int32_t)(bits << (31 - o)) >> 31; }
+// `yes` where the mask is all ones, `no` where it is zero
+THRUST_AMD_DEVICE int32_t set_pick(int32_t mask, int32_t yes, int32_t no) { return (yes & mask) | (no & ~mask); }
+
 template <typename T, typename V, bool HAS_VALUES, typename Comp>
 struct SetArgs {
   const T* a;
@@ -166,22 +194,43 @@ struct SetArgs {
   Comp comp;
 };
 
+// Reads the tile's `ca` elements at pa and `count - ca` elements at pb into LDS, A's part first.
+// A wave's 64 consecutive elements of one round nearly always lie in one range: then the
+// address is the wave's base plus the lane, with nothing to select.
+template <int BLOCK, int ITEMS, typename E>
+THRUST_AMD_DEVICE void set_stage(const E* __restrict__ pa, const E* __restrict__ pb, uint32_t ca, uint32_t count,
+                                 bool with_b, uint32_t wave, uint32_t lane, E* s_items) {
+  E in[ITEMS];
+#pragma unroll
+  for (int q = 0; q < ITEMS; ++q) {
+    const uint32_t row = (uint32_t)q * BLOCK + wave * WAVE;  // the same for the whole wave
+    if (row + WAVE <= ca) {
+      in[q] = pa[row + lane];
+    } else if (with_b && row >= ca && row + WAVE <= count) {
+      in[q] = pb[(row - ca) + lane];
+    } else {
+      const uint32_t e = row + lane;
+      in[q] = (e < ca) ? pa[e] : (with_b && e < count) ? pb[e - ca] : E{};
+    }
+  }
+#pragma unroll
+  for (int q = 0; q < ITEMS; ++q) s_items[(uint32_t)q * BLOCK + wave * WAVE + lane] = in[q];
+}
+
 template <typename T, typename V, bool HAS_VALUES, typename Comp>
 __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V, HAS_VALUES>::WAVES_PER_SIMD)) void set_op_kernel(SetArgs<T, V, HAS_VALUES, Comp> g) {
   using Shape = SetShape<T, V, HAS_VALUES>;
   constexpr int SET_BLOCK = Shape::BLOCK;
   constexpr int SET_TILE = Shape::TILE;
   constexpr int SET_WAVES = SET_BLOCK / WAVE;
+  static_assert(SET_TILE <= 0x7fff && SET_ITEMS == 16, "positions travel in 16 bits, flags in 16-bit masks");
   // one buffer for the staged keys, the compacted keys and (later) the staged values
   __shared__ __attribute__((aligned(16))) unsigned char s_raw[(size_t)(SET_TILE + 1) * Shape::ITEM];
   T* s_keys = reinterpret_cast<T*>(s_raw);
   V* s_vals = reinterpret_cast<V*>(s_raw);
   __shared__ uint16_t s_src[HAS_VALUES ? SET_TILE : 1];
-  __shared__ __attribute__((aligned(16))) unsigned char s_edge_raw[SET_BLOCK * sizeof(T)];  // keys may be structs of the caller
-  T* s_edge_key = reinterpret_cast<T*>(s_edge_raw);
-  __shared__ uint8_t s_edge_b[SET_BLOCK];
-  __shared__ uint64_t s_pair[SET_BLOCK];
-  __shared__ uint64_t s_scan64[SET_WAVES];
+  __shared__ uint32_t s_fwd[SET_WAVES];
+  __shared__ uint32_t s_bwd[SET_WAVES];
   __shared__ uint32_t s_scan32[SET_WAVES];
   __shared__ uint32_t s_tile;
   __shared__ uint64_t s_base;
@@ -189,7 +238,10 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
   Comp& comp = g.comp;
   if (threadIdx.x == 0) s_tile = atomicAdd(g.ticket, 1u);
   __syncthreads();
-  const uint64_t tile = s_tile;
+  // the ticket and what follows from it are the same for the whole workgroup: scalar registers
+  const uint64_t tile = (uint32_t)__builtin_amdgcn_readfirstlane((int)s_tile);
+  const uint32_t wave = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x / WAVE));
+  const uint32_t lane = threadIdx.x % WAVE;
   const uint64_t total = g.na + g.nb;
   const uint64_t d0 = tile * SET_TILE;
   const uint64_t d1 = (d0 + SET_TILE < total) ? d0 + SET_TILE : total;
@@ -198,50 +250,58 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
   const uint32_t ca = (uint32_t)(a1 - a0), cb = (uint32_t)(b1 - b0);
   const uint32_t count = ca + cb;  // == d1 - d0, 1 .. SET_TILE
 
-  // The run the tile starts in, and the run the next tile starts in (the only runs that can
-  // reach outside the tile).  With rs / rm / re the merged positions where such a run
-  // starts, where its B part starts and where it ends, its element at merged position P
-  // has rank P - rs >= (re - rm) [A] or P - rm >= (rm - rs) [B] exactly when its tile-local
-  // position is at or past a threshold that is the same for the whole tile.
-  const T f0_key = g.key[tile];
+  // The run the tile starts in is the only one that can begin before the tile.  With rs / rm /
+  // re the merged positions where it starts, where its B part starts and where it ends, its
+  // element at merged position P has rank P - rs >= (re - rm) [A] or P - rm >= (rm - rs) [B]
+  // exactly when its tile-local position is at or past a threshold (used when that run
+  // covers the whole tile; otherwise its start and its B part seed the lanes' states below).
+  constexpr uint32_t FAR = 4u * SET_TILE;  // counts at or above this decide like any larger one
   const bool f1_valid = d1 < total;
-  const T f1_key = f1_valid ? g.key[tile + 1] : f0_key;
-  auto local_threshold = [&](uint64_t global_pos) -> uint32_t {
-    if (global_pos <= d0) return 0u;
-    const uint64_t rel = global_pos - d0;
-    return rel > (uint64_t)SET_TILE ? (uint32_t)SET_TILE + 1u : (uint32_t)rel;
-  };
-  uint32_t thr_a0, thr_b0, thr_a1 = 0, thr_b1 = 0;
+  uint32_t thr_a0, thr_b0;
+  int32_t first_start;   // local position where the tile's first run starts (<= 0), bounded below
+  bool first_b_before;   // its B part starts before the tile
   {
     const uint64_t rs = g.run[3 * tile], rm = g.run[3 * tile + 1], re = g.run[3 * tile + 2];
+    auto local_threshold = [&](uint64_t global_pos) -> uint32_t {
+      if (global_pos <= d0) return 0u;
+      const uint64_t rel = global_pos - d0;
+      return rel > (uint64_t)SET_TILE ? (uint32_t)SET_TILE + 1u : (uint32_t)rel;
+    };
     thr_a0 = local_threshold(rs + (re - rm));
     thr_b0 = local_threshold(rm + (rm - rs));
-  }
-  if (f1_valid) {
-    const uint64_t rs = g.run[3 * (tile + 1)], rm = g.run[3 * (tile + 1) + 1], re = g.run[3 * (tile + 1) + 2];
-    thr_a1 = local_threshold(rs + (re - rm));
-    thr_b1 = local_threshold(rm + (rm - rs));
+    const uint64_t back = d0 - rs;
+    first_start = -(int32_t)(back < (uint64_t)SET_TILE + 1u ? (uint32_t)back : (uint32_t)SET_TILE + 1u);
+    first_b_before = rm < d0;
   }
 
   // ---- stage the keys: A's part first, then B's
-  {
-    T in[SET_ITEMS];
-#pragma unroll
-    for (int q = 0; q < SET_ITEMS; ++q) {
-      const uint32_t e = q * SET_BLOCK + threadIdx.x;
-      in[q] = (e < ca) ? g.a[a0 + e] : (e < count) ? g.b[b0 + (e - ca)] : T{};
-    }
-#pragma unroll
-    for (int q = 0; q < SET_ITEMS; ++q) s_keys[q * SET_BLOCK + threadIdx.x] = in[q];
-    if (threadIdx.x == 0) s_keys[SET_TILE] = T{};
-  }
+  set_stage<SET_BLOCK, SET_ITEMS>(g.a + a0, g.b + b0, ca, count, true, wave, lane, s_keys);
+  if (threadIdx.x == 0) s_keys[SET_TILE] = T{};
   __syncthreads();
 
   // ---- this lane's start on the path, then a serial merge of ITEMS elements
   const uint32_t run0 = threadIdx.x * SET_ITEMS;
   const uint32_t diag = run0 < count ? run0 : count;
-  uint32_t i = (uint32_t)set_merge_path<T>(s_keys, (uint64_t)ca, s_keys + ca, (uint64_t)cb, (uint64_t)diag, comp);
+  uint32_t i;
+  {
+    uint32_t lo = diag > cb ? diag - cb : 0u, hi = diag < ca ? diag : ca;
+    while (lo < hi) {
+      const uint32_t mid = (lo + hi) >> 1;
+      if (!comp(s_keys[ca + diag - 1 - mid], s_keys[mid])) lo = mid + 1;
+      else hi = mid;
+    }
+    i = lo;
+  }
   uint32_t j = ca + (diag - i);
+  // the element before this lane's first one is the later of the two last ones taken so far (B after A on ties)
+  bool prev_is_b;
+  T prev_key;
+  {
+    const T last_a = s_keys[i > 0 ? i - 1 : 0], last_b = s_keys[j > ca ? j - 1 : ca];
+    prev_is_b = (j > ca) && (i == 0 || !comp(last_b, last_a));
+    prev_key = prev_is_b ? last_b : last_a;
+    if (threadIdx.x == 0) prev_is_b = first_b_before;  // the element before the tile, if it belongs to the same run
+  }
   T k[SET_ITEMS];
   uint32_t slot[SET_ITEMS];
   uint32_t is_b = 0;  // bit o: merged element o of this lane comes from B
@@ -263,120 +323,123 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
   // valid elements of this lane: merged positions run0 + o < count
   const uint32_t live = (run0 >= count) ? 0u : ((count - run0 >= (uint32_t)SET_ITEMS) ? 0xffffu : ((1u << (count - run0)) - 1u));
 
-  // does the tile's last run go on in the next tile?  (the last merged key is the later of
-  // the two parts' last keys; only its equivalence class matters)
-  bool tail_continues = false;
+  // B elements of the tile's last run that lie in later tiles (the last merged key is the later
+  // of the two parts' last keys; only its equivalence class matters)
+  uint32_t tail_b = 0;
   if (f1_valid) {
     const T last_a = s_keys[ca ? ca - 1 : 0], last_b = s_keys[count - 1];
     const T last = (cb == 0) ? last_a : (ca == 0) ? last_b : (comp(last_b, last_a) ? last_a : last_b);
-    tail_continues = !comp(last, f1_key);
+    const T f1_key = g.key[tile + 1];
+    if (!comp(last, f1_key)) {
+      const uint64_t rm = g.run[3 * (tile + 1) + 1], re = g.run[3 * (tile + 1) + 2];
+      const uint64_t beyond = re - (rm > d1 ? rm : d1);
+      tail_b = beyond < (uint64_t)FAR ? (uint32_t)beyond : FAR;
+    }
   }
 
   // ---- head flags on the merged order: bit o set when valid element o starts a run (local
-  // position 0 counts as a start); e2: first B of a run
-  s_edge_key[threadIdx.x] = k[SET_ITEMS - 1];
-  s_edge_b[threadIdx.x] = (uint8_t)((is_b >> (SET_ITEMS - 1)) & 1u);
-  __syncthreads();
+  // position 0 never counts: the first run's start is known from the partition); e2: first
+  // B of a run, i.e. a B whose predecessor is an A or that starts a run
   uint32_t head = 0;
   {
-    T prev = (threadIdx.x > 0) ? s_edge_key[threadIdx.x - 1] : k[0];
+    T prev = (threadIdx.x > 0) ? prev_key : k[0];
 #pragma unroll
     for (int o = 0; o < SET_ITEMS; ++o) {
       head |= (uint32_t)comp(prev, k[o]) << o;
       prev = k[o];
     }
-    if (threadIdx.x == 0) head |= 1u;
     head &= live;
   }
-  // first B of a run: a B whose predecessor is an A, or that starts a run
-  const uint32_t prev_b_bits = (is_b << 1) | ((threadIdx.x > 0) ? (uint32_t)s_edge_b[threadIdx.x - 1] : 0u);
+  const uint32_t prev_b_bits = (is_b << 1) | (uint32_t)prev_is_b;
   const uint32_t e2 = is_b & (head | ~prev_b_bits) & live;
 
-  // ---- last run start / B-part start at or before each element (forward scan), next ones
-  // after it (backward scan).  Positions are stored +1 so that 0 means "none" in the forward
-  // scan; the backward scan runs over mirrored positions (SET_TILE - p) and mirrored lanes.
-  uint64_t fwd_in, bwd_in, fwd_all, bwd_all;
+  // ---- for every lane: the last run start and B-part start before its elements (positions
+  // + 1, 0 = none) and the next ones after them (SET_TILE - position, 0 = none)
+  uint32_t fwd_in, bwd_in, fwd_all;
   {
-    const uint32_t head_after0 = (threadIdx.x == 0) ? (head & ~1u) : head;  // position 0 is never "next"
     const uint32_t last_h = head ? run0 + (31 - __builtin_clz(head)) + 1 : 0u;
     const uint32_t last_e2 = e2 ? run0 + (31 - __builtin_clz(e2)) + 1 : 0u;
-    const uint32_t first_h = head_after0 ? SET_TILE - (run0 + __builtin_ctz(head_after0)) : 0u;
+    const uint32_t first_h = head ? SET_TILE - (run0 + __builtin_ctz(head)) : 0u;
     const uint32_t first_e2 = e2 ? SET_TILE - (run0 + __builtin_ctz(e2)) : 0u;
-    fwd_in = set_block_exclusive<SET_WAVES, uint64_t>(((uint64_t)last_h << 32) | last_e2, OpMaxPair{}, (uint64_t)0,
-                                                      s_scan64, &fwd_all);
-    // mirrored lanes: thread t contributes as thread BLOCK - 1 - t
-    s_pair[SET_BLOCK - 1 - threadIdx.x] = ((uint64_t)first_h << 32) | first_e2;
-    __syncthreads();
-    const uint64_t mirrored = s_pair[threadIdx.x];
-    __syncthreads();  // s_scan64 and s_pair are reused below
-    const uint64_t r = set_block_exclusive<SET_WAVES, uint64_t>(mirrored, OpMaxPair{}, (uint64_t)0, s_scan64, &bwd_all);
-    s_pair[SET_BLOCK - 1 - threadIdx.x] = r;
-    __syncthreads();
-    bwd_in = s_pair[threadIdx.x];
+    set_block_both_ways<SET_WAVES>((last_h << 16) | last_e2, (first_h << 16) | first_e2, s_fwd, s_bwd, fwd_in, bwd_in,
+                                   fwd_all);
   }
-  // the first run of the tile ends where the first later run starts; the last run starts at
-  // the last run start (position 0 is one, so there always is one)
-  const uint32_t first_end = (uint32_t)(bwd_all >> 32) ? SET_TILE - (uint32_t)(bwd_all >> 32) : count;
-  const uint32_t last_start = (uint32_t)(fwd_all >> 32) - 1u;
 
-  // ---- decide every element
-  // backward pass: the number of B elements of the element's run that lie after it (for an
-  // element of A that is the size of the run's B part, because all of them follow it);
-  // two 16-bit counts per register
-  uint32_t b_after[SET_ITEMS / 2];
-  {
-    // mirrored value v = SET_TILE - p, 0 = none  ->  position, `count` when there is none
-    const uint32_t nh = (uint32_t)(bwd_in >> 32), ne = (uint32_t)bwd_in;
-    uint32_t cur_h = nh ? SET_TILE - nh : count;  // next run start after this element
-    uint32_t cur_e = ne ? SET_TILE - ne : count;  // next B-part start after this element
+  // ---- decide every element: lt_a / lt_b, bit o = element o (of A / of B) has a rank inside
+  // its own part of the run that is below the size of the other part.  Positions are
+  // relative to the lane's first element from here on, and signed.
+  const bool need_a = g.op != THRUST_AMD_SET_UNION;  // union keeps every element of A
+  const bool need_b = g.op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE || g.op == THRUST_AMD_SET_UNION;
+  uint32_t lt_a = 0, lt_b = 0;
+  if ((fwd_all >> 16) == 0) {
+    // no run starts inside the tile: the first run covers it, and the thresholds decide
+    auto below = [&](uint32_t thr) -> uint32_t {
+      const uint32_t c = thr > run0 ? (thr - run0 < (uint32_t)SET_ITEMS ? thr - run0 : (uint32_t)SET_ITEMS) : 0u;
+      return (1u << c) - 1u;
+    };
+    lt_a = below(thr_a0);
+    lt_b = below(thr_b0);
+  } else {
+    const uint32_t h_in = fwd_in >> 16, e_in = fwd_in & 0xffffu;
+    const int32_t start = h_in ? (int32_t)h_in - 1 - (int32_t)run0 : first_start - (int32_t)run0;
+    if (need_b) {
+      // an element of B at position p, in a run that starts at s and whose B part starts at m,
+      // has rank p - m and faces m - s elements of A: below exactly when p < 2m - s
+      int32_t s = start;
+      int32_t tb = (e_in != 0 && e_in >= h_in) ? 2 * ((int32_t)e_in - 1 - (int32_t)run0) - s
+                   : (h_in == 0 && first_b_before) ? (int32_t)thr_b0 - (int32_t)run0
+                                                   : 0x10000;  // no B of this run yet: the first one sets it
+      uint32_t acc = 0;
 #pragma unroll
-    for (int o = SET_ITEMS - 1; o >= 0; --o) {
-      const uint32_t nb_run = (cur_e < cur_h) ? cur_h - cur_e : 0u;
-      if (o & 1) b_after[o / 2] = nb_run << 16;
-      else b_after[o / 2] |= nb_run;
-      const uint32_t p = run0 + o;
-      if ((head >> o) & 1u) cur_h = p;
-      if ((e2 >> o) & 1u) cur_e = p;
+      for (int o = 0; o < SET_ITEMS; ++o) {
+        s = set_pick(set_bit_mask(head, o), o, s);
+        tb = set_pick(set_bit_mask(e2, o), 2 * o - s, tb);
+        acc = __builtin_amdgcn_alignbit(acc, (uint32_t)(o - tb), 31);  // shifts the sign in: o < tb
+      }
+      lt_b = __builtin_bitreverse32(acc) >> 16;
+    }
+    if (need_a) {
+      // an element of A at position p has rank p - s and faces all B elements of its run, which
+      // come after it: those in this lane, and after the lane those up to the next run start
+      const uint32_t nh_m = bwd_in >> 16, ne_m = bwd_in & 0xffffu;
+      const uint32_t end_l = run0 + SET_ITEMS < count ? run0 + SET_ITEMS : count;
+      const bool last_is_b = (is_b & live) > (live >> 1);
+      uint32_t nb;
+      if (nh_m) nb = last_is_b ? (SET_TILE - nh_m) - end_l : (ne_m > nh_m ? ne_m - nh_m : 0u);
+      else nb = (last_is_b ? count - end_l : (ne_m ? count - (SET_TILE - ne_m) : 0u)) + tail_b;
+      uint32_t facing[SET_ITEMS];
+      const uint32_t not_head = ~head;
+#pragma unroll
+      for (int o = SET_ITEMS - 1; o >= 0; --o) {
+        facing[o] = nb;
+        nb += (is_b >> o) & 1u;
+        nb &= (uint32_t)set_bit_mask(not_head, o);
+      }
+      int32_t s = start;
+      uint32_t acc = 0;
+#pragma unroll
+      for (int o = 0; o < SET_ITEMS; ++o) {
+        s = set_pick(set_bit_mask(head, o), o, s);
+        acc = __builtin_amdgcn_alignbit(acc, (uint32_t)((o - s) - (int32_t)facing[o]), 31);  // rank < facing
+      }
+      lt_a = __builtin_bitreverse32(acc) >> 16;
     }
   }
-  // what is kept, by side and by "rank inside the own part >= size of the other part"
-  const bool a_ge = g.op != THRUST_AMD_SET_INTERSECTION;                                  // A, rank >= |B part|
-  const bool a_lt = g.op == THRUST_AMD_SET_INTERSECTION || g.op == THRUST_AMD_SET_UNION;  // A, rank <  |B part|
-  const bool b_ge = g.op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE || g.op == THRUST_AMD_SET_UNION;
-  uint32_t keep = 0;
-  {
-    uint32_t cur_h = (uint32_t)(fwd_in >> 32);  // p + 1 of the last run start at or before the element
-    uint32_t cur_e = (uint32_t)fwd_in;          // p + 1 of the last B-part start at or before it
-#pragma unroll
-    for (int o = 0; o < SET_ITEMS; ++o) {
-      const uint32_t p = run0 + o;
-      if ((head >> o) & 1u) cur_h = p + 1;
-      if ((e2 >> o) & 1u) cur_e = p + 1;
-      const bool bo = (is_b >> o) & 1u;
-      // an interior run starts inside the tile (cur_h >= 1); for a B, the run's first B is at or before p
-      const uint32_t n_b = (o & 1) ? (b_after[o / 2] >> 16) : (b_after[o / 2] & 0xffffu);
-      const uint32_t own_start = (bo ? cur_e : cur_h) - 1u;
-      const uint32_t other = bo ? cur_e - cur_h : n_b;
-      const bool ge_local = p - own_start >= other;
-      const bool ge_first = p >= (bo ? thr_b0 : thr_a0);
-      const bool ge_next = p >= (bo ? thr_b1 : thr_a1);
-      const bool ge = (p < first_end) ? ge_first : ((tail_continues && p >= last_start) ? ge_next : ge_local);
-      const bool kp = bo ? (b_ge && ge) : (ge ? a_ge : a_lt);
-      keep |= (uint32_t)kp << o;
-    }
-    keep &= live;
-  }
+  // difference: A at or above; intersection: A below; symmetric difference: A and B at or
+  // above; union: all of A, B at or above
+  const uint32_t keep_a = g.op == THRUST_AMD_SET_INTERSECTION ? lt_a : (need_a ? ~lt_a : ~0u);
+  const uint32_t keep_b = need_b ? ~lt_b : 0u;
+  const uint32_t keep = ((~is_b & keep_a) | (is_b & keep_b)) & live;
 
   // ---- ranks inside the tile, then the tile's place in the output
-  uint32_t tile_cnt = 0;
-  __syncthreads();  // s_scan32 is fresh, but s_keys is about to be overwritten: all merges are done
+  uint32_t tile_cnt_v = 0;
   const uint32_t mine = __builtin_popcount(keep);
-  const uint32_t excl = set_block_exclusive<SET_WAVES, uint32_t>(mine, OpPlus{}, 0u, s_scan32, &tile_cnt);
+  const uint32_t excl = set_block_exclusive<SET_WAVES, uint32_t>(mine, OpPlus{}, 0u, s_scan32, &tile_cnt_v);
+  const uint32_t tile_cnt = (uint32_t)__builtin_amdgcn_readfirstlane((int)tile_cnt_v);
 
   constexpr int W = TileWords<uint64_t>::W;
   uint64_t* my_slot = g.status + (size_t)tile * W;
   if (threadIdx.x < WAVE) {
-    const int lane = threadIdx.x;
     uint64_t before = 0;
     if (tile == 0) {
       if (lane == 0) tile_publish<uint64_t>(my_slot, TS_INCLUSIVE, (uint64_t)tile_cnt);
@@ -391,7 +454,7 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
     }
   }
 
-  // ---- compaction through LDS (the staging area is free: every lane has merged)
+  // ---- compaction through LDS (the staging area is free: every lane has merged, two barriers ago)
   {
     uint32_t r = excl;
 #pragma unroll
@@ -404,32 +467,33 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
     }
   }
   __syncthreads();
-  const uint64_t base = s_base;
+  uint64_t base;
+  {
+    const uint64_t b64 = s_base;
+    base = ((uint64_t)(uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(b64 >> 32)) << 32) |
+           (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)b64);
+  }
+  {
+    T* dst = g.out + base;
 #pragma unroll
-  for (int q = 0; q < SET_ITEMS; ++q) {
-    const uint32_t e = q * SET_BLOCK + threadIdx.x;
-    if (e < tile_cnt) g.out[base + e] = s_keys[e];
+    for (int q = 0; q < SET_ITEMS; ++q) {
+      const uint32_t row = (uint32_t)q * SET_BLOCK + wave * WAVE;
+      if (row + WAVE <= tile_cnt) dst[row + lane] = s_keys[row + lane];
+      else if (row + lane < tile_cnt) dst[row + lane] = s_keys[row + lane];
+    }
   }
   if constexpr (HAS_VALUES) {
     // values: the two sub-ranges are staged like the keys were (A's part, then B's, so a
     // key's staging slot is its value's), then gathered by slot in output order
-    const bool keeps_b = g.op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE || g.op == THRUST_AMD_SET_UNION;
     __syncthreads();  // the compacted keys have been read
-    {
-      V in[SET_ITEMS];
-#pragma unroll
-      for (int q = 0; q < SET_ITEMS; ++q) {
-        const uint32_t e = q * SET_BLOCK + threadIdx.x;
-        in[q] = (e < ca) ? g.va[a0 + e] : (keeps_b && e < count) ? g.vb[b0 + (e - ca)] : V{};
-      }
-#pragma unroll
-      for (int q = 0; q < SET_ITEMS; ++q) s_vals[q * SET_BLOCK + threadIdx.x] = in[q];
-    }
+    set_stage<SET_BLOCK, SET_ITEMS>(g.va + a0, g.vb + b0, ca, count, need_b, wave, lane, s_vals);
     __syncthreads();
+    V* dst = g.vout + base;
 #pragma unroll
     for (int q = 0; q < SET_ITEMS; ++q) {
-      const uint32_t e = q * SET_BLOCK + threadIdx.x;
-      if (e < tile_cnt) g.vout[base + e] = s_vals[s_src[e]];  // s_src[e] < count
+      const uint32_t row = (uint32_t)q * SET_BLOCK + wave * WAVE;
+      if (row + WAVE <= tile_cnt) dst[row + lane] = s_vals[s_src[row + lane]];
+      else if (row + lane < tile_cnt) dst[row + lane] = s_vals[s_src[row + lane]];  // s_src[e] < count
     }
   }
 }

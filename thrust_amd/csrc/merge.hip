@@ -9,10 +9,11 @@
 namespace ta {
 using namespace ::thrust::system::hip::merging;
 
+// The direction is part of the type: a comparison is one instruction in the kernels' inner loops.
+template <bool DESCENDING>
 struct OrderComp {
-  bool descending;
   template <typename T>
-  TA_DEVICE bool operator()(const T& x, const T& y) const { return descending ? (y < x) : (x < y); }
+  TA_DEVICE bool operator()(const T& x, const T& y) const { return DESCENDING ? (y < x) : (x < y); }
 };
 
 template <typename T, typename V, bool HAS_VALUES>
@@ -31,10 +32,13 @@ static int merge_run(void* temp, size_t* temp_bytes, const void* a, uint64_t na,
   if (total == 0) return 0;
   if ((na && !a) || (nb && !b) || !out) return (int)hipErrorInvalidValue;
   if (HAS_VALUES && ((na && !va) || (nb && !vb) || !vout)) return (int)hipErrorInvalidValue;
-  return merge_launch<T, V, HAS_VALUES>(static_cast<uint64_t*>(temp), static_cast<const T*>(a), na,
-                                        static_cast<const T*>(b), nb, static_cast<const V*>(va),
-                                        static_cast<const V*>(vb), static_cast<T*>(out), static_cast<V*>(vout),
-                                        OrderComp{descending != 0}, stream);
+  auto launch = [&](auto comp) {
+    return merge_launch<T, V, HAS_VALUES>(static_cast<uint64_t*>(temp), static_cast<const T*>(a), na,
+                                          static_cast<const T*>(b), nb, static_cast<const V*>(va),
+                                          static_cast<const V*>(vb), static_cast<T*>(out), static_cast<V*>(vout),
+                                          comp, stream);
+  };
+  return descending ? launch(OrderComp<true>{}) : launch(OrderComp<false>{});
 }
 
 }  // namespace ta

@@ -9,10 +9,11 @@
 namespace ta {
 using namespace ::thrust::system::hip::setops;
 
+// The direction is part of the type: a comparison is one instruction in the kernels' inner loops.
+template <bool DESCENDING>
 struct SetOrder {
-  bool descending;
   template <typename T>
-  TA_DEVICE bool operator()(const T& x, const T& y) const { return descending ? (y < x) : (x < y); }
+  TA_DEVICE bool operator()(const T& x, const T& y) const { return DESCENDING ? (y < x) : (x < y); }
 };
 
 template <typename T, typename V, bool HAS_VALUES>
@@ -32,10 +33,13 @@ static int set_run(void* temp, size_t* temp_bytes, int op, const void* a, uint64
   const bool keeps_b = op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE || op == THRUST_AMD_SET_UNION;
   if (HAS_VALUES && ((na && !va) || (nb && keeps_b && !vb) || (total && !vout)))
     return (int)hipErrorInvalidValue;
-  return set_launch<T, V, HAS_VALUES>(static_cast<char*>(temp), op, static_cast<const T*>(a), na,
-                                      static_cast<const T*>(b), nb, static_cast<const V*>(va),
-                                      static_cast<const V*>(vb), static_cast<T*>(out), static_cast<V*>(vout), d_num,
-                                      SetOrder{descending != 0}, stream);
+  auto launch = [&](auto comp) {
+    return set_launch<T, V, HAS_VALUES>(static_cast<char*>(temp), op, static_cast<const T*>(a), na,
+                                        static_cast<const T*>(b), nb, static_cast<const V*>(va),
+                                        static_cast<const V*>(vb), static_cast<T*>(out), static_cast<V*>(vout), d_num,
+                                        comp, stream);
+  };
+  return descending ? launch(SetOrder<true>{}) : launch(SetOrder<false>{});
 }
 
 inline bool valid_set_op(int op) { return op >= 0 && op < THRUST_AMD_SET_OP_COUNT; }
