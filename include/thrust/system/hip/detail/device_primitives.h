@@ -235,6 +235,64 @@ THRUST_AMD_DEVICE uint64_t aligned_partition_point(uint64_t lo, uint64_t hi, Pre
   return lo;
 }
 
+// ------------------------------------------------------------------ merging inside a tile
+// A tile of a merge holds two sorted parts side by side in LDS: s[0, ca) from the first range and
+// s[ca, count) from the second.  (The set operations use these; the merge and merge sort kernels
+// keep their own predicated staging, which measured faster for them with 8-byte keys and values.)
+
+// Stages the tile: element e of the tile is pa[e] for e < ca and pb[e - ca] after that; thread t
+// loads the elements t, t + BLOCK, ...  Slots from `count` up to BLOCK * ITEMS receive a copy of
+// the tile's last element (count >= 1), so that every slot holds a value of the input.
+// One select of the base address and one 64-bit add per element.
+template <int BLOCK, int ITEMS, typename E>
+THRUST_AMD_DEVICE void stage_two_parts(const E* __restrict__ pa, const E* __restrict__ pb, uint32_t ca, uint32_t count,
+                                       E* s) {
+  // (the arithmetic stays on pointers so that the loads are known to go to global memory)
+  const E* const base_b = pb - ca;  // only indexed from ca on
+  E in[ITEMS];
+#pragma unroll
+  for (int q = 0; q < ITEMS; ++q) {
+    uint32_t e = (uint32_t)q * BLOCK + threadIdx.x;
+    e = e < count ? e : count - 1;
+    in[q] = (e < ca ? pa : base_b)[e];
+  }
+#pragma unroll
+  for (int q = 0; q < ITEMS; ++q) s[(uint32_t)q * BLOCK + threadIdx.x] = in[q];
+}
+
+// Number of elements of the first part among the first `diag` elements of the merged order
+// (an element of the second part is taken only when it is before the first part's: ties go to the first).
+template <typename T, typename Comp>
+THRUST_AMD_DEVICE uint32_t merge_path_in_tile(const T* s, uint32_t ca, uint32_t count, uint32_t diag, Comp& comp) {
+  const uint32_t cb = count - ca;
+  uint32_t lo = diag > cb ? diag - cb : 0u, hi = diag < ca ? diag : ca;
+  while (lo < hi) {
+    const uint32_t mid = (lo + hi) >> 1;
+    if (!comp(s[ca + diag - 1 - mid], s[mid])) lo = mid + 1;
+    else hi = mid;
+  }
+  return lo;
+}
+
+// ITEMS steps of the merge from slot i of the first part and slot j of the second (i + j - ca elements
+// are already merged).  emit(o, element, slot, from_second) receives the steps in order.  The
+// comparator only sees elements of the parts (candidates past their ends are not compared); slots
+// read stay at or below count + ITEMS.
+template <int ITEMS, typename T, typename Comp, typename Emit>
+THRUST_AMD_DEVICE void merge_steps(const T* s, uint32_t i, uint32_t j, uint32_t ca, uint32_t count, Comp& comp,
+                                   Emit emit) {
+  T ka = s[i], kb = s[j];
+#pragma unroll
+  for (int o = 0; o < ITEMS; ++o) {
+    const bool take_b = (j < count) && (i >= ca || comp(kb, ka));
+    emit(o, take_b ? kb : ka, take_b ? j : i, take_b);
+    const uint32_t next = take_b ? ++j : ++i;
+    const T nk = s[next];
+    if (take_b) kb = nk;
+    else ka = nk;
+  }
+}
+
 // ------------------------------------------------------------------ tile status
 // A tile publishes W 32-bit payload words, each inside its own 64-bit word together
 // with the status, using relaxed agent-scope atomics.  A reader accepts a descriptor

@@ -194,29 +194,6 @@ struct SetArgs {
   Comp comp;
 };
 
-// Reads the tile's `ca` elements at pa and `count - ca` elements at pb into LDS, A's part first.
-// A wave's 64 consecutive elements of one round nearly always lie in one range: then the
-// address is the wave's base plus the lane, with nothing to select.
-template <int BLOCK, int ITEMS, typename E>
-THRUST_AMD_DEVICE void set_stage(const E* __restrict__ pa, const E* __restrict__ pb, uint32_t ca, uint32_t count,
-                                 bool with_b, uint32_t wave, uint32_t lane, E* s_items) {
-  E in[ITEMS];
-#pragma unroll
-  for (int q = 0; q < ITEMS; ++q) {
-    const uint32_t row = (uint32_t)q * BLOCK + wave * WAVE;  // the same for the whole wave
-    if (row + WAVE <= ca) {
-      in[q] = pa[row + lane];
-    } else if (with_b && row >= ca && row + WAVE <= count) {
-      in[q] = pb[(row - ca) + lane];
-    } else {
-      const uint32_t e = row + lane;
-      in[q] = (e < ca) ? pa[e] : (with_b && e < count) ? pb[e - ca] : E{};
-    }
-  }
-#pragma unroll
-  for (int q = 0; q < ITEMS; ++q) s_items[(uint32_t)q * BLOCK + wave * WAVE + lane] = in[q];
-}
-
 template <typename T, typename V, bool HAS_VALUES, typename Comp>
 __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V, HAS_VALUES>::WAVES_PER_SIMD)) void set_op_kernel(SetArgs<T, V, HAS_VALUES, Comp> g) {
   using Shape = SetShape<T, V, HAS_VALUES>;
@@ -225,7 +202,8 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
   constexpr int SET_WAVES = SET_BLOCK / WAVE;
   static_assert(SET_TILE <= 0x7fff && SET_ITEMS == 16, "positions travel in 16 bits, flags in 16-bit masks");
   // one buffer for the staged keys, the compacted keys and (later) the staged values
-  __shared__ __attribute__((aligned(16))) unsigned char s_raw[(size_t)(SET_TILE + 1) * Shape::ITEM];
+  // (lanes past the end of a short tile read up to SET_ITEMS slots past it)
+  __shared__ __attribute__((aligned(16))) unsigned char s_raw[(size_t)(SET_TILE + SET_ITEMS) * Shape::ITEM];
   T* s_keys = reinterpret_cast<T*>(s_raw);
   V* s_vals = reinterpret_cast<V*>(s_raw);
   __shared__ uint16_t s_src[HAS_VALUES ? SET_TILE : 1];
@@ -275,24 +253,14 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
   }
 
   // ---- stage the keys: A's part first, then B's
-  set_stage<SET_BLOCK, SET_ITEMS>(g.a + a0, g.b + b0, ca, count, true, wave, lane, s_keys);
-  if (threadIdx.x == 0) s_keys[SET_TILE] = T{};
+  stage_two_parts<SET_BLOCK, SET_ITEMS>(g.a + a0, g.b + b0, ca, count, s_keys);
   __syncthreads();
 
   // ---- this lane's start on the path, then a serial merge of ITEMS elements
   const uint32_t run0 = threadIdx.x * SET_ITEMS;
   const uint32_t diag = run0 < count ? run0 : count;
-  uint32_t i;
-  {
-    uint32_t lo = diag > cb ? diag - cb : 0u, hi = diag < ca ? diag : ca;
-    while (lo < hi) {
-      const uint32_t mid = (lo + hi) >> 1;
-      if (!comp(s_keys[ca + diag - 1 - mid], s_keys[mid])) lo = mid + 1;
-      else hi = mid;
-    }
-    i = lo;
-  }
-  uint32_t j = ca + (diag - i);
+  const uint32_t i = merge_path_in_tile(s_keys, ca, count, diag, comp);
+  const uint32_t j = ca + (diag - i);
   // the element before this lane's first one is the later of the two last ones taken so far (B after A on ties)
   bool prev_is_b;
   T prev_key;
@@ -305,21 +273,11 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
   T k[SET_ITEMS];
   uint32_t slot[SET_ITEMS];
   uint32_t is_b = 0;  // bit o: merged element o of this lane comes from B
-  {
-    T ka = s_keys[i];
-    T kb = s_keys[j];
-#pragma unroll
-    for (int o = 0; o < SET_ITEMS; ++o) {
-      const bool take_b = (j < count) && (i >= ca || comp(kb, ka));
-      k[o] = take_b ? kb : ka;
-      slot[o] = take_b ? j : i;
-      is_b |= (uint32_t)take_b << o;
-      const uint32_t next = take_b ? ++j : ++i;
-      const T nk = s_keys[next];  // next <= count <= SET_TILE
-      if (take_b) kb = nk;
-      else ka = nk;
-    }
-  }
+  merge_steps<SET_ITEMS>(s_keys, i, j, ca, count, comp, [&](int o, const T& x, uint32_t from, bool take_b) {
+    k[o] = x;
+    slot[o] = from;
+    is_b |= (uint32_t)take_b << o;
+  });
   // valid elements of this lane: merged positions run0 + o < count
   const uint32_t live = (run0 >= count) ? 0u : ((count - run0 >= (uint32_t)SET_ITEMS) ? 0xffffu : ((1u << (count - run0)) - 1u));
 
@@ -486,7 +444,9 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
     // values: the two sub-ranges are staged like the keys were (A's part, then B's, so a
     // key's staging slot is its value's), then gathered by slot in output order
     __syncthreads();  // the compacted keys have been read
-    set_stage<SET_BLOCK, SET_ITEMS>(g.va + a0, g.vb + b0, ca, count, need_b, wave, lane, s_vals);
+    // (B's values are only read by the operations that can keep an element of B)
+    if (need_b) stage_two_parts<SET_BLOCK, SET_ITEMS>(g.va + a0, g.vb + b0, ca, count, s_vals);
+    else if (ca) stage_two_parts<SET_BLOCK, SET_ITEMS>(g.va + a0, g.va + a0, ca, ca, s_vals);
     __syncthreads();
     V* dst = g.vout + base;
 #pragma unroll
