@@ -52,7 +52,7 @@ struct SetShape {
   static constexpr int TILE = BLOCK * SET_ITEMS;
   // waves per SIMD the register allocation aims at: the merge of 8-byte items does not fit
   // the 128 registers that four would leave
-  static constexpr int WAVES_PER_SIMD = ITEM > 4 ? 3 : 4;
+  static constexpr int WAVES_PER_SIMD = ITEM > 4 ? 3 : (HAS_VALUES ? 4 : 8);
 };
 
 // Per tile boundary t (t = 0 .. tiles), found by one thread: split[t] = elements of A before
