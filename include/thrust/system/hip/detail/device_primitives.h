@@ -235,6 +235,48 @@ THRUST_AMD_DEVICE uint64_t aligned_partition_point(uint64_t lo, uint64_t hi, Pre
   return lo;
 }
 
+// The same partition point, for a caller that knows an index `from` (lo <= from <= hi) near it: steps of
+// doubling length away from `from` bracket the point, a bisection inside the bracket finds it.  The
+// number of probes grows with the logarithm of the distance, not of the range.
+template <typename Pred>
+THRUST_AMD_DEVICE uint64_t nearby_partition_point(uint64_t lo, uint64_t hi, uint64_t from, Pred pred) {
+  from = from < lo ? lo : (from > hi ? hi : from);
+  uint64_t l, r;
+  if (from < hi && pred(from)) {  // the point lies after `from`
+    l = from + 1;
+    r = hi;
+    for (uint64_t step = 1;; step <<= 1) {
+      if (hi - l < step) break;  // the probe would be hi or later
+      const uint64_t probe = l + step - 1;
+      if (pred(probe)) {
+        l = probe + 1;
+      } else {
+        r = probe;
+        break;
+      }
+    }
+  } else {  // the point lies at or before `from`
+    l = lo;
+    r = from;
+    for (uint64_t step = 1;; step <<= 1) {
+      if (r - lo < step) break;  // the probe would lie before lo
+      const uint64_t probe = r - step;
+      if (!pred(probe)) {
+        r = probe;
+      } else {
+        l = probe + 1;
+        break;
+      }
+    }
+  }
+  while (l < r) {
+    const uint64_t mid = l + ((r - l) >> 1);
+    if (pred(mid)) l = mid + 1;
+    else r = mid;
+  }
+  return l;
+}
+
 // ------------------------------------------------------------------ merging inside a tile
 // A tile of a merge holds two sorted parts side by side in LDS: s[0, ca) from the first range and
 // s[ca, count) from the second.  (The set operations use these; the merge and merge sort kernels

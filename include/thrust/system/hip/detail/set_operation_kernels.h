@@ -16,16 +16,22 @@
 // the run starts, where its B part starts and where it ends.
 //
 //   partition  one thread per tile boundary: the merge-path split, and the three
-//              positions (by binary search over the whole ranges) of the run that
+//              positions (searched outward from the split) of the run that
 //              contains the first element of the tile -- the only run of a tile that can
 //              start before it, and, read from the next boundary, the only one that can
 //              end after it
 //   tile       stages its two sub-ranges in LDS and merges them serially per lane as
-//              the merge kernel does; head flags on the merged order and two workgroup scans
-//              (last / next run start and B-part start) give the three positions of
-//              every interior run; keep flags -> ranks -> decoupled look-back over the
-//              tiles' counts (dynamic tickets) -> compaction through LDS -> coalesced
-//              stores; values are gathered from the range their key came from
+//              the merge kernel does; head flags on the merged order (a lane's predecessor
+//              key is the later of the two elements before its merge-path split); the last run
+//              start and B-part start before every lane, and the next ones after it, travel
+//              as pairs of 16-bit positions through one forward and one backward max-scan
+//              behind a single barrier; each lane then walks its 16 elements once per side
+//              that the operation can keep (A: rank against the B elements that follow in
+//              the run; B: position against a threshold fixed where the B part starts), in
+//              lane-relative positions, collecting the outcomes as sign bits; keep flags ->
+//              ranks -> decoupled look-back over the tiles' counts (dynamic tickets) ->
+//              compaction through LDS -> coalesced stores; values are gathered from the
+//              range their key came from
 //
 // Equivalent keys need not be identical (-0.0 and +0.0 under operator<), the copy that is kept is the one the rule above names.
 // HBM traffic: (na + nb) keys read, the result written, values read only where kept.
@@ -81,11 +87,12 @@ __global__ __launch_bounds__(256) void set_partition_kernel(const T* __restrict_
   T x;
   if (as < na && (bs >= nb || !comp(b[bs], a[as]))) x = a[as];
   else x = b[bs];
-  // first index whose element is not before x / is after x, in each range
-  const uint64_t lb_a = aligned_partition_point(0, na, [&](uint64_t i) { return comp(a[i], x); });
-  const uint64_t ub_a = aligned_partition_point(lb_a, na, [&](uint64_t i) { return !comp(x, a[i]); });
-  const uint64_t lb_b = aligned_partition_point(0, nb, [&](uint64_t i) { return comp(b[i], x); });
-  const uint64_t ub_b = aligned_partition_point(lb_b, nb, [&](uint64_t i) { return !comp(x, b[i]); });
+  // first index whose element is not before x / is after x, in each range: the run of x lies
+  // around the split, a few elements long unless the input repeats itself
+  const uint64_t lb_a = nearby_partition_point(0, na, as, [&](uint64_t i) { return comp(a[i], x); });
+  const uint64_t ub_a = nearby_partition_point(lb_a, na, as, [&](uint64_t i) { return !comp(x, a[i]); });
+  const uint64_t lb_b = nearby_partition_point(0, nb, bs, [&](uint64_t i) { return comp(b[i], x); });
+  const uint64_t ub_b = nearby_partition_point(lb_b, nb, bs, [&](uint64_t i) { return !comp(x, b[i]); });
   key[t] = x;
   run[3 * t + 0] = lb_a + lb_b;
   run[3 * t + 1] = ub_a + lb_b;
