@@ -108,6 +108,50 @@ def test_set_operation_by_key(dev, oracle, op, vdtype):
         assert cnt == rk.size and np.array_equal(ko.numpy()[:cnt], rk) and np.array_equal(vo.numpy()[:cnt], rv), (op, na, nb)
 
 
+def _origin_values(na, nb, vdtype=np.uint32):
+    """Values that name their origin: the index, plus the top bit for the second range."""
+    top = np.uint64(1) << np.uint64(8 * np.dtype(vdtype).itemsize - 1)
+    va = (np.arange(na, dtype=np.uint64) % top).astype(vdtype)
+    vb = ((np.arange(nb, dtype=np.uint64) % top) + top).astype(vdtype)
+    return va, vb
+
+
+@pytest.mark.parametrize("op", OPS)
+def test_set_operation_by_key_long_runs_name_the_surviving_copies(dev, oracle, op):
+    """Runs longer than a tile, starting before a tile and ending after it, in A, in B and in both:
+    the values tell which copies of the equal keys were kept."""
+    shapes = [
+        (np.zeros(20000, np.int32), np.zeros(9000, np.int32)),
+        (np.zeros(9000, np.int32), np.zeros(20000, np.int32)),
+        (np.repeat(np.arange(3, dtype=np.int32), [5000, 1, 7000]), np.repeat(np.arange(1, 4, dtype=np.int32), [3000, 6000, 2])),
+        (np.r_[np.zeros(8192, np.int32), np.ones(100, np.int32)], np.r_[np.ones(8192, np.int32), np.full(3, 2, np.int32)]),
+        (np.repeat(np.arange(3, dtype=np.int32), [30000, 1, 17000]), np.repeat(np.arange(1, 4, dtype=np.int32), [9000, 26000, 2])),
+        (np.repeat(np.arange(6, dtype=np.int32), [8190, 3, 8192, 1, 16384, 5]), np.repeat(np.arange(6, dtype=np.int32), [2, 8191, 1, 8192, 7, 16390])),
+        (np.repeat(np.arange(700, dtype=np.int32), 13), np.repeat(np.arange(700, dtype=np.int32), 17)),
+    ]
+    for ka, kb in shapes:
+        va, vb = _origin_values(ka.size, kb.size)
+        ko, vo, cnt = dev.set_operation_by_key(op, dev.DeviceArray.from_numpy(ka), dev.DeviceArray.from_numpy(kb),
+                                               dev.DeviceArray.from_numpy(va), dev.DeviceArray.from_numpy(vb))
+        rk, rv = oracle.set_operation_by_key(op, ka, kb, va, vb)
+        assert cnt == rk.size and np.array_equal(ko.numpy()[:cnt], rk) and np.array_equal(vo.numpy()[:cnt], rv), (op, ka.size, kb.size)
+
+
+@pytest.mark.parametrize("kdtype", [np.uint64, np.float64, np.int16, np.uint8])
+@pytest.mark.parametrize("op", OPS)
+def test_set_operation_by_key_other_key_widths_and_descending(dev, oracle, op, kdtype):
+    """8-byte keys take the 256-thread tile, 1- and 2-byte keys repeat themselves by the thousand."""
+    for na, nb, descending in [(5, 7, False), (4096, 4097, False), (40000, 23456, True), (1 << 16, (1 << 16) + 3, False)]:
+        spread = 1 if np.dtype(kdtype).itemsize == 1 else 3
+        ka, kb = _sorted(na, kdtype, 77, spread, descending), _sorted(nb, kdtype, 78, spread, descending)
+        va, vb = _origin_values(na, nb)
+        ko, vo, cnt = dev.set_operation_by_key(op, dev.DeviceArray.from_numpy(ka), dev.DeviceArray.from_numpy(kb),
+                                               dev.DeviceArray.from_numpy(va), dev.DeviceArray.from_numpy(vb),
+                                               descending=descending)
+        rk, rv = oracle.set_operation_by_key(op, ka, kb, va, vb, descending)
+        assert cnt == rk.size and np.array_equal(ko.numpy()[:cnt], rk) and np.array_equal(vo.numpy()[:cnt], rv), (op, kdtype, na, nb)
+
+
 def test_set_operation_signed_zero_keeps_the_copy_of_the_named_side(dev, oracle):
     """-0.0 and +0.0 are equivalent keys with different bits: the kept copy is the one the
     reference's loop emits."""
