@@ -308,12 +308,23 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   const int nbits = (geo.end_bit - shift) < RADIX_BITS ? (geo.end_bit - shift) : RADIX_BITS;
   const uint32_t dmask = (1u << nbits) - 1u;
 
-  // ---- load (wave-striped) and encode; slots past the end sort last inside the tile
+  // Keys travel between the passes in their encoded form: the first pass that runs encodes them as
+  // it loads, the last one decodes them as it stores (unsigned ascending keys need no transform).
+  bool encodes = false, decodes = false;  // uniform
+  if (!codec.plain) {
+    encodes = decodes = true;
+    for (int p = 0; p < pass; ++p)
+      if (!ctl->skip[p]) encodes = false;
+    for (int p = pass + 1; p < geo.passes; ++p)
+      if (!ctl->skip[p]) decodes = false;
+  }
+
+  // ---- load (wave-striped); slots past the end sort last inside the tile
   K e[ITEMS];
   if (valid == (uint32_t)TILE) {
 #pragma unroll
     for (int r = 0; r < ITEMS; ++r) e[r] = keys_in[tile_base + span + r * WAVE];
-    if (!codec.plain) {  // uniform branch: unsigned ascending keys need no transform
+    if (encodes) {
 #pragma unroll
       for (int r = 0; r < ITEMS; ++r) e[r] = codec.encode(e[r]);
     }
@@ -321,7 +332,12 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
 #pragma unroll
     for (int r = 0; r < ITEMS; ++r) {
       const uint32_t pos = span + r * WAVE;
-      e[r] = (pos < valid) ? codec.encode(keys_in[tile_base + pos]) : (K)~(K)0;
+      K x = (K)~(K)0;
+      if (pos < valid) {
+        x = keys_in[tile_base + pos];
+        if (encodes) x = codec.encode(x);
+      }
+      e[r] = x;
     }
   }
 
@@ -483,7 +499,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k)
       gpos[k] = s_scatter_base[(uint32_t)(ek[k] >> shift) & dmask] + (uint32_t)k * BLOCK + threadIdx.x;
-    if (!codec.plain) {
+    if (decodes) {
 #pragma unroll
       for (int k = 0; k < ITEMS; ++k) ek[k] = codec.decode(ek[k]);
     }
