@@ -84,3 +84,11 @@ def test_placeholder_expressions_as_functors():
     # thrust::transform on both systems, and as predicates / operators of count_if, copy_if, partition, reduce, inner_product
     out = _run("test_placeholders")
     assert "PASSED" in out
+
+
+def test_searches_and_extrema():
+    # min_element / max_element / minmax_element (first of equivalent extremes), find / find_if / find_if_not,
+    # all_of / any_of / none_of, mismatch and equal: the reference's literal vectors on both systems, then the device
+    # system against the host system over the size list
+    out = _run("test_searches_and_extrema")
+    assert "PASSED" in out
