@@ -1,0 +1,81 @@
+// thrust::adjacent_difference: result[0] = x[0], result[i] = x[i] - x[i-1] (or op(x[i], x[i-1]));
+// the output may be the input (thrust/system/detail/generic/adjacent_difference.inl:35-78,
+// thrust/system/cuda/detail/adjacent_difference.h; testing/adjacent_difference.cu).  On the device
+// system: one binary transform over the range and itself shifted by one, from a copy of the input
+// when the output is the input.
+#pragma once
+#include <cstddef>
+
+#include <thrust/copy.h>
+#include <thrust/device_vector.h>
+#include <thrust/functional.h>
+#include <thrust/host_vector.h>
+#include <thrust/transform.h>
+
+namespace thrust {
+
+template <typename D, typename In, typename Out, typename Op>
+Out adjacent_difference(const detail::execution_policy_base<D>& exec, In first, In last, Out result, Op op);
+
+namespace system {
+namespace cpp {
+template <typename D, typename In, typename Out, typename Op>
+Out adjacent_difference(execution_policy<D>&, In first, In last, Out result, Op op) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  if (first == last) return result;
+  V previous = *first;
+  *result = previous;
+  for (++first, ++result; first != last; ++first, ++result) {
+    const V current = *first;  // read before the write: the output may be the input
+    *result = op(current, previous);
+    previous = current;
+  }
+  return result;
+}
+}  // namespace cpp
+
+namespace hip {
+namespace detail {
+template <typename A, typename B>
+inline bool same_position(const A&, const B&) { return false; }
+template <typename A>
+inline bool same_position(const A& a, const A& b) { return a == b; }
+}  // namespace detail
+
+template <typename D, typename In, typename Out, typename Op>
+Out adjacent_difference(execution_policy<D>& exec, In first, In last, Out result, Op op) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  const std::ptrdiff_t n = last - first;
+  if (n == 0) return result;
+  if (detail::same_position(first, result)) {
+    thrust::device_vector<V> input(first, last);
+    thrust::transform(exec, input.begin() + 1, input.end(), input.begin(), result + 1, op);
+    return result + n;  // result[0] already is x[0]
+  }
+  thrust::copy(exec, first, first + 1, result);
+  thrust::transform(exec, first + 1, last, first, result + 1, op);
+  return result + n;
+}
+}  // namespace hip
+}  // namespace system
+
+template <typename D, typename In, typename Out, typename Op>
+Out adjacent_difference(const detail::execution_policy_base<D>& exec, In first, In last, Out result, Op op) {
+  return adjacent_difference(detail::derived_cast(detail::strip_const(exec)), first, last, result, op);
+}
+template <typename D, typename In, typename Out>
+Out adjacent_difference(const detail::execution_policy_base<D>& exec, In first, In last, Out result) {
+  typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
+  return thrust::adjacent_difference(exec, first, last, result, thrust::minus<V>());
+}
+template <typename In, typename Out, typename Op,
+          typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>
+Out adjacent_difference(In first, In last, Out result, Op op) {
+  return thrust::adjacent_difference(detail::policy_for<Out>(), first, last, result, op);
+}
+template <typename In, typename Out>
+Out adjacent_difference(In first, In last, Out result) {
+  return thrust::adjacent_difference(detail::policy_for<Out>(), first, last, result);
+}
+
+}  // namespace thrust

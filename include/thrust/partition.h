@@ -10,6 +10,7 @@
 #include <vector>
 
 #include <thrust/copy.h>
+#include <thrust/logical.h>
 #include <thrust/pair.h>
 
 namespace thrust {
@@ -275,5 +276,28 @@ THRUST_AMD_PARTITION_ENTRY(stable_partition)
 THRUST_AMD_PARTITION_COPY_ENTRY(partition_copy)
 THRUST_AMD_PARTITION_COPY_ENTRY(stable_partition_copy)
 #undef THRUST_AMD_PARTITION_COPY_ENTRY
+
+// ------------------------------------------------------------------ is_partitioned, partition_point
+// partition_point: the end of the leading elements that satisfy the predicate, for a range that is
+// partitioned by it; is_partitioned: no element after that point satisfies it
+// (thrust/system/detail/generic/partition.inl:163-214; testing/partition_point.cu, is_partitioned.cu).
+template <typename D, typename It, typename Pred>
+It partition_point(const detail::execution_policy_base<D>& exec, It first, It last, Pred pred) {
+  return thrust::find_if_not(exec, first, last, pred);
+}
+template <typename It, typename Pred, typename = typename std::enable_if<!detail::is_execution_policy<It>::value>::type>
+It partition_point(It first, It last, Pred pred) {
+  return thrust::partition_point(detail::policy_for<It>(), first, last, pred);
+}
+template <typename D, typename It, typename Pred>
+bool is_partitioned(const detail::execution_policy_base<D>& exec, It first, It last, Pred pred) {
+  const It mid = thrust::find_if_not(exec, first, last, pred);
+  if (mid == last) return true;
+  return thrust::none_of(exec, mid + 1, last, pred);
+}
+template <typename It, typename Pred, typename = typename std::enable_if<!detail::is_execution_policy<It>::value>::type>
+bool is_partitioned(It first, It last, Pred pred) {
+  return thrust::is_partitioned(detail::policy_for<It>(), first, last, pred);
+}
 
 }  // namespace thrust

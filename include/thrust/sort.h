@@ -17,7 +17,10 @@
 #include <tuple>
 #include <vector>
 
+#include <thrust/find.h>
 #include <thrust/functional.h>
+#include <thrust/iterator/zip_iterator.h>
+#include <thrust/tuple.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/device_input.h>
 #include <thrust/iterator/counting_iterator.h>
@@ -386,5 +389,56 @@ THRUST_AMD_SORT_ENTRY(stable_sort)
 THRUST_AMD_SORT_BY_KEY_ENTRY(sort_by_key)
 THRUST_AMD_SORT_BY_KEY_ENTRY(stable_sort_by_key)
 #undef THRUST_AMD_SORT_BY_KEY_ENTRY
+
+// ------------------------------------------------------------------ is_sorted, is_sorted_until
+// is_sorted_until: the end of the longest sorted prefix, i.e. the first position whose element is
+// before its predecessor, `last` if there is none (thrust/system/detail/generic/sort.inl:155-196: a
+// find over the range zipped with itself shifted by one; testing/is_sorted_until.cu, is_sorted.cu).
+namespace detail {
+template <typename Comp>
+struct out_of_order {
+  mutable Comp comp;  // a caller's comparison need not be const-callable
+  template <typename Tuple>
+  __host__ __device__ bool operator()(const Tuple& t) const { return comp(thrust::get<1>(t), thrust::get<0>(t)); }
+};
+}  // namespace detail
+
+template <typename D, typename It, typename Comp>
+It is_sorted_until(const detail::execution_policy_base<D>& exec, It first, It last, Comp comp) {
+  const std::ptrdiff_t n = last - first;
+  if (n < 2) return last;
+  auto pairs = thrust::make_zip_iterator(thrust::make_tuple(first, first + 1));
+  const detail::out_of_order<Comp> breaks = {comp};
+  return first + ((thrust::find_if(exec, pairs, pairs + (n - 1), breaks) - pairs) + 1);
+}
+template <typename D, typename It>
+It is_sorted_until(const detail::execution_policy_base<D>& exec, It first, It last) {
+  typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
+  return thrust::is_sorted_until(exec, first, last, thrust::less<V>());
+}
+template <typename It, typename Comp, typename = typename std::enable_if<!detail::is_execution_policy<It>::value>::type>
+It is_sorted_until(It first, It last, Comp comp) {
+  return thrust::is_sorted_until(detail::policy_for<It>(), first, last, comp);
+}
+template <typename It>
+It is_sorted_until(It first, It last) {
+  return thrust::is_sorted_until(detail::policy_for<It>(), first, last);
+}
+template <typename D, typename It, typename Comp>
+bool is_sorted(const detail::execution_policy_base<D>& exec, It first, It last, Comp comp) {
+  return thrust::is_sorted_until(exec, first, last, comp) == last;
+}
+template <typename D, typename It>
+bool is_sorted(const detail::execution_policy_base<D>& exec, It first, It last) {
+  return thrust::is_sorted_until(exec, first, last) == last;
+}
+template <typename It, typename Comp, typename = typename std::enable_if<!detail::is_execution_policy<It>::value>::type>
+bool is_sorted(It first, It last, Comp comp) {
+  return thrust::is_sorted(detail::policy_for<It>(), first, last, comp);
+}
+template <typename It>
+bool is_sorted(It first, It last) {
+  return thrust::is_sorted(detail::policy_for<It>(), first, last);
+}
 
 }  // namespace thrust

@@ -92,3 +92,11 @@ def test_searches_and_extrema():
     # system against the host system over the size list
     out = _run("test_searches_and_extrema")
     assert "PASSED" in out
+
+
+def test_elementwise_callers_and_order_checks():
+    # is_sorted / is_sorted_until, is_partitioned / partition_point, adjacent_difference (also in place), the replace
+    # family with and without stencils, generate(_n), tabulate, reverse(_copy), swap_ranges, uninitialized_fill / _copy:
+    # the reference's literal vectors on both systems, then the device system against the host system
+    out = _run("test_elementwise_callers")
+    assert "PASSED" in out
