@@ -100,3 +100,10 @@ def test_elementwise_callers_and_order_checks():
     # the reference's literal vectors on both systems, then the device system against the host system
     out = _run("test_elementwise_callers")
     assert "PASSED" in out
+
+
+def test_binary_searches():
+    # lower_bound / upper_bound / binary_search / equal_range for one value and for ranges of values, ascending and
+    # under thrust::greater: the reference's literal vectors on both systems, then device against host on sorted inputs
+    out = _run("test_binary_search")
+    assert "PASSED" in out
