@@ -9,6 +9,7 @@
 #pragma once
 #include <thrust/iterator/detail/fancy_iterator_base.h>
 #include <thrust/iterator/permutation_iterator.h>
+#include <thrust/iterator/reverse_iterator.h>
 #include <thrust/iterator/zip_iterator.h>
 #include <thrust/system/hip/detail/backend.h>
 #if defined(__HIPCC__)
@@ -43,6 +44,10 @@ struct is_device_output<thrust::zip_iterator<thrust::tuple<H, T...> > >
 template <typename E, typename I>
 struct is_device_output<thrust::permutation_iterator<E, I> >
     : std::integral_constant<bool, is_device_output<E>::value && is_device_input<I>::value> {};
+
+// a range of something writable, walked backwards
+template <typename It>
+struct is_device_output<thrust::reverse_iterator<It> > : is_device_output<It> {};
 
 template <typename It>
 struct fancy_needs_hipcc : std::false_type {};

@@ -11,6 +11,8 @@
 #include <thrust/iterator/counting_iterator.h>
 #include <thrust/iterator/permutation_iterator.h>
 #include <thrust/iterator/transform_iterator.h>
+#include <thrust/iterator/zip_iterator.h>
+#include <thrust/tuple.h>
 #include <thrust/system/hip/detail/device_input.h>
 
 namespace thrust {
@@ -242,6 +244,139 @@ void scatter(const detail::execution_policy_base<D>& exec, In first, In last, Ma
 template <typename In, typename MapIt, typename Out>
 void scatter(In first, In last, MapIt map, Out output) {
   thrust::scatter(detail::policy_for<Out>(), first, last, map, output);
+}
+
+// ------------------------------------------------------------------ the conditional forms
+// transform_if, gather_if, scatter_if write an element only where the predicate holds for the input
+// element (transform_if without a stencil) or for the stencil; for_each_n is for_each over a count
+// (thrust/system/detail/generic/transform.inl:79-190, gather.inl:60-105, scatter.inl:48-96,
+// for_each.h; testing/transform.cu, gather.cu, scatter.cu, for_each.cu).  All of them are one
+// for_each over the zipped ranges, so they run on either system.
+namespace detail {
+template <typename Op, typename Pred>
+struct writes_if {
+  mutable Op op;  // a caller's functors need not be const-callable
+  mutable Pred pred;
+  // (input, output): the input decides
+  template <typename A, typename O>
+  __host__ __device__ void operator()(thrust::tuple<A, O> t) const {
+    if (pred(thrust::get<0>(t))) thrust::get<1>(t) = op(thrust::get<0>(t));
+  }
+  // (input, stencil, output)
+  template <typename A, typename S, typename O>
+  __host__ __device__ void operator()(thrust::tuple<A, S, O> t) const {
+    if (pred(thrust::get<1>(t))) thrust::get<2>(t) = op(thrust::get<0>(t));
+  }
+  // (input 1, input 2, stencil, output)
+  template <typename A, typename B, typename S, typename O>
+  __host__ __device__ void operator()(thrust::tuple<A, B, S, O> t) const {
+    if (pred(thrust::get<2>(t))) thrust::get<3>(t) = op(thrust::get<0>(t), thrust::get<1>(t));
+  }
+};
+struct passes_on {
+  template <typename V>
+  __host__ __device__ const V& operator()(const V& x) const { return x; }
+};
+struct is_nonzero {
+  template <typename V>
+  __host__ __device__ bool operator()(const V& x) const { return x ? true : false; }
+};
+}  // namespace detail
+
+template <typename D, typename In, typename Out, typename Op, typename Pred>
+Out transform_if(const detail::execution_policy_base<D>& exec, In first, In last, Out result, Op op, Pred pred) {
+  const std::ptrdiff_t n = last - first;
+  auto zipped = thrust::make_zip_iterator(thrust::make_tuple(first, result));
+  const detail::writes_if<Op, Pred> f = {op, pred};
+  thrust::for_each(exec, zipped, zipped + n, f);
+  return result + n;
+}
+template <typename D, typename In, typename St, typename Out, typename Op, typename Pred>
+Out transform_if(const detail::execution_policy_base<D>& exec, In first, In last, St stencil, Out result, Op op,
+                 Pred pred) {
+  const std::ptrdiff_t n = last - first;
+  auto zipped = thrust::make_zip_iterator(thrust::make_tuple(first, stencil, result));
+  const detail::writes_if<Op, Pred> f = {op, pred};
+  thrust::for_each(exec, zipped, zipped + n, f);
+  return result + n;
+}
+template <typename D, typename In1, typename In2, typename St, typename Out, typename Op, typename Pred>
+Out transform_if(const detail::execution_policy_base<D>& exec, In1 first1, In1 last1, In2 first2, St stencil, Out result,
+                 Op op, Pred pred) {
+  const std::ptrdiff_t n = last1 - first1;
+  auto zipped = thrust::make_zip_iterator(thrust::make_tuple(first1, first2, stencil, result));
+  const detail::writes_if<Op, Pred> f = {op, pred};
+  thrust::for_each(exec, zipped, zipped + n, f);
+  return result + n;
+}
+template <typename In, typename Out, typename Op, typename Pred,
+          typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>
+Out transform_if(In first, In last, Out result, Op op, Pred pred) {
+  return thrust::transform_if(detail::policy_for<Out>(), first, last, result, op, pred);
+}
+template <typename In, typename St, typename Out, typename Op, typename Pred,
+          typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>
+Out transform_if(In first, In last, St stencil, Out result, Op op, Pred pred) {
+  return thrust::transform_if(detail::policy_for<Out>(), first, last, stencil, result, op, pred);
+}
+template <typename In1, typename In2, typename St, typename Out, typename Op, typename Pred,
+          typename = typename std::enable_if<!detail::is_execution_policy<In1>::value>::type>
+Out transform_if(In1 first1, In1 last1, In2 first2, St stencil, Out result, Op op, Pred pred) {
+  return thrust::transform_if(detail::policy_for<Out>(), first1, last1, first2, stencil, result, op, pred);
+}
+
+template <typename D, typename MapIt, typename St, typename In, typename Out, typename Pred>
+Out gather_if(const detail::execution_policy_base<D>& exec, MapIt map_first, MapIt map_last, St stencil, In input,
+              Out result, Pred pred) {
+  return thrust::transform_if(exec, thrust::make_permutation_iterator(input, map_first),
+                              thrust::make_permutation_iterator(input, map_last), stencil, result, detail::passes_on(),
+                              pred);
+}
+template <typename D, typename MapIt, typename St, typename In, typename Out>
+Out gather_if(const detail::execution_policy_base<D>& exec, MapIt map_first, MapIt map_last, St stencil, In input,
+              Out result) {
+  return thrust::gather_if(exec, map_first, map_last, stencil, input, result, detail::is_nonzero());
+}
+template <typename MapIt, typename St, typename In, typename Out, typename Pred,
+          typename = typename std::enable_if<!detail::is_execution_policy<MapIt>::value>::type>
+Out gather_if(MapIt map_first, MapIt map_last, St stencil, In input, Out result, Pred pred) {
+  return thrust::gather_if(detail::policy_for<Out>(), map_first, map_last, stencil, input, result, pred);
+}
+template <typename MapIt, typename St, typename In, typename Out,
+          typename = typename std::enable_if<!detail::is_execution_policy<MapIt>::value>::type>
+Out gather_if(MapIt map_first, MapIt map_last, St stencil, In input, Out result) {
+  return thrust::gather_if(detail::policy_for<Out>(), map_first, map_last, stencil, input, result);
+}
+
+template <typename D, typename In, typename MapIt, typename St, typename Out, typename Pred>
+void scatter_if(const detail::execution_policy_base<D>& exec, In first, In last, MapIt map, St stencil, Out output,
+                Pred pred) {
+  thrust::transform_if(exec, first, last, stencil, thrust::make_permutation_iterator(output, map), detail::passes_on(),
+                       pred);
+}
+template <typename D, typename In, typename MapIt, typename St, typename Out>
+void scatter_if(const detail::execution_policy_base<D>& exec, In first, In last, MapIt map, St stencil, Out output) {
+  thrust::scatter_if(exec, first, last, map, stencil, output, detail::is_nonzero());
+}
+template <typename In, typename MapIt, typename St, typename Out, typename Pred,
+          typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>
+void scatter_if(In first, In last, MapIt map, St stencil, Out output, Pred pred) {
+  thrust::scatter_if(detail::policy_for<Out>(), first, last, map, stencil, output, pred);
+}
+template <typename In, typename MapIt, typename St, typename Out,
+          typename = typename std::enable_if<!detail::is_execution_policy<In>::value>::type>
+void scatter_if(In first, In last, MapIt map, St stencil, Out output) {
+  thrust::scatter_if(detail::policy_for<Out>(), first, last, map, stencil, output);
+}
+
+template <typename D, typename It, typename Size, typename F>
+It for_each_n(const detail::execution_policy_base<D>& exec, It first, Size n, F f) {
+  return thrust::for_each(exec, first, first + (std::ptrdiff_t)n, f);
+}
+template <typename It, typename Size, typename F,
+          typename = typename std::enable_if<!detail::is_execution_policy<It>::value>::type>
+It for_each_n(It first, Size n, F f) {
+  return thrust::for_each(detail::policy_for<It>(), first, first + (std::ptrdiff_t)n, f);
 }
 
 }  // namespace thrust

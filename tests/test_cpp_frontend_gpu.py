@@ -107,3 +107,10 @@ def test_binary_searches():
     # under thrust::greater: the reference's literal vectors on both systems, then device against host on sorted inputs
     out = _run("test_binary_search")
     assert "PASSED" in out
+
+
+def test_conditional_forms_and_reverse_iterator():
+    # transform_if (input decides / stencil decides / two inputs), gather_if, scatter_if, for_each_n, and
+    # thrust::reverse_iterator as input and output of copy, transform, reduce, scan and sort
+    out = _run("test_conditional_forms")
+    assert "PASSED" in out
