@@ -16,6 +16,8 @@
 #include <thrust/iterator/zip_iterator.h>
 #include <thrust/pair.h>
 #include <thrust/reduce.h>
+#include <thrust/system/hip/detail/backend.h>
+#include <thrust/system/hip/detail/device_input.h>
 #include <thrust/tuple.h>
 
 namespace thrust {
@@ -53,70 +55,98 @@ thrust::pair<It, It> minmax_element(execution_policy<D>& exec, It first, It last
 
 namespace hip {
 namespace detail {
-// An element and where it stands; index < 0: nothing seen yet.
-template <typename V>
+// An element and where it stands.  Positions are 32-bit while the range allows it: the pair is
+// what every step of the reduction carries.
+template <typename V, typename I>
 struct located {
   V value;
-  long long index;
+  I index;
 };
-template <typename V>
+template <typename V, typename I>
 struct locates {
   template <typename Tuple>
-  __host__ __device__ located<V> operator()(const Tuple& t) const {
-    located<V> r = {(V)thrust::get<0>(t), (long long)thrust::get<1>(t)};
+  __host__ __device__ located<V, I> operator()(const Tuple& t) const {
+    located<V, I> r = {(V)thrust::get<0>(t), (I)thrust::get<1>(t)};
     return r;
   }
 };
-// Of two located elements the more extreme; of equivalent ones the earlier.
-template <typename V, typename Comp, bool LARGEST>
+// Of two located elements the more extreme; of equivalent ones the earlier
+// (thrust/system/detail/generic/extrema.inl:53-108).
+template <typename V, typename I, typename Comp, bool LARGEST>
 struct picks_extreme {
   mutable Comp comp;  // a caller's comparison need not be const-callable
-  __host__ __device__ located<V> operator()(const located<V>& a, const located<V>& b) const {
-    if (a.index < 0) return b;
-    if (b.index < 0) return a;
-    const bool a_first = a.index < b.index;
-    const located<V>& early = a_first ? a : b;
-    const located<V>& late = a_first ? b : a;
-    const bool late_wins = LARGEST ? (bool)comp(early.value, late.value) : (bool)comp(late.value, early.value);
-    return late_wins ? late : early;
+  __host__ __device__ located<V, I> operator()(const located<V, I>& a, const located<V, I>& b) const {
+    // selects, not branches: this runs once per element in the reduction's inner loop
+    const bool a_before = comp(a.value, b.value), b_before = comp(b.value, a.value);
+    const bool b_earlier = b.index < a.index;
+    const bool take_b = LARGEST ? (a_before | (!b_before & b_earlier)) : (b_before | (!a_before & b_earlier));
+    located<V, I> r;
+    r.value = take_b ? b.value : a.value;
+    r.index = take_b ? b.index : a.index;
+    return r;
   }
 };
 // Both extremes in one pass.
-template <typename V>
+template <typename V, typename I>
 struct located_pair {
-  located<V> smallest, largest;
+  located<V, I> smallest, largest;
 };
-template <typename V>
+template <typename V, typename I>
 struct locates_pair {
   template <typename Tuple>
-  __host__ __device__ located_pair<V> operator()(const Tuple& t) const {
-    located<V> r = {(V)thrust::get<0>(t), (long long)thrust::get<1>(t)};
-    located_pair<V> p = {r, r};
+  __host__ __device__ located_pair<V, I> operator()(const Tuple& t) const {
+    located<V, I> r = {(V)thrust::get<0>(t), (I)thrust::get<1>(t)};
+    located_pair<V, I> p = {r, r};
     return p;
   }
 };
-template <typename V, typename Comp>
+template <typename V, typename I, typename Comp>
 struct picks_both {
   Comp comp;
-  __host__ __device__ located_pair<V> operator()(const located_pair<V>& a, const located_pair<V>& b) const {
-    const picks_extreme<V, Comp, false> lo = {comp};
-    const picks_extreme<V, Comp, true> hi = {comp};
-    located_pair<V> r = {lo(a.smallest, b.smallest), hi(a.largest, b.largest)};
+  __host__ __device__ located_pair<V, I> operator()(const located_pair<V, I>& a, const located_pair<V, I>& b) const {
+    const picks_extreme<V, I, Comp, false> lo = {comp};
+    const picks_extreme<V, I, Comp, true> hi = {comp};
+    located_pair<V, I> r = {lo(a.smallest, b.smallest), hi(a.largest, b.largest)};
     return r;
   }
 };
 
+// The range's first element on the host: what the reduction starts from.
+template <typename V, typename D, typename It>
+V first_value(execution_policy<D>& exec, It first) {
+  void* stream = stream_of(exec);
+  device_input<It> head(stream, temp_source_of(exec), first, 1);  // a computed element is written out first
+  return read_scalar<V>(head.ptr(), stream, "extrema: first element");
+}
+
+template <bool LARGEST, typename I, typename D, typename It, typename Comp>
+std::ptrdiff_t extreme_position(execution_policy<D>& exec, It first, std::ptrdiff_t n, Comp comp) {
+  typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
+  auto zipped = thrust::make_zip_iterator(thrust::make_tuple(first, thrust::counting_iterator<I>(0)));
+  const located<V, I> start = {first_value<V>(exec, first), 0};
+  const picks_extreme<V, I, Comp, LARGEST> pick = {comp};
+  const located<V, I> found = thrust::reduce(exec, thrust::make_transform_iterator(zipped, locates<V, I>()),
+                                             thrust::make_transform_iterator(zipped + n, locates<V, I>()), start, pick);
+  return (std::ptrdiff_t)found.index;
+}
 template <bool LARGEST, typename D, typename It, typename Comp>
 It extreme_element(execution_policy<D>& exec, It first, It last, Comp comp) {
-  typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
   if (first == last) return last;
   const std::ptrdiff_t n = last - first;
-  auto zipped = thrust::make_zip_iterator(thrust::make_tuple(first, thrust::counting_iterator<long long>(0)));
-  const located<V> nothing = {V(), -1};
-  const picks_extreme<V, Comp, LARGEST> pick = {comp};
-  const located<V> found = thrust::reduce(exec, thrust::make_transform_iterator(zipped, locates<V>()),
-                                          thrust::make_transform_iterator(zipped + n, locates<V>()), nothing, pick);
-  return first + (std::ptrdiff_t)found.index;
+  return first + (n <= 0x7fffffff ? extreme_position<LARGEST, int>(exec, first, n, comp)
+                                  : extreme_position<LARGEST, long long>(exec, first, n, comp));
+}
+template <typename I, typename D, typename It, typename Comp>
+thrust::pair<It, It> both_extremes(execution_policy<D>& exec, It first, std::ptrdiff_t n, Comp comp) {
+  typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
+  auto zipped = thrust::make_zip_iterator(thrust::make_tuple(first, thrust::counting_iterator<I>(0)));
+  const located<V, I> one = {first_value<V>(exec, first), 0};
+  const located_pair<V, I> start = {one, one};
+  const picks_both<V, I, Comp> pick = {comp};
+  const located_pair<V, I> found =
+      thrust::reduce(exec, thrust::make_transform_iterator(zipped, locates_pair<V, I>()),
+                     thrust::make_transform_iterator(zipped + n, locates_pair<V, I>()), start, pick);
+  return thrust::pair<It, It>(first + (std::ptrdiff_t)found.smallest.index, first + (std::ptrdiff_t)found.largest.index);
 }
 }  // namespace detail
 
@@ -130,17 +160,10 @@ It max_element(execution_policy<D>& exec, It first, It last, Comp comp) {
 }
 template <typename D, typename It, typename Comp>
 thrust::pair<It, It> minmax_element(execution_policy<D>& exec, It first, It last, Comp comp) {
-  typedef typename std::remove_const<typename iterator_value<It>::type>::type V;
   if (first == last) return thrust::pair<It, It>(last, last);
   const std::ptrdiff_t n = last - first;
-  auto zipped = thrust::make_zip_iterator(thrust::make_tuple(first, thrust::counting_iterator<long long>(0)));
-  const detail::located<V> nothing = {V(), -1};
-  const detail::located_pair<V> none = {nothing, nothing};
-  const detail::picks_both<V, Comp> pick = {comp};
-  const detail::located_pair<V> found =
-      thrust::reduce(exec, thrust::make_transform_iterator(zipped, detail::locates_pair<V>()),
-                     thrust::make_transform_iterator(zipped + n, detail::locates_pair<V>()), none, pick);
-  return thrust::pair<It, It>(first + (std::ptrdiff_t)found.smallest.index, first + (std::ptrdiff_t)found.largest.index);
+  return n <= 0x7fffffff ? detail::both_extremes<int>(exec, first, n, comp)
+                         : detail::both_extremes<long long>(exec, first, n, comp);
 }
 }  // namespace hip
 }  // namespace system

@@ -9,8 +9,12 @@
 // written once).
 //
 //   tests/cpp/bin/test_user_functor_paths [log2 of the element count, default 27]
+#include <thrust/adjacent_difference.h>
+#include <thrust/binary_search.h>
 #include <thrust/copy.h>
 #include <thrust/device_vector.h>
+#include <thrust/extrema.h>
+#include <thrust/find.h>
 #include <thrust/functional.h>
 #include <thrust/host_vector.h>
 #include <thrust/iterator/counting_iterator.h>
@@ -234,6 +238,35 @@ int main(int argc, char** argv) {
   expect(same_prefix(out, out2, n), "sort");
   std::printf("%-34s user %8.3f ms (merge sort, %.2f Gkeys/s)   library %8.3f ms (radix sort, %.2f Gkeys/s)\n", "sort", tu,
               n / tu / 1e6, tl, n / tl / 1e6);
+  // the callers around the path (one reduction or one element-wise pass each); `out2` holds x sorted
+  {
+    auto single = [&](const char* what, double ms, double bytes) {
+      std::printf("%-34s      %8.3f ms %5.1f%%\n", what, ms, bytes / ms / 1e6 / 80.0);
+    };
+    size_t at = 0;
+    double t = best_ms([&] { at = thrust::min_element(x.begin(), x.end()) - x.begin(); });
+    const unsigned smallest = x[at];
+    expect(smallest == (unsigned)out2[0], "min_element");
+    single("min_element", t, 4.0 * n);
+    t = best_ms([&] { at = thrust::max_element(x.begin(), x.end(), my_less()) - x.begin(); });
+    expect((unsigned)x[at] == (unsigned)out2[n - 1], "max_element");
+    single("max_element, user comparator", t, 4.0 * n);
+    const my_below never = {0u};
+    t = best_ms([&] { at = thrust::find_if(x.begin(), x.end(), never) - x.begin(); });
+    expect(at == n, "find_if of an absent element");
+    single("find_if, nothing found", t, 4.0 * n);
+    bool sorted = false;
+    t = best_ms([&] { sorted = thrust::is_sorted(out2.begin(), out2.begin() + n); });
+    expect(sorted, "is_sorted");
+    single("is_sorted", t, 4.0 * n);  // every element is read once (twice by address, once from memory)
+    t = best_ms([&] { thrust::adjacent_difference(x.begin(), x.end(), out.begin()); });
+    single("adjacent_difference", t, 8.0 * n);
+    // every element of x looked up in the sorted copy of x: it is found, at a position that holds it
+    t = best_ms([&] { thrust::lower_bound(out2.begin(), out2.begin() + n, x.begin(), x.end(), vout.begin()); });
+    const unsigned probe = x[n / 3], where = vout[n / 3];
+    expect((unsigned)out2[where] == probe && (where == 0 || (unsigned)out2[where - 1] < probe), "lower_bound");
+    single("lower_bound, n values in n sorted", t, 8.0 * n);
+  }
   std::printf("%d mismatches\n", g_failed);
   std::printf(g_failed ? "FAILED\n" : "PASSED\n");
   return g_failed ? 1 : 0;
