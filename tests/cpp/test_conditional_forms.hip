@@ -14,6 +14,9 @@
 #include <thrust/sequence.h>
 #include <thrust/sort.h>
 #include <thrust/transform.h>
+#include <thrust/advance.h>
+#include <thrust/iterator/zip_iterator.h>
+#include <thrust/zip_function.h>
 
 #include <hip/hip_runtime.h>
 
@@ -173,6 +176,39 @@ static void ReverseIterator() {
   ASSERT_EQUAL((T)twice[3], T(4));
 }
 
+struct sum_and_difference {
+  template <typename T>
+  __host__ __device__ void operator()(const T& a, const T& b, T& sum, T& difference) const {
+    sum = a + b;
+    difference = a - b;
+  }
+};
+struct multiply_add {
+  template <typename T>
+  __host__ __device__ T operator()(const T& a, const T& b, const T& c) const { return a * b + c; }
+};
+
+template <typename Vector>
+static void ZipFunctionAndAdvance() {
+  typedef typename Vector::value_type T;
+  g_test = "zip_function / advance";
+  Vector a(4), b(4), c(4), sum(4), difference(4), out(4);
+  for (int i = 0; i < 4; ++i) { a[i] = T(10 * i); b[i] = T(i + 1); c[i] = T(100); }
+  // testing/zip_function.cu: a function of the elements applied to the zipped ranges
+  auto zipped = thrust::make_zip_iterator(thrust::make_tuple(a.begin(), b.begin(), c.begin()));
+  thrust::transform(zipped, zipped + 4, out.begin(), thrust::make_zip_function(multiply_add()));
+  ASSERT_TRUE(holds(out, {100, 120, 160, 220}));
+  auto four = thrust::make_zip_iterator(thrust::make_tuple(a.begin(), b.begin(), sum.begin(), difference.begin()));
+  thrust::for_each(four, four + 4, thrust::make_zip_function(sum_and_difference()));
+  ASSERT_TRUE(holds(sum, {1, 12, 23, 34}));
+  ASSERT_TRUE(holds(difference, {-1, 8, 17, 26}));
+  auto it = a.begin();
+  thrust::advance(it, 3);
+  ASSERT_EQUAL(it - a.begin(), 3);
+  thrust::advance(it, -2);
+  ASSERT_EQUAL((T)*it, T(10));
+}
+
 template <typename T>
 static void AgainstHost() {
   g_test = "conditional forms: device against host";
@@ -219,6 +255,9 @@ int main() {
   ReverseIterator<thrust::host_vector<int> >();
   ReverseIterator<thrust::device_vector<int> >();
   ReverseIterator<thrust::device_vector<long long> >();
+  ZipFunctionAndAdvance<thrust::host_vector<int> >();
+  ZipFunctionAndAdvance<thrust::device_vector<int> >();
+  ZipFunctionAndAdvance<thrust::device_vector<float> >();
   AgainstHost<int>();
   AgainstHost<long long>();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
