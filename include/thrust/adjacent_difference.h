@@ -40,6 +40,22 @@ template <typename A, typename B>
 inline bool same_position(const A&, const B&) { return false; }
 template <typename A>
 inline bool same_position(const A& a, const A& b) { return a == b; }
+
+#if defined(__HIPCC__)
+// arrays of 4- and 8-byte elements: one kernel that moves 16 bytes per access
+template <typename ViewIn, typename ViewOut, typename Op>
+inline bool adjacent_packed(void*, ViewIn, ViewOut, uint64_t, Op&) { return false; }
+template <typename A, typename O, typename Op>
+inline typename std::enable_if<is_packable<typename std::remove_const<A>::type>::value && is_packable<O>::value &&
+                                   !std::is_const<O>::value, bool>::type
+adjacent_packed(void* stream, A* in, O* out, uint64_t n, Op& op) {
+  constexpr int PER = (sizeof(A) == 8 || sizeof(O) == 8) ? 2 : 4;
+  if (n < 4096 || !pack_aligned(in, PER) || !pack_aligned(out, PER)) return false;
+  hipLaunchKernelGGL((adjacent_packed_kernel<typename std::remove_const<A>::type, O, Op, PER>),
+                     dim3(elementwise_grid(n / PER)), dim3(ELEMENTWISE_BLOCK), 0, (hipStream_t)stream, in, out, n, op);
+  return true;
+}
+#endif
 }  // namespace detail
 
 template <typename D, typename In, typename Out, typename Op>
@@ -49,9 +65,16 @@ Out adjacent_difference(execution_policy<D>& exec, In first, In last, Out result
   if (n == 0) return result;
   if (detail::same_position(first, result)) {
     thrust::device_vector<V> input(first, last);
-    thrust::transform(exec, input.begin() + 1, input.end(), input.begin(), result + 1, op);
-    return result + n;  // result[0] already is x[0]
+    return thrust::adjacent_difference(exec, input.begin(), input.end(), result, op);
   }
+#if defined(__HIPCC__)
+  if (detail::adjacent_packed(detail::stream_of(exec), thrust::detail::device_view(first),
+                              thrust::detail::device_view(result), (uint64_t)n, op)) {
+    detail::throw_on_error(detail::launch_status(), "adjacent_difference: kernel launch");
+    detail::synchronize(detail::stream_of(exec), "adjacent_difference: synchronize");
+    return result + n;
+  }
+#endif
   thrust::copy(exec, first, first + 1, result);
   thrust::transform(exec, first + 1, last, first, result + 1, op);
   return result + n;

@@ -5,6 +5,7 @@
 // util.h:527-561 LoadIterator, parallel_for.h).  HBM traffic: what the iterators read and
 // one write per element.
 #pragma once
+#include <type_traits>
 #if !defined(__HIPCC__)
 #error "thrust/system/hip/detail/fancy_kernels.h is HIP code: compile this translation unit with hipcc"
 #endif
@@ -55,6 +56,96 @@ template <typename ViewIn, typename ViewMap, typename OutView>
 __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void scatter_kernel(ViewIn in, ViewMap map, OutView out, uint64_t n) {
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[map[i]] = in[i];
+}
+
+// ---- arrays of 4- and 8-byte elements: every thread takes PER consecutive elements with 16-byte
+// accesses.  The functor still receives the element itself (a copy in registers); an input that
+// it changed is written back, so a functor that modifies its argument behaves as in the plain
+// kernels above.
+template <typename T, int N>
+struct alignas(sizeof(T) * N >= 16 ? 16 : sizeof(T) * N) element_pack {
+  T v[N];
+};
+template <typename T>
+struct is_packable : std::integral_constant<bool, std::is_trivially_copyable<T>::value && (sizeof(T) == 4 || sizeof(T) == 8)> {};
+template <typename T, int N>
+__device__ __forceinline__ bool same_bytes(const element_pack<T, N>& a, const element_pack<T, N>& b) {
+  uint32_t x[sizeof(a) / 4], y[sizeof(b) / 4];  // copied, not aliased: T may be any 4- or 8-byte type
+  __builtin_memcpy(x, &a, sizeof(a));
+  __builtin_memcpy(y, &b, sizeof(b));
+  uint32_t differ = 0;
+#pragma unroll
+  for (unsigned w = 0; w < sizeof(a) / 4; ++w) differ |= x[w] ^ y[w];
+  return differ == 0;
+}
+template <typename A>
+__device__ __forceinline__ void write_back(const A*, uint64_t, const void*, const void*) {}  // read-only input
+template <typename A, int PER>
+__device__ __forceinline__ void write_back(A* in, uint64_t p, const element_pack<A, PER>* now,
+                                           const element_pack<A, PER>* before) {
+  if (!same_bytes(*now, *before)) reinterpret_cast<element_pack<A, PER>*>(in)[p] = *now;
+}
+
+template <typename PA, typename O, typename F, int PER>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform1_packed_kernel(PA in, O* out, uint64_t n, F f) {
+  typedef typename std::remove_const<typename std::remove_pointer<PA>::type>::type A;
+  const uint64_t packs = n / PER;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; p < packs; p += stride) {
+    element_pack<A, PER> a = reinterpret_cast<const element_pack<A, PER>*>(in)[p];
+    const element_pack<A, PER> before = a;
+    element_pack<O, PER> o;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) o.v[k] = f(a.v[k]);
+    reinterpret_cast<element_pack<O, PER>*>(out)[p] = o;
+    write_back(in, p, &a, &before);
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    for (uint64_t i = packs * PER; i < n; ++i) out[i] = f(in[i]);
+}
+template <typename PA, typename PB, typename O, typename F, int PER>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform2_packed_kernel(PA ina, PB inb, O* out, uint64_t n, F f) {
+  typedef typename std::remove_const<typename std::remove_pointer<PA>::type>::type A;
+  typedef typename std::remove_const<typename std::remove_pointer<PB>::type>::type B;
+  const uint64_t packs = n / PER;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; p < packs; p += stride) {
+    element_pack<A, PER> a = reinterpret_cast<const element_pack<A, PER>*>(ina)[p];
+    element_pack<B, PER> b = reinterpret_cast<const element_pack<B, PER>*>(inb)[p];
+    const element_pack<A, PER> a_before = a;
+    const element_pack<B, PER> b_before = b;
+    element_pack<O, PER> o;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) o.v[k] = f(a.v[k], b.v[k]);
+    reinterpret_cast<element_pack<O, PER>*>(out)[p] = o;
+    write_back(ina, p, &a, &a_before);
+    write_back(inb, p, &b, &b_before);
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    for (uint64_t i = packs * PER; i < n; ++i) out[i] = f(ina[i], inb[i]);
+}
+// out[0] = in[0], out[i] = f(in[i], in[i - 1]); `in` and `out` do not overlap
+template <typename A, typename O, typename F, int PER>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void adjacent_packed_kernel(const A* in, O* out, uint64_t n, F f) {
+  const uint64_t packs = n / PER;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; p < packs; p += stride) {
+    const element_pack<A, PER> a = reinterpret_cast<const element_pack<A, PER>*>(in)[p];
+    element_pack<O, PER> o;
+    if (p == 0) o.v[0] = a.v[0];
+    else o.v[0] = f(a.v[0], in[p * PER - 1]);
+#pragma unroll
+    for (int k = 1; k < PER; ++k) o.v[k] = f(a.v[k], a.v[k - 1]);
+    reinterpret_cast<element_pack<O, PER>*>(out)[p] = o;
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    for (uint64_t i = packs * PER; i < n; ++i) out[i] = i ? (O)f(in[i], in[i - 1]) : (O)in[i];
+}
+
+template <typename T>
+inline bool pack_aligned(const T* p, int per) {
+  const size_t bytes = sizeof(T) * (size_t)per;
+  return reinterpret_cast<uintptr_t>(p) % (bytes >= 16 ? 16 : bytes) == 0;
 }
 
 inline int launch_status() { return (int)hipPeekAtLastError(); }

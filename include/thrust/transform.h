@@ -58,6 +58,38 @@ struct sequence_value {  // element i of thrust::sequence(first, last, init, ste
 };
 }  // namespace detail
 
+#if defined(__HIPCC__)
+namespace detail {
+// Arrays of 4- and 8-byte elements, suitably aligned, go through the kernels that move 16 bytes per
+// access; everything else (fancy iterators, zips, other element sizes) through the plain ones.
+template <typename ViewIn, typename ViewOut, typename F>
+inline bool transform_packed(void*, ViewIn, ViewOut, uint64_t, F&) { return false; }
+template <typename A, typename O, typename F>
+inline typename std::enable_if<is_packable<typename std::remove_const<A>::type>::value && is_packable<O>::value &&
+                                   !std::is_const<O>::value, bool>::type
+transform_packed(void* stream, A* in, O* out, uint64_t n, F& f) {
+  constexpr int PER = (sizeof(A) == 8 || sizeof(O) == 8) ? 2 : 4;
+  if (n < 4096 || !pack_aligned(in, PER) || !pack_aligned(out, PER)) return false;
+  hipLaunchKernelGGL((transform1_packed_kernel<A*, O, F, PER>), dim3(elementwise_grid(n / PER)), dim3(ELEMENTWISE_BLOCK),
+                     0, (hipStream_t)stream, in, out, n, f);
+  return true;
+}
+template <typename ViewA, typename ViewB, typename ViewOut, typename F>
+inline bool transform_packed(void*, ViewA, ViewB, ViewOut, uint64_t, F&) { return false; }
+template <typename A, typename B, typename O, typename F>
+inline typename std::enable_if<is_packable<typename std::remove_const<A>::type>::value &&
+                                   is_packable<typename std::remove_const<B>::type>::value && is_packable<O>::value &&
+                                   !std::is_const<O>::value, bool>::type
+transform_packed(void* stream, A* ina, B* inb, O* out, uint64_t n, F& f) {
+  constexpr int PER = (sizeof(A) == 8 || sizeof(B) == 8 || sizeof(O) == 8) ? 2 : 4;
+  if (n < 4096 || !pack_aligned(ina, PER) || !pack_aligned(inb, PER) || !pack_aligned(out, PER)) return false;
+  hipLaunchKernelGGL((transform2_packed_kernel<A*, B*, O, F, PER>), dim3(elementwise_grid(n / PER)),
+                     dim3(ELEMENTWISE_BLOCK), 0, (hipStream_t)stream, ina, inb, out, n, f);
+  return true;
+}
+}  // namespace detail
+#endif
+
 template <typename D, typename In, typename Out, typename F>
 Out transform(execution_policy<D>& exec, In first, In last, Out result, F f) {
   static_assert(detail::is_device_input<In>::value && detail::is_device_output<Out>::value,
@@ -66,10 +98,11 @@ Out transform(execution_policy<D>& exec, In first, In last, Out result, F f) {
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;
 #if defined(__HIPCC__)
-  hipLaunchKernelGGL((detail::transform1_kernel<typename thrust::detail::device_view_of<In>::type,
-                                                typename thrust::detail::device_view_of<Out>::type, F>),
-                     dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
-                     thrust::detail::device_view(first), thrust::detail::device_view(result), n, f);
+  if (!detail::transform_packed(stream, thrust::detail::device_view(first), thrust::detail::device_view(result), n, f))
+    hipLaunchKernelGGL((detail::transform1_kernel<typename thrust::detail::device_view_of<In>::type,
+                                                  typename thrust::detail::device_view_of<Out>::type, F>),
+                       dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
+                       thrust::detail::device_view(first), thrust::detail::device_view(result), n, f);
   detail::throw_on_error(detail::launch_status(), "transform: kernel launch");
   detail::synchronize(stream, "transform: synchronize");
 #else
@@ -87,12 +120,14 @@ Out transform(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, Out 
   const uint64_t n = (uint64_t)(last1 - first1);
   if (n == 0) return result;
 #if defined(__HIPCC__)
-  hipLaunchKernelGGL((detail::transform2_kernel<typename thrust::detail::device_view_of<In1>::type,
-                                                typename thrust::detail::device_view_of<In2>::type,
-                                                typename thrust::detail::device_view_of<Out>::type, F>),
-                     dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
-                     thrust::detail::device_view(first1), thrust::detail::device_view(first2),
-                     thrust::detail::device_view(result), n, f);
+  if (!detail::transform_packed(stream, thrust::detail::device_view(first1), thrust::detail::device_view(first2),
+                                thrust::detail::device_view(result), n, f))
+    hipLaunchKernelGGL((detail::transform2_kernel<typename thrust::detail::device_view_of<In1>::type,
+                                                  typename thrust::detail::device_view_of<In2>::type,
+                                                  typename thrust::detail::device_view_of<Out>::type, F>),
+                       dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
+                       thrust::detail::device_view(first1), thrust::detail::device_view(first2),
+                       thrust::detail::device_view(result), n, f);
   detail::throw_on_error(detail::launch_status(), "transform: kernel launch");
   detail::synchronize(stream, "transform: synchronize");
 #else

@@ -338,7 +338,63 @@ static void IsSortedAgainstHost() {
   }
 }
 
+struct times_three_plus_one {
+  template <typename T>
+  __host__ __device__ T operator()(const T& x) const { return (T)(x * 3 + 1); }
+};
+struct widens {
+  __host__ __device__ long long operator()(int x) const { return (long long)x * 1000000007ll; }
+};
+struct bumps_and_doubles {  // changes its argument: the input must change too
+  __host__ __device__ int operator()(int& x) const { x += 1; return 2 * x; }
+};
+
+// thrust::transform over plain arrays takes kernels that move 16 bytes per access when the arrays are
+// aligned for it: sizes around the switch, tails, offsets that break the alignment, 8-byte and mixed
+// element sizes, in place, and a functor that modifies its argument
+template <typename T>
+static void TransformShapes() {
+  g_test = "transform: array shapes";
+  const size_t sizes[] = {1, 3, 4095, 4096, 4097, 4099, 10001, 65536 + 3, (1u << 20) + 5};
+  for (size_t n : sizes) {
+    for (size_t offset : {size_t(0), size_t(1), size_t(2)}) {
+      thrust::host_vector<T> h = samples<T>(n + offset, 101 + n, 1000), h2 = samples<T>(n + offset, 102 + n, 1000);
+      thrust::host_vector<T> ho(n + offset, T(7));
+      thrust::device_vector<T> d = h, d2 = h2, dout = ho;
+      thrust::transform(h.begin() + offset, h.end(), ho.begin() + offset, times_three_plus_one());
+      thrust::transform(d.begin() + offset, d.end(), dout.begin() + offset, times_three_plus_one());
+      ASSERT_TRUE(same(thrust::host_vector<T>(dout), ho));
+      thrust::transform(h.begin() + offset, h.end(), h2.begin(), ho.begin() + offset, thrust::minus<T>());
+      thrust::transform(d.begin() + offset, d.end(), d2.begin(), dout.begin() + offset, thrust::minus<T>());
+      ASSERT_TRUE(same(thrust::host_vector<T>(dout), ho));
+      thrust::transform(h.begin(), h.end(), h.begin(), times_three_plus_one());  // in place
+      thrust::transform(d.begin(), d.end(), d.begin(), times_three_plus_one());
+      ASSERT_TRUE(same(thrust::host_vector<T>(d), h));
+      thrust::adjacent_difference(h.begin() + offset, h.end(), ho.begin() + offset);
+      thrust::adjacent_difference(d.begin() + offset, d.end(), dout.begin() + offset);
+      ASSERT_TRUE(same(thrust::host_vector<T>(dout), ho));
+    }
+  }
+  thrust::host_vector<int> hi = samples<int>(70001, 7, 100000);
+  thrust::device_vector<int> di = hi;
+  thrust::host_vector<long long> hw(hi.size());
+  thrust::device_vector<long long> dw(hi.size());
+  thrust::transform(hi.begin(), hi.end(), hw.begin(), widens());
+  thrust::transform(di.begin(), di.end(), dw.begin(), widens());
+  ASSERT_TRUE(same(thrust::host_vector<long long>(dw), hw));
+  thrust::host_vector<int> hb(hi.size());
+  thrust::device_vector<int> db(hi.size());
+  thrust::transform(hi.begin(), hi.end(), hb.begin(), bumps_and_doubles());
+  thrust::transform(di.begin(), di.end(), db.begin(), bumps_and_doubles());
+  ASSERT_TRUE(same(thrust::host_vector<int>(db), hb));
+  ASSERT_TRUE(same(thrust::host_vector<int>(di), hi));  // both inputs were bumped
+}
+
 int main() {
+  TransformShapes<int>();
+  TransformShapes<float>();
+  TransformShapes<long long>();
+  TransformShapes<double>();
   IsSorted<thrust::host_vector<int> >();
   IsSorted<thrust::device_vector<int> >();
   IsSorted<thrust::device_vector<float> >();

@@ -26,6 +26,7 @@
 #include <thrust/scan.h>
 #include <thrust/set_operations.h>
 #include <thrust/sort.h>
+#include <thrust/transform.h>
 #include <thrust/unique.h>
 
 #include <hip/hip_runtime.h>
@@ -259,6 +260,13 @@ int main(int argc, char** argv) {
     t = best_ms([&] { sorted = thrust::is_sorted(out2.begin(), out2.begin() + n); });
     expect(sorted, "is_sorted");
     single("is_sorted", t, 4.0 * n);  // every element is read once (twice by address, once from memory)
+    const modulo by_thousand = {1000u};
+    t = best_ms([&] { thrust::transform(x.begin(), x.end(), out.begin(), by_thousand); });
+    expect((unsigned)out[n / 3] == (unsigned)x[n / 3] % 1000u && (unsigned)out[n - 1] == (unsigned)x[n - 1] % 1000u, "transform");
+    single("transform, one input", t, 8.0 * n);
+    t = best_ms([&] { thrust::transform(x.begin(), x.end(), vals.begin(), out.begin(), my_plus()); });
+    expect((unsigned)out[n / 3] == (unsigned)x[n / 3] + (unsigned)vals[n / 3], "transform of two inputs");
+    single("transform, two inputs", t, 12.0 * n);
     t = best_ms([&] { thrust::adjacent_difference(x.begin(), x.end(), out.begin()); });
     single("adjacent_difference", t, 8.0 * n);
     // every element of x looked up in the sorted copy of x: it is found, at a position that holds it
