@@ -124,6 +124,22 @@ __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform2_packed_kernel(PA
   if (blockIdx.x == 0 && threadIdx.x == 0)
     for (uint64_t i = packs * PER; i < n; ++i) out[i] = f(ina[i], inb[i]);
 }
+template <typename PA, typename F, int PER>
+__global__ __launch_bounds__(ELEMENTWISE_BLOCK) void for_each_packed_kernel(PA first, uint64_t n, F f) {
+  typedef typename std::remove_const<typename std::remove_pointer<PA>::type>::type A;
+  const uint64_t packs = n / PER;
+  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
+  for (uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; p < packs; p += stride) {
+    element_pack<A, PER> a = reinterpret_cast<const element_pack<A, PER>*>(first)[p];
+    const element_pack<A, PER> before = a;
+#pragma unroll
+    for (int k = 0; k < PER; ++k) f(a.v[k]);
+    write_back(first, p, &a, &before);
+  }
+  if (blockIdx.x == 0 && threadIdx.x == 0)
+    for (uint64_t i = packs * PER; i < n; ++i) f(first[i]);
+}
+
 // out[0] = in[0], out[i] = f(in[i], in[i - 1]); `in` and `out` do not overlap
 template <typename A, typename O, typename F, int PER>
 __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void adjacent_packed_kernel(const A* in, O* out, uint64_t n, F f) {

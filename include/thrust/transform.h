@@ -74,6 +74,17 @@ transform_packed(void* stream, A* in, O* out, uint64_t n, F& f) {
                      0, (hipStream_t)stream, in, out, n, f);
   return true;
 }
+template <typename View, typename F>
+inline bool for_each_packed(void*, View, uint64_t, F&) { return false; }
+template <typename A, typename F>
+inline typename std::enable_if<is_packable<typename std::remove_const<A>::type>::value, bool>::type
+for_each_packed(void* stream, A* first, uint64_t n, F& f) {
+  constexpr int PER = sizeof(A) == 8 ? 2 : 4;
+  if (n < 4096 || !pack_aligned(first, PER)) return false;
+  hipLaunchKernelGGL((for_each_packed_kernel<A*, F, PER>), dim3(elementwise_grid(n / PER)), dim3(ELEMENTWISE_BLOCK), 0,
+                     (hipStream_t)stream, first, n, f);
+  return true;
+}
 template <typename ViewA, typename ViewB, typename ViewOut, typename F>
 inline bool transform_packed(void*, ViewA, ViewB, ViewOut, uint64_t, F&) { return false; }
 template <typename A, typename B, typename O, typename F>
@@ -145,9 +156,10 @@ It for_each(execution_policy<D>& exec, It first, It last, F f) {
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return last;
 #if defined(__HIPCC__)
-  hipLaunchKernelGGL((detail::for_each_kernel<typename thrust::detail::device_view_of<It>::type, F>),
-                     dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
-                     thrust::detail::device_view(first), n, f);
+  if (!detail::for_each_packed(stream, thrust::detail::device_view(first), n, f))
+    hipLaunchKernelGGL((detail::for_each_kernel<typename thrust::detail::device_view_of<It>::type, F>),
+                       dim3(detail::elementwise_grid(n)), dim3(detail::ELEMENTWISE_BLOCK), 0, (hipStream_t)stream,
+                       thrust::detail::device_view(first), n, f);
   detail::throw_on_error(detail::launch_status(), "for_each: kernel launch");
   detail::synchronize(stream, "for_each: synchronize");
 #else

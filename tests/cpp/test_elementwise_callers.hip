@@ -338,6 +338,10 @@ static void IsSortedAgainstHost() {
   }
 }
 
+struct adds_one_in_place {
+  template <typename T>
+  __host__ __device__ void operator()(T& x) const { x = x + T(1); }
+};
 struct times_three_plus_one {
   template <typename T>
   __host__ __device__ T operator()(const T& x) const { return (T)(x * 3 + 1); }
@@ -373,6 +377,18 @@ static void TransformShapes() {
       thrust::adjacent_difference(h.begin() + offset, h.end(), ho.begin() + offset);
       thrust::adjacent_difference(d.begin() + offset, d.end(), dout.begin() + offset);
       ASSERT_TRUE(same(thrust::host_vector<T>(dout), ho));
+    }
+  }
+  for (size_t n : sizes) {
+    for (size_t offset : {size_t(0), size_t(1)}) {
+      thrust::host_vector<T> h = samples<T>(n + offset, 111 + n, 1000);
+      thrust::device_vector<T> d = h;
+      thrust::for_each(h.begin() + offset, h.end(), adds_one_in_place());
+      thrust::for_each(d.begin() + offset, d.end(), adds_one_in_place());
+      ASSERT_TRUE(same(thrust::host_vector<T>(d), h));
+      thrust::generate(d.begin() + offset, d.end(), return_value<T>{T(5)});
+      thrust::fill(h.begin() + offset, h.end(), T(5));
+      ASSERT_TRUE(same(thrust::host_vector<T>(d), h));
     }
   }
   thrust::host_vector<int> hi = samples<int>(70001, 7, 100000);
