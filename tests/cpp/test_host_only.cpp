@@ -5,6 +5,22 @@
 #include <cstdlib>
 #include <vector>
 
+#include <thrust/adjacent_difference.h>
+#include <thrust/binary_search.h>
+#include <thrust/equal.h>
+#include <thrust/extrema.h>
+#include <thrust/find.h>
+#include <thrust/iterator/reverse_iterator.h>
+#include <thrust/logical.h>
+#include <thrust/mismatch.h>
+#include <thrust/partition.h>
+#include <thrust/replace.h>
+#include <thrust/reverse.h>
+#include <thrust/sort.h>
+#include <thrust/swap.h>
+#include <thrust/tabulate.h>
+#include <thrust/uninitialized_copy.h>
+#include <thrust/uninitialized_fill.h>
 #include <thrust/device_free.h>
 #include <thrust/device_malloc.h>
 #include <thrust/device_reference.h>
@@ -96,7 +112,50 @@ static void TestDistance() {
   CHECK(thrust::distance(p, p + 5) == 5);
 }
 
+// The callers around the path on the host system, in a translation unit compiled by g++: the
+// reference's vectors (testing/min_element.cu:6-30, find.cu:44-60, is_sorted.cu:6-40,
+// binary_search.cu:50-90, adjacent_difference.cu:6-40, replace.cu:6-40, reverse.cu:6-40, tabulate.cu:6-40).
+static void TestCallersAroundThePath() {
+  thrust::host_vector<int> v(6), w(6);
+  v[0] = 3; v[1] = 5; v[2] = 1; v[3] = 2; v[4] = 5; v[5] = 1;
+  CHECK(thrust::min_element(v.begin(), v.end()) - v.begin() == 2);
+  CHECK(thrust::max_element(thrust::host, v.begin(), v.end()) - v.begin() == 1);
+  CHECK(thrust::minmax_element(v.begin(), v.end()).second - v.begin() == 1);
+  CHECK(thrust::find(v.begin(), v.end(), 2) - v.begin() == 3);
+  CHECK(thrust::find(v.begin(), v.end(), 7) == v.end());
+  CHECK(thrust::any_of(v.begin(), v.end(), thrust::identity<int>()));
+  CHECK(thrust::all_of(v.begin(), v.end(), thrust::identity<int>()));
+  CHECK(!thrust::none_of(v.begin(), v.end(), thrust::identity<int>()));
+  CHECK(!thrust::is_sorted(v.begin(), v.end()));
+  CHECK(thrust::is_sorted_until(v.begin(), v.end()) - v.begin() == 2);
+  thrust::sort(v.begin(), v.end());  // 1 1 2 3 5 5
+  CHECK(thrust::is_sorted(v.begin(), v.end()));
+  CHECK(thrust::lower_bound(v.begin(), v.end(), 5) - v.begin() == 4);
+  CHECK(thrust::upper_bound(v.begin(), v.end(), 1) - v.begin() == 2);
+  CHECK(thrust::binary_search(v.begin(), v.end(), 3) && !thrust::binary_search(v.begin(), v.end(), 4));
+  CHECK(thrust::equal_range(v.begin(), v.end(), 5).second == v.end());
+  thrust::adjacent_difference(v.begin(), v.end(), w.begin());
+  CHECK(w[0] == 1 && w[1] == 0 && w[2] == 1 && w[3] == 1 && w[4] == 2 && w[5] == 0);
+  thrust::reverse(v.begin(), v.end());
+  CHECK(v[0] == 5 && v[5] == 1);
+  thrust::replace(v.begin(), v.end(), 5, 9);
+  CHECK(v[0] == 9 && v[1] == 9 && v[2] == 3);
+  CHECK(thrust::equal(v.begin(), v.end(), v.begin()) && !thrust::equal(v.begin(), v.end(), w.begin()));
+  CHECK(thrust::mismatch(v.begin(), v.end(), w.begin()).first == v.begin());
+  thrust::swap_ranges(v.begin(), v.end(), w.begin());
+  CHECK(w[0] == 9 && v[0] == 1);
+  thrust::tabulate(v.begin(), v.end(), thrust::negate<std::ptrdiff_t>());
+  CHECK(v[2] == -2 && v[5] == -5);
+  CHECK(*thrust::make_reverse_iterator(v.end()) == -5);
+  CHECK(thrust::partition_point(w.begin(), w.end(), thrust::identity<int>()) == w.end());
+  CHECK(thrust::is_partitioned(w.begin(), w.end(), thrust::identity<int>()));
+  thrust::uninitialized_fill(v.begin(), v.end(), 4);
+  thrust::uninitialized_copy(v.begin(), v.begin() + 2, w.begin());
+  CHECK(w[0] == 4 && w[1] == 4 && w[2] == 3);
+}
+
 int main() {
+  TestCallersAroundThePath();
   TestFunctors();
   TestDistance();
   TestReduceByKeyComparesWithTheRunsFirstKey();
