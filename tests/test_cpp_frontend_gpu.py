@@ -114,3 +114,11 @@ def test_conditional_forms_and_reverse_iterator():
     # thrust::reverse_iterator as input and output of copy, transform, reduce, scan and sort
     out = _run("test_conditional_forms")
     assert "PASSED" in out
+
+
+def test_random_engines_and_distributions():
+    # thrust::random: the 10000th draw of minstd_rand0 / minstd_rand (the standard's validation values) on the host and
+    # in device code, discard against drawing, equality, the ranges of uniform_real / uniform_int, normal deviates, and
+    # the stream made by one seed-discard-draw functor per element (identical on both sides)
+    out = _run("test_random")
+    assert "PASSED" in out
