@@ -1,0 +1,42 @@
+// thrust::device_new_allocator: an allocator over device_new / device_delete
+// (thrust/device_new_allocator.h:45-170).
+#pragma once
+#include <cstddef>
+#include <limits>
+#include <new>
+
+#include <thrust/device_delete.h>
+#include <thrust/device_new.h>
+#include <thrust/device_ptr.h>
+#include <thrust/device_reference.h>
+
+namespace thrust {
+
+template <typename T>
+class device_new_allocator {
+ public:
+  typedef T value_type;
+  typedef device_ptr<T> pointer;
+  typedef device_ptr<const T> const_pointer;
+  typedef device_reference<T> reference;
+  typedef device_reference<const T> const_reference;
+  typedef std::size_t size_type;
+  typedef std::ptrdiff_t difference_type;
+  template <typename U>
+  struct rebind { typedef device_new_allocator<U> other; };
+
+  device_new_allocator() {}
+  template <typename U>
+  device_new_allocator(const device_new_allocator<U>&) {}
+  pointer address(reference r) { return &r; }
+  pointer allocate(size_type n, const void* = nullptr) {
+    if (n > max_size()) throw std::bad_alloc();
+    return thrust::device_new<T>(n);
+  }
+  void deallocate(pointer p, size_type n) { thrust::device_delete(p, n); }
+  size_type max_size() const { return (std::numeric_limits<size_type>::max)() / sizeof(T); }
+  bool operator==(const device_new_allocator&) const { return true; }
+  bool operator!=(const device_new_allocator& other) const { return !(*this == other); }
+};
+
+}  // namespace thrust

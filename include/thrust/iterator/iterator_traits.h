@@ -27,6 +27,15 @@ template <typename It>
 struct iterator_value { typedef typename thrust::iterator_traits<It>::value_type type; };
 template <typename It>
 struct iterator_difference { typedef typename detail::difference_of<thrust::iterator_traits<It> >::type type; };
+namespace detail {
+// The element type an algorithm hands to an output iterator: the iterator's own, or, for an
+// iterator that names none (transform_output_iterator), what the algorithm computes in.
+template <typename Out, typename Computed>
+struct output_value {
+  typedef typename std::conditional<std::is_void<typename iterator_value<Out>::type>::value, Computed,
+                                    typename iterator_value<Out>::type>::type type;
+};
+}  // namespace detail
 
 // The system an iterator belongs to: device_ptr -> device system, anything else -> host.
 template <typename It>

@@ -214,7 +214,7 @@ Out scan_generic(execution_policy<D>& exec, In first, In last, Out result, A ini
   namespace gk = thrust::system::hip::generic;
   typedef typename thrust::detail::device_view_of<In>::type View;
   typedef typename thrust::detail::device_view_of<Out>::type OutView;
-  typedef typename iterator_value<Out>::type U;
+  typedef typename thrust::detail::output_value<Out, A>::type U;
   void* stream = stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return result;

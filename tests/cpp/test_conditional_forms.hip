@@ -14,7 +14,14 @@
 #include <thrust/sequence.h>
 #include <thrust/sort.h>
 #include <thrust/transform.h>
+#include <thrust/addressof.h>
 #include <thrust/advance.h>
+#include <thrust/device_delete.h>
+#include <thrust/device_malloc_allocator.h>
+#include <thrust/device_new.h>
+#include <thrust/device_new_allocator.h>
+#include <thrust/iterator/transform_output_iterator.h>
+#include <thrust/limits.h>
 #include <thrust/iterator/zip_iterator.h>
 #include <thrust/zip_function.h>
 
@@ -209,6 +216,49 @@ static void ZipFunctionAndAdvance() {
   ASSERT_EQUAL((T)*it, T(10));
 }
 
+struct doubles {
+  template <typename T>
+  __host__ __device__ T operator()(const T& x) const { return x + x; }
+};
+
+template <typename Vector>
+static void TransformOutputIterator() {
+  typedef typename Vector::value_type T;
+  g_test = "transform_output_iterator";
+  // testing/transform_output_iterator.cu: what is written arrives transformed
+  Vector input(4), output(4, T(0));
+  for (int i = 0; i < 4; ++i) input[i] = T(i + 1);
+  auto doubled = thrust::make_transform_output_iterator(output.begin(), doubles());
+  thrust::copy(input.begin(), input.end(), doubled);
+  ASSERT_TRUE(holds(output, {2, 4, 6, 8}));
+  thrust::transform(input.begin(), input.end(), doubled, thrust::negate<T>());
+  ASSERT_TRUE(holds(output, {-2, -4, -6, -8}));
+  thrust::inclusive_scan(input.begin(), input.end(), doubled);
+  ASSERT_TRUE(holds(output, {2, 6, 12, 20}));
+  ASSERT_EQUAL((doubled + 3) - doubled, 3);
+}
+
+static void DeviceNewAndAllocators() {
+  g_test = "device_new / device_delete / allocators";
+  thrust::device_ptr<int> p = thrust::device_new<int>(5);
+  for (int i = 0; i < 5; ++i) ASSERT_EQUAL((int)p[i], 0);
+  p[2] = 7;
+  ASSERT_EQUAL(thrust::reduce(p, p + 5), 7);
+  thrust::device_delete(p, 5);
+  thrust::device_ptr<void> raw = thrust::device_malloc(4 * sizeof(float));
+  thrust::device_ptr<float> q = thrust::device_new<float>(raw, 2.5f, 4);
+  ASSERT_EQUAL(thrust::reduce(q, q + 4), 10.0f);
+  thrust::device_delete(q, 4);
+  thrust::device_vector<int, thrust::device_malloc_allocator<int> > a(100, 3);
+  ASSERT_EQUAL(thrust::reduce(a.begin(), a.end()), 300);
+  thrust::device_vector<int, thrust::device_new_allocator<int> > b(50, 2);
+  b.resize(80, 1);
+  ASSERT_EQUAL(thrust::reduce(b.begin(), b.end()), 130);
+  int on_host = 4;
+  ASSERT_TRUE(thrust::addressof(on_host) == &on_host);
+  ASSERT_EQUAL(thrust::numeric_limits<int>::max(), std::numeric_limits<int>::max());
+}
+
 template <typename T>
 static void AgainstHost() {
   g_test = "conditional forms: device against host";
@@ -258,6 +308,10 @@ int main() {
   ZipFunctionAndAdvance<thrust::host_vector<int> >();
   ZipFunctionAndAdvance<thrust::device_vector<int> >();
   ZipFunctionAndAdvance<thrust::device_vector<float> >();
+  TransformOutputIterator<thrust::host_vector<int> >();
+  TransformOutputIterator<thrust::device_vector<int> >();
+  TransformOutputIterator<thrust::device_vector<double> >();
+  DeviceNewAndAllocators();
   AgainstHost<int>();
   AgainstHost<long long>();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
