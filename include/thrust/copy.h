@@ -228,7 +228,7 @@ class tested_stream {
 
  private:
   device_input<St> input_;
-  Pred pred_;
+  mutable Pred pred_;  // a caller's predicate need not be const-callable
   bool has_stencil_;
 };
 template <typename St, typename Pred>

@@ -46,7 +46,7 @@ namespace hip {
 namespace detail {
 template <typename Pred>
 struct counts_one {  // a user predicate as a 0 / 1 summand
-  Pred pred;
+  mutable Pred pred;  // a caller's predicate need not be const-callable
   template <typename V>
   __host__ __device__ long long operator()(const V& x) const { return pred(x) ? 1 : 0; }
 };

@@ -29,6 +29,27 @@ class memory_resource : public thrust::mr::memory_resource<thrust::device_ptr<vo
 
 typedef system::hip::memory_resource device_memory_resource;
 
+// A resource whose pointers are device_ptr over one whose pointers are the system's own
+// (thrust/device_allocator.h:46-95).  The device system's pointers are device_ptr already, so
+// this forwards.
+template <typename Upstream>
+class device_ptr_memory_resource final : public thrust::mr::memory_resource<thrust::device_ptr<void> > {
+ public:
+  device_ptr_memory_resource() : upstream_(thrust::mr::get_global_resource<Upstream>()) {}
+  device_ptr_memory_resource(Upstream* upstream) : upstream_(upstream) {}
+
+ protected:
+  thrust::device_ptr<void> do_allocate(std::size_t bytes, std::size_t alignment) override {
+    return thrust::device_ptr<void>(raw_pointer_cast(upstream_->allocate(bytes, alignment)));
+  }
+  void do_deallocate(thrust::device_ptr<void> p, std::size_t bytes, std::size_t alignment) override {
+    upstream_->deallocate(typename Upstream::pointer(p.get()), bytes, alignment);
+  }
+
+ private:
+  Upstream* upstream_;
+};
+
 template <typename T>
 class device_allocator : public thrust::mr::stateless_resource_allocator<T, device_memory_resource> {
  public:

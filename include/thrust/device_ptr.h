@@ -12,6 +12,7 @@
 #include <iterator>
 #include <type_traits>
 
+#include <thrust/detail/config.h>
 #include <thrust/detail/execution_policy.h>
 #include <thrust/system_error.h>
 
@@ -24,40 +25,50 @@ class device_reference {
  public:
   typedef typename std::remove_const<T>::type value_type;
   typedef device_ptr<T> pointer;
-  explicit device_reference(T* p) : ptr_(p) {}
-  explicit device_reference(const device_ptr<T>& p);  // defined below device_ptr
+  __host__ __device__ explicit device_reference(T* p) : ptr_(p) {}
+  __host__ __device__ explicit device_reference(const device_ptr<T>& p);  // defined below device_ptr
   device_reference(const device_reference&) = default;
   // a reference to const from a reference to non-const
   template <typename U, typename = typename std::enable_if<std::is_same<const U, T>::value>::type>
-  device_reference(const device_reference<U>& o) : ptr_((&o).get()) {}
+  __host__ __device__ device_reference(const device_reference<U>& o) : ptr_((&o).get()) {}
 
-  operator value_type() const {
+  // (in device code the referent is ordinary memory: a functor handed device_vector iterators
+  // may dereference them, thrust/detail/reference.h of the reference)
+  __host__ __device__ operator value_type() const {
+#if defined(__HIP_DEVICE_COMPILE__)
+    return *ptr_;
+#else
     value_type v;
     system::hip::detail::throw_on_error(
         thrust_amd_memcpy(static_cast<void*>(&v), ptr_, sizeof(value_type), THRUST_AMD_D2H, nullptr), "device_reference read");
     return v;
+#endif
   }
-  device_reference& operator=(const value_type& v) {
+  __host__ __device__ device_reference& operator=(const value_type& v) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    *const_cast<value_type*>(ptr_) = v;
+#else
     system::hip::detail::throw_on_error(
         thrust_amd_memcpy(const_cast<value_type*>(ptr_), &v, sizeof(value_type), THRUST_AMD_H2D, nullptr),
         "device_reference write");
+#endif
     return *this;
   }
-  device_reference& operator=(const device_reference& other) { return *this = (value_type)other; }
+  __host__ __device__ device_reference& operator=(const device_reference& other) { return *this = (value_type)other; }
   // from a reference to another element type: converted on the way
   template <typename U>
-  device_reference& operator=(const device_reference<U>& other) {
+  __host__ __device__ device_reference& operator=(const device_reference<U>& other) {
     return *this = static_cast<value_type>((typename device_reference<U>::value_type)other);
   }
-  device_ptr<T> operator&() const { return device_ptr<T>(ptr_); }
+  __host__ __device__ device_ptr<T> operator&() const { return device_ptr<T>(ptr_); }
   // exchanges the two referents
-  void swap(device_reference& other) {
+  __host__ __device__ void swap(device_reference& other) {
     const value_type mine = *this, theirs = other;
     *this = theirs;
     other = mine;
   }
 #define THRUST_AMD_REF_COMPOUND(OP)                               \
-  device_reference& operator OP##=(const value_type& v) {         \
+  __host__ __device__ device_reference& operator OP##=(const value_type& v) {         \
     value_type t = *this;                                         \
     t OP##= v;                                                    \
     return *this = t;                                             \
@@ -66,14 +77,14 @@ class device_reference {
   THRUST_AMD_REF_COMPOUND(%) THRUST_AMD_REF_COMPOUND(<<) THRUST_AMD_REF_COMPOUND(>>) THRUST_AMD_REF_COMPOUND(&)
   THRUST_AMD_REF_COMPOUND(|) THRUST_AMD_REF_COMPOUND(^)
 #undef THRUST_AMD_REF_COMPOUND
-  device_reference& operator++() { return *this += value_type(1); }
-  device_reference& operator--() { return *this -= value_type(1); }
-  value_type operator++(int) {
+  __host__ __device__ device_reference& operator++() { return *this += value_type(1); }
+  __host__ __device__ device_reference& operator--() { return *this -= value_type(1); }
+  __host__ __device__ value_type operator++(int) {
     const value_type before = *this;
     *this = before + value_type(1);
     return before;
   }
-  value_type operator--(int) {
+  __host__ __device__ value_type operator--(int) {
     const value_type before = *this;
     *this = before - value_type(1);
     return before;
@@ -84,7 +95,7 @@ class device_reference {
 };
 // thrust::swap of two references exchanges what they refer to (the references are proxies, taken by value)
 template <typename T>
-inline void swap(device_reference<T> a, device_reference<T> b) { a.swap(b); }
+__host__ __device__ inline void swap(device_reference<T> a, device_reference<T> b) { a.swap(b); }
 
 template <typename T>
 class device_ptr {
@@ -97,78 +108,78 @@ class device_ptr {
   typedef T element_type;
   typedef thrust::device_system_tag system_tag;
 
-  device_ptr() : ptr_(nullptr) {}
-  device_ptr(std::nullptr_t) : ptr_(nullptr) {}
-  explicit device_ptr(T* p) : ptr_(p) {}
+  __host__ __device__ device_ptr() : ptr_(nullptr) {}
+  __host__ __device__ device_ptr(std::nullptr_t) : ptr_(nullptr) {}
+  __host__ __device__ explicit device_ptr(T* p) : ptr_(p) {}
   template <typename U, typename = typename std::enable_if<std::is_convertible<U*, T*>::value>::type>
-  device_ptr(const device_ptr<U>& o) : ptr_(o.get()) {}
+  __host__ __device__ device_ptr(const device_ptr<U>& o) : ptr_(o.get()) {}
 
-  T* get() const { return ptr_; }
-  reference operator*() const { return reference(ptr_); }
-  reference operator[](difference_type i) const { return reference(ptr_ + i); }
-  T* operator->() const { return ptr_; }
-  explicit operator bool() const { return ptr_ != nullptr; }
+  __host__ __device__ T* get() const { return ptr_; }
+  __host__ __device__ reference operator*() const { return reference(ptr_); }
+  __host__ __device__ reference operator[](difference_type i) const { return reference(ptr_ + i); }
+  __host__ __device__ T* operator->() const { return ptr_; }
+  __host__ __device__ explicit operator bool() const { return ptr_ != nullptr; }
 
-  device_ptr& operator++() { ++ptr_; return *this; }
-  device_ptr operator++(int) { device_ptr t(*this); ++ptr_; return t; }
-  device_ptr& operator--() { --ptr_; return *this; }
-  device_ptr operator--(int) { device_ptr t(*this); --ptr_; return t; }
-  device_ptr& operator=(std::nullptr_t) { ptr_ = nullptr; return *this; }
+  __host__ __device__ device_ptr& operator++() { ++ptr_; return *this; }
+  __host__ __device__ device_ptr operator++(int) { device_ptr t(*this); ++ptr_; return t; }
+  __host__ __device__ device_ptr& operator--() { --ptr_; return *this; }
+  __host__ __device__ device_ptr operator--(int) { device_ptr t(*this); --ptr_; return t; }
+  __host__ __device__ device_ptr& operator=(std::nullptr_t) { ptr_ = nullptr; return *this; }
   // (templates on the integer type: an unsigned or 64-bit offset would otherwise be ambiguous
   // between the offset form and the conversion of the offset to a pointer difference)
   template <typename I, typename = typename std::enable_if<std::is_integral<I>::value>::type>
-  device_ptr& operator+=(I n) { ptr_ += (difference_type)n; return *this; }
+  __host__ __device__ device_ptr& operator+=(I n) { ptr_ += (difference_type)n; return *this; }
   template <typename I, typename = typename std::enable_if<std::is_integral<I>::value>::type>
-  device_ptr& operator-=(I n) { ptr_ -= (difference_type)n; return *this; }
+  __host__ __device__ device_ptr& operator-=(I n) { ptr_ -= (difference_type)n; return *this; }
   template <typename I, typename = typename std::enable_if<std::is_integral<I>::value>::type>
-  device_ptr operator+(I n) const { return device_ptr(ptr_ + (difference_type)n); }
+  __host__ __device__ device_ptr operator+(I n) const { return device_ptr(ptr_ + (difference_type)n); }
   template <typename I, typename = typename std::enable_if<std::is_integral<I>::value>::type>
-  device_ptr operator-(I n) const { return device_ptr(ptr_ - (difference_type)n); }
-  difference_type operator-(const device_ptr& o) const { return ptr_ - o.ptr_; }
-  bool operator==(const device_ptr& o) const { return ptr_ == o.ptr_; }
-  bool operator!=(const device_ptr& o) const { return ptr_ != o.ptr_; }
-  bool operator<(const device_ptr& o) const { return ptr_ < o.ptr_; }
-  bool operator>(const device_ptr& o) const { return ptr_ > o.ptr_; }
-  bool operator<=(const device_ptr& o) const { return ptr_ <= o.ptr_; }
-  bool operator>=(const device_ptr& o) const { return ptr_ >= o.ptr_; }
-  bool operator==(std::nullptr_t) const { return ptr_ == nullptr; }
-  bool operator!=(std::nullptr_t) const { return ptr_ != nullptr; }
+  __host__ __device__ device_ptr operator-(I n) const { return device_ptr(ptr_ - (difference_type)n); }
+  __host__ __device__ difference_type operator-(const device_ptr& o) const { return ptr_ - o.ptr_; }
+  __host__ __device__ bool operator==(const device_ptr& o) const { return ptr_ == o.ptr_; }
+  __host__ __device__ bool operator!=(const device_ptr& o) const { return ptr_ != o.ptr_; }
+  __host__ __device__ bool operator<(const device_ptr& o) const { return ptr_ < o.ptr_; }
+  __host__ __device__ bool operator>(const device_ptr& o) const { return ptr_ > o.ptr_; }
+  __host__ __device__ bool operator<=(const device_ptr& o) const { return ptr_ <= o.ptr_; }
+  __host__ __device__ bool operator>=(const device_ptr& o) const { return ptr_ >= o.ptr_; }
+  __host__ __device__ bool operator==(std::nullptr_t) const { return ptr_ == nullptr; }
+  __host__ __device__ bool operator!=(std::nullptr_t) const { return ptr_ != nullptr; }
 
  private:
   T* ptr_;
 };
 template <typename T>
-inline bool operator==(std::nullptr_t, const device_ptr<T>& p) { return p.get() == nullptr; }
+__host__ __device__ inline bool operator==(std::nullptr_t, const device_ptr<T>& p) { return p.get() == nullptr; }
 template <typename T>
-inline bool operator!=(std::nullptr_t, const device_ptr<T>& p) { return p.get() != nullptr; }
+__host__ __device__ inline bool operator!=(std::nullptr_t, const device_ptr<T>& p) { return p.get() != nullptr; }
 template <typename T>
-inline device_reference<T>::device_reference(const device_ptr<T>& p) : ptr_(p.get()) {}
+__host__ __device__ inline device_reference<T>::device_reference(const device_ptr<T>& p) : ptr_(p.get()) {}
 
 template <>
 class device_ptr<void> {
  public:
-  device_ptr() : ptr_(nullptr) {}
-  explicit device_ptr(void* p) : ptr_(p) {}
-  void* get() const { return ptr_; }
+  __host__ __device__ device_ptr() : ptr_(nullptr) {}
+  __host__ __device__ explicit device_ptr(void* p) : ptr_(p) {}
+  __host__ __device__ void* get() const { return ptr_; }
 
  private:
   void* ptr_;
 };
 
 template <typename T>
-inline device_ptr<T> operator+(std::ptrdiff_t n, const device_ptr<T>& p) { return p + n; }
+__host__ __device__ inline device_ptr<T> operator+(std::ptrdiff_t n, const device_ptr<T>& p) { return p + n; }
 
 template <typename T>
-inline device_ptr<T> device_pointer_cast(T* p) { return device_ptr<T>(p); }
+__host__ __device__ inline device_ptr<T> device_pointer_cast(T* p) { return device_ptr<T>(p); }
 template <typename T>
-inline device_ptr<T> device_pointer_cast(const device_ptr<T>& p) { return p; }
+__host__ __device__ inline device_ptr<T> device_pointer_cast(const device_ptr<T>& p) { return p; }
 
 template <typename T>
-inline T* raw_pointer_cast(const device_ptr<T>& p) { return p.get(); }
+__host__ __device__ inline T* raw_pointer_cast(const device_ptr<T>& p) { return p.get(); }
 template <typename T>
-inline T* raw_pointer_cast(T* p) { return p; }
+__host__ __device__ inline T* raw_pointer_cast(T* p) { return p; }
 template <typename T>
-inline T* raw_pointer_cast(const device_reference<T>& r) { return (&r).get(); }
+__host__ __device__ inline T* raw_pointer_cast(const device_reference<T>& r) { return (&r).get(); }
 
 // Allocation through the device system (cuda_cub::malloc / free in the reference,
 // thrust/system/cuda/detail/malloc_and_free.h:51-100).

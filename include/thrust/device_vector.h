@@ -377,3 +377,13 @@ template <typename T, typename DA>
 inline bool operator!=(const detail::contiguous_vector<T>& a, const device_vector<T, DA>& b) { return !(b == a); }
 
 }  // namespace thrust
+
+// Programs written for the reference reach these through its vector headers
+// (thrust/detail/vector_base.inl:19-40 includes the algorithms the container is built from).
+#include <thrust/advance.h>
+#include <thrust/copy.h>
+#include <thrust/distance.h>
+#include <thrust/equal.h>
+#include <thrust/fill.h>
+#include <thrust/reduce.h>
+#include <thrust/swap.h>

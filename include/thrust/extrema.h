@@ -10,6 +10,7 @@
 #pragma once
 #include <cstddef>
 
+#include <thrust/detail/minmax.h>
 #include <thrust/functional.h>
 #include <thrust/iterator/counting_iterator.h>
 #include <thrust/iterator/transform_iterator.h>
@@ -102,7 +103,7 @@ struct locates_pair {
 };
 template <typename V, typename I, typename Comp>
 struct picks_both {
-  Comp comp;
+  mutable Comp comp;
   __host__ __device__ located_pair<V, I> operator()(const located_pair<V, I>& a, const located_pair<V, I>& b) const {
     const picks_extreme<V, I, Comp, false> lo = {comp};
     const picks_extreme<V, I, Comp, true> hi = {comp};

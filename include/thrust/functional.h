@@ -11,6 +11,7 @@
 //   unary transforms   identity, negate, square          (transform_reduce, transform scans)
 #pragma once
 #include <thrust/detail/config.h>
+#include <thrust/detail/minmax.h>
 #include <thrust/detail/placeholder_expressions.h>
 
 namespace thrust {

@@ -6,8 +6,11 @@
 
 namespace thrust {
 
-template <typename T>
-class counting_iterator : public detail::fancy_iterator_base<counting_iterator<T>, T> {
+// System: the system the range belongs to when no policy says so (host_system_tag for the
+// sequential loops); Traversal and Difference are accepted for source compatibility
+// (thrust/iterator/counting_iterator.h:135-139).
+template <typename T, typename System = use_default, typename Traversal = use_default, typename Difference = use_default>
+class counting_iterator : public detail::fancy_iterator_base<counting_iterator<T, System, Traversal, Difference>, T> {
  public:
   typedef std::ptrdiff_t difference_type;
   __host__ __device__ counting_iterator() : value_() {}
@@ -25,7 +28,9 @@ class counting_iterator : public detail::fancy_iterator_base<counting_iterator<T
 template <typename T>
 __host__ __device__ inline counting_iterator<T> make_counting_iterator(T v) { return counting_iterator<T>(v); }
 
-template <typename T>
-struct iterator_system<counting_iterator<T> > { typedef thrust::device_system_tag type; };
+template <typename T, typename S, typename Tr, typename D>
+struct iterator_system<counting_iterator<T, S, Tr, D> > {
+  typedef typename std::conditional<std::is_same<S, use_default>::value, thrust::device_system_tag, S>::type type;
+};
 
 }  // namespace thrust

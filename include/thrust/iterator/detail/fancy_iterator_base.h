@@ -15,6 +15,9 @@
 #include <thrust/iterator/iterator_traits.h>
 
 namespace thrust {
+// "Work it out from the other arguments" (thrust/iterator/iterator_adaptor.h of the reference).
+struct use_default {};
+
 namespace detail {
 
 // Derived provides: Reference at(difference_type i) const  (element i from the current position)

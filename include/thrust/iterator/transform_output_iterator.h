@@ -45,7 +45,7 @@ class transform_output_iterator
 
  private:
   Out out_;
-  F f_;
+  mutable F f_;
 };
 template <typename F, typename Out>
 inline transform_output_iterator<F, Out> make_transform_output_iterator(Out out, F f) {

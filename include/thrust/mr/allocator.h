@@ -7,6 +7,7 @@
 #include <new>
 
 #include <thrust/mr/memory_resource.h>
+#include <thrust/mr/polymorphic_adaptor.h>
 
 namespace thrust {
 template <typename T> class device_ptr;
@@ -65,6 +66,19 @@ class stateless_resource_allocator : public allocator<T, MR> {
   stateless_resource_allocator() : allocator<T, MR>(get_global_resource<MR>()) {}
   template <typename U>
   stateless_resource_allocator(const stateless_resource_allocator<U, MR>&) : allocator<T, MR>(get_global_resource<MR>()) {}
+};
+
+// An allocator over whichever resource is behind a polymorphic_adaptor_resource
+// (thrust/mr/allocator.h:215-240).
+template <typename T, typename Pointer = void*>
+class polymorphic_allocator : public allocator<T, polymorphic_adaptor_resource<Pointer> > {
+ public:
+  template <typename U> struct rebind { typedef polymorphic_allocator<U, Pointer> other; };
+  polymorphic_allocator(polymorphic_adaptor_resource<Pointer>* resource)
+      : allocator<T, polymorphic_adaptor_resource<Pointer> >(resource) {}
+  template <typename U>
+  polymorphic_allocator(const polymorphic_allocator<U, Pointer>& o)
+      : allocator<T, polymorphic_adaptor_resource<Pointer> >(o.resource()) {}
 };
 
 }  // namespace mr

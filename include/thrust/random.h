@@ -8,15 +8,13 @@
 // Provided: linear_congruential_engine, minstd_rand0, minstd_rand, default_random_engine,
 // uniform_real_distribution, uniform_int_distribution, normal_distribution.
 #pragma once
+#include <iostream>  // as the reference's header does: its users print what they draw
 #include <cmath>
 #include <cstdint>
 #include <limits>
 
 #include <thrust/detail/config.h>
 #include <thrust/pair.h>
-
-// between a member named min / max and its parentheses: keeps function-like macros of those names out
-#define THRUST_AMD_NO_MACRO
 
 namespace thrust {
 namespace random {
@@ -240,4 +238,3 @@ using random::uniform_real_distribution;
 
 }  // namespace thrust
 
-#undef THRUST_AMD_NO_MACRO

@@ -96,17 +96,17 @@ struct has_bit_rank : std::integral_constant<bool, std::is_same<K, float>::value
 // CODE: 0 = thrust::less<K>, 1 = thrust::greater<K> on an arithmetic K, < 0 anything else
 template <int CODE, typename K, typename Comp>
 struct key_order {
-  Comp comp;
+  mutable Comp comp;
   bool operator()(const K& a, const K& b) const { return comp(a, b); }
 };
 template <typename K, typename Comp>
 struct key_order<0, K, Comp> {
-  Comp comp;
+  mutable Comp comp;
   bool operator()(const K& a, const K& b) const { return rank(a, has_bit_rank<K>()) < rank(b, has_bit_rank<K>()); }
 };
 template <typename K, typename Comp>
 struct key_order<1, K, Comp> {
-  Comp comp;
+  mutable Comp comp;
   bool operator()(const K& a, const K& b) const { return rank(b, has_bit_rank<K>()) < rank(a, has_bit_rank<K>()); }
 };
 template <typename K, typename Comp>

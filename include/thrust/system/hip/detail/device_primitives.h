@@ -115,11 +115,11 @@ template <int CTRL, int ROW_MASK = 0xf, int BANK_MASK = 0xf, typename T>
 THRUST_AMD_DEVICE T dpp_move(T old, T src) {
   if constexpr (sizeof(T) <= 4) {
     uint32_t o = 0, s = 0;
-    __builtin_memcpy(&o, &old, sizeof(T));
-    __builtin_memcpy(&s, &src, sizeof(T));
+    __builtin_memcpy(&o, (const void*)&old, sizeof(T));
+    __builtin_memcpy(&s, (const void*)&src, sizeof(T));
     uint32_t r = (uint32_t)__builtin_amdgcn_update_dpp((int)o, (int)s, CTRL, ROW_MASK, BANK_MASK, false);
     T out;
-    __builtin_memcpy(&out, &r, sizeof(T));
+    __builtin_memcpy((void*)&out, &r, sizeof(T));
     return out;
   } else {
     static_assert(sizeof(T) % 4 == 0, "dpp_move: size must be a multiple of 4 bytes");
@@ -131,7 +131,7 @@ THRUST_AMD_DEVICE T dpp_move(T old, T src) {
     for (int i = 0; i < WORDS; ++i)
       r[i] = (uint32_t)__builtin_amdgcn_update_dpp((int)o[i], (int)s[i], CTRL, ROW_MASK, BANK_MASK, false);
     T out;
-    __builtin_memcpy(&out, r, sizeof(T));
+    __builtin_memcpy((void*)&out, r, sizeof(T));
     return out;
   }
 }
@@ -140,10 +140,10 @@ template <typename T>
 THRUST_AMD_DEVICE T readlane(T v, int lane) {
   if constexpr (sizeof(T) <= 4) {
     uint32_t s = 0;
-    __builtin_memcpy(&s, &v, sizeof(T));
+    __builtin_memcpy(&s, (const void*)&v, sizeof(T));
     uint32_t r = (uint32_t)__builtin_amdgcn_readlane((int)s, lane);
     T out;
-    __builtin_memcpy(&out, &r, sizeof(T));
+    __builtin_memcpy((void*)&out, &r, sizeof(T));
     return out;
   } else {
     static_assert(sizeof(T) % 4 == 0, "readlane: size must be a multiple of 4 bytes");
@@ -153,7 +153,7 @@ THRUST_AMD_DEVICE T readlane(T v, int lane) {
 #pragma unroll
     for (int i = 0; i < WORDS; ++i) r[i] = (uint32_t)__builtin_amdgcn_readlane((int)s[i], lane);
     T out;
-    __builtin_memcpy(&out, r, sizeof(T));
+    __builtin_memcpy((void*)&out, r, sizeof(T));
     return out;
   }
 }
@@ -375,7 +375,7 @@ THRUST_AMD_DEVICE uint32_t tile_try_load(const uint64_t* slot, P& payload) {
     if (i == 0) status = s;
     else same = same && (s == status);
   }
-  __builtin_memcpy(&payload, words, sizeof(P));
+  __builtin_memcpy((void*)&payload, words, sizeof(P));
   return same ? status : (uint32_t)TS_INVALID;
 }
 

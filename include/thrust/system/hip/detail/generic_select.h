@@ -14,6 +14,8 @@
 #endif
 #include <type_traits>
 
+#include <thrust/pair.h>
+#include <thrust/tuple.h>
 #include <thrust/system/hip/detail/backend.h>
 #include <thrust/system/hip/detail/select_kernels.h>
 
@@ -46,9 +48,23 @@ struct run_flagger {
 // copyable in full: the kernel assigns elements to registers and to staging memory that no
 // constructor has run on, which a type with an assignment operator of its own may not survive
 // (such a type has its predicate evaluated into flags first and is then moved as bytes).
+// A thrust::tuple or thrust::pair of such values counts: its assignment operator is its own (a
+// tuple of references assigns through) but assigns member by member, which is the same bytes.
+template <typename S>
+struct is_bytewise_copyable : std::is_trivially_copyable<S> {};
+template <>
+struct is_bytewise_copyable<thrust::tuple<> > : std::true_type {};
+template <typename H, typename... T>
+struct is_bytewise_copyable<thrust::tuple<H, T...> >
+    : std::integral_constant<bool, !std::is_reference<H>::value && is_bytewise_copyable<H>::value &&
+                                       is_bytewise_copyable<thrust::tuple<T...> >::value> {};
+template <typename A, typename B>
+struct is_bytewise_copyable<thrust::pair<A, B> >
+    : std::integral_constant<bool, !std::is_reference<A>::value && !std::is_reference<B>::value &&
+                                       is_bytewise_copyable<A>::value && is_bytewise_copyable<B>::value> {};
 template <typename S>
 struct is_kernel_item
-    : std::integral_constant<bool, std::is_trivially_copyable<S>::value && std::is_default_constructible<S>::value &&
+    : std::integral_constant<bool, is_bytewise_copyable<S>::value && std::is_default_constructible<S>::value &&
                                        (sizeof(S) == 1 || sizeof(S) == 2 || sizeof(S) == 4 || sizeof(S) == 8 ||
                                         sizeof(S) == 16) &&
                                        (alignof(S) <= 16)> {};

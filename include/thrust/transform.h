@@ -149,9 +149,11 @@ Out transform(execution_policy<D>& exec, In1 first1, In1 last1, In2 first2, Out 
 }
 template <typename D, typename It, typename F>
 It for_each(execution_policy<D>& exec, It first, It last, F f) {
-  static_assert(detail::is_device_output<It>::value,
+  // (something a kernel can read is enough: the functor of a for_each over counting_iterator
+  // works through pointers of its own)
+  static_assert(detail::is_device_output<It>::value || detail::is_device_input<It>::value,
                 "thrust::for_each on the device system needs device_ptr / device_vector iterators, raw device pointers "
-                "or a zip of them");
+                "or fancy iterators over them");
   void* stream = detail::stream_of(exec);
   const uint64_t n = (uint64_t)(last - first);
   if (n == 0) return last;

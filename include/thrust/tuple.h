@@ -30,7 +30,8 @@ template <typename H, typename... T>
 class tuple<H, T...> {
  public:
   H head;
-  tuple<T...> tail;
+  // the empty tuple that ends every chain takes no room: tuple<float, float> is 8 bytes
+  [[no_unique_address]] tuple<T...> tail;
 
   struct cons_tag {};
   __host__ __device__ tuple() : head(), tail() {}

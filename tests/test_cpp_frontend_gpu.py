@@ -122,3 +122,12 @@ def test_random_engines_and_distributions():
     # the stream made by one seed-discard-draw functor per element (identical on both sides)
     out = _run("test_random")
     assert "PASSED" in out
+
+
+def test_reference_idioms():
+    # what programs written for the reference lean on beside the algorithms: thrust::min / max, distance, the storage
+    # calls of thrust/memory.h, transform_input_output_iterator, transform_iterator with named types, device_vector
+    # iterators dereferenced inside a functor, fill through a strided view, callables that are not const, unique over
+    # tuples, allocators over run-time chosen resources, and the algorithms the vector headers bring along
+    out = _run("test_reference_idioms")
+    assert "PASSED" in out
