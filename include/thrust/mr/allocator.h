@@ -5,6 +5,7 @@
 #pragma once
 #include <cstddef>
 #include <new>
+#include <type_traits>
 
 #include <thrust/mr/memory_resource.h>
 #include <thrust/mr/polymorphic_adaptor.h>
