@@ -37,9 +37,14 @@ struct output_value {
 };
 }  // namespace detail
 
-// The system an iterator belongs to: device_ptr -> device system, anything else -> host.
-template <typename It>
+// The system an iterator belongs to: device_ptr -> device system, an iterator that names one
+// (those built on thrust::iterator_facade do) -> that one, anything else -> host.
+template <typename It, typename = void>
 struct iterator_system { typedef thrust::host_system_tag type; };
+template <typename It>
+struct iterator_system<It, typename std::enable_if<!std::is_void<typename It::facade_system>::value>::type> {
+  typedef typename It::facade_system type;
+};
 template <typename T>
 struct iterator_system<device_ptr<T> > { typedef thrust::device_system_tag type; };
 

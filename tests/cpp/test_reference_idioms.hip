@@ -6,7 +6,8 @@
 // counting_iterator with a named system, device_vector iterators dereferenced inside a functor
 // (raw_reference_cast), fill through a strided view, predicates that are not const-callable,
 // unique over tuples, allocators over run-time chosen resources (thrust/mr/polymorphic_adaptor.h),
-// and what the vector headers bring along.
+// iterators of the caller's own built on iterator_adaptor / iterator_facade, and what the vector
+// headers bring along.
 #include <thrust/device_vector.h>
 #include <thrust/host_vector.h>
 // (nothing else before the first test on purpose: fill, copy, reduce, distance and equal are reached
@@ -42,6 +43,8 @@ static void ReachedThroughTheVectorHeaders() {
 #include <thrust/gather.h>
 #include <thrust/iterator/constant_iterator.h>
 #include <thrust/iterator/counting_iterator.h>
+#include <thrust/iterator/iterator_adaptor.h>
+#include <thrust/iterator/iterator_facade.h>
 #include <thrust/iterator/permutation_iterator.h>
 #include <thrust/iterator/transform_input_output_iterator.h>
 #include <thrust/iterator/transform_iterator.h>
@@ -402,6 +405,117 @@ static void AllocatorsOverChosenResources() {
   }
 }
 
+// Each element of the wrapped range `times` times over: only dereference() is written anew
+// (the use the documentation of thrust/iterator/iterator_adaptor.h shows).
+template <typename It>
+class repeats : public thrust::iterator_adaptor<repeats<It>, It> {
+ public:
+  typedef thrust::iterator_adaptor<repeats<It>, It> super_t;
+  __host__ __device__ repeats(const It& x, int times) : super_t(x), begin_(x), times_(times) {}
+  friend class thrust::iterator_core_access;
+
+ private:
+  It begin_;
+  int times_;
+  __host__ __device__ typename super_t::reference dereference() const {
+    return *(begin_ + (this->base() - begin_) / times_);
+  }
+};
+// Every `stride`-th element of the wrapped range: movement is written anew, dereference is the
+// wrapped iterator's, so the view can be written through.
+template <typename It>
+class strides_over : public thrust::iterator_adaptor<strides_over<It>, It> {
+ public:
+  typedef thrust::iterator_adaptor<strides_over<It>, It> super_t;
+  typedef typename super_t::difference_type difference_type;
+  __host__ __device__ strides_over(const It& x, difference_type stride) : super_t(x), stride_(stride) {}
+  friend class thrust::iterator_core_access;
+
+ private:
+  difference_type stride_;
+  __host__ __device__ void advance(difference_type n) { this->base_reference() += n * stride_; }
+  __host__ __device__ void increment() { this->base_reference() += stride_; }
+  __host__ __device__ void decrement() { this->base_reference() -= stride_; }
+  __host__ __device__ difference_type distance_to(const strides_over& o) const {
+    return (o.base() - this->base()) / stride_;
+  }
+};
+// a * i + b for i = 0, 1, ...: nothing wrapped, every member written here
+template <typename System>
+class affine : public thrust::iterator_facade<affine<System>, long long, System, thrust::random_access_traversal_tag,
+                                              long long, std::ptrdiff_t> {
+ public:
+  __host__ __device__ affine(long long a, long long b, std::ptrdiff_t i = 0) : a_(a), b_(b), i_(i) {}
+  friend class thrust::iterator_core_access;
+
+ private:
+  long long a_, b_;
+  std::ptrdiff_t i_;
+  __host__ __device__ long long dereference() const { return a_ * i_ + b_; }
+  __host__ __device__ bool equal(const affine& o) const { return i_ == o.i_; }
+  __host__ __device__ void increment() { ++i_; }
+  __host__ __device__ void decrement() { --i_; }
+  __host__ __device__ void advance(std::ptrdiff_t n) { i_ += n; }
+  __host__ __device__ std::ptrdiff_t distance_to(const affine& o) const { return o.i_ - i_; }
+};
+
+template <typename Vector, typename System>
+static void IteratorsOfTheCallersOwn() {
+  g_test = "IteratorsOfTheCallersOwn";
+  typedef typename Vector::iterator It;
+  static_assert(std::is_same<typename thrust::iterator_system<repeats<It> >::type, System>::value, "the wrapped iterator's system");
+  static_assert(std::is_same<typename thrust::iterator_value<repeats<It> >::type, int>::value, "the wrapped iterator's value");
+  const int few[] = {10, 20, 30, 40};
+  Vector v(few, few + 4);
+  repeats<It> first(v.begin(), 3), last(v.end(), 3);
+  ASSERT_EQUAL(first[0], 10);
+  ASSERT_EQUAL(first[2], 10);
+  ASSERT_EQUAL(first[3], 20);
+  ASSERT_EQUAL(*(first + 11), 40);
+  ASSERT_EQUAL((first + 12) - first, 12);
+  Vector out(12);
+  thrust::copy(first, first + 12, out.begin());
+  const int gold[] = {10, 10, 10, 20, 20, 20, 30, 30, 30, 40, 40, 40};
+  ASSERT_TRUE(same(out, thrust::host_vector<int>(gold, gold + 12)));
+  ASSERT_EQUAL(thrust::reduce(first, first + 12), 300);
+  (void)last;
+  // a long one, against the closed form
+  Vector big(5000);
+  thrust::sequence(big.begin(), big.end());
+  repeats<It> rb(big.begin(), 7);
+  ASSERT_EQUAL(thrust::reduce(rb, rb + 35000, 0ll), 7ll * 4999 * 5000 / 2);
+  using namespace thrust::placeholders;
+  Vector twice(35000);
+  thrust::transform(rb, rb + 35000, twice.begin(), _1 * 2);
+  ASSERT_EQUAL((int)twice[34999], 9998);
+  ASSERT_EQUAL((int)twice[7], 2);
+
+  // written through: every third element
+  Vector w(30, 1);
+  strides_over<It> s(w.begin(), 3);
+  ASSERT_EQUAL((s + 10) - s, 10);
+  thrust::fill(s, s + 10, 5);
+  ASSERT_EQUAL(thrust::reduce(w.begin(), w.end()), 20 + 50);
+  ASSERT_EQUAL((int)w[0], 5);
+  ASSERT_EQUAL((int)w[1], 1);
+  ASSERT_EQUAL((int)w[27], 5);
+  thrust::transform(s, s + 10, thrust::counting_iterator<int>(0), s, _1 + _2);  // in place through the view
+  ASSERT_EQUAL((int)w[27], 14);
+  ASSERT_EQUAL((int)w[28], 1);
+  ASSERT_EQUAL(thrust::reduce(s, s + 10), 50 + 45);
+
+  // nothing wrapped
+  affine<System> a(3, 1);
+  ASSERT_EQUAL(*a, 1);
+  ASSERT_EQUAL(a[4], 13);
+  ASSERT_EQUAL(thrust::reduce(a, a + 100000), 3ll * 99999 * 100000 / 2 + 100000);
+  thrust::host_vector<long long> got(5);
+  thrust::copy(a + 2, a + 7, got.begin());
+  ASSERT_EQUAL(got[0], 7);
+  ASSERT_EQUAL(got[4], 19);
+  ASSERT_EQUAL(thrust::count_if(a, a + 1000, _1 % 2 == 0), 500);
+}
+
 int main() {
   ReachedThroughTheVectorHeaders();
   MinAndMax<int>();
@@ -427,6 +541,8 @@ int main() {
   ExpandByCounts<thrust::host_vector<int> >();
   ExpandByCounts<thrust::device_vector<int> >();
   AllocatorsOverChosenResources();
+  IteratorsOfTheCallersOwn<thrust::host_vector<int>, thrust::host_system_tag>();
+  IteratorsOfTheCallersOwn<thrust::device_vector<int>, thrust::device_system_tag>();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
   std::printf(g_failed ? "FAILED\n" : "PASSED\n");
   return g_failed ? 1 : 0;
