@@ -1,5 +1,19 @@
-// Named by the API this front end mirrors and not provided by it.  The header exists so that
-// including it stops the build here, instead of the compiler picking up a file of the same name
-// from another Thrust installation on its include path and mixing two implementations.
+// thrust::device_make_unique<T>(args...): one T in device memory, a copy of T(args...) built on
+// the host, owned by a std::unique_ptr that gives the storage back to thrust::device_allocator
+// (thrust/device_make_unique.h:40-58; testing/async_reduce_into.cu:383 uses it for result slots).
 #pragma once
-#error "thrust::device_make_unique is not provided by this Thrust front end (MI355X device system: the sort / scan / reduce / select / merge path and its callers)"
+#include <utility>
+
+#include <thrust/allocate_unique.h>
+#include <thrust/device_allocator.h>
+#include <thrust/device_new.h>
+#include <thrust/device_ptr.h>
+
+namespace thrust {
+template <typename T, typename... Args>
+inline auto device_make_unique(Args&&... args) -> decltype(uninitialized_allocate_unique<T>(device_allocator<T>())) {
+  auto p = uninitialized_allocate_unique<T>(device_allocator<T>());
+  device_new<T>(thrust::device_ptr<void>(p.get().get()), T(std::forward<Args>(args)...));
+  return p;
+}
+}  // namespace thrust

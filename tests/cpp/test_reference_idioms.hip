@@ -6,7 +6,8 @@
 // counting_iterator with a named system, device_vector iterators dereferenced inside a functor
 // (raw_reference_cast), fill through a strided view, predicates that are not const-callable,
 // unique over tuples, allocators over run-time chosen resources (thrust/mr/polymorphic_adaptor.h),
-// iterators of the caller's own built on iterator_adaptor / iterator_facade, and what the vector
+// iterators of the caller's own built on iterator_adaptor / iterator_facade, allocate_unique and
+// device_make_unique, and what the vector
 // headers bring along.
 #include <thrust/device_vector.h>
 #include <thrust/host_vector.h>
@@ -35,7 +36,11 @@ static void ReachedThroughTheVectorHeaders() {
   assert(h[999] == 3);  // <cassert> comes with the headers too
 }
 
+#include <thrust/allocate_unique.h>
 #include <thrust/count.h>
+#include <thrust/device_make_unique.h>
+#include <thrust/universal_ptr.h>
+#include <thrust/universal_vector.h>
 #include <thrust/detail/raw_reference_cast.h>
 #include <thrust/extrema.h>
 #include <thrust/for_each.h>
@@ -516,6 +521,65 @@ static void IteratorsOfTheCallersOwn() {
   ASSERT_EQUAL(thrust::count_if(a, a + 1000, _1 % 2 == 0), 500);
 }
 
+template <typename T>
+struct holds {
+  T held;
+  holds(T x) : held(x) {}
+  __host__ __device__ T getter() const { return held; }
+};
+template <typename T>
+static void OwnedThroughUniquePtr() {
+  g_test = "OwnedThroughUniquePtr";
+  {  // storage the host addresses too: read through the pointer (testing/universal_memory.cu:35-66)
+    auto raw = thrust::allocate_unique<T>(thrust::universal_allocator<T>(), 42);
+    auto obj = thrust::allocate_unique<holds<T> >(thrust::universal_allocator<holds<T> >(), 42);
+    static_assert(std::is_same<decltype(raw.get()), thrust::universal_ptr<T> >::value, "the allocator's pointer");
+    static_assert(std::is_same<decltype(obj.get()), thrust::universal_ptr<holds<T> > >::value, "the allocator's pointer");
+    // (through get(): std::unique_ptr's own operator* wants a plain T&, and what a device_ptr
+    // yields on the host is a proxy)
+    ASSERT_EQUAL((T)*raw.get(), T(42));
+    ASSERT_EQUAL((T)raw.get()[0], T(42));
+    ASSERT_EQUAL(obj->getter(), T(42));
+    ASSERT_EQUAL(obj.get()->getter(), T(42));
+    auto array = thrust::allocate_unique_n<T>(thrust::universal_allocator<T>(), 6, 42);
+    static_assert(std::is_same<decltype(array.get()), thrust::universal_ptr<T> >::value, "the allocator's pointer");
+    ASSERT_EQUAL(thrust::reduce(array.get(), array.get() + 6), T(6 * 42));
+    ASSERT_EQUAL(array.get_deleter().size(), 6u);
+    for (int i = 0; i < 6; ++i) array.get()[i] = T(i);  // written by the host ...
+    ASSERT_EQUAL(thrust::reduce(array.get(), array.get() + 6), T(15));  // ... summed by the device
+  }
+  {  // device memory
+    auto one = thrust::device_make_unique<T>(T(7));
+    static_assert(std::is_same<decltype(one.get()), thrust::device_ptr<T> >::value, "device_allocator's pointer");
+    ASSERT_EQUAL((T)*one.get(), T(7));
+    auto zero = thrust::device_make_unique<T>();
+    ASSERT_EQUAL((T)*zero.get(), T());
+    auto many = thrust::allocate_unique_n<T>(thrust::device_allocator<T>(), 1000, 3);
+    ASSERT_EQUAL(thrust::reduce(many.get(), many.get() + 1000), T(3000));
+    auto blank = thrust::uninitialized_allocate_unique_n<T>(thrust::device_allocator<T>(), 1000);
+    thrust::copy(many.get(), many.get() + 1000, blank.get());
+    ASSERT_TRUE(thrust::equal(many.get(), many.get() + 1000, blank.get()));
+    one.reset();  // gives the storage back now
+    ASSERT_TRUE(!one);
+  }
+  {  // the host's allocator: constructed in place, destroyed on release
+    static int alive;
+    alive = 0;
+    struct counted {
+      counted(int) { ++alive; }
+      counted(const counted&) { ++alive; }
+      ~counted() { --alive; }
+    };
+    {
+      auto one = thrust::allocate_unique<counted>(std::allocator<counted>(), 1);
+      ASSERT_EQUAL(alive, 1);
+      auto five = thrust::allocate_unique_n<counted>(std::allocator<counted>(), 5, 1);
+      ASSERT_EQUAL(alive, 6);
+    }
+    ASSERT_EQUAL(alive, 0);
+  }
+}
+
 int main() {
   ReachedThroughTheVectorHeaders();
   MinAndMax<int>();
@@ -543,6 +607,8 @@ int main() {
   AllocatorsOverChosenResources();
   IteratorsOfTheCallersOwn<thrust::host_vector<int>, thrust::host_system_tag>();
   IteratorsOfTheCallersOwn<thrust::device_vector<int>, thrust::device_system_tag>();
+  OwnedThroughUniquePtr<int>();
+  OwnedThroughUniquePtr<double>();
   std::printf("%d checks, %d failed\n", g_checks, g_failed);
   std::printf(g_failed ? "FAILED\n" : "PASSED\n");
   return g_failed ? 1 : 0;
