@@ -12,6 +12,7 @@
 #include <cmath>
 #include <cstdint>
 #include <limits>
+#include <type_traits>
 
 #include <thrust/detail/config.h>
 #include <thrust/pair.h>
@@ -105,6 +106,215 @@ template <typename U, U a, U c, U m> const U linear_congruential_engine<U, a, c,
 typedef linear_congruential_engine<std::uint32_t, 16807, 0, 2147483647> minstd_rand0;
 typedef linear_congruential_engine<std::uint32_t, 48271, 0, 2147483647> minstd_rand;
 typedef minstd_rand default_random_engine;
+
+// ------------------------------------------------------------------ the other engines
+// A Tausworthe generator (thrust/random/linear_feedback_shift_engine.h:50-200,
+// detail/linear_feedback_shift_engine.inl:27-60).
+template <typename UIntType, std::size_t w, std::size_t k, std::size_t q, std::size_t s>
+class linear_feedback_shift_engine {
+ public:
+  typedef UIntType result_type;
+  static const std::size_t word_size = w, exponent1 = k, exponent2 = q, step_size = s;
+  // bits 1 .. w-1: the mask the reference builds leaves bit 0 out
+  // (random/detail/linear_feedback_shift_engine_wordmask.h:27-40), and the validation value of
+  // taus88 is the one this mask gives
+  static const result_type wordmask =
+      (result_type)((w < 8 * sizeof(UIntType) ? (result_type)((result_type)1 << (w % (8 * sizeof(UIntType)))) : (result_type)0) - 2);
+  static const result_type min = 0;
+  static const result_type max = wordmask;
+  static const result_type default_seed = 341u;
+
+  __host__ __device__ explicit linear_feedback_shift_engine(result_type value = default_seed) { seed(value); }
+  __host__ __device__ void seed(result_type value = default_seed) { x_ = value; }
+  __host__ __device__ result_type operator()() {
+    const UIntType b = (UIntType)((((x_ << q) ^ x_) & wordmask) >> (k - s));
+    const UIntType mask = (UIntType)(((~static_cast<UIntType>(0)) << (w - k)) & wordmask);
+    x_ = (UIntType)(((x_ & mask) << s) ^ b);
+    return x_;
+  }
+  __host__ __device__ void discard(unsigned long long z) {
+    for (; z > 0; --z) (*this)();
+  }
+  __host__ __device__ friend bool operator==(const linear_feedback_shift_engine& a, const linear_feedback_shift_engine& b) {
+    return a.x_ == b.x_;
+  }
+  __host__ __device__ friend bool operator!=(const linear_feedback_shift_engine& a, const linear_feedback_shift_engine& b) {
+    return !(a == b);
+  }
+
+ private:
+  result_type x_;
+};
+template <typename U, std::size_t w, std::size_t k, std::size_t q, std::size_t s>
+const U linear_feedback_shift_engine<U, w, k, q, s>::wordmask;
+template <typename U, std::size_t w, std::size_t k, std::size_t q, std::size_t s>
+const U linear_feedback_shift_engine<U, w, k, q, s>::min;
+template <typename U, std::size_t w, std::size_t k, std::size_t q, std::size_t s>
+const U linear_feedback_shift_engine<U, w, k, q, s>::max;
+template <typename U, std::size_t w, std::size_t k, std::size_t q, std::size_t s>
+const U linear_feedback_shift_engine<U, w, k, q, s>::default_seed;
+
+// x_i = (x_{i-s} - x_{i-r} - carry) mod 2^w (thrust/random/subtract_with_carry_engine.h:55-215,
+// detail/subtract_with_carry_engine.inl:30-85).  The r words of state are seeded with one draw
+// each of a 40014 / 2147483563 congruential engine, which is the reference's rule (and not the
+// C++ standard's, whose engines of the same names give other numbers).
+template <typename UIntType, std::size_t w, std::size_t s, std::size_t r>
+class subtract_with_carry_engine {
+ public:
+  typedef UIntType result_type;
+  static const std::size_t word_size = w, short_lag = s, long_lag = r;
+  static const result_type modulus = (result_type)((result_type)1 << w);
+  static const result_type min = 0;
+  static const result_type max = modulus - 1;
+  static const result_type default_seed = 19780503u;
+
+  __host__ __device__ explicit subtract_with_carry_engine(result_type value = default_seed) { seed(value); }
+  __host__ __device__ void seed(result_type value = default_seed) {
+    linear_congruential_engine<result_type, 40014u, 0u, 2147483563u> e(value == 0u ? (result_type)default_seed : value);
+    for (std::size_t i = 0; i < r; ++i) x_[i] = (result_type)(e() % modulus);
+    carry_ = x_[r - 1] == 0;
+    k_ = 0;
+  }
+  __host__ __device__ result_type operator()() {
+    int short_index = k_ - (int)s;
+    if (short_index < 0) short_index += (int)r;
+    result_type xi;
+    if (x_[short_index] >= x_[k_] + carry_) {
+      xi = x_[short_index] - x_[k_] - carry_;
+      carry_ = 0;
+    } else {
+      xi = modulus - x_[k_] - carry_ + x_[short_index];
+      carry_ = 1;
+    }
+    x_[k_] = xi;
+    if (++k_ >= (int)r) k_ = 0;
+    return xi;
+  }
+  __host__ __device__ void discard(unsigned long long z) {
+    for (; z > 0; --z) (*this)();
+  }
+  // the same future: the same words in the same order from where each one stands, and the same carry
+  __host__ __device__ friend bool operator==(const subtract_with_carry_engine& a, const subtract_with_carry_engine& b) {
+    bool same = a.carry_ == b.carry_;
+    for (std::size_t i = 0; i < r; ++i) same = same && a.x_[(i + a.k_) % r] == b.x_[(i + b.k_) % r];
+    return same;
+  }
+  __host__ __device__ friend bool operator!=(const subtract_with_carry_engine& a, const subtract_with_carry_engine& b) {
+    return !(a == b);
+  }
+
+ private:
+  result_type x_[r];
+  result_type carry_;
+  int k_;
+};
+template <typename U, std::size_t w, std::size_t s, std::size_t r> const U subtract_with_carry_engine<U, w, s, r>::modulus;
+template <typename U, std::size_t w, std::size_t s, std::size_t r> const U subtract_with_carry_engine<U, w, s, r>::min;
+template <typename U, std::size_t w, std::size_t s, std::size_t r> const U subtract_with_carry_engine<U, w, s, r>::max;
+template <typename U, std::size_t w, std::size_t s, std::size_t r> const U subtract_with_carry_engine<U, w, s, r>::default_seed;
+
+// Of every p draws of Engine the first r (thrust/random/discard_block_engine.h:45-200,
+// detail/discard_block_engine.inl:27-90).
+template <typename Engine, std::size_t p, std::size_t r>
+class discard_block_engine {
+ public:
+  typedef Engine base_type;
+  typedef typename base_type::result_type result_type;
+  static const std::size_t block_size = p, used_block = r;
+  static const result_type min = base_type::min;
+  static const result_type max = base_type::max;
+
+  __host__ __device__ discard_block_engine() : e_(), n_(0) {}
+  __host__ __device__ explicit discard_block_engine(result_type s) : e_(s), n_(0) {}
+  __host__ __device__ explicit discard_block_engine(const base_type& urng) : e_(urng), n_(0) {}
+  __host__ __device__ void seed() { e_.seed(); n_ = 0; }
+  __host__ __device__ void seed(result_type s) { e_.seed(s); n_ = 0; }
+  __host__ __device__ result_type operator()() {
+    if (n_ >= r) {
+      e_.discard(p - n_);
+      n_ = 0;
+    }
+    ++n_;
+    return e_();
+  }
+  __host__ __device__ void discard(unsigned long long z) {
+    for (; z > 0; --z) (*this)();
+  }
+  __host__ __device__ const base_type& base() const { return e_; }
+  __host__ __device__ friend bool operator==(const discard_block_engine& a, const discard_block_engine& b) {
+    return a.e_ == b.e_ && a.n_ == b.n_;
+  }
+  __host__ __device__ friend bool operator!=(const discard_block_engine& a, const discard_block_engine& b) { return !(a == b); }
+
+ private:
+  base_type e_;
+  unsigned int n_;
+};
+template <typename E, std::size_t p, std::size_t r> const typename E::result_type discard_block_engine<E, p, r>::min;
+template <typename E, std::size_t p, std::size_t r> const typename E::result_type discard_block_engine<E, p, r>::max;
+
+// The draws of two engines, shifted and combined by exclusive or
+// (thrust/random/xor_combine_engine.h:50-230, detail/xor_combine_engine.inl:27-120).
+template <typename Engine1, std::size_t s1, typename Engine2, std::size_t s2 = 0u>
+class xor_combine_engine {
+ public:
+  typedef Engine1 base1_type;
+  typedef Engine2 base2_type;
+  typedef typename std::conditional<(sizeof(typename base2_type::result_type) > sizeof(typename base1_type::result_type)),
+                                    typename base2_type::result_type, typename base1_type::result_type>::type result_type;
+  static const std::size_t shift1 = s1, shift2 = s2;
+  static const result_type min = 0;
+
+ private:
+  // all ones up to the highest bit either side can set: the exact bound for the engines whose
+  // ranges end one below a power of two or, as taus88's parts do, two below
+  static constexpr result_type ones_up_to(result_type x) {
+    return x == 0 ? 0 : (result_type)(ones_up_to((result_type)(x >> 1)) << 1 | 1);
+  }
+
+ public:
+  static const result_type max = ones_up_to((result_type)(((result_type)(base1_type::max - base1_type::min) << s1) |
+                                                           ((result_type)(base2_type::max - base2_type::min) << s2)));
+
+  __host__ __device__ xor_combine_engine() : b1_(), b2_() {}
+  __host__ __device__ xor_combine_engine(const base1_type& urng1, const base2_type& urng2) : b1_(urng1), b2_(urng2) {}
+  __host__ __device__ explicit xor_combine_engine(result_type s) : b1_(s), b2_(s) {}
+  __host__ __device__ void seed() { b1_.seed(); b2_.seed(); }
+  __host__ __device__ void seed(result_type s) { b1_.seed(s); b2_.seed(s); }
+  __host__ __device__ const base1_type& base1() const { return b1_; }
+  __host__ __device__ const base2_type& base2() const { return b2_; }
+  __host__ __device__ result_type operator()() {
+    return (result_type)((result_type(b1_() - base1_type::min) << shift1) ^ (result_type(b2_() - base2_type::min) << shift2));
+  }
+  __host__ __device__ void discard(unsigned long long z) {
+    for (; z > 0; --z) (*this)();
+  }
+  __host__ __device__ friend bool operator==(const xor_combine_engine& a, const xor_combine_engine& b) {
+    return a.b1_ == b.b1_ && a.b2_ == b.b2_;
+  }
+  __host__ __device__ friend bool operator!=(const xor_combine_engine& a, const xor_combine_engine& b) { return !(a == b); }
+
+ private:
+  base1_type b1_;
+  base2_type b2_;
+};
+template <typename E1, std::size_t s1, typename E2, std::size_t s2>
+const typename xor_combine_engine<E1, s1, E2, s2>::result_type xor_combine_engine<E1, s1, E2, s2>::min;
+template <typename E1, std::size_t s1, typename E2, std::size_t s2>
+const typename xor_combine_engine<E1, s1, E2, s2>::result_type xor_combine_engine<E1, s1, E2, s2>::max;
+
+// The engines with predefined parameters and the 10000th draw of a default-constructed one
+// (thrust/random.h:60-100, subtract_with_carry_engine.h:225-245): ranlux24_base 7937952,
+// ranlux48_base 192113843633948, ranlux24 9901578, ranlux48 88229545517833, taus88 3535848941.
+typedef subtract_with_carry_engine<std::uint32_t, 24, 10, 24> ranlux24_base;
+typedef subtract_with_carry_engine<std::uint64_t, 48, 5, 12> ranlux48_base;
+typedef discard_block_engine<ranlux24_base, 223, 23> ranlux24;
+typedef discard_block_engine<ranlux48_base, 389, 11> ranlux48;
+typedef xor_combine_engine<linear_feedback_shift_engine<std::uint32_t, 32u, 31u, 13u, 12u>, 0,
+                           xor_combine_engine<linear_feedback_shift_engine<std::uint32_t, 32u, 29u, 2u, 4u>, 0,
+                                              linear_feedback_shift_engine<std::uint32_t, 32u, 28u, 3u, 17u>, 0>,
+                           0>
+    taus88;
 
 // A real number in [a, b): the engine's draw, shifted to start at zero, over the number of values it can take.
 template <typename RealType = double>
@@ -229,6 +439,15 @@ class normal_distribution {
 }  // namespace random
 
 using random::default_random_engine;
+using random::discard_block_engine;
+using random::linear_feedback_shift_engine;
+using random::ranlux24;
+using random::ranlux24_base;
+using random::ranlux48;
+using random::ranlux48_base;
+using random::subtract_with_carry_engine;
+using random::taus88;
+using random::xor_combine_engine;
 using random::linear_congruential_engine;
 using random::minstd_rand;
 using random::minstd_rand0;

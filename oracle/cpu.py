@@ -337,6 +337,19 @@ class Reference(_Base):
                  "reduce_mixed")
         return out[0]
 
+    # thrust::shuffle_copy / thrust::shuffle with thrust::default_random_engine(seed).
+    def shuffle_copy(self, x, seed):
+        x = _c(x)
+        out = np.empty_like(x)
+        self._ok(self._fn("shuffle_copy")(_p(x), _p(out), ctypes.c_uint64(x.size), _code(x), ctypes.c_uint32(seed)),
+                 "shuffle_copy")
+        return out
+
+    def shuffle(self, x, seed):
+        out = _c(x).copy()
+        self._ok(self._fn("shuffle")(_p(out), ctypes.c_uint64(out.size), _code(out), ctypes.c_uint32(seed)), "shuffle")
+        return out
+
     def _scan_mixed(self, x, out_dtype, exclusive, init):
         x = _c(x)
         out = np.empty(x.size, out_dtype)

@@ -23,7 +23,9 @@
 #include <thrust/partition.h>
 #include <thrust/reduce.h>
 #include <thrust/scan.h>
+#include <thrust/random.h>
 #include <thrust/set_operations.h>
+#include <thrust/shuffle.h>
 #include <thrust/sort.h>
 #include <thrust/transform_reduce.h>
 #include <thrust/transform_scan.h>
@@ -586,3 +588,24 @@ REF_API int ref_exclusive_scan_by_key(const void* keys, const void* values, void
     });
   });
 }
+
+// thrust::shuffle_copy with thrust::default_random_engine(seed): the permutation the library
+// draws for that generator (in and out may not overlap).
+REF_API int ref_shuffle_copy(const void* in, void* out, uint64_t n, int dtype, uint32_t seed) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    thrust::default_random_engine g(seed);
+    thrust::shuffle_copy(DRIVER_POLICY, dp<T>(in), dp<T>(in) + n, dp<T>(out), g);
+    return 0;
+  });
+}
+// thrust::shuffle in place, same generator.
+REF_API int ref_shuffle(void* data, uint64_t n, int dtype, uint32_t seed) {
+  return with_dtype(dtype, [&](auto z) {
+    using T = decltype(z);
+    thrust::default_random_engine g(seed);
+    thrust::shuffle(DRIVER_POLICY, dp<T>(data), dp<T>(data) + n, g);
+    return 0;
+  });
+}
+

@@ -7,6 +7,9 @@
 #include <thrust/host_vector.h>
 #include <thrust/iterator/counting_iterator.h>
 #include <thrust/random.h>
+#include <thrust/sequence.h>
+#include <thrust/shuffle.h>
+#include <thrust/sort.h>
 #include <thrust/transform.h>
 #include <thrust/transform_reduce.h>
 
@@ -120,6 +123,25 @@ struct squared_distance_from_ten {
   __host__ __device__ double operator()(double x) const { return (x - 10.0) * (x - 10.0); }
 };
 
+// what holds for any engine: discard against drawing, equality of equal histories, reseeding
+template <typename Engine>
+struct validate_histories {
+  __host__ __device__ bool operator()() const {
+    Engine e0, e1;
+    bool ok = e0 == e1;
+    for (int i = 0; i < 1000; ++i) e0();
+    ok &= e0 != e1;
+    e1.discard(1000);
+    ok &= e0 == e1 && e0() == e1();
+    Engine e2(13), e3(13), e4(7);
+    ok &= e2 == e3 && e2 != e4 && e2() == e3();
+    e4.seed(13);
+    e4();
+    ok &= e4 == e2;
+    return ok;
+  }
+};
+
 template <typename Vector, typename Check>
 static bool holds_on(Check check) {
   Vector flag(1);
@@ -148,6 +170,104 @@ int main() {
     thrust::linear_congruential_engine<std::uint32_t, 1664525u, 1013904223u, 0u> skipped(1);
     skipped.discard(2);
     ASSERT_TRUE(skipped == lcg);
+  }
+
+  g_test = "the other engines";
+  // the 10000th draw of each engine with predefined parameters (thrust/random.h:60-100,
+  // thrust/random/subtract_with_carry_engine.h:225-245; testing/random.cu:237-360)
+  ASSERT_TRUE((holds_on<thrust::host_vector<bool> >(validate_engine<thrust::ranlux24_base>{7937952u})));
+  ASSERT_TRUE((holds_on<thrust::device_vector<bool> >(validate_engine<thrust::ranlux24_base>{7937952u})));
+  ASSERT_TRUE((holds_on<thrust::host_vector<bool> >(validate_engine<thrust::ranlux48_base>{192113843633948ull})));
+  ASSERT_TRUE((holds_on<thrust::device_vector<bool> >(validate_engine<thrust::ranlux48_base>{192113843633948ull})));
+  ASSERT_TRUE((holds_on<thrust::host_vector<bool> >(validate_engine<thrust::ranlux24>{9901578u})));
+  ASSERT_TRUE((holds_on<thrust::device_vector<bool> >(validate_engine<thrust::ranlux24>{9901578u})));
+  ASSERT_TRUE((holds_on<thrust::host_vector<bool> >(validate_engine<thrust::ranlux48>{88229545517833ull})));
+  ASSERT_TRUE((holds_on<thrust::device_vector<bool> >(validate_engine<thrust::ranlux48>{88229545517833ull})));
+  ASSERT_TRUE((holds_on<thrust::host_vector<bool> >(validate_engine<thrust::taus88>{3535848941u})));
+  ASSERT_TRUE((holds_on<thrust::device_vector<bool> >(validate_engine<thrust::taus88>{3535848941u})));
+  ASSERT_TRUE((holds_on<thrust::host_vector<bool> >(validate_by_drawing<thrust::ranlux24>{9901578u})));
+  ASSERT_TRUE((holds_on<thrust::device_vector<bool> >(validate_by_drawing<thrust::taus88>{3535848941u})));
+  ASSERT_TRUE((holds_on<thrust::host_vector<bool> >(validate_histories<thrust::ranlux24_base>())));
+  ASSERT_TRUE((holds_on<thrust::device_vector<bool> >(validate_histories<thrust::ranlux24_base>())));
+  ASSERT_TRUE((holds_on<thrust::host_vector<bool> >(validate_histories<thrust::ranlux48>())));
+  ASSERT_TRUE((holds_on<thrust::device_vector<bool> >(validate_histories<thrust::ranlux48>())));
+  ASSERT_TRUE((holds_on<thrust::host_vector<bool> >(validate_histories<thrust::taus88>())));
+  ASSERT_TRUE((holds_on<thrust::device_vector<bool> >(validate_histories<thrust::taus88>())));
+  ASSERT_EQUAL(thrust::ranlux24_base::max, (1u << 24) - 1);
+  ASSERT_EQUAL(thrust::ranlux48::max, (1ull << 48) - 1);
+  ASSERT_EQUAL(thrust::taus88::min, 0u);
+
+  g_test = "shuffle";
+  {
+    // every element once, and the copying form draws what the in-place form draws
+    // (testing/shuffle.cu:327-360)
+    thrust::device_vector<int> data(5), shuffled(5), again(5);
+    thrust::sequence(data.begin(), data.end());
+    shuffled = data;
+    thrust::default_random_engine g(2);
+    thrust::shuffle(shuffled.begin(), shuffled.end(), g);
+    g.seed(2);
+    thrust::shuffle_copy(data.begin(), data.end(), again.begin(), g);
+    ASSERT_TRUE(shuffled == again);
+    thrust::sort(shuffled.begin(), shuffled.end());
+    ASSERT_TRUE(shuffled == data);
+    // the permutation the reference draws for this generator (its CPP system, five elements, seed 2)
+    const int drawn[] = {3, 0, 1, 2, 4};
+    ASSERT_TRUE(again == thrust::host_vector<int>(drawn, drawn + 5));
+    // the generator has moved on by the sixteen keys of the network
+    thrust::default_random_engine sixteen(2);
+    sixteen.discard(16);
+    ASSERT_TRUE(g == sixteen);
+  }
+  for (size_t m : {size_t(0), size_t(1), size_t(2), size_t(3), size_t(31), size_t(32), size_t(33), size_t(1000), size_t(4097),
+                   size_t(100000), size_t(1) << 20}) {
+    // host and device draw the same permutation (testing/shuffle.cu:362-376), of any element type
+    thrust::host_vector<long long> h(m);
+    thrust::sequence(h.begin(), h.end());
+    thrust::device_vector<long long> d(h);
+    thrust::default_random_engine host_g(183), device_g(183);
+    thrust::shuffle(h.begin(), h.end(), host_g);
+    thrust::shuffle(d.begin(), d.end(), device_g);
+    ASSERT_TRUE(d == h);
+    ASSERT_TRUE(host_g == device_g);
+    thrust::sort(d.begin(), d.end());
+    bool every = true;
+    thrust::host_vector<long long> sorted(d);
+    for (size_t i = 0; i < m; ++i) every &= sorted[i] == (long long)i;
+    ASSERT_TRUE(every);
+    if (m > 32) {  // not the identity, and not the same for another seed
+      thrust::host_vector<long long> other(m);
+      thrust::sequence(other.begin(), other.end());
+      thrust::default_random_engine other_g(184);
+      thrust::shuffle(other.begin(), other.end(), other_g);
+      ASSERT_TRUE(!(other == h));
+      ASSERT_TRUE(!(sorted == h));
+    }
+  }
+  {
+    // the network is a bijection of [0, 2^bits) and knows its length (testing/shuffle.cu:378-425)
+    thrust::default_random_engine g(0xD5);
+    ASSERT_EQUAL(thrust::detail::feistel_bijection(3, g).nearest_power_of_two(), 4u);
+    ASSERT_EQUAL(thrust::detail::feistel_bijection(2, g).nearest_power_of_two(), 2u);
+    ASSERT_EQUAL(thrust::detail::feistel_bijection(0, g).nearest_power_of_two(), 1u);
+    for (std::uint64_t m : {5ull, 64ull, 1000ull, 40000ull}) {
+      thrust::default_random_engine host_g(0xD5), device_g(0xD5);
+      const thrust::detail::image_under host_f = {thrust::detail::feistel_bijection(m, host_g)};
+      const thrust::detail::image_under device_f = {thrust::detail::feistel_bijection(m, device_g)};
+      const std::uint64_t n = host_f.bijection.nearest_power_of_two();
+      thrust::host_vector<std::uint64_t> hr(n);
+      thrust::device_vector<std::uint64_t> dr(n);
+      thrust::sequence(hr.begin(), hr.end());
+      thrust::sequence(dr.begin(), dr.end());
+      thrust::transform(hr.begin(), hr.end(), hr.begin(), host_f);
+      thrust::transform(dr.begin(), dr.end(), dr.begin(), device_f);
+      ASSERT_TRUE(dr == hr);
+      thrust::sort(dr.begin(), dr.end());
+      thrust::host_vector<std::uint64_t> once(dr);
+      bool every = true;
+      for (std::uint64_t i = 0; i < n; ++i) every &= once[i] == i;
+      ASSERT_TRUE(every);
+    }
   }
 
   g_test = "distributions";

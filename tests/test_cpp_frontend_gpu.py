@@ -119,7 +119,10 @@ def test_conditional_forms_and_reverse_iterator():
 def test_random_engines_and_distributions():
     # thrust::random: the 10000th draw of minstd_rand0 / minstd_rand (the standard's validation values) on the host and
     # in device code, discard against drawing, equality, the ranges of uniform_real / uniform_int, normal deviates, and
-    # the stream made by one seed-discard-draw functor per element (identical on both sides)
+    # the stream made by one seed-discard-draw functor per element (identical on both sides); the 10000th draw of
+    # ranlux24_base, ranlux48_base, ranlux24, ranlux48 and taus88 on both sides; thrust::shuffle / shuffle_copy: a
+    # permutation, the same on host and device, the one the reference draws for five elements and seed 2, the generator
+    # advanced by sixteen draws, and the Feistel network a bijection of the same images on both sides
     out = _run("test_random")
     assert "PASSED" in out
 

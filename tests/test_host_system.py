@@ -256,3 +256,31 @@ def test_host_only_program():
     res = subprocess.run([prog], capture_output=True, text=True, timeout=60)
     assert res.returncode == 0, res.stdout + res.stderr
     assert " 0 failed" in res.stdout
+
+
+# ------------------------------------------------------------------ shuffle
+SHUFFLE_FIXTURE = os.path.join(HERE, "golden", "shuffle_permutations.npz")
+
+
+def test_shuffle_copy_draws_the_permutations_the_reference_drew(front):
+    # tests/golden/shuffle_permutations.npz: the real reference's shuffle_copy of 0 .. n-1 with
+    # default_random_engine(seed) (tests/golden/make_shuffle_vectors.py made it)
+    with np.load(SHUFFLE_FIXTURE) as z:
+        assert len(z.files) == 12
+        for name in z.files:
+            n, seed = int(name.split("_")[0][1:]), int(name.split("seed")[1])
+            x = np.arange(n, dtype=np.uint32)
+            same(front.shuffle_copy(x, seed), z[name])
+            same(front.shuffle(x, seed), z[name])  # in place: the same draw
+            assert np.array_equal(np.sort(z[name]), x)
+
+
+@pytest.mark.parametrize("dtype", [np.uint8, np.int16, np.float32, np.int64, np.float64])
+@pytest.mark.parametrize("n,seed", [(1, 3), (6, 0), (255, 77), (1025, 2), (30000, 99)])
+def test_shuffle_against_the_real_reference(front, dtype, n, seed):
+    if not cpu.ref_available("cpp"):
+        pytest.skip("the reference build is not here; the fixture test above holds its permutations")
+    want = cpu.Reference("cpp")
+    x = (rng(seed).integers(0, 200, n)).astype(dtype)
+    same(front.shuffle_copy(x, seed), want.shuffle_copy(x, seed))
+    same(front.shuffle(x, seed), want.shuffle(x, seed))
