@@ -92,6 +92,26 @@ class linear_congruential_engine {
     return l.x_ != r.x_;
   }
 
+  // the state as text, and back (thrust/random/detail/*_engine.inl: stream_out / stream_in)
+  template <typename CharT, typename Traits>
+  friend std::basic_ostream<CharT, Traits>& operator<<(std::basic_ostream<CharT, Traits>& os, const linear_congruential_engine& e) {
+    const typename std::basic_ostream<CharT, Traits>::fmtflags flags = os.flags();
+    const CharT fill = os.fill();
+    os.flags(std::ios_base::dec | std::ios_base::fixed | std::ios_base::left);
+    os.fill(os.widen(' '));
+    os << e.x_;
+    os.flags(flags);
+    os.fill(fill);
+    return os;
+  }
+  template <typename CharT, typename Traits>
+  friend std::basic_istream<CharT, Traits>& operator>>(std::basic_istream<CharT, Traits>& is, linear_congruential_engine& e) {
+    const typename std::basic_istream<CharT, Traits>::fmtflags flags = is.flags();
+    is.flags(std::ios_base::dec | std::ios_base::skipws);
+    is >> e.x_;
+    is.flags(flags);
+    return is;
+  }
  private:
   result_type x_;
 };
@@ -142,6 +162,26 @@ class linear_feedback_shift_engine {
     return !(a == b);
   }
 
+  // the state as text, and back (thrust/random/detail/*_engine.inl: stream_out / stream_in)
+  template <typename CharT, typename Traits>
+  friend std::basic_ostream<CharT, Traits>& operator<<(std::basic_ostream<CharT, Traits>& os, const linear_feedback_shift_engine& e) {
+    const typename std::basic_ostream<CharT, Traits>::fmtflags flags = os.flags();
+    const CharT fill = os.fill();
+    os.flags(std::ios_base::dec | std::ios_base::fixed | std::ios_base::left);
+    os.fill(os.widen(' '));
+    os << e.x_;
+    os.flags(flags);
+    os.fill(fill);
+    return os;
+  }
+  template <typename CharT, typename Traits>
+  friend std::basic_istream<CharT, Traits>& operator>>(std::basic_istream<CharT, Traits>& is, linear_feedback_shift_engine& e) {
+    const typename std::basic_istream<CharT, Traits>::fmtflags flags = is.flags();
+    is.flags(std::ios_base::dec | std::ios_base::skipws);
+    is >> e.x_;
+    is.flags(flags);
+    return is;
+  }
  private:
   result_type x_;
 };
@@ -203,6 +243,29 @@ class subtract_with_carry_engine {
     return !(a == b);
   }
 
+  // the state as text, and back (thrust/random/detail/*_engine.inl: stream_out / stream_in)
+  template <typename CharT, typename Traits>
+  friend std::basic_ostream<CharT, Traits>& operator<<(std::basic_ostream<CharT, Traits>& os, const subtract_with_carry_engine& e) {
+    const typename std::basic_ostream<CharT, Traits>::fmtflags flags = os.flags();
+    const CharT fill = os.fill();
+    os.flags(std::ios_base::dec | std::ios_base::fixed | std::ios_base::left);
+    os.fill(os.widen(' '));
+    for (std::size_t i = 0; i < r; ++i) os << e.x_[(i + e.k_) % r] << os.widen(' ');
+    os << e.carry_;
+    os.flags(flags);
+    os.fill(fill);
+    return os;
+  }
+  template <typename CharT, typename Traits>
+  friend std::basic_istream<CharT, Traits>& operator>>(std::basic_istream<CharT, Traits>& is, subtract_with_carry_engine& e) {
+    const typename std::basic_istream<CharT, Traits>::fmtflags flags = is.flags();
+    is.flags(std::ios_base::dec | std::ios_base::skipws);
+    for (std::size_t i = 0; i < r; ++i) is >> e.x_[i];
+    is >> e.carry_;
+    e.k_ = 0;
+    is.flags(flags);
+    return is;
+  }
  private:
   result_type x_[r];
   result_type carry_;
@@ -246,6 +309,26 @@ class discard_block_engine {
   }
   __host__ __device__ friend bool operator!=(const discard_block_engine& a, const discard_block_engine& b) { return !(a == b); }
 
+  // the state as text, and back (thrust/random/detail/*_engine.inl: stream_out / stream_in)
+  template <typename CharT, typename Traits>
+  friend std::basic_ostream<CharT, Traits>& operator<<(std::basic_ostream<CharT, Traits>& os, const discard_block_engine& e) {
+    const typename std::basic_ostream<CharT, Traits>::fmtflags flags = os.flags();
+    const CharT fill = os.fill();
+    os.flags(std::ios_base::dec | std::ios_base::fixed | std::ios_base::left);
+    os.fill(os.widen(' '));
+    os << e.e_ << os.widen(' ') << e.n_;
+    os.flags(flags);
+    os.fill(fill);
+    return os;
+  }
+  template <typename CharT, typename Traits>
+  friend std::basic_istream<CharT, Traits>& operator>>(std::basic_istream<CharT, Traits>& is, discard_block_engine& e) {
+    const typename std::basic_istream<CharT, Traits>::fmtflags flags = is.flags();
+    is.flags(std::ios_base::dec | std::ios_base::skipws);
+    is >> e.e_ >> e.n_;
+    is.flags(flags);
+    return is;
+  }
  private:
   base_type e_;
   unsigned int n_;
@@ -294,6 +377,26 @@ class xor_combine_engine {
   }
   __host__ __device__ friend bool operator!=(const xor_combine_engine& a, const xor_combine_engine& b) { return !(a == b); }
 
+  // the state as text, and back (thrust/random/detail/*_engine.inl: stream_out / stream_in)
+  template <typename CharT, typename Traits>
+  friend std::basic_ostream<CharT, Traits>& operator<<(std::basic_ostream<CharT, Traits>& os, const xor_combine_engine& e) {
+    const typename std::basic_ostream<CharT, Traits>::fmtflags flags = os.flags();
+    const CharT fill = os.fill();
+    os.flags(std::ios_base::dec | std::ios_base::fixed | std::ios_base::left);
+    os.fill(os.widen(' '));
+    os << e.b1_ << os.widen(' ') << e.b2_;
+    os.flags(flags);
+    os.fill(fill);
+    return os;
+  }
+  template <typename CharT, typename Traits>
+  friend std::basic_istream<CharT, Traits>& operator>>(std::basic_istream<CharT, Traits>& is, xor_combine_engine& e) {
+    const typename std::basic_istream<CharT, Traits>::fmtflags flags = is.flags();
+    is.flags(std::ios_base::dec | std::ios_base::skipws);
+    is >> e.b1_ >> e.b2_;
+    is.flags(flags);
+    return is;
+  }
  private:
   base1_type b1_;
   base2_type b2_;
@@ -346,6 +449,26 @@ class uniform_real_distribution {
     return !(l == r);
   }
 
+  // the parameters as text, and back (the two parameters)
+  template <typename CharT, typename Traits>
+  friend std::basic_ostream<CharT, Traits>& operator<<(std::basic_ostream<CharT, Traits>& os, const uniform_real_distribution& e) {
+    const typename std::basic_ostream<CharT, Traits>::fmtflags flags = os.flags();
+    const CharT fill = os.fill();
+    os.flags(std::ios_base::dec | std::ios_base::fixed | std::ios_base::left);
+    os.fill(os.widen(' '));
+    os << e.param_.first << os.widen(' ') << e.param_.second;
+    os.flags(flags);
+    os.fill(fill);
+    return os;
+  }
+  template <typename CharT, typename Traits>
+  friend std::basic_istream<CharT, Traits>& operator>>(std::basic_istream<CharT, Traits>& is, uniform_real_distribution& e) {
+    const typename std::basic_istream<CharT, Traits>::fmtflags flags = is.flags();
+    is.flags(std::ios_base::dec | std::ios_base::skipws);
+    is >> e.param_.first >> e.param_.second;
+    is.flags(flags);
+    return is;
+  }
  private:
   param_type param_;
 };
@@ -380,6 +503,26 @@ class uniform_int_distribution {
     return !(l == r);
   }
 
+  // the parameters as text, and back (the two parameters)
+  template <typename CharT, typename Traits>
+  friend std::basic_ostream<CharT, Traits>& operator<<(std::basic_ostream<CharT, Traits>& os, const uniform_int_distribution& e) {
+    const typename std::basic_ostream<CharT, Traits>::fmtflags flags = os.flags();
+    const CharT fill = os.fill();
+    os.flags(std::ios_base::dec | std::ios_base::fixed | std::ios_base::left);
+    os.fill(os.widen(' '));
+    os << e.param_.first << os.widen(' ') << e.param_.second;
+    os.flags(flags);
+    os.fill(fill);
+    return os;
+  }
+  template <typename CharT, typename Traits>
+  friend std::basic_istream<CharT, Traits>& operator>>(std::basic_istream<CharT, Traits>& is, uniform_int_distribution& e) {
+    const typename std::basic_istream<CharT, Traits>::fmtflags flags = is.flags();
+    is.flags(std::ios_base::dec | std::ios_base::skipws);
+    is >> e.param_.first >> e.param_.second;
+    is.flags(flags);
+    return is;
+  }
  private:
   param_type param_;
 };
@@ -430,6 +573,26 @@ class normal_distribution {
     return !(l == r);
   }
 
+  // the parameters as text, and back (mean and standard deviation)
+  template <typename CharT, typename Traits>
+  friend std::basic_ostream<CharT, Traits>& operator<<(std::basic_ostream<CharT, Traits>& os, const normal_distribution& e) {
+    const typename std::basic_ostream<CharT, Traits>::fmtflags flags = os.flags();
+    const CharT fill = os.fill();
+    os.flags(std::ios_base::dec | std::ios_base::fixed | std::ios_base::left);
+    os.fill(os.widen(' '));
+    os << e.param_.first << os.widen(' ') << e.param_.second;
+    os.flags(flags);
+    os.fill(fill);
+    return os;
+  }
+  template <typename CharT, typename Traits>
+  friend std::basic_istream<CharT, Traits>& operator>>(std::basic_istream<CharT, Traits>& is, normal_distribution& e) {
+    const typename std::basic_istream<CharT, Traits>::fmtflags flags = is.flags();
+    is.flags(std::ios_base::dec | std::ios_base::skipws);
+    is >> e.param_.first >> e.param_.second;
+    is.flags(flags);
+    return is;
+  }
  private:
   param_type param_;
   RealType r1_, r2_, rho_;

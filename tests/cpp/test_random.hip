@@ -18,6 +18,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <sstream>
 
 static int g_failed = 0, g_checks = 0;
 static const char* g_test = "";
@@ -142,6 +143,20 @@ struct validate_histories {
   }
 };
 
+// written out after 10000 draws and read into an engine with another history: the same engine
+// (testing/random.cu: the save / restore cases of every engine)
+template <typename Engine>
+static bool saves_and_restores() {
+  Engine e0;
+  e0.discard(10000);
+  std::stringstream text;
+  text << e0;
+  Engine e1(7);
+  e1.discard(3);
+  text >> e1;
+  return e0 == e1 && e0() == e1();
+}
+
 template <typename Vector, typename Check>
 static bool holds_on(Check check) {
   Vector flag(1);
@@ -196,6 +211,27 @@ int main() {
   ASSERT_EQUAL(thrust::ranlux24_base::max, (1u << 24) - 1);
   ASSERT_EQUAL(thrust::ranlux48::max, (1ull << 48) - 1);
   ASSERT_EQUAL(thrust::taus88::min, 0u);
+
+  g_test = "save and restore";
+  ASSERT_TRUE(saves_and_restores<thrust::minstd_rand0>());
+  ASSERT_TRUE(saves_and_restores<thrust::minstd_rand>());
+  ASSERT_TRUE(saves_and_restores<thrust::ranlux24_base>());
+  ASSERT_TRUE(saves_and_restores<thrust::ranlux48_base>());
+  ASSERT_TRUE(saves_and_restores<thrust::ranlux24>());
+  ASSERT_TRUE(saves_and_restores<thrust::ranlux48>());
+  ASSERT_TRUE(saves_and_restores<thrust::taus88>());
+  {
+    std::stringstream text;
+    text << thrust::uniform_real_distribution<float>(2.0f, 5.0f) << ' ' << thrust::uniform_int_distribution<int>(-3, 9) << ' '
+         << thrust::normal_distribution<double>(1.5, 2.5);
+    thrust::uniform_real_distribution<float> real;
+    thrust::uniform_int_distribution<int> whole;
+    thrust::normal_distribution<double> normal;
+    text >> real >> whole >> normal;
+    ASSERT_TRUE(real.a() == 2.0f && real.b() == 5.0f);
+    ASSERT_TRUE(whole.a() == -3 && whole.b() == 9);
+    ASSERT_TRUE(normal.mean() == 1.5 && normal.stddev() == 2.5);
+  }
 
   g_test = "shuffle";
   {
