@@ -13,7 +13,7 @@
 //
 // Ranking inside a tile uses the wave64 match pattern: for each of the 8 digit bits one
 // ballot, folded into a 64-bit peer mask with v_bitop3; rank = wave-private LDS counter
-// + number of peers in lower lanes.  Lanes hold keys wave-striped (lane l of wave w holds
+// + number of peers in lower lanes (v_mbcnt accumulates onto the counter's value).  Lanes hold keys wave-striped (lane l of wave w holds
 // keys l, 64+l, ... of the wave's span), so (round, lane) order is memory order and the
 // pass is stable.  Keys and values are then exchanged through LDS so that global stores
 // are contiguous per digit run.
@@ -264,7 +264,10 @@ struct PassShape {
 // Tile descriptors fetched together per look-back round by each digit thread.
 constexpr int LOOKBACK_WINDOW = 4;
 
-template <typename K, typename V, bool HAS_VALUES, int BLOCK, int ITEMS, typename D>
+// OFF32: every key and value of the call lies within 4 GiB of its array's start, so that
+// global addresses are a scalar base plus a 32-bit byte offset (one vector instruction per
+// access less than with 64-bit address arithmetic).
+template <typename K, typename V, bool HAS_VALUES, int BLOCK, int ITEMS, typename D, bool OFF32>
 __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     K* __restrict__ keys_a, K* __restrict__ keys_b, V* __restrict__ vals_a, V* __restrict__ vals_b,
     uint32_t n, int pass, SortGeometry geo, KeyCodec<K> codec,
@@ -297,7 +300,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   }
   for (int i = threadIdx.x; i < WAVES * RADIX_SIZE; i += BLOCK) s_cnt[i] = 0;
   __syncthreads();
-  const uint32_t tile = s_tile;
+  const uint32_t tile = __builtin_amdgcn_readfirstlane(s_tile);
   const uint32_t tile_base = tile * (uint32_t)TILE;
   const uint32_t valid = (n - tile_base < (uint32_t)TILE) ? (n - tile_base) : (uint32_t)TILE;
   const int wave = threadIdx.x / WAVE;
@@ -307,6 +310,20 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   const int shift = geo.begin_bit + pass * RADIX_BITS;
   const int nbits = (geo.end_bit - shift) < RADIX_BITS ? (geo.end_bit - shift) : RADIX_BITS;
   const uint32_t dmask = (1u << nbits) - 1u;
+  auto digit_of = [&](K x) -> uint32_t {
+    if constexpr (sizeof(K) == 8) return __builtin_amdgcn_ubfe((uint32_t)(x >> shift), 0u, (uint32_t)nbits);
+    else return __builtin_amdgcn_ubfe((uint32_t)x, (uint32_t)shift, (uint32_t)nbits);
+  };
+  // element i of an array, addressed the cheaper way where the offsets allow it
+  auto at = [&](auto* base, uint32_t i) -> auto& {
+    using T = std::remove_reference_t<decltype(*base)>;
+    if constexpr (OFF32) {
+      using B = std::conditional_t<std::is_const<T>::value, const char, char>;
+      return *reinterpret_cast<T*>(reinterpret_cast<B*>(base) + (uint32_t)(i * (uint32_t)sizeof(T)));
+    } else {
+      return base[i];
+    }
+  };
 
   // Keys travel between the passes in their encoded form: the first pass that runs encodes them as
   // it loads, the last one decodes them as it stores (unsigned ascending keys need no transform).
@@ -322,8 +339,9 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   // ---- load (wave-striped); slots past the end sort last inside the tile
   K e[ITEMS];
   if (valid == (uint32_t)TILE) {
+    const K* __restrict__ tile_keys = keys_in + tile_base;  // scalar
 #pragma unroll
-    for (int r = 0; r < ITEMS; ++r) e[r] = keys_in[tile_base + span + r * WAVE];
+    for (int r = 0; r < ITEMS; ++r) e[r] = at(tile_keys, span + r * WAVE);
     if (encodes) {
 #pragma unroll
       for (int r = 0; r < ITEMS; ++r) e[r] = codec.encode(e[r]);
@@ -349,8 +367,9 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     if (valid == (uint32_t)TILE) {
       // whole tile: no predicates, so that all loads are in flight together (a predicated
       // load makes the compiler wait for it before issuing the next one)
+      const V* __restrict__ tile_vals = vals_in + tile_base;  // scalar
 #pragma unroll
-      for (int r = 0; r < ITEMS; ++r) v[r] = vals_in[tile_base + span + r * WAVE];
+      for (int r = 0; r < ITEMS; ++r) v[r] = at(tile_vals, span + r * WAVE);
     } else {
 #pragma unroll
       for (int r = 0; r < ITEMS; ++r) {
@@ -362,16 +381,17 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
 
   // ---- rank inside the wave by digit
   // Per digit bit: v_bfe_i32 (lane's bit as 0 / -1), one ballot, and two v_bitop3 folding
-  // "same bit as mine" into the 64-bit peer mask.  The wave-private counter is read, then
-  // bumped by one per peer with an LDS atomic; LDS executes a wave's instructions in
-  // order, so the next round reads the updated count.
+  // "same bit as mine" into the 64-bit peer mask.  The wave-private counter is read by every
+  // lane and then raised by the size of the peer group; LDS executes a wave's instructions
+  // in order, so the next round reads the updated count.
   uint32_t* my_cnt = s_cnt + wave * RADIX_SIZE;
   // ranks are < TILE <= 65536: two per register
   static_assert(TILE <= 65536 && ITEMS % 2 == 0, "rank packing");
   uint32_t rank2[ITEMS / 2];
 #pragma unroll
   for (int r = 0; r < ITEMS; ++r) {
-    const uint32_t d = (uint32_t)(e[r] >> shift) & dmask;
+    const uint32_t d = digit_of(e[r]);
+    const uint32_t old = my_cnt[d];
     uint32_t peers_lo = ~0u, peers_hi = ~0u;
 #pragma unroll
     for (int b = 0; b < RADIX_BITS; ++b) {
@@ -382,11 +402,14 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
       peers_lo = __builtin_amdgcn_bitop3_b32(peers_lo, (uint32_t)m, (uint32_t)sb, BITOP_AND_XNOR);
       peers_hi = __builtin_amdgcn_bitop3_b32(peers_hi, (uint32_t)(m >> 32), (uint32_t)sb, BITOP_AND_XNOR);
     }
-    const uint32_t below = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, 0u));
-    const uint32_t old = my_cnt[d];
-    __hip_atomic_fetch_add(&my_cnt[d], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (r % 2 == 0) rank2[r / 2] = old + below;
-    else rank2[r / 2] |= (old + below) << 16;
+    // the count of peers in lower lanes is accumulated onto the counter's value
+    const uint32_t rank = __builtin_amdgcn_mbcnt_hi(peers_hi, __builtin_amdgcn_mbcnt_lo(peers_lo, old));
+    // The lowest lane of every group of peers bumps the counter for all of them: one LDS
+    // write per distinct digit instead of an atomic per key, which an LDS bank serialises
+    // when many lanes hold the same digit (float exponents, skewed keys).
+    if (rank == old) my_cnt[d] = old + (uint32_t)__builtin_popcount(peers_lo) + (uint32_t)__builtin_popcount(peers_hi);
+    if (r % 2 == 0) rank2[r / 2] = rank;
+    else rank2[r / 2] |= rank << 16;
     // pin the packed rank here: otherwise the add is sunk past the barrier and `old` and
     // `below` of every round stay live
     asm volatile("" : "+v"(rank2[r / 2]));
@@ -434,7 +457,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   // ---- final position of every key inside the tile
 #pragma unroll
   for (int r = 0; r < ITEMS; ++r) {
-    const uint32_t d = (uint32_t)(e[r] >> shift) & dmask;
+    const uint32_t d = digit_of(e[r]);
     rank2[r / 2] += my_cnt[d] << (16 * (r % 2));  // no carry: each half stays < TILE
   }
   __syncthreads();  // all reads of s_cnt done: the exchange buffer may overwrite it
@@ -485,7 +508,8 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     }
     __hip_atomic_store(my_status + d, (D)(Desc::INCLUSIVE | (D)(uint32_t)(excl + digit_count)), __ATOMIC_RELAXED,
                        __HIP_MEMORY_SCOPE_AGENT);
-    s_scatter_base[d] = excl - local_base;
+    // (in bytes of a key where the offsets are 32-bit)
+    s_scatter_base[d] = OFF32 ? (excl - local_base) * (uint32_t)sizeof(K) : excl - local_base;
   }
   __syncthreads();
 
@@ -496,20 +520,27 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     K ek[ITEMS];
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) ek[k] = s_keys[(uint32_t)k * BLOCK + threadIdx.x];
+    // gpos: the key's place in the output, as a byte offset where those fit 32 bits
+    auto key_slot = [&](uint32_t g) -> K& {
+      if constexpr (OFF32) return *reinterpret_cast<K*>(reinterpret_cast<char*>(keys_out) + g);
+      else return keys_out[g];
+    };
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k)
-      gpos[k] = s_scatter_base[(uint32_t)(ek[k] >> shift) & dmask] + (uint32_t)k * BLOCK + threadIdx.x;
+      gpos[k] = s_scatter_base[digit_of(ek[k])] +
+                (OFF32 ? (uint32_t)(threadIdx.x * sizeof(K)) + (uint32_t)(k * BLOCK * sizeof(K))
+                       : (uint32_t)k * BLOCK + threadIdx.x);
     if (decodes) {
 #pragma unroll
       for (int k = 0; k < ITEMS; ++k) ek[k] = codec.decode(ek[k]);
     }
     if (valid == (uint32_t)TILE) {
 #pragma unroll
-      for (int k = 0; k < ITEMS; ++k) keys_out[gpos[k]] = ek[k];
+      for (int k = 0; k < ITEMS; ++k) key_slot(gpos[k]) = ek[k];
     } else {
 #pragma unroll
       for (int k = 0; k < ITEMS; ++k)
-        if ((uint32_t)k * BLOCK + threadIdx.x < valid) keys_out[gpos[k]] = ek[k];
+        if ((uint32_t)k * BLOCK + threadIdx.x < valid) key_slot(gpos[k]) = ek[k];
     }
   }
   if constexpr (HAS_VALUES) {
@@ -520,7 +551,14 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
 #pragma unroll
     for (int k = 0; k < ITEMS; ++k) {
       const uint32_t q = (uint32_t)k * BLOCK + threadIdx.x;
-      if (q < valid) vals_out[gpos[k]] = s_vals[q];
+      if constexpr (OFF32) {
+        uint32_t vbyte;
+        if constexpr (sizeof(V) >= sizeof(K)) vbyte = gpos[k] * (uint32_t)(sizeof(V) / sizeof(K));
+        else vbyte = gpos[k] / (uint32_t)(sizeof(K) / sizeof(V));
+        if (q < valid) *reinterpret_cast<V*>(reinterpret_cast<char*>(vals_out) + vbyte) = s_vals[q];
+      } else {
+        if (q < valid) vals_out[gpos[k]] = s_vals[q];
+      }
     }
   }
 }
@@ -584,6 +622,8 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
   const size_t off_ctl = lay.add(sizeof(SortCtl));
   // contiguous zero-initialised region: tickets, histograms, tile descriptors
   const bool wide = n > SORT_MAX_N_NARROW;  // prefixes need more than 30 bits: 64-bit descriptors
+  // every key and value within 4 GiB of its array's start: 32-bit byte offsets
+  const bool off32 = !wide && n * (uint64_t)((HAS_VALUES && sizeof(V) > sizeof(K)) ? sizeof(V) : sizeof(K)) <= (1ull << 32);
   const size_t zero_words = (size_t)MAX_PASSES + (size_t)MAX_PASSES * RADIX_SIZE +
                             (size_t)geo.passes * tiles * RADIX_SIZE * (wide ? 2 : 1);
   const size_t off_zero = lay.add(zero_words * sizeof(uint32_t));
@@ -626,10 +666,12 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
   TA_CHECK_LAUNCH();
   for (int p = 0; p < geo.passes; ++p) {
     const size_t status_off = (size_t)p * tiles * RADIX_SIZE;  // in descriptor words
-    if (wide) {
-      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint64_t>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, reinterpret_cast<uint64_t*>(status) + status_off, tickets + p, (const SortCtl*)ctl);
+    if (off32) {
+      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint32_t, true>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + status_off, tickets + p, (const SortCtl*)ctl);
+    } else if (wide) {
+      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint64_t, false>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, reinterpret_cast<uint64_t*>(status) + status_off, tickets + p, (const SortCtl*)ctl);
     } else {
-      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint32_t>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + status_off, tickets + p, (const SortCtl*)ctl);
+      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint32_t, false>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + status_off, tickets + p, (const SortCtl*)ctl);
     }
     TA_CHECK_LAUNCH();
   }
