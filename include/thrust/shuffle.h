@@ -27,59 +27,58 @@ template <typename D, typename It, typename Out, typename URBG>
 void shuffle_copy(const detail::execution_policy_base<D>& exec, It first, It last, Out result, URBG&& g);
 
 namespace detail {
-// A keyed bijection of [0, 2^bits) (generic/shuffle.inl:34-140).
-class feistel_bijection {
- public:
-  template <typename URBG>
-  __host__ __device__ feistel_bijection(std::uint64_t m, URBG&& g) {
-    const std::uint64_t total_bits = cipher_bits(m);
-    left_side_bits_ = total_bits / 2;
-    left_side_mask_ = (1ull << left_side_bits_) - 1;
-    right_side_bits_ = total_bits - left_side_bits_;
-    right_side_mask_ = (1ull << right_side_bits_) - 1;
-    for (int i = 0; i < ROUNDS; ++i) key_[i] = g();
-  }
-  __host__ __device__ std::uint64_t nearest_power_of_two() const { return 1ull << (left_side_bits_ + right_side_bits_); }
-  __host__ __device__ std::uint64_t operator()(std::uint64_t val) const {
-    std::uint32_t left = static_cast<std::uint32_t>(val >> right_side_bits_);
-    std::uint32_t right = static_cast<std::uint32_t>(val & right_side_mask_);
-    for (int i = 0; i < ROUNDS; ++i) {
-      const std::uint32_t new_left = static_cast<std::uint32_t>(right & left_side_mask_);
-      const std::uint32_t mixed = left ^ round_function(right, key_[i]);
-      // an odd number of bits: the right side is one wider and keeps its top bit in place
-      right = right_side_bits_ != left_side_bits_
-                  ? static_cast<std::uint32_t>((static_cast<std::uint64_t>(mixed) << 1ull) | (right >> left_side_bits_))
-                  : mixed;
-      left = new_left;
-    }
-    return (static_cast<std::uint64_t>(left) << right_side_bits_) | right;
-  }
-
- private:
-  static const int ROUNDS = 16;
-  __host__ __device__ static std::uint64_t cipher_bits(std::uint64_t m) {
-    if (m == 0) return 0;
-    std::uint64_t i = 0;
-    for (--m; m != 0; m >>= 1) ++i;
-    return i;
-  }
-  __host__ __device__ static std::uint64_t hash_combine(std::uint64_t lhs, std::uint64_t rhs) {
-    lhs ^= rhs + 0x9e3779b9 + (lhs << 6) + (lhs >> 2);
-    return lhs;
-  }
-  __host__ __device__ std::uint32_t round_function(std::uint64_t value, std::uint64_t key) const {
-    const std::uint64_t hash0 = thrust::random::taus88(static_cast<std::uint32_t>(value))();
-    const std::uint64_t hash1 = thrust::random::ranlux48(value)();
-    return static_cast<std::uint32_t>(hash_combine(hash_combine(hash0, key), hash1) & left_side_mask_);
-  }
-
-  std::uint64_t right_side_bits_, left_side_bits_, right_side_mask_, left_side_mask_;
-  std::uint64_t key_[ROUNDS];
+// The keyed permutation of [0, 2^w), w = bits needed for m - 1, that the reference draws its shuffle
+// from (generic/shuffle.inl:34-140 states the arithmetic; tests/golden/shuffle_permutations.npz pins
+// it).  An index is split into a high part of floor(w / 2) bits and a low part of the remaining
+// bits.  Sixteen times over, the low part's narrow bits move up to become the high part, and the old
+// high part, xor-ed with a keyed hash of the whole low part, moves down; when w is odd the low
+// part's extra top bit stays at the bottom of the new low part.  The sixteen keys are the first
+// sixteen draws of the caller's generator.
+struct index_cipher {
+  std::uint64_t round_key[16];
+  unsigned narrow;  // bits of the high part
+  unsigned wide;    // bits of the low part: narrow, or narrow + 1
 };
 
+template <typename URBG>
+__host__ __device__ index_cipher make_index_cipher(std::uint64_t m, URBG&& g) {
+  unsigned w = 0;
+  for (std::uint64_t top = m > 0 ? m - 1 : 0; top != 0; top >>= 1) ++w;
+  index_cipher c;
+  c.narrow = w / 2;
+  c.wide = w - c.narrow;
+  for (std::uint64_t& k : c.round_key) k = g();
+  return c;
+}
+
+__host__ __device__ inline std::uint64_t cipher_domain(const index_cipher& c) { return 1ull << (c.narrow + c.wide); }
+
+// a ^= b + golden ratio + (a << 6) + (a >> 2): how the round function folds its three ingredients
+__host__ __device__ inline std::uint64_t fold_into(std::uint64_t a, std::uint64_t b) {
+  return a ^ (b + 0x9e3779b9 + (a << 6) + (a >> 2));
+}
+
+__host__ __device__ inline std::uint64_t encipher(const index_cipher& c, std::uint64_t index) {
+  const std::uint32_t narrow_mask = static_cast<std::uint32_t>((1ull << c.narrow) - 1);
+  std::uint32_t hi = static_cast<std::uint32_t>(index >> c.wide);
+  std::uint32_t lo = static_cast<std::uint32_t>(index & ((1ull << c.wide) - 1));
+  for (const std::uint64_t key : c.round_key) {
+    // the first draw of a taus88 seeded with the low part, the round's key, and the first draw of
+    // a ranlux48 seeded with the low part
+    const std::uint64_t from_taus = thrust::random::taus88(lo)();
+    const std::uint64_t from_ranlux = thrust::random::ranlux48(static_cast<std::uint64_t>(lo))();
+    const std::uint32_t mask = static_cast<std::uint32_t>(fold_into(fold_into(from_taus, key), from_ranlux)) & narrow_mask;
+    // (lo >> narrow is the extra top bit of an odd split and zero otherwise)
+    const std::uint32_t next_lo = ((hi ^ mask) << (c.wide - c.narrow)) | (lo >> c.narrow);
+    hi = lo & narrow_mask;
+    lo = next_lo;
+  }
+  return (static_cast<std::uint64_t>(hi) << c.wide) | lo;
+}
+
 struct image_under {
-  feistel_bijection bijection;
-  __host__ __device__ std::uint64_t operator()(std::uint64_t i) const { return bijection(i); }
+  index_cipher cipher;
+  __host__ __device__ std::uint64_t operator()(std::uint64_t i) const { return encipher(cipher, i); }
 };
 struct falls_below {
   std::uint64_t m;
@@ -97,11 +96,11 @@ template <typename Keys, typename Policy, typename It, typename Out, typename UR
 inline void shuffle_copy_with(Policy& exec, It first, It last, Out result, URBG&& g) {
   typedef typename std::remove_const<typename thrust::iterator_value<It>::type>::type V;
   const std::uint64_t m = (std::uint64_t)(last - first);
-  const feistel_bijection bijection(m, g);  // (draws its keys also for an empty range, as the reference does)
+  const index_cipher cipher = make_index_cipher(m, g);  // (draws its keys also for an empty range, as the reference does)
   if (m == 0) return;
-  const std::uint64_t n = bijection.nearest_power_of_two();
+  const std::uint64_t n = cipher_domain(cipher);
   Keys keys(n);
-  const image_under image = {bijection};
+  const image_under image = {cipher};
   thrust::transform(exec, thrust::counting_iterator<std::uint64_t>(0), thrust::counting_iterator<std::uint64_t>(n),
                     keys.begin(), image);
   const fetches_at<It, V> fetch = {first, m};

@@ -283,14 +283,14 @@ int main() {
   {
     // the network is a bijection of [0, 2^bits) and knows its length (testing/shuffle.cu:378-425)
     thrust::default_random_engine g(0xD5);
-    ASSERT_EQUAL(thrust::detail::feistel_bijection(3, g).nearest_power_of_two(), 4u);
-    ASSERT_EQUAL(thrust::detail::feistel_bijection(2, g).nearest_power_of_two(), 2u);
-    ASSERT_EQUAL(thrust::detail::feistel_bijection(0, g).nearest_power_of_two(), 1u);
+    ASSERT_EQUAL(thrust::detail::cipher_domain(thrust::detail::make_index_cipher(3, g)), 4u);
+    ASSERT_EQUAL(thrust::detail::cipher_domain(thrust::detail::make_index_cipher(2, g)), 2u);
+    ASSERT_EQUAL(thrust::detail::cipher_domain(thrust::detail::make_index_cipher(0, g)), 1u);
     for (std::uint64_t m : {5ull, 64ull, 1000ull, 40000ull}) {
       thrust::default_random_engine host_g(0xD5), device_g(0xD5);
-      const thrust::detail::image_under host_f = {thrust::detail::feistel_bijection(m, host_g)};
-      const thrust::detail::image_under device_f = {thrust::detail::feistel_bijection(m, device_g)};
-      const std::uint64_t n = host_f.bijection.nearest_power_of_two();
+      const thrust::detail::image_under host_f = {thrust::detail::make_index_cipher(m, host_g)};
+      const thrust::detail::image_under device_f = {thrust::detail::make_index_cipher(m, device_g)};
+      const std::uint64_t n = thrust::detail::cipher_domain(host_f.cipher);
       thrust::host_vector<std::uint64_t> hr(n);
       thrust::device_vector<std::uint64_t> dr(n);
       thrust::sequence(hr.begin(), hr.end());

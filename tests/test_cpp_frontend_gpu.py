@@ -134,3 +134,10 @@ def test_reference_idioms():
     # tuples, allocators over run-time chosen resources, and the algorithms the vector headers bring along
     out = _run("test_reference_idioms")
     assert "PASSED" in out
+
+
+def test_bandwidth_ceiling_kernels_run():
+    # plain read / write / copy kernels over 1 GiB: the ceiling the library's bandwidth fractions can be read against
+    # (profiles/copy_ceiling.txt holds their rocprofv3 durations); here only that they run and give sane rates
+    out = _run("bandwidth_ceiling")
+    assert "PASSED" in out and "best copy" in out
