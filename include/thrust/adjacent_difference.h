@@ -41,6 +41,21 @@ inline bool same_position(const A&, const B&) { return false; }
 template <typename A>
 inline bool same_position(const A& a, const A& b) { return a == b; }
 
+// Whether writing n results from `out` on may change inputs that later results still read.  Two
+// ranges in memory are compared by address, whatever their iterator types (a const iterator and
+// a plain one of the same vector, a raw pointer and a device_ptr); other iterators by equality
+// where they are of one type.
+template <typename A, typename B>
+inline bool output_reaches_input(A* in, B* out, std::size_t n) {
+  const char* in_begin = reinterpret_cast<const char*>(in);
+  const char* in_end = reinterpret_cast<const char*>(in + n);
+  const char* out_begin = reinterpret_cast<const char*>(out);
+  const char* out_end = reinterpret_cast<const char*>(out + n);
+  return out_begin < in_end && in_begin < out_end;
+}
+template <typename ViewIn, typename ViewOut>
+inline bool output_reaches_input(const ViewIn&, const ViewOut&, std::size_t) { return false; }
+
 #if defined(__HIPCC__)
 // arrays of 4- and 8-byte elements: one kernel that moves 16 bytes per access
 template <typename ViewIn, typename ViewOut, typename Op>
@@ -63,7 +78,8 @@ Out adjacent_difference(execution_policy<D>& exec, In first, In last, Out result
   typedef typename std::remove_const<typename iterator_value<In>::type>::type V;
   const std::ptrdiff_t n = last - first;
   if (n == 0) return result;
-  if (detail::same_position(first, result)) {
+  if (detail::same_position(first, result) ||
+      detail::output_reaches_input(thrust::detail::device_view(first), thrust::detail::device_view(result), (std::size_t)n)) {
     thrust::device_vector<V> input(first, last);
     return thrust::adjacent_difference(exec, input.begin(), input.end(), result, op);
   }

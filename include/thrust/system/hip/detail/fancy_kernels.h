@@ -58,83 +58,62 @@ __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void scatter_kernel(ViewIn in, V
   for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride) out[map[i]] = in[i];
 }
 
-// ---- arrays of 4- and 8-byte elements: every thread takes PER consecutive elements with 16-byte
-// accesses.  The functor still receives the element itself (a copy in registers); an input that
-// it changed is written back, so a functor that modifies its argument behaves as in the plain
-// kernels above.
+// ---- arrays of 4- and 8-byte elements: every thread takes PER consecutive elements, 16 bytes at a
+// time.  The functor receives the element where it lies in memory, exactly as in the plain kernels
+// above (it may take its address, or change it: thrust/system/cuda/detail/for_each.h:58 hands it
+// raw_reference_cast(input[idx])); the element accesses of one thread are adjacent and 16-byte
+// aligned, which is what lets the compiler fetch them with one load.  Results leave as one 16-byte
+// store after the thread's PER calls, so an output that is the input ends up holding the results,
+// as in `*result = f(*first)`.
 template <typename T, int N>
 struct alignas(sizeof(T) * N >= 16 ? 16 : sizeof(T) * N) element_pack {
   T v[N];
 };
 template <typename T>
 struct is_packable : std::integral_constant<bool, std::is_trivially_copyable<T>::value && (sizeof(T) == 4 || sizeof(T) == 8)> {};
-template <typename T, int N>
-__device__ __forceinline__ bool same_bytes(const element_pack<T, N>& a, const element_pack<T, N>& b) {
-  uint32_t x[sizeof(a) / 4], y[sizeof(b) / 4];  // copied, not aliased: T may be any 4- or 8-byte type
-  __builtin_memcpy(x, &a, sizeof(a));
-  __builtin_memcpy(y, &b, sizeof(b));
-  uint32_t differ = 0;
-#pragma unroll
-  for (unsigned w = 0; w < sizeof(a) / 4; ++w) differ |= x[w] ^ y[w];
-  return differ == 0;
-}
-template <typename A>
-__device__ __forceinline__ void write_back(const A*, uint64_t, const void*, const void*) {}  // read-only input
-template <typename A, int PER>
-__device__ __forceinline__ void write_back(A* in, uint64_t p, const element_pack<A, PER>* now,
-                                           const element_pack<A, PER>* before) {
-  if (!same_bytes(*now, *before)) reinterpret_cast<element_pack<A, PER>*>(in)[p] = *now;
+template <typename T, int PER>
+__device__ __forceinline__ T* pack_at(T* base, uint64_t p) {
+  constexpr size_t BYTES = sizeof(T) * PER >= 16 ? 16 : sizeof(T) * PER;
+  return static_cast<T*>(__builtin_assume_aligned(base, BYTES)) + p * PER;
 }
 
 template <typename PA, typename O, typename F, int PER>
 __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform1_packed_kernel(PA in, O* out, uint64_t n, F f) {
-  typedef typename std::remove_const<typename std::remove_pointer<PA>::type>::type A;
   const uint64_t packs = n / PER;
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; p < packs; p += stride) {
-    element_pack<A, PER> a = reinterpret_cast<const element_pack<A, PER>*>(in)[p];
-    const element_pack<A, PER> before = a;
+    auto* a = pack_at<typename std::remove_pointer<PA>::type, PER>(in, p);
     element_pack<O, PER> o;
 #pragma unroll
-    for (int k = 0; k < PER; ++k) o.v[k] = f(a.v[k]);
+    for (int k = 0; k < PER; ++k) o.v[k] = f(a[k]);
     reinterpret_cast<element_pack<O, PER>*>(out)[p] = o;
-    write_back(in, p, &a, &before);
   }
   if (blockIdx.x == 0 && threadIdx.x == 0)
     for (uint64_t i = packs * PER; i < n; ++i) out[i] = f(in[i]);
 }
 template <typename PA, typename PB, typename O, typename F, int PER>
 __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void transform2_packed_kernel(PA ina, PB inb, O* out, uint64_t n, F f) {
-  typedef typename std::remove_const<typename std::remove_pointer<PA>::type>::type A;
-  typedef typename std::remove_const<typename std::remove_pointer<PB>::type>::type B;
   const uint64_t packs = n / PER;
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; p < packs; p += stride) {
-    element_pack<A, PER> a = reinterpret_cast<const element_pack<A, PER>*>(ina)[p];
-    element_pack<B, PER> b = reinterpret_cast<const element_pack<B, PER>*>(inb)[p];
-    const element_pack<A, PER> a_before = a;
-    const element_pack<B, PER> b_before = b;
+    auto* a = pack_at<typename std::remove_pointer<PA>::type, PER>(ina, p);
+    auto* b = pack_at<typename std::remove_pointer<PB>::type, PER>(inb, p);
     element_pack<O, PER> o;
 #pragma unroll
-    for (int k = 0; k < PER; ++k) o.v[k] = f(a.v[k], b.v[k]);
+    for (int k = 0; k < PER; ++k) o.v[k] = f(a[k], b[k]);
     reinterpret_cast<element_pack<O, PER>*>(out)[p] = o;
-    write_back(ina, p, &a, &a_before);
-    write_back(inb, p, &b, &b_before);
   }
   if (blockIdx.x == 0 && threadIdx.x == 0)
     for (uint64_t i = packs * PER; i < n; ++i) out[i] = f(ina[i], inb[i]);
 }
 template <typename PA, typename F, int PER>
 __global__ __launch_bounds__(ELEMENTWISE_BLOCK) void for_each_packed_kernel(PA first, uint64_t n, F f) {
-  typedef typename std::remove_const<typename std::remove_pointer<PA>::type>::type A;
   const uint64_t packs = n / PER;
   const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
   for (uint64_t p = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; p < packs; p += stride) {
-    element_pack<A, PER> a = reinterpret_cast<const element_pack<A, PER>*>(first)[p];
-    const element_pack<A, PER> before = a;
+    auto* a = pack_at<typename std::remove_pointer<PA>::type, PER>(first, p);
 #pragma unroll
-    for (int k = 0; k < PER; ++k) f(a.v[k]);
-    write_back(first, p, &a, &before);
+    for (int k = 0; k < PER; ++k) f(a[k]);
   }
   if (blockIdx.x == 0 && threadIdx.x == 0)
     for (uint64_t i = packs * PER; i < n; ++i) f(first[i]);

@@ -184,6 +184,17 @@ static void AdjacentDifferenceAgainstHost() {
     ASSERT_TRUE(same(thrust::host_vector<T>(d), ho));
     thrust::adjacent_difference(h.begin(), h.end(), h.begin());
     ASSERT_TRUE(same(h, ho));
+    // in place through iterators of different types: a const and a plain iterator of one vector, a raw
+    // pointer and a device_ptr of one array
+    thrust::device_vector<T> d2 = samples<T>(n, 41 + n, 1000);
+    thrust::adjacent_difference(d2.cbegin(), d2.cend(), d2.begin());
+    ASSERT_TRUE(same(thrust::host_vector<T>(d2), ho));
+    thrust::device_vector<T> d3 = samples<T>(n, 41 + n, 1000);
+    if (n > 0) {
+      const T* raw = thrust::raw_pointer_cast(d3.data());
+      thrust::adjacent_difference(thrust::device, raw, raw + n, d3.data());
+      ASSERT_TRUE(same(thrust::host_vector<T>(d3), ho));
+    }
     // the differences of a scan give the input back
     thrust::host_vector<T> again(n);
     thrust::device_vector<T> scanned = ho;
@@ -353,6 +364,15 @@ struct bumps_and_doubles {  // changes its argument: the input must change too
   __host__ __device__ int operator()(int& x) const { x += 1; return 2 * x; }
 };
 
+struct position_writer {
+  const int* base;
+  __host__ __device__ void operator()(int& x) const { x = (int)(&x - base); }
+};
+struct position_reader {
+  const int* base;
+  __host__ __device__ int operator()(const int& x) const { return (int)(&x - base); }
+};
+
 // thrust::transform over plain arrays takes kernels that move 16 bytes per access when the arrays are
 // aligned for it: sizes around the switch, tails, offsets that break the alignment, 8-byte and mixed
 // element sizes, in place, and a functor that modifies its argument
@@ -404,6 +424,24 @@ static void TransformShapes() {
   thrust::transform(di.begin(), di.end(), db.begin(), bumps_and_doubles());
   ASSERT_TRUE(same(thrust::host_vector<int>(db), hb));
   ASSERT_TRUE(same(thrust::host_vector<int>(di), hi));  // both inputs were bumped
+  // the same functor with the output on the input: the results, not the bumped inputs, stay
+  thrust::transform(hi.begin(), hi.end(), hi.begin(), bumps_and_doubles());
+  thrust::transform(di.begin(), di.end(), di.begin(), bumps_and_doubles());
+  ASSERT_TRUE(same(thrust::host_vector<int>(di), hi));
+  // a functor is handed the element where it lies: its address gives the element's position
+  // (thrust/system/cuda/detail/for_each.h:58), on aligned arrays of any size as well
+  for (size_t n : {size_t(5), size_t(4096), size_t(70001)}) {
+    thrust::device_vector<int> where(n, -1);
+    const position_writer writes = {thrust::raw_pointer_cast(where.data())};
+    thrust::for_each(where.begin(), where.end(), writes);
+    thrust::host_vector<int> expect(n);
+    thrust::sequence(expect.begin(), expect.end());
+    ASSERT_TRUE(same(thrust::host_vector<int>(where), expect));
+    thrust::device_vector<int> from(n, 3), positions(n);
+    const position_reader reads = {thrust::raw_pointer_cast(from.data())};
+    thrust::transform(from.begin(), from.end(), positions.begin(), reads);
+    ASSERT_TRUE(same(thrust::host_vector<int>(positions), expect));
+  }
 }
 
 int main() {
