@@ -28,10 +28,31 @@ HBM_PEAK_GBS = 8000.0  # MI355X HBM3E, published
 N_SORT = 1 << 28
 N_C1 = 1 << 28
 
-# HBM bytes per onesweep pass launch at n = 2^28 uint32, from rocprofv3 --pmc FETCH_SIZE /
-# WRITE_SIZE, each scaled by what the same counter reads for kernels of known size in the
-# same run (reduce: 1 GiB read, scan: 1 GiB read + 1 GiB written).
-PASS_TRAFFIC_BYTES = 2.318e9  # profiles/sort_u32_2p28_hbm_traffic.txt
+# HBM bytes per onesweep pass launch at n = 2^28 uint32 come from the committed counter summary:
+# rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE of this very command, each scaled by what the same counter
+# reads for kernels of known size in the same run (FETCH_SIZE reports half the KiB fetched: x2.0 from
+# the reduce kernel's 1 GiB; WRITE_SIZE x1.0 from the scan kernel's 1 GiB).
+PMC_SUMMARY = os.path.join("profiles", "bench_kernels_pmc_counters.txt")
+FETCH_SCALE, WRITE_SCALE = 2.0, 1.0
+
+
+def pass_traffic_from_profile():
+    """(bytes per launch, "file:line") of the uint32 keys-only onesweep pass in the committed counter
+    summary, or (None, reason) when the file or the line is not there."""
+    import re
+    path = os.path.join(ROOT, PMC_SUMMARY)
+    try:
+        lines = open(path).read().splitlines()
+    except OSError:
+        return None, f"{PMC_SUMMARY} not found"
+    for i, text in enumerate(lines):
+        if text.startswith("onesweep_pass_kernel<unsigned int, unsigned int, false"):
+            for j in range(i + 1, min(i + 4, len(lines))):
+                m = re.search(r"FETCH (\d+) KiB WRITE (\d+) KiB", lines[j])
+                if m:
+                    nbytes = (FETCH_SCALE * int(m.group(1)) + WRITE_SCALE * int(m.group(2))) * 1024.0
+                    return nbytes, f"{PMC_SUMMARY}:{j + 1}"
+    return None, f"no onesweep_pass line in {PMC_SUMMARY}"
 
 
 def device_random_u32(torch, n, seed):
@@ -91,7 +112,7 @@ def bench_sort(torch, capi, steps, warmup, want_host_copy):
 class C1:
     """reduce and inclusive_scan over 2^28 int32: buffers made once and measured twice -- before and
     after the sort -- so that a disturbance at either end of the run does not decide the figure;
-    the better pass is reported, both are printed."""
+    the mean of the two passes is the figure reported, the better pass and both passes are printed."""
 
     def __init__(self, torch, capi, want_host_copy):
         from thrust_amd import datagen_device
@@ -112,6 +133,7 @@ class C1:
             raise SystemExit("bench: inclusive_scan total differs from the int64 sum modulo 2^32")
         self.host = x.cpu().numpy() if want_host_copy else None
         self.passes = []
+        self.copy_ms = []
 
     def measure(self, steps, warmup):
         # calls of 0.2 - 0.4 ms: at least 50 back to back, so that the one synchronisation at the end
@@ -120,7 +142,14 @@ class C1:
         capi = self.capi
         ms_reduce = time_region(self.torch, lambda i, w: capi.reduce(self.d, temp=self.t_r, out=self.out1), reps, warmup)
         ms_scan = time_region(self.torch, lambda i, w: capi.inclusive_scan(self.d, out=self.outn, temp=self.t_s), reps, warmup)
+        # a plain device copy of the same 1 GiB into the same output (torch's copy kernel): what moving the
+        # scan's bytes costs with no scan in between
+        src_t, dst_t = self.d.storage, self.outn.storage
+        self.copy_ms.append(time_region(self.torch, lambda i, w: dst_t.copy_(src_t), reps, warmup))
         self.passes.append((ms_reduce, ms_scan))
+
+    def mean(self):
+        return sum(p[0] for p in self.passes) / len(self.passes), sum(p[1] for p in self.passes) / len(self.passes)
 
     def best(self):
         return min(p[0] for p in self.passes), min(p[1] for p in self.passes)
@@ -224,7 +253,9 @@ def main():
     c1.measure(args.steps, args.warmup)
     ms_sort, pass_ms, kernels_ms, host_keys = bench_sort(torch, capi, args.steps, args.warmup, want_host)
     c1.measure(args.steps, args.warmup)
-    ms_reduce, ms_scan = c1.best()
+    ms_reduce, ms_scan = c1.mean()
+    best_reduce, best_scan = c1.best()
+    ms_copy = sum(c1.copy_ms) / len(c1.copy_ms)
     host_c1 = c1.host
     c1_passes = [{"reduce_ms": round(r, 4), "scan_ms": round(sc, 4)} for r, sc in c1.passes]
     del c1
@@ -237,6 +268,7 @@ def main():
     gkeys = n / ms_sort / 1e6
     pass_bytes = 2.0 * 4.0 * n  # keys read + keys written by one digit-binning pass
     pass_gbs = pass_bytes / pass_ms / 1e6
+    traffic, traffic_source = pass_traffic_from_profile()
     line = {
         "metric": "sort Gkeys/s (2^28 u32) + scan/reduce GB/s as % of HBM peak, 1 GPU",
         "value": round(gkeys, 3),
@@ -254,14 +286,26 @@ def main():
                                "uniform over the full range (seeded), in place, keys resident in HBM"},
         "sort_model_bytes_pct_of_peak": round(36.0 * n / ms_sort / 1e6 / HBM_PEAK_GBS * 100, 2),
         "sort_kernels_ms": {k: round(v, 4) for k, v in kernels_ms.items()},
+        "sort_kernels_ms_note": "each launch of a separate profiled run bracketed by its own pair of events: the pairs "
+                                "add about 4 % per launch, so these sum to more than ms_per_step, which has none",
         "reduce_i32_2p28": {"ms": round(ms_reduce, 4), "GBps": round(4.0 * N_C1 / ms_reduce / 1e6, 1),
-                            "pct_of_peak": round(4.0 * N_C1 / ms_reduce / 1e6 / HBM_PEAK_GBS * 100, 2)},
+                            "pct_of_peak": round(4.0 * N_C1 / ms_reduce / 1e6 / HBM_PEAK_GBS * 100, 2),
+                            "ms_best": round(best_reduce, 4),
+                            "pct_of_peak_best": round(4.0 * N_C1 / best_reduce / 1e6 / HBM_PEAK_GBS * 100, 2)},
         "inclusive_scan_i32_2p28": {"ms": round(ms_scan, 4), "GBps": round(8.0 * N_C1 / ms_scan / 1e6, 1),
-                                    "pct_of_peak": round(8.0 * N_C1 / ms_scan / 1e6 / HBM_PEAK_GBS * 100, 2)},
-        "reduce_scan_passes": c1_passes,  # before and after the sort; the better pass is the one reported
+                                    "pct_of_peak": round(8.0 * N_C1 / ms_scan / 1e6 / HBM_PEAK_GBS * 100, 2),
+                                    "ms_best": round(best_scan, 4),
+                                    "pct_of_peak_best": round(8.0 * N_C1 / best_scan / 1e6 / HBM_PEAK_GBS * 100, 2),
+                                    # beside it: a plain copy of the same bytes in this run, and the best hand-written
+                                    # copy kernel of profiles/copy_ceiling.txt (256 threads x 16 bytes: 0.3459 ms)
+                                    "torch_copy_ms": round(ms_copy, 4),
+                                    "pct_of_torch_copy": round(ms_copy / ms_scan * 100, 1),
+                                    "pct_of_best_copy_kernel": round(0.3459 / ms_scan * 100, 1)},
+        # before and after the sort, each the mean of >= 50 back-to-back calls; "ms" above is the mean of the two
+        "reduce_scan_passes": c1_passes,
         "roofline": {"bound": "hbm", "kernel": "onesweep_pass (one of 4 per sort)",
                      "achieved": round(pass_gbs, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(pass_gbs / HBM_PEAK_GBS, 4), "traffic": PASS_TRAFFIC_BYTES,
+                     "frac": round(pass_gbs / HBM_PEAK_GBS, 4), "traffic": traffic, "traffic_source": traffic_source,
                      "launch_ms": round(pass_ms, 4)},
     }
     if config_rows is not None:

@@ -110,9 +110,13 @@ def run_c3(torch, capi, reps):
             and bool((vo[1:][same] > vo[:-1][same]).all().item())
         if not ok:
             _fail(f"C3 sort_by_key {kind}")
+        # passes over a digit that is the same in every key move nothing (the reference's sequential radix
+        # sort skips them too): the bytes of the call are the histogram read and the passes that run
+        passes_run = sum(1 for p in range(8) if int(((keys >> (8 * p)) & 0xFF).min().item())
+                         != int(((keys >> (8 * p)) & 0xFF).max().item()))
         rows[f"c3_sort_by_key_u64_u32_2p27_{kind}"] = _row(
-            med, mn, 200 * m, Gpairs_per_s=round(m / med / 1e6, 2),
-            model="200 B/pair: histogram read + 8 passes x 24 B; passes over a constant digit are skipped")
+            med, mn, (8 + 24 * passes_run) * m, Gpairs_per_s=round(m / med / 1e6, 2), passes_run=passes_run,
+            model="8 B/pair histogram read + 24 B/pair per pass that runs (all 8: 200 B/pair)")
         del keys, vals, sk, sv, wk, wv, t, ko, vo, o, same
     return rows
 
@@ -178,7 +182,11 @@ def run_c5(torch, capi, reps):
         got = work.storage.view(torch.float32)
         if cnt != cnt_want or not torch.equal(got[:cnt], want_true) or not torch.equal(got[cnt:], x[~mask]):
             _fail(f"C5 stable_partition {tag}")
-        rows[f"c5_stable_partition_{tag}"] = _row(med, mn, 8 * n, selected=cnt)
+        # in place the smaller side is parked in temporary storage and copied back: 8 bytes more per parked element
+        moved = 8 * n + 8 * min(cnt, n - cnt)
+        rows[f"c5_stable_partition_{tag}"] = _row(
+            med, mn, 8 * n, selected=cnt, bytes_moved=int(moved),
+            pct_of_peak_moved=round(moved / med / 1e6 / HBM_PEAK_GBS * 100, 2))
         del mask, want_true, got
     del x, dx, out, work, t, tp
 
