@@ -251,11 +251,16 @@ int thrust_amd_inclusive_scan(void* temp, size_t* temp_bytes, const void* in, vo
  * tight serving loops, harnesses that forbid hipMalloc): same result, no temporary storage
  * argument.  It has no counterpart in the reference.  The tile descriptors live in a fixed
  * 1 MiB array inside the library's device image (one copy per GPU, held until the process
- * ends), cleared by a small kernel at every call; the call performs no hipMalloc / hipFree.
+ * ends); the call performs no hipMalloc / hipFree.  The array is all zero when the library is
+ * loaded and the scan kernel clears what it used before it ends, so the call is ONE kernel
+ * launch (the entry point with temporary storage needs a clearing launch first).
  * n is limited by that array: up to 131040 tiles (about 6.4e9 elements of 4 bytes or less,
  * 1.6e9 of 8 bytes); a larger n returns hipErrorInvalidValue and launches nothing.  Every
- * call on a GPU shares that GPU's array: calls that may overlap in time on one GPU (two
- * streams, two host threads) race and must be serialised by the caller. */
+ * call on a GPU shares that GPU's array.  The library orders such calls itself: each call's
+ * stream first waits (on the device) for an event recorded behind the previous call on that GPU,
+ * whatever stream or host thread made it.  A stream under capture is left out of that ordering:
+ * replays of a graph that holds this call must not overlap other calls of it on the same GPU.
+ * The first call on a GPU also looks up the array's address and creates that event. */
 int thrust_amd_inclusive_scan_static(const void* in, void* out, uint64_t n, int dtype, int op,
                                      void* stream);
 

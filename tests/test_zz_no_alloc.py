@@ -33,6 +33,9 @@ def test_static_scan_matches_the_temp_storage_entry_point(dev, oracle, dtype, op
         assert np.array_equal(got.view(np.uint8), want.view(np.uint8)), (dtype, op, n)
         if n <= 100003 and np.dtype(dtype).kind != "f":
             assert np.array_equal(got, oracle.inclusive_scan(x, op)), (dtype, op, n)
+        if op == 0 and np.dtype(dtype).kind != "f":
+            # every size against the definition as well: the running sum modulo 2^bits
+            assert np.array_equal(got, np.cumsum(x, dtype=dtype)), (dtype, n)
 
 
 def test_static_scan_in_place_and_empty(dev):
@@ -51,10 +54,45 @@ def test_static_scan_refuses_sizes_beyond_its_scratch(dev):
     out = dev.DeviceArray(16, dev.I32)
     # 2^40 elements need more tile descriptors than the fixed array holds; the pointers are
     # never dereferenced because the call is refused before any launch
-    rc = lib.thrust_amd_inclusive_scan_static(d.ptr, out.ptr, 1 << 40, dev.I32, dev.PLUS, dev.stream_ptr())
-    assert rc != 0
+    # the library's launch log shows that nothing was launched by the refused calls
+    dev.profile_collect()
+    dev.profile_enable(True)
+    try:
+        rc = lib.thrust_amd_inclusive_scan_static(d.ptr, out.ptr, 1 << 40, dev.I32, dev.PLUS, dev.stream_ptr())
+        assert rc != 0
+        rc = lib.thrust_amd_inclusive_scan_static(d.ptr, out.ptr, 16, 99, dev.PLUS, dev.stream_ptr())
+        assert rc != 0  # invalid dtype
+        assert dev.profile_collect() == {}
+    finally:
+        dev.profile_enable(False)
     assert np.array_equal(d.numpy(), np.arange(16, dtype=np.int32))
-    rc = lib.thrust_amd_inclusive_scan_static(d.ptr, out.ptr, 16, 99, dev.PLUS, dev.stream_ptr())
-    assert rc != 0  # invalid dtype
     # and the entry point still works afterwards
     assert np.array_equal(dev.inclusive_scan_static(d).numpy(), np.cumsum(np.arange(16, dtype=np.int32)))
+
+
+def test_static_scan_is_one_launch_and_calls_from_two_streams_follow_each_other(dev):
+    import torch
+    x = _ints((1 << 24) + 77, np.int32, 9)
+    d = dev.DeviceArray.from_numpy(x)
+    want = np.cumsum(x, dtype=np.int32)
+    dev.profile_collect()
+    dev.profile_enable(True)
+    try:
+        got = dev.inclusive_scan_static(d).numpy()
+        log = dev.profile_collect()
+    finally:
+        dev.profile_enable(False)
+    assert np.array_equal(got, want)
+    assert sum(v[0] for v in log.values()) == 1, log  # the scan kernel alone: no clearing launch
+    # calls issued on two streams without any synchronisation in between share the scratch array;
+    # the library puts them one behind the other
+    lib = dev.load()
+    outs = [dev.DeviceArray(d.n, dev.I32) for _ in range(6)]
+    streams = [torch.cuda.Stream(), torch.cuda.Stream()]
+    torch.cuda.synchronize()
+    for i, o in enumerate(outs):
+        rc = lib.thrust_amd_inclusive_scan_static(d.ptr, o.ptr, d.n, dev.I32, dev.PLUS, streams[i % 2].cuda_stream)
+        assert rc == 0
+    torch.cuda.synchronize()
+    for o in outs:
+        assert np.array_equal(o.numpy(), want)

@@ -39,10 +39,15 @@ TA_DEVICE T wave_shift_up(T v, T id) {
   return dpp_move<0x138 /* wave_shr:1 */>(id, v);
 }
 
+// `finished`, when given, makes the kernel leave its descriptors the way it found them: every tile
+// counts itself in once its look-back is over, and the tile that completes the count clears the
+// descriptors, the ticket and the counter again.  Storage that is only ever used that way (the
+// library's own, all zero when the module is loaded) needs no clearing launch in front of the kernel.
 template <typename T, typename Op, typename Pre, bool EXCLUSIVE, bool ALIGNED, typename Shape>
 __global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out, uint64_t n, T init,
                                                           uint64_t* __restrict__ status,
-                                                          uint32_t* __restrict__ ticket) {
+                                                          uint32_t* __restrict__ ticket,
+                                                          uint32_t* __restrict__ finished) {
   constexpr int SCAN_BLOCK = Shape::BLOCK;
   constexpr int SCAN_CHUNKS = Shape::CHUNKS;
   constexpr int VEC = Vec16<T>::N;
@@ -57,8 +62,12 @@ __global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out,
   __shared__ uint32_t s_tile;
   __shared__ T s_wave_agg[WAVES];
   __shared__ T s_prefix;
+  __shared__ uint32_t s_last;
 
-  if (threadIdx.x == 0) s_tile = atomicAdd(ticket, 1u);
+  if (threadIdx.x == 0) {
+    s_tile = atomicAdd(ticket, 1u);
+    s_last = 0;
+  }
   __syncthreads();
   const uint32_t tile = s_tile;
   const uint64_t tile_base = (uint64_t)tile * TILE;
@@ -145,7 +154,18 @@ __global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out,
       tile_excl = tile_lookback<T>(status, tile, op, id);
       if (lane == 0) tile_publish<T>(my_slot, TS_INCLUSIVE, op(tile_excl, block_agg));
     }
-    if (lane == 0) s_prefix = tile_excl;
+    if (lane == 0) {
+      s_prefix = tile_excl;
+      // Counted in only after this tile's last descriptor store has been acknowledged (the wait
+      // below; descriptor stores and this counter are agent-scope accesses that bypass the
+      // non-coherent caches, so no cache write-back is involved -- a release fence here would
+      // write back the L2 with the kernel's output in it, once per tile).  Whoever completes the
+      // count knows that no descriptor will be read or written again.
+      if (finished != nullptr) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        s_last = __hip_atomic_fetch_add(finished, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == gridDim.x - 1;
+      }
+    }
   }
   __syncthreads();
   T prefix = s_prefix;
@@ -172,19 +192,29 @@ __global__ __launch_bounds__(Shape::BLOCK) void scan_kernel(const T* in, T* out,
       }
     }
   }
+  if (s_last) {
+    const uint64_t words = (uint64_t)gridDim.x * W;
+    for (uint64_t i = threadIdx.x; i < words; i += SCAN_BLOCK) status[i] = 0;
+    if (threadIdx.x == 0) {
+      *ticket = 0;
+      *finished = 0;
+    }
+  }
 }
 
 template <bool EXCLUSIVE, typename Pre>
 struct ScanLaunch {
+  // kept_clean: `temp` is storage of the library's own that only this function uses and that was all
+  // zero to begin with; the kernel then clears up after itself and no clearing launch precedes it.
   template <typename T, typename Op, typename Shape>
   static int run_shape(void* temp, size_t* temp_bytes, const void* in, void* out, uint64_t n,
-                       const void* init, hipStream_t stream) {
+                       const void* init, hipStream_t stream, bool kept_clean = false) {
     constexpr int W = TileWords<T>::W;
     constexpr uint64_t TILE = (uint64_t)Shape::BLOCK * Shape::CHUNKS * Vec16<T>::N;
     const uint64_t tiles = (n + TILE - 1) / TILE;
     if (tiles > 0xffffffffull) return (int)hipErrorInvalidValue;
     TempLayout lay;
-    const size_t off_ticket = lay.add(sizeof(uint32_t));
+    const size_t off_ticket = lay.add(2 * sizeof(uint32_t));  // the ticket and the count of finished tiles
     const size_t off_status = lay.add((size_t)tiles * W * sizeof(uint64_t));
     if (temp == nullptr) {
       *temp_bytes = lay.total;
@@ -201,24 +231,27 @@ struct ScanLaunch {
     uint32_t* ticket = reinterpret_cast<uint32_t*>(static_cast<char*>(temp) + off_ticket);
     uint64_t* status = reinterpret_cast<uint64_t*>(static_cast<char*>(temp) + off_status);
     const uint64_t words = tiles * W;
-    TA_LAUNCH("tile_state_init", stream, tile_state_init_kernel, dim3((uint32_t)((words + 255) / 256)), dim3(256), status, words, ticket, 1u);
-    TA_CHECK_LAUNCH();
+    uint32_t* finished = kept_clean ? ticket + 1 : nullptr;
+    if (!kept_clean) {
+      TA_LAUNCH("tile_state_init", stream, tile_state_init_kernel, dim3((uint32_t)((words + 255) / 256)), dim3(256), status, words, ticket, 2u);
+      TA_CHECK_LAUNCH();
+    }
     const T* src = static_cast<const T*>(in);
     T* dst = static_cast<T*>(out);
     if (is_aligned16(in) && is_aligned16(out))
-      TA_LAUNCH("scan", stream, (scan_kernel<T, Op, Pre, EXCLUSIVE, true, Shape>), dim3((uint32_t)tiles), dim3(Shape::BLOCK), src, dst, n, init_v, status, ticket);
+      TA_LAUNCH("scan", stream, (scan_kernel<T, Op, Pre, EXCLUSIVE, true, Shape>), dim3((uint32_t)tiles), dim3(Shape::BLOCK), src, dst, n, init_v, status, ticket, finished);
     else
-      TA_LAUNCH("scan", stream, (scan_kernel<T, Op, Pre, EXCLUSIVE, false, Shape>), dim3((uint32_t)tiles), dim3(Shape::BLOCK), src, dst, n, init_v, status, ticket);
+      TA_LAUNCH("scan", stream, (scan_kernel<T, Op, Pre, EXCLUSIVE, false, Shape>), dim3((uint32_t)tiles), dim3(Shape::BLOCK), src, dst, n, init_v, status, ticket, finished);
     TA_CHECK_LAUNCH();
     return 0;
   }
 
   template <typename T, typename Op>
   static int run(void* temp, size_t* temp_bytes, const void* in, void* out, uint64_t n,
-                 const void* init, hipStream_t stream) {
+                 const void* init, hipStream_t stream, bool kept_clean = false) {
     if (n * sizeof(T) >= SCAN_LARGE_MIN_BYTES)
-      return run_shape<T, Op, ScanShapeLarge>(temp, temp_bytes, in, out, n, init, stream);
-    return run_shape<T, Op, ScanShapeSmall>(temp, temp_bytes, in, out, n, init, stream);
+      return run_shape<T, Op, ScanShapeLarge>(temp, temp_bytes, in, out, n, init, stream, kept_clean);
+    return run_shape<T, Op, ScanShapeSmall>(temp, temp_bytes, in, out, n, init, stream, kept_clean);
   }
 };
 
