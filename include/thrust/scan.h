@@ -414,16 +414,7 @@ Out exclusive_scan_by_key_library(execution_policy<D>& exec, KIt kf, KIt kl, VIt
   const uint64_t n = (uint64_t)(kl - kf);
   if (n == 0) return result;
   const void* values = thrust::detail::raw(vf);
-  void* out = thrust::detail::raw(result);
-  // the device entry point reads values[i-1] while other tiles write: an in-place call
-  // scans from a copy of the values
-  detail::temp_storage copy(stream, detail::temp_source_of(exec));
-  if (values == out) {
-    copy.ensure(n * sizeof(V));
-    detail::throw_on_error(thrust_amd_memcpy(copy.ptr(), values, n * sizeof(V), THRUST_AMD_D2D, stream),
-                           "exclusive_scan_by_key: copy of the values");
-    values = copy.ptr();
-  }
+  void* out = thrust::detail::raw(result);  // may be the values themselves
   detail::temp_storage temp(stream, detail::temp_source_of(exec));
   detail::run(temp, 0, "exclusive_scan_by_key failed", [&](void* t, std::size_t* b) {
     return thrust_amd_exclusive_scan_by_key(t, b, thrust::detail::raw(kf), values, out, n,

@@ -259,15 +259,7 @@ Out scan_by_key_one_pass(execution_policy<D>& exec, KIt kf, KIt kl, VIt vf, Out 
   device_input<KIt> keys(stream, temp_source_of(exec), kf, n);
   device_input<VIt> values(stream, temp_source_of(exec), vf, n);
   const A* in = (const A*)values.ptr();
-  A* out = (A*)thrust::detail::raw(result);
-  // the exclusive form reads values[i-1] across tile borders: in place it scans a copy of the values
-  temp_storage copy(stream, temp_source_of(exec));
-  if (EXCLUSIVE && (const A*)out == in) {
-    copy.ensure((std::size_t)n * sizeof(A));
-    throw_on_error(thrust_amd_memcpy(copy.ptr(), in, n * sizeof(A), THRUST_AMD_D2D, stream),
-                   "exclusive_scan_by_key: copy of the values");
-    in = static_cast<const A*>(copy.ptr());
-  }
+  A* out = (A*)thrust::detail::raw(result);  // either form may write onto its values
   const seg::SbkTemp<K, A> lay(n);
   temp_storage temp(stream, temp_source_of(exec));
   temp.ensure(lay.total);

@@ -7,10 +7,11 @@
 // Same machinery as reduce_by_key: every element carries the pair (heads, value) and
 // pairs combine with (h1, v1) (+) (h2, v2) = (h1 + h2, h2 ? v2 : v1 OP v2); the scan runs
 // lane -> wave (DPP) -> workgroup (LDS) -> grid (decoupled look-back, dynamic ticket),
-// and here every element's inclusive value is written out.  The exclusive form scans
-// the input shifted one to the right with init at every segment head, exactly as the
-// reference states it (thrust/system/detail/generic/scan_by_key.inl:216-234), so
-// out[i] = init at a head and init OP v[s] OP ... OP v[i-1] elsewhere.
+// and here every element's inclusive value is written out.  The exclusive form writes
+// init at a head and init OP (running value of the segment before the element) elsewhere:
+// what the reference's scan of the right-shifted input with init at every head gives
+// (thrust/system/detail/generic/scan_by_key.inl:216-234), out[i] = init OP v[s] OP ... OP v[i-1],
+// without reading any element twice -- so that form, too, may write onto its input.
 //
 // Inside a segment the values are folded in a tree order: floating-point results agree
 // with the reference's strict left fold (the OMP back end's scan is sequential,
@@ -132,15 +133,10 @@ __global__ __launch_bounds__(SBK_BLOCK, 4) void sbk_kernel(SbkArgs<K, V, Eq, Op>
   for (int j = 0; j < CHUNKS; ++j) {
     const uint64_t first = tile_base + lane_off + j * (WAVE * VEC);
     K prev = dpp_move<0x138 /* wave_shr:1 */>(k[j].v[VEC - 1], k[j].v[VEC - 1]);
-    V prev_value = dpp_move<0x138>(v[j].v[VEC - 1], v[j].v[VEC - 1]);
     bool first_of_all = false;
     if (lane == 0) {
-      if (first == 0) {
-        first_of_all = true;
-      } else if (first < a.n) {
-        prev = a.keys[first - 1];
-        if (a.exclusive) prev_value = a.values[first - 1];
-      }
+      if (first == 0) first_of_all = true;
+      else if (first < a.n) prev = a.keys[first - 1];
     }
     uint32_t h = 0;
 #pragma unroll
@@ -150,13 +146,6 @@ __global__ __launch_bounds__(SBK_BLOCK, 4) void sbk_kernel(SbkArgs<K, V, Eq, Op>
       h |= (uint32_t)hd << i;
     }
     head[j] = h;
-    if (a.exclusive) {  // uniform
-#pragma unroll
-      for (int i = VEC - 1; i >= 0; --i) {
-        const V left = (i == 0) ? prev_value : v[j].v[i > 0 ? i - 1 : 0];
-        v[j].v[i] = ((h >> i) & 1u) ? a.init : left;
-      }
-    }
     Pair agg{h & 1u, (WV)v[j].v[0]};
 #pragma unroll
     for (int i = 1; i < VEC; ++i) agg = sop(agg, Pair{(h >> i) & 1u, (WV)v[j].v[i]});
@@ -201,8 +190,12 @@ __global__ __launch_bounds__(SBK_BLOCK, 4) void sbk_kernel(SbkArgs<K, V, Eq, Op>
     VV o;
 #pragma unroll
     for (int i = 0; i < VEC; ++i) {
-      run = sop(run, Pair{(head[j] >> i) & 1u, (WV)v[j].v[i]});
-      o.v[i] = (V)run.value;
+      const bool hd = (head[j] >> i) & 1u;
+      // exclusive form: init at a head, else init combined with the running value of the
+      // elements before this one in its segment (the element itself is folded in afterwards)
+      if (a.exclusive) o.v[i] = hd ? a.init : (V)a.op(a.init, (V)run.value);
+      run = sop(run, Pair{(uint32_t)hd, (WV)v[j].v[i]});
+      if (!a.exclusive) o.v[i] = (V)run.value;
     }
     const uint32_t e0 = lane_off + j * (WAVE * VEC);
     if (full && a.aligned) {
@@ -233,13 +226,13 @@ struct SbkTemp {
 };
 
 // Launches the init kernel and the scan into `temp` (SbkTemp<K, V>(n).total bytes); 0 < n < 2^32 - 1.
-// The exclusive form reads values[i-1] across tile borders: its output must not be its input.
+// Both forms may run in place (out == values): a tile stores only after all its loads have returned, and
+// nothing outside the tile's own elements and the tile descriptors is read.
 template <typename K, typename V, typename Eq, typename Op>
 inline int sbk_launch(char* temp, const K* keys, const V* values, V* out, uint64_t n, bool exclusive, V init, Eq eq,
                       Op op, hipStream_t stream) {
   const SbkTemp<K, V> lay(n);
   if (lay.tiles > 0xffffffffull || n >= 0xffffffffull) return (int)hipErrorInvalidValue;
-  if (exclusive && (const V*)out == values) return (int)hipErrorInvalidValue;
   constexpr size_t VALIGN = alignof(RbkValueVec<V, SbkTemp<K, V>::VEC>);
   SbkArgs<K, V, Eq, Op> a{keys,
                           values,

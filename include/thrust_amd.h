@@ -292,8 +292,7 @@ int thrust_amd_inclusive_scan_by_key(void* temp, size_t* temp_bytes, const void*
                                      int value_dtype, int op, void* stream);
 
 /* out[i] = *init at the first element of a segment, else init OP (the segment's values
- * before i).  `init` is a host pointer to one value_dtype element.  out must not alias
- * values.
+ * before i).  `init` is a host pointer to one value_dtype element.  out may alias values.
  * Replaces cuda_cub::exclusive_scan_by_key (thrust/system/cuda/detail/scan_by_key.h:885-1000;
  * generic form thrust/system/detail/generic/scan_by_key.inl:190-238). */
 int thrust_amd_exclusive_scan_by_key(void* temp, size_t* temp_bytes, const void* keys,

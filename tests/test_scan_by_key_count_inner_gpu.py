@@ -73,11 +73,15 @@ def test_inclusive_scan_by_key_in_place(dev, oracle):
     assert np.array_equal(dv.numpy(), oracle.inclusive_scan_by_key(k, v))
 
 
-def test_exclusive_scan_by_key_rejects_in_place(dev):
-    k = np.zeros(100, np.int32)
-    dk, dv = dev.DeviceArray.from_numpy(k), dev.DeviceArray.from_numpy(k.copy())
-    with pytest.raises(dev.ThrustAmdError):
-        dev.exclusive_scan_by_key(dk, dv, out=dv)
+@pytest.mark.parametrize("n", [100, (1 << 18) + 9, (1 << 22) + 5])
+def test_exclusive_scan_by_key_in_place(dev, oracle, n):
+    # the output on the values themselves, as testing/scan_by_key.cu:463-490 runs it: many tiles, whose first
+    # elements continue segments of the tile before them
+    k = _keys(n, np.int32, 8, 300)
+    v = (datagen.splitmix64(4, n) % np.uint64(1000)).astype(np.int64)
+    dk, dv = dev.DeviceArray.from_numpy(k), dev.DeviceArray.from_numpy(v)
+    dev.exclusive_scan_by_key(dk, dv, init=7, out=dv)
+    assert np.array_equal(dv.numpy(), oracle.exclusive_scan_by_key(k, v, init=7))
 
 
 def test_scan_by_key_unaligned(dev, oracle):
