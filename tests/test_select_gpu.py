@@ -143,6 +143,21 @@ def test_stable_partition_stencil(dev, oracle):
         assert cnt == rcnt and np.array_equal(d.numpy(), ref)
 
 
+@pytest.mark.parametrize("sdtype", [np.int8, np.uint16, np.int32, np.float32, np.uint64, np.float64])
+def test_stable_partition_stencil_in_place_one_pass(dev, oracle, sdtype):
+    """The in-place form tests the stencil in its own type with the items as payload (no flag array): every item width,
+    selectivities that make the sweep run from either end, sizes of many tiles with a ragged last one."""
+    for item in (np.uint8, np.int16, np.float32, np.int64):
+        for n, thr in ((70001, 10), ((1 << 21) + 77, 150), ((1 << 21) + 77, 100)):
+            x = _vals(n, item, 23)
+            st = _vals(n, sdtype, 29)
+            d, ds = dev.DeviceArray.from_numpy(x), dev.DeviceArray.from_numpy(st)
+            cnt = dev.stable_partition(d, dev.LT, thr, stencil=ds)
+            ref, rcnt = oracle.stable_partition(x, dev.LT, thr, stencil=st)
+            assert cnt == rcnt and np.array_equal(d.numpy(), ref), (sdtype, item, n, thr)
+            assert np.array_equal(ds.numpy(), st)  # the stencil is only read
+
+
 def test_config5_full_size(dev):
     """Config 5 at N=2^28 float32, t = 0.5 and 0.05: compared with numpy's boolean filter
     (the definition of an order-preserving selection)."""

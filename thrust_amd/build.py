@@ -24,7 +24,7 @@ FLAGS = [
 # Sources that take longest to compile (many template instances) go first, so that the
 # worker pool does not end on one of them.
 SLOWEST_FIRST = ["transform_scan.hip", "transform_scan_exclusive.hip", "merge_sort.hip", "scan.hip",
-                 "reduce_by_key.hip", "radix_sort.hip", "scan_by_key.hip", "transform_reduce.hip"]
+                 "reduce_by_key.hip", "radix_sort.hip", "select_stencil_in_place.hip", "scan_by_key.hip", "transform_reduce.hip"]
 
 
 def sources():

@@ -10,26 +10,6 @@
 
 namespace ta {
 
-// Stencil forms: flags[i] = stencil[i] CMP threshold as one byte each.
-template <typename T>
-__global__ __launch_bounds__(256) void select_flag_kernel(const T* __restrict__ stencil, uint64_t n,
-                                                          int cmp, T threshold,
-                                                          uint8_t* __restrict__ flags) {
-  const uint64_t stride = (uint64_t)gridDim.x * blockDim.x;
-  for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += stride)
-    flags[i] = apply_cmp(cmp, stencil[i], threshold) ? 1 : 0;
-}
-
-
-// One element per lane up to 2^28 elements: many short workgroups keep more memory requests
-// in flight than a few that loop (the loop only starts beyond that size).
-static uint32_t stride_grid(uint64_t n) {
-  uint64_t blocks = (n + 255) / 256;
-  const uint64_t cap = (uint64_t)1 << 20;
-  if (blocks < 1) blocks = 1;
-  return (uint32_t)(blocks < cap ? blocks : cap);
-}
-
 // Shared body of copy_if / partition_copy / stable_partition.
 //   in_place: out_true == in, rejected elements are parked in temp and moved back.
 static int select_by_predicate(void* temp, size_t* temp_bytes, const void* in, const void* stencil,
@@ -79,51 +59,10 @@ static int select_by_predicate(void* temp, size_t* temp_bytes, const void* in, c
   if (!in_place)
     return select_by_stencil(temp, temp_bytes, in, stencil, out_true, out_false, d_num, n, item_bytes, stencil_dtype,
                              cmp, threshold, stream);
-  // stencil form in place: byte flags first (the sweep may run from either end, and the
-  // items of a tile are parked or written over before the stencil's turn would come),
-  // then compaction of the items under those flags
-  return with_item_bytes(item_bytes, [&](auto ut) {
-    using U = typename decltype(ut)::type;
-    const size_t flag_bytes = align_up((size_t)n, 256);
-    const SelectTemp lay = select_layout<uint8_t>(n, flag_bytes + park_bytes);
-    if (!temp) {
-      *temp_bytes = lay.total;
-      return 0;
-    }
-    if (*temp_bytes < lay.total || !d_num || (n && (!in || !out_true))) return (int)hipErrorInvalidValue;
-    char* base = static_cast<char*>(temp);
-    uint8_t* flags = reinterpret_cast<uint8_t*>(base + lay.off_extra);
-    U* parked = reinterpret_cast<U*>(base + lay.off_extra + flag_bytes);
-    if (n) {
-      int rc = with_dtype(stencil_dtype, [&](auto tt) {
-        using T = typename decltype(tt)::type;
-        T thr{};
-        if (threshold) __builtin_memcpy(&thr, threshold, sizeof(T));
-        TA_LAUNCH("select_flag", stream, (select_flag_kernel<T>), dim3(stride_grid(n)), dim3(256),
-                  static_cast<const T*>(stencil), n, cmp, thr, flags);
-        TA_CHECK_LAUNCH();
-        return 0;
-      });
-      if (rc) return rc;
-    }
-    SelectArgs<uint8_t, U, ByteFlagger> a{};
-    a.tested = flags;
-    a.payload = static_cast<const U*>(in);
-    a.payload_true = static_cast<U*>(out_true);
-    a.payload_false = in_place ? parked : static_cast<U*>(out_false);
-    a.d_num_true = d_num;
-    a.n = n;
-    if (!in_place)
-      return a.payload_false ? select_launch<uint8_t, U, FLAG_BYTE, true, true>(base, lay, a, stream)
-                             : select_launch<uint8_t, U, FLAG_BYTE, true>(base, lay, a, stream);
-    int rc = select_launch<uint8_t, U, FLAG_BYTE, true, true, true>(base, lay, a, stream);
-    if (rc || n == 0) return rc;
-    TA_LAUNCH("partition_tail", stream, (partition_tail_kernel<U>), dim3(tail_grid<U>(n)), dim3(TAIL_BLOCK),
-              static_cast<U*>(out_true), (const U*)parked, n, (const uint64_t*)d_num,
-              (const uint32_t*)(reinterpret_cast<uint32_t*>(base + lay.off_ticket) + 16));
-    TA_CHECK_LAUNCH();
-    return 0;
-  });
+  // stencil form in place: the same one pass, the sweep from whichever end parks the smaller side
+  // (select_stencil_in_place.hip)
+  return partition_in_place_by_stencil(temp, temp_bytes, out_true, stencil, d_num, n, item_bytes, stencil_dtype, cmp,
+                                       threshold, stream);
 }
 
 }  // namespace ta

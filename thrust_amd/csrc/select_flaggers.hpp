@@ -47,4 +47,10 @@ int select_by_stencil(void* temp, size_t* temp_bytes, const void* in, const void
                       void* out_false, uint64_t* d_num, uint64_t n, size_t item_bytes, int stencil_dtype, int cmp,
                       const void* threshold, hipStream_t stream);
 
+// stable_partition by stencil in place, in one pass (select_stencil_in_place.hip): `data` is both the
+// items and where the selected ones end up.
+int partition_in_place_by_stencil(void* temp, size_t* temp_bytes, void* data, const void* stencil,
+                                  uint64_t* d_num, uint64_t n, size_t item_bytes, int stencil_dtype, int cmp,
+                                  const void* threshold, hipStream_t stream);
+
 }  // namespace ta
