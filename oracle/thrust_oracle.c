@@ -15,7 +15,8 @@
  *     (tests/golden/known_answers.json),
  *   - against outputs of the real reference built from its sources (oracle/_ref, both
  *     the OMP and the CPP device system) on seeded inputs (tests/golden/ fixtures and, where
- *     oracle/_ref is present, live in tests/test_oracle_vs_ref.py),
+ *     oracle/_ref is present, live in tests/test_oracle.py:
+ *     test_oracle_matches_live_reference_on_ragged_sizes),
  *   - against independent definitions (numpy cumsum mod 2^k, np.sort(kind="stable"),
  *     brute-force filters, float64 folds) in tests/test_oracle.py.
  */
