@@ -197,6 +197,13 @@ THRUST_AMD_DEVICE T wave_inclusive_scan(T v, Op op) {
   return wave_inclusive_scan(v, op, Op::template identity<T>());
 }
 
+// A 64-bit value that is the same in every lane of the wave, moved to scalar registers.
+THRUST_AMD_DEVICE uint64_t wave_uniform(uint64_t v) {
+  const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+  const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+  return ((uint64_t)hi << 32) | lo;
+}
+
 THRUST_AMD_DEVICE int lane_id() { return (int)__builtin_amdgcn_mbcnt_hi(~0u, __builtin_amdgcn_mbcnt_lo(~0u, 0u)); }
 
 // ------------------------------------------------------------------ search
@@ -277,6 +284,25 @@ THRUST_AMD_DEVICE uint64_t nearby_partition_point(uint64_t lo, uint64_t hi, uint
   return l;
 }
 
+// The element at an address of global memory that was computed as an integer (the compiler
+// cannot tell where such an address points and would use the slower generic load).  Elements
+// of the usual sizes travel as one integer of their size; E is trivially copyable.
+template <typename E>
+THRUST_AMD_DEVICE E load_global(uintptr_t address) {
+  if constexpr ((sizeof(E) == 1 || sizeof(E) == 2 || sizeof(E) == 4 || sizeof(E) == 8) && alignof(E) >= sizeof(E)) {
+    using Raw = std::conditional_t<sizeof(E) == 1, uint8_t,
+                                   std::conditional_t<sizeof(E) == 2, uint16_t,
+                                                      std::conditional_t<sizeof(E) == 4, uint32_t, uint64_t>>>;
+    typedef const Raw __attribute__((address_space(1))) * in_global_memory;
+    const Raw raw = *reinterpret_cast<in_global_memory>(address);
+    E e;
+    __builtin_memcpy(&e, &raw, sizeof(E));
+    return e;
+  } else {
+    return *reinterpret_cast<const E*>(address);
+  }
+}
+
 // ------------------------------------------------------------------ merging inside a tile
 // A tile of a merge holds two sorted parts side by side in LDS: s[0, ca) from the first range and
 // s[ca, count) from the second.  (The set operations use these; the merge and merge sort kernels
@@ -285,18 +311,39 @@ THRUST_AMD_DEVICE uint64_t nearby_partition_point(uint64_t lo, uint64_t hi, uint
 // Stages the tile: element e of the tile is pa[e] for e < ca and pb[e - ca] after that; thread t
 // loads the elements t, t + BLOCK, ...  Slots from `count` up to BLOCK * ITEMS receive a copy of
 // the tile's last element (count >= 1), so that every slot holds a value of the input.
-// One select of the base address and one 64-bit add per element.
 template <int BLOCK, int ITEMS, typename E>
 THRUST_AMD_DEVICE void stage_two_parts(const E* __restrict__ pa, const E* __restrict__ pb, uint32_t ca, uint32_t count,
                                        E* s) {
-  // (the arithmetic stays on pointers so that the loads are known to go to global memory)
-  const E* const base_b = pb - ca;  // only indexed from ca on
   E in[ITEMS];
+  if (count == (uint32_t)BLOCK * ITEMS) {
+    // A full tile.  The 64 elements a wave loads per step are consecutive, so all but at most one
+    // of its steps lie inside one part: there the address is a base that is the same for the
+    // whole wave (scalar arithmetic) plus the lane's offset, and nothing is computed per lane.
+    // The caller's arguments are the same in every lane; saying so keeps them in scalar registers.
+    const uint32_t lane = threadIdx.x % WAVE;
+    const uint32_t first = (uint32_t)__builtin_amdgcn_readfirstlane((int)(threadIdx.x - lane));
+    const uint32_t ca_u = (uint32_t)__builtin_amdgcn_readfirstlane((int)ca);
+    const uintptr_t base_a = wave_uniform(reinterpret_cast<uintptr_t>(pa)) + (uintptr_t)first * sizeof(E);
+    const uintptr_t base_b = wave_uniform(reinterpret_cast<uintptr_t>(pb)) +
+                             (uintptr_t)(((intptr_t)first - (intptr_t)ca_u) * (intptr_t)sizeof(E));
+    const uint32_t off = lane * (uint32_t)sizeof(E);
 #pragma unroll
-  for (int q = 0; q < ITEMS; ++q) {
-    uint32_t e = (uint32_t)q * BLOCK + threadIdx.x;
-    e = e < count ? e : count - 1;
-    in[q] = (e < ca ? pa : base_b)[e];
+    for (int q = 0; q < ITEMS; ++q) {
+      const int32_t lanes_of_a = (int32_t)ca_u - (int32_t)((uint32_t)q * BLOCK + first);
+      const uintptr_t step = (uintptr_t)q * BLOCK * sizeof(E);
+      if (lanes_of_a >= WAVE) in[q] = load_global<E>(base_a + step + off);
+      else if (lanes_of_a <= 0) in[q] = load_global<E>(base_b + step + off);
+      else in[q] = load_global<E>(((int32_t)lane < lanes_of_a ? base_a : base_b) + step + off);
+    }
+  } else {
+    // (the arithmetic stays on pointers so that the loads are known to go to global memory)
+    const E* const base_b = pb - ca;  // only indexed from ca on
+#pragma unroll
+    for (int q = 0; q < ITEMS; ++q) {
+      uint32_t e = (uint32_t)q * BLOCK + threadIdx.x;
+      e = e < count ? e : count - 1;
+      in[q] = (e < ca ? pa : base_b)[e];
+    }
   }
 #pragma unroll
   for (int q = 0; q < ITEMS; ++q) s[(uint32_t)q * BLOCK + threadIdx.x] = in[q];

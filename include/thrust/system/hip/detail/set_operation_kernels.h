@@ -13,7 +13,13 @@
 //   union                 every A_r     and B_r with r >= m
 // so an element is decided by its rank r inside its own part of the run and by the size
 // of the other part.  Both follow from three positions per run on the merge path: where
-// the run starts, where its B part starts and where it ends.
+// the run starts, where its B part starts and where it ends.  An element of the part that
+// comes second in the run has everything it needs before it on the path; an element of the
+// first part needs to know how many elements of the second part follow.  Difference and
+// intersection only ever keep elements of A, so for them the two ranges change places (ties
+// go to B, a run is B_0 .. B_{n-1} A_0 .. A_{m-1}) and nothing has to look ahead; only the
+// symmetric difference decides elements of both parts and pays for the look ahead.  Below,
+// "A" and "B" name the ranges in the order the kernels receive them.
 //
 //   partition  one thread per tile boundary: the merge-path split, and the three
 //              positions (searched outward from the split) of the run that
@@ -25,8 +31,9 @@
 //              key is the later of the two elements before its merge-path split); the last run
 //              start and B-part start before every lane, and the next ones after it, travel
 //              as pairs of 16-bit positions through one forward and one backward max-scan
-//              behind a single barrier; each lane then walks its 16 elements once per side
-//              that the operation can keep (A: rank against the B elements that follow in
+//              behind a single barrier (the backward one only for the symmetric difference);
+//              each lane then walks its 16 elements once per side that the operation
+//              decides (A: rank against the B elements that follow in
 //              the run; B: position against a threshold fixed where the B part starts), in
 //              lane-relative positions, collecting the outcomes as sign bits; keep flags ->
 //              ranks -> decoupled look-back over the tiles' counts (dynamic tickets) ->
@@ -146,30 +153,35 @@ THRUST_AMD_DEVICE V set_block_exclusive(V v, Op op, V id, V* buf, V* total) {
 }
 
 // Two scans of position pairs behind one barrier: `before` = the fold of `fwd` over the
-// threads before this one, `after` = the fold of `bwd` over the threads after it, `all` =
-// the fold of `fwd` over the workgroup.  0 is the identity.
+// threads before this one, `after` = the fold of `bwd` over the threads after it (0 unless
+// `backward`, which is the same for the whole workgroup), `all` = the fold of `fwd` over the
+// workgroup.  0 is the identity.
 template <int WAVES>
-THRUST_AMD_DEVICE void set_block_both_ways(uint32_t fwd, uint32_t bwd, uint32_t* buf_fwd, uint32_t* buf_bwd,
-                                           uint32_t& before, uint32_t& after, uint32_t& all) {
+THRUST_AMD_DEVICE void set_block_both_ways(uint32_t fwd, uint32_t bwd, bool backward, uint32_t* buf_fwd,
+                                           uint32_t* buf_bwd, uint32_t& before, uint32_t& after, uint32_t& all) {
   const int wave = threadIdx.x / WAVE, lane = threadIdx.x % WAVE;
   const OpMaxPair16 op;
   const int mirror = (WAVE - 1 - lane) * 4;
   const uint32_t incl_f = wave_inclusive_scan(fwd, op, 0u);
-  const uint32_t incl_b = wave_inclusive_scan((uint32_t)__builtin_amdgcn_ds_bpermute(mirror, (int)bwd), op, 0u);
-  if (lane == WAVE - 1) {
-    buf_fwd[wave] = incl_f;
-    buf_bwd[wave] = incl_b;
-  }
+  if (lane == WAVE - 1) buf_fwd[wave] = incl_f;
   const uint32_t excl_f = dpp_move<0x138 /* wave_shr:1 */>(0u, incl_f);
-  const uint32_t excl_b =
-      (uint32_t)__builtin_amdgcn_ds_bpermute(mirror, (int)dpp_move<0x138 /* wave_shr:1 */>(0u, incl_b));
+  uint32_t excl_b = 0;
+  if (backward) {
+    const uint32_t incl_b = wave_inclusive_scan((uint32_t)__builtin_amdgcn_ds_bpermute(mirror, (int)bwd), op, 0u);
+    if (lane == WAVE - 1) buf_bwd[wave] = incl_b;
+    excl_b = (uint32_t)__builtin_amdgcn_ds_bpermute(mirror, (int)dpp_move<0x138 /* wave_shr:1 */>(0u, incl_b));
+  }
   __syncthreads();
   uint32_t prefix = 0, total = 0, suffix = 0;
 #pragma unroll
   for (int w = 0; w < WAVES; ++w) {
     if (w == wave) prefix = total;
     total = op(total, buf_fwd[w]);
-    if (w > wave) suffix = op(suffix, buf_bwd[w]);
+  }
+  if (backward) {
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w)
+      if (w > wave) suffix = op(suffix, buf_bwd[w]);
   }
   before = op(prefix, excl_f);
   after = op(suffix, excl_b);
@@ -259,6 +271,12 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
     first_b_before = rm < d0;
   }
 
+  // Only the symmetric difference decides elements of the first range (their rank against the
+  // elements of the second range, which follow them in the run); elements of the second range
+  // are decided by every operation, against what came before them.
+  const bool need_a = g.op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE;
+  constexpr bool need_b = true;
+
   // ---- stage the keys: A's part first, then B's
   stage_two_parts<SET_BLOCK, SET_ITEMS>(g.a + a0, g.b + b0, ca, count, s_keys);
   __syncthreads();
@@ -291,7 +309,7 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
   // B elements of the tile's last run that lie in later tiles (the last merged key is the later
   // of the two parts' last keys; only its equivalence class matters)
   uint32_t tail_b = 0;
-  if (f1_valid) {
+  if (need_a && f1_valid) {
     const T last_a = s_keys[ca ? ca - 1 : 0], last_b = s_keys[count - 1];
     const T last = (cb == 0) ? last_a : (ca == 0) ? last_b : (comp(last_b, last_a) ? last_a : last_b);
     const T f1_key = g.key[tile + 1];
@@ -326,15 +344,13 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
     const uint32_t last_e2 = e2 ? run0 + (31 - __builtin_clz(e2)) + 1 : 0u;
     const uint32_t first_h = head ? SET_TILE - (run0 + __builtin_ctz(head)) : 0u;
     const uint32_t first_e2 = e2 ? SET_TILE - (run0 + __builtin_ctz(e2)) : 0u;
-    set_block_both_ways<SET_WAVES>((last_h << 16) | last_e2, (first_h << 16) | first_e2, s_fwd, s_bwd, fwd_in, bwd_in,
-                                   fwd_all);
+    set_block_both_ways<SET_WAVES>((last_h << 16) | last_e2, (first_h << 16) | first_e2, need_a, s_fwd, s_bwd, fwd_in,
+                                   bwd_in, fwd_all);
   }
 
   // ---- decide every element: lt_a / lt_b, bit o = element o (of A / of B) has a rank inside
   // its own part of the run that is below the size of the other part.  Positions are
   // relative to the lane's first element from here on, and signed.
-  const bool need_a = g.op != THRUST_AMD_SET_UNION;  // union keeps every element of A
-  const bool need_b = g.op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE || g.op == THRUST_AMD_SET_UNION;
   uint32_t lt_a = 0, lt_b = 0;
   if ((fwd_all >> 16) == 0) {
     // no run starts inside the tile: the first run covers it, and the thresholds decide
@@ -390,10 +406,11 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
       lt_a = __builtin_bitreverse32(acc) >> 16;
     }
   }
-  // difference: A at or above; intersection: A below; symmetric difference: A and B at or
-  // above; union: all of A, B at or above
-  const uint32_t keep_a = g.op == THRUST_AMD_SET_INTERSECTION ? lt_a : (need_a ? ~lt_a : ~0u);
-  const uint32_t keep_b = need_b ? ~lt_b : 0u;
+  // union: all of the first range, of the second those at or above; symmetric difference: of both
+  // those at or above; difference and intersection (whose first range is the caller's second):
+  // nothing of the first range, of the second those at or above / those below
+  const uint32_t keep_a = g.op == THRUST_AMD_SET_UNION ? ~0u : (need_a ? ~lt_a : 0u);
+  const uint32_t keep_b = g.op == THRUST_AMD_SET_INTERSECTION ? lt_b : ~lt_b;
   const uint32_t keep = ((~is_b & keep_a) | (is_b & keep_b)) & live;
 
   // ---- ranks inside the tile, then the tile's place in the output
@@ -451,9 +468,23 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
     // values: the two sub-ranges are staged like the keys were (A's part, then B's, so a
     // key's staging slot is its value's), then gathered by slot in output order
     __syncthreads();  // the compacted keys have been read
-    // (B's values are only read by the operations that can keep an element of B)
-    if (need_b) stage_two_parts<SET_BLOCK, SET_ITEMS>(g.va + a0, g.vb + b0, ca, count, s_vals);
-    else if (ca) stage_two_parts<SET_BLOCK, SET_ITEMS>(g.va + a0, g.va + a0, ca, ca, s_vals);
+    // (the first range's values are only read by the operations that can keep one of its elements)
+    if (g.op == THRUST_AMD_SET_UNION || g.op == THRUST_AMD_SET_SYMMETRIC_DIFFERENCE) {
+      stage_two_parts<SET_BLOCK, SET_ITEMS>(g.va + a0, g.vb + b0, ca, count, s_vals);
+    } else {
+      const V* const second = g.vb + b0;
+      V in[SET_ITEMS];
+#pragma unroll
+      for (int q = 0; q < SET_ITEMS; ++q) {
+        const uint32_t e = (uint32_t)q * SET_BLOCK + threadIdx.x;
+        if (e >= ca && e < count) in[q] = second[e - ca];
+      }
+#pragma unroll
+      for (int q = 0; q < SET_ITEMS; ++q) {
+        const uint32_t e = (uint32_t)q * SET_BLOCK + threadIdx.x;
+        if (e >= ca && e < count) s_vals[e] = in[q];
+      }
+    }
     __syncthreads();
     V* dst = g.vout + base;
 #pragma unroll
@@ -488,6 +519,21 @@ template <typename T, typename V, bool HAS_VALUES, typename Comp>
 inline int set_launch(char* temp, int op, const T* a, uint64_t na, const T* b, uint64_t nb, const V* va, const V* vb,
                       T* out, V* vout, uint64_t* d_num, Comp comp, hipStream_t stream) {
   using Shape = SetShape<T, V, HAS_VALUES>;
+  // Difference and intersection keep elements of A only, each decided by its rank against the
+  // number of equivalent elements of B.  The kernel decides the elements of its second range
+  // from what precedes them on the merge path, so for these two the ranges change places: ties
+  // then go to B, and an element of A has all of its run's elements of B before it.
+  if (op == THRUST_AMD_SET_DIFFERENCE || op == THRUST_AMD_SET_INTERSECTION) {
+    const T* const ta = a;
+    a = b;
+    b = ta;
+    const V* const tv = va;
+    va = vb;
+    vb = tv;
+    const uint64_t tn = na;
+    na = nb;
+    nb = tn;
+  }
   const uint64_t total = na + nb;
   const SetTemp<T, V, HAS_VALUES> lay(total);
   const uint64_t tiles = lay.tiles;
