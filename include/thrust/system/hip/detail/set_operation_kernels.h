@@ -363,7 +363,19 @@ __global__ __launch_bounds__((SetShape<T, V, HAS_VALUES>::BLOCK), (SetShape<T, V
   } else {
     const uint32_t h_in = fwd_in >> 16, e_in = fwd_in & 0xffffu;
     const int32_t start = h_in ? (int32_t)h_in - 1 - (int32_t)run0 : first_start - (int32_t)run0;
-    if (need_b) {
+    // Most elements of B need no positions: one that starts a run faces no element of A and is
+    // not below; one that follows an element of A in its run has rank 0 and is below; one that
+    // follows an element of B that is not below is not below either.  Only an element of B after
+    // an element of B that may be below (one that does not start the run) has to count, and a wave
+    // without such an element decides with three bit operations.  (The element before a wave's
+    // first one counts as one that may be below.)
+    const uint32_t head_all = head | (uint32_t)(threadIdx.x == 0 && first_start == 0);  // the tile's first element too
+    const uint32_t head_before =
+        (head_all << 1) | (lane == 0 ? 0u : dpp_move<0x138 /* wave_shr:1 */>(0u, (head_all >> (SET_ITEMS - 1)) & 1u));
+    const uint32_t counts = is_b & ~head_all & prev_b_bits & ~head_before & live;
+    if (__builtin_amdgcn_ballot_w64(counts != 0) == 0) {
+      lt_b = is_b & ~head_all & ~prev_b_bits;
+    } else {
       // an element of B at position p, in a run that starts at s and whose B part starts at m,
       // has rank p - m and faces m - s elements of A: below exactly when p < 2m - s
       int32_t s = start;

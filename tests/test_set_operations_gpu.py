@@ -152,6 +152,29 @@ def test_set_operation_by_key_other_key_widths_and_descending(dev, oracle, op, k
         assert cnt == rk.size and np.array_equal(ko.numpy()[:cnt], rk) and np.array_equal(vo.numpy()[:cnt], rv), (op, kdtype, na, nb)
 
 
+@pytest.mark.parametrize("op", OPS)
+def test_set_operation_mostly_distinct_keys_with_a_few_repeated(dev, oracle, op):
+    """Ranges that are sets but for a few hundred keys with multiplicities 0..3 on either side:
+    nearly every wave decides its elements without counting, the planted keys land anywhere
+    (inside lanes, across lanes, waves and tiles) and must be counted."""
+    for seed in (91, 92, 93):
+        pool = np.unique(datagen.splitmix64(seed, 300000) >> np.uint64(33)).astype(np.uint32)
+        side = datagen.splitmix64(seed + 10, pool.size) % np.uint64(4)  # 0: A only, 1: B only, 2 and 3: both
+        ma = (side != 1).astype(np.int64)
+        mb = (side != 0).astype(np.int64)
+        planted = (datagen.splitmix64(seed + 20, 400) % np.uint64(pool.size)).astype(np.int64)
+        ma[planted] = (datagen.splitmix64(seed + 30, 400) % np.uint64(4)).astype(np.int64)
+        mb[planted] = (datagen.splitmix64(seed + 40, 400) % np.uint64(4)).astype(np.int64)
+        a, b = np.repeat(pool, ma), np.repeat(pool, mb)
+        va, vb = _origin_values(a.size, b.size)
+        ko, vo, cnt = dev.set_operation_by_key(op, dev.DeviceArray.from_numpy(a), dev.DeviceArray.from_numpy(b),
+                                               dev.DeviceArray.from_numpy(va), dev.DeviceArray.from_numpy(vb))
+        rk, rv = oracle.set_operation_by_key(op, a, b, va, vb)
+        assert cnt == rk.size and np.array_equal(ko.numpy()[:cnt], rk) and np.array_equal(vo.numpy()[:cnt], rv), (op, seed)
+        out, cnt = dev.set_operation(op, dev.DeviceArray.from_numpy(a), dev.DeviceArray.from_numpy(b))
+        assert cnt == rk.size and np.array_equal(out.numpy()[:cnt], rk), (op, seed)
+
+
 def test_set_operation_signed_zero_keeps_the_copy_of_the_named_side(dev, oracle):
     """-0.0 and +0.0 are equivalent keys with different bits: the kept copy is the one the
     reference's loop emits."""
