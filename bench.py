@@ -140,6 +140,9 @@ class C1:
         # calls of 0.2 - 0.4 ms: at least 50 back to back, so that the one synchronisation at the end
         # of the timed region does not weigh on the figure
         reps = max(steps, 50)
+        # and at least 20 untimed calls first (a few ms of work): three calls of 0.2 ms end before the
+        # device has left its idle clocks
+        warmup = max(warmup, 20)
         capi = self.capi
         ms_reduce = time_region(self.torch, lambda i, w: capi.reduce(self.d, temp=self.t_r, out=self.out1), reps, warmup)
         ms_scan = time_region(self.torch, lambda i, w: capi.inclusive_scan(self.d, out=self.outn, temp=self.t_s), reps, warmup)
