@@ -260,7 +260,8 @@ int thrust_amd_inclusive_scan(void* temp, size_t* temp_bytes, const void* in, vo
  * stream first waits (on the device) for an event recorded behind the previous call on that GPU,
  * whatever stream or host thread made it.  A stream under capture is left out of that ordering:
  * replays of a graph that holds this call must not overlap other calls of it on the same GPU.
- * The first call on a GPU also looks up the array's address and creates that event. */
+ * The first call on a GPU also looks up the array's address and creates that event (under the
+ * relaxed capture mode, should the calling thread be capturing). */
 int thrust_amd_inclusive_scan_static(const void* in, void* out, uint64_t n, int dtype, int op,
                                      void* stream);
 

@@ -88,8 +88,15 @@ TA_EXPORT int thrust_amd_inclusive_scan_static(const void* in, void* out, uint64
   if (device < 0 || device >= SCAN_STATIC_MAX_DEVICES) return (int)hipErrorInvalidDevice;
   ScanStaticDevice& dev = g_scan_static[device];
   std::lock_guard<std::mutex> guard(dev.lock);
-  const int rs = scan_static_setup(dev);
-  if (rs) return rs;
+  if (!dev.scratch) {
+    // The set-up calls are not stream work.  Should this first call come from a thread that is
+    // capturing a stream, they run under the relaxed capture mode, which allows them there.
+    hipStreamCaptureMode mode = hipStreamCaptureModeRelaxed;
+    const bool exchanged = hipThreadExchangeStreamCaptureMode(&mode) == hipSuccess;
+    const int rs = scan_static_setup(dev);
+    if (exchanged) (void)hipThreadExchangeStreamCaptureMode(&mode);
+    if (rs) return rs;
+  }
   hipStream_t s = (hipStream_t)stream;
   hipStreamCaptureStatus capture = hipStreamCaptureStatusNone;
   if (hipStreamIsCapturing(s, &capture) != hipSuccess) capture = hipStreamCaptureStatusNone;
