@@ -144,15 +144,6 @@ class C1:
         # idle clocks
         warmup = max(warmup, 20)
         capi = self.capi
-        # The pass in front of the sort is the first memory-bound work of the process.  On some boxes the
-        # reduce read 3.5 % slower there than after the sort even behind 20 untimed calls (0.1836 against
-        # 0.1777 ms): the memory clocks follow the load over tens of milliseconds.  So the device first
-        # streams for about 60 ms (untimed scans of the same buffers), as it has when the second pass runs.
-        t_end = time.perf_counter() + 0.06
-        while time.perf_counter() < t_end:
-            for _ in range(20):
-                capi.inclusive_scan(self.d, out=self.outn, temp=self.t_s)
-            self.torch.cuda.synchronize()
         ms_reduce = time_region(self.torch, lambda i, w: capi.reduce(self.d, temp=self.t_r, out=self.out1), reps, warmup)
         ms_scan = time_region(self.torch, lambda i, w: capi.inclusive_scan(self.d, out=self.outn, temp=self.t_s), reps, warmup)
         # a plain device copy of the same 1 GiB into the same output (torch's copy kernel): what moving the
