@@ -141,3 +141,12 @@ def test_bandwidth_ceiling_kernels_run():
     # (profiles/copy_ceiling.txt holds their rocprofv3 durations); here only that they run and give sane rates
     out = _run("bandwidth_ceiling")
     assert "PASSED" in out and "best copy" in out
+
+
+def test_pass_pattern_ceiling_kernels_run():
+    # the memory accesses of one radix-sort pass and nothing else (tiles read in order, written as 256 runs): the
+    # ceiling the sort pass can be read against (profiles/scatter_ceiling.txt holds the rocprofv3 durations); every
+    # variant is checked to be a permutation of its input
+    out = _run("scatter_ceiling")
+    assert "PASSED" in out and "NOT A PERMUTATION" not in out and "256 runs of 72 keys" in out
+
