@@ -73,7 +73,44 @@ struct SortCtl {
   uint32_t skip[MAX_PASSES];     // pass moves nothing
   uint32_t src_alt[MAX_PASSES];  // pass reads the alternate buffer
   uint32_t final_in_alt;         // result sits in the alternate buffer after the last pass
+  uint32_t gave_up;              // a tile stopped waiting for its predecessors (see LOOKBACK_SPIN_LIMIT)
 };
+
+// ------------------------------------------------------------------ which tile a workgroup takes
+// The digit runs of tile t + 1 continue those of tile t in memory, and the cache line in which
+// one ends and the other begins is written in part by both.  When both tiles run on the same
+// XCD the two parts meet in that XCD's L2 and leave as one line; otherwise each costs a
+// partial-line write to memory -- for 288-byte runs a third of a pass (a kernel with nothing
+// but a pass's memory accesses: 0.60 ms, 0.54 ms with neighbouring tiles on one XCD).
+// Workgroups go to the XCDs in turn (workgroup i to XCD i % 8), so the workgroups of class
+// k = i % 8 draw their tickets from a counter of their own and ticket c of class k stands for
+// tile class_tile(k, c): 8 consecutive tiles, then the 8 tiles 64 further on, ...; the tiles
+// past the last whole group of 64 are dealt to the classes in order, each as many as it has
+// workgroups left.  With exactly `tiles` workgroups every tile is taken exactly once whatever
+// the hardware does; inside a class tiles are taken in rising order.
+constexpr uint32_t TILES_PER_GROUP = 8;
+constexpr uint32_t TICKET_CLASSES = 8;
+constexpr uint32_t TICKET_STRIDE = 32;  // words between the counters of two classes: a cache line each
+constexpr uint32_t TICKET_WORDS = MAX_PASSES * TICKET_CLASSES * TICKET_STRIDE;
+
+__host__ __device__ inline uint32_t class_tile(uint32_t k, uint32_t c, uint32_t tiles) {
+  constexpr uint32_t G = TILES_PER_GROUP, S = TICKET_CLASSES * G;
+  const uint32_t whole = tiles / S;  // groups of 64 tiles that are complete
+  if (c < whole * G) return ((c / G) * TICKET_CLASSES + k) * G + c % G;
+  // class k has tiles / 8 workgroups, one more if k < tiles % 8; `rest` of them are past the whole groups
+  const uint32_t rest = tiles / TICKET_CLASSES - whole * G, extra = tiles % TICKET_CLASSES;
+  const uint32_t before = k * rest + (k < extra ? k : extra);  // tail tiles of the classes before k
+  return whole * S + before + (c - whole * G);
+}
+
+// A tile waits for its predecessors' counts in a loop.  Every predecessor is taken by a running
+// workgroup as long as every class keeps receiving its workgroups while slots are free -- which
+// holds when workgroups are bound to XCDs in turn, and when they are dispatched in order to at
+// least 64 slots.  Should neither hold, a tile that has polled this often stops waiting: it
+// uses what it has summed so far (its positions stay inside the array: a prefix can only be too
+// small), sets SortCtl::gave_up, and every tile that sees the flag does the same, so the
+// kernel ends -- with keys out of order -- instead of hanging.
+constexpr uint32_t LOOKBACK_SPIN_LIMIT = 1u << 21;
 
 struct SortGeometry {
   int passes;
@@ -244,7 +281,10 @@ __global__ __launch_bounds__(RADIX_SIZE) void sort_scan_kernel(uint32_t* __restr
     parity ^= (skip ? 0u : 1u);
     __syncthreads();
   }
-  if (d == 0) ctl->final_in_alt = parity;
+  if (d == 0) {
+    ctl->final_in_alt = parity;
+    ctl->gave_up = 0;
+  }
 }
 
 // ------------------------------------------------------------------ onesweep pass
@@ -273,7 +313,9 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
     uint32_t n, int pass, SortGeometry geo, KeyCodec<K> codec,
     const uint32_t* __restrict__ bin_base,  // [RADIX_SIZE] global digit offsets of this pass
     D* __restrict__ status,                 // [tiles][RADIX_SIZE]
-    uint32_t* __restrict__ ticket, const SortCtl* __restrict__ ctl) {
+    uint32_t* __restrict__ ticket,          // [TICKET_CLASSES] counters of this pass, TICKET_STRIDE words apart
+    const SortCtl* __restrict__ ctl,
+    uint32_t* __restrict__ gave_up) {       // &SortCtl::gave_up, the one field the passes write
   using Shape = PassShape<K, V, HAS_VALUES, BLOCK, ITEMS>;
   using Desc = Descriptor<D>;
   constexpr int WAVES = Shape::WAVES;
@@ -296,7 +338,8 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
   V* s_vals = reinterpret_cast<V*>(s_union);
 
   if (threadIdx.x == 0) {
-    s_tile = atomicAdd(ticket, 1u);
+    const uint32_t k = blockIdx.x % TICKET_CLASSES;
+    s_tile = class_tile(k, atomicAdd(ticket + k * TICKET_STRIDE, 1u), gridDim.x);
   }
   for (int i = threadIdx.x; i < WAVES * RADIX_SIZE; i += BLOCK) s_cnt[i] = 0;
   __syncthreads();
@@ -479,6 +522,7 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
       uint32_t acc = 0;
       int t = (int)tile - 1;  // tile counts stay below 2^20
       const D* my_col = status + d;
+      uint32_t spins = 0;
       for (;;) {
         D s[LOOKBACK_WINDOW];
 #pragma unroll
@@ -502,7 +546,16 @@ __global__ __launch_bounds__(BLOCK) void onesweep_pass_kernel(
         }
         if (done) break;
         t -= used;
-        if (used < LOOKBACK_WINDOW) __builtin_amdgcn_s_sleep(1);
+        if (used < LOOKBACK_WINDOW) {
+          __builtin_amdgcn_s_sleep(1);
+          ++spins;
+          if (spins >= LOOKBACK_SPIN_LIMIT ||
+              (spins % 1024u == 0 &&
+               __hip_atomic_load(gave_up, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+            __hip_atomic_store(gave_up, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            break;
+          }
+        }
       }
       excl = acc;
     }
@@ -624,7 +677,7 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
   const bool wide = n > SORT_MAX_N_NARROW;  // prefixes need more than 30 bits: 64-bit descriptors
   // every key and value within 4 GiB of its array's start: 32-bit byte offsets
   const bool off32 = !wide && n * (uint64_t)((HAS_VALUES && sizeof(V) > sizeof(K)) ? sizeof(V) : sizeof(K)) <= (1ull << 32);
-  const size_t zero_words = (size_t)MAX_PASSES + (size_t)MAX_PASSES * RADIX_SIZE +
+  const size_t zero_words = (size_t)TICKET_WORDS + (size_t)MAX_PASSES * RADIX_SIZE +
                             (size_t)geo.passes * tiles * RADIX_SIZE * (wide ? 2 : 1);
   const size_t off_zero = lay.add(zero_words * sizeof(uint32_t));
   const size_t off_keys = lay.add((size_t)n * sizeof(K));
@@ -641,7 +694,7 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
   SortCtl* ctl = reinterpret_cast<SortCtl*>(base + off_ctl);
   uint32_t* zero = reinterpret_cast<uint32_t*>(base + off_zero);
   uint32_t* tickets = zero;
-  uint32_t* hist = zero + MAX_PASSES;
+  uint32_t* hist = zero + TICKET_WORDS;
   uint32_t* status = hist + MAX_PASSES * RADIX_SIZE;
   K* keys_a = static_cast<K*>(keys);
   K* keys_b = reinterpret_cast<K*>(base + off_keys);
@@ -667,11 +720,11 @@ static int sort_impl(void* temp, size_t* temp_bytes, void* keys, void* values, u
   for (int p = 0; p < geo.passes; ++p) {
     const size_t status_off = (size_t)p * tiles * RADIX_SIZE;  // in descriptor words
     if (off32) {
-      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint32_t, true>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + status_off, tickets + p, (const SortCtl*)ctl);
+      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint32_t, true>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + status_off, tickets + (size_t)p * TICKET_CLASSES * TICKET_STRIDE, (const SortCtl*)ctl, &ctl->gave_up);
     } else if (wide) {
-      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint64_t, false>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, reinterpret_cast<uint64_t*>(status) + status_off, tickets + p, (const SortCtl*)ctl);
+      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint64_t, false>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, reinterpret_cast<uint64_t*>(status) + status_off, tickets + (size_t)p * TICKET_CLASSES * TICKET_STRIDE, (const SortCtl*)ctl, &ctl->gave_up);
     } else {
-      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint32_t, false>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + status_off, tickets + p, (const SortCtl*)ctl);
+      TA_LAUNCH("onesweep_pass", stream, (onesweep_pass_kernel<K, V, HAS_VALUES, Plan::BLOCK, Plan::ITEMS, uint32_t, false>), dim3((uint32_t)tiles), dim3(Plan::BLOCK), keys_a, keys_b, vals_a, vals_b, (uint32_t)n, p, geo, codec, hist + p * RADIX_SIZE, status + status_off, tickets + (size_t)p * TICKET_CLASSES * TICKET_STRIDE, (const SortCtl*)ctl, &ctl->gave_up);
     }
     TA_CHECK_LAUNCH();
   }
