@@ -68,3 +68,16 @@ def test_size_queries_and_argument_errors_need_no_gpu(lib):
     assert lib.thrust_amd_sort_keys(None, ctypes.byref(n), None, 1 << 32, 5, 0, 0, 32, None) != 0  # n too large
     assert lib.thrust_amd_copy_if(None, ctypes.byref(n), None, None, None, None, 10, 3, 8, 0, None, None) != 0  # item size
     assert lib.thrust_amd_reduce(None, None, None, 10, 4, 0, None, None, None) != 0                # no size slot
+
+
+def test_sort_pass_tickets_take_every_tile_once_and_never_get_stuck():
+    """tests/cpp/test_sort_tickets.cpp compiles the rule by which the workgroups of a radix-sort pass take
+    their tiles (thrust_amd/csrc/sort_tickets.hpp, the function the kernel calls) for the host: every tile
+    exactly once for every tile count, and no schedule of two dispatcher models leaves a pass stuck."""
+    import subprocess
+    cpp = os.path.join(ROOT, "tests", "cpp")
+    prog = os.path.join(cpp, "bin", "test_sort_tickets")
+    subprocess.run(["make", "-C", cpp, prog], check=True, capture_output=True)
+    res = subprocess.run([prog], capture_output=True, text=True, timeout=120)
+    assert res.returncode == 0 and "PASSED" in res.stdout, res.stdout + res.stderr
+
