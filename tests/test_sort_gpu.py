@@ -214,3 +214,32 @@ def test_sort_beyond_2p30_keys_properties(dev):
     same = ko[1:] == ko[:-1]
     assert bool((vo[1:][same] > vo[:-1][same]).all().item())  # ascending inside every key: stable
     assert bool((keys[vo.to(torch.int64)] == ko).all().item())  # every value still carries its key
+
+
+def test_sorts_in_flight_on_several_streams(dev):
+    """Twelve sorts issued on four streams without any synchronisation in between share the device:
+    the passes of different calls run side by side, each with a part of the workgroup slots, and each
+    call's tiles still find their predecessors (the ticket rule of the passes must not depend on a
+    call having the device to itself)."""
+    import torch
+    sizes = [(1 << 22) + 5, (1 << 21) + 12345, 3000017]
+    streams = [torch.cuda.Stream() for _ in range(4)]
+    jobs = []
+    for si, st in enumerate(streams):
+        for ni, n in enumerate(sizes):
+            k = _keys(n, np.uint32, 100 + 10 * si + ni)
+            v = np.arange(n, dtype=np.uint32)
+            jobs.append((st, k, dev.DeviceArray.from_numpy(k), dev.DeviceArray.from_numpy(v), dev.Temp()))
+    for st, k, dk, dv, t in jobs:  # sizes the temporary storage of every job: no allocation in the timed part
+        with torch.cuda.stream(st):
+            dev.sort_pairs(dev.DeviceArray.from_numpy(k), dev.DeviceArray.from_numpy(np.arange(k.size, dtype=np.uint32)), temp=t)
+    torch.cuda.synchronize()
+    for st, k, dk, dv, t in jobs:
+        with torch.cuda.stream(st):
+            dev.sort_pairs(dk, dv, temp=t)
+    torch.cuda.synchronize()
+    for st, k, dk, dv, t in jobs:
+        order = np.argsort(k, kind="stable")
+        assert np.array_equal(dk.numpy(), k[order])
+        assert np.array_equal(dv.numpy(), order.astype(np.uint32))
+
